@@ -1,0 +1,120 @@
+/* C ABI of libmxq_gfx950.so -- MI355X (gfx950) kernels for microxcaling's MX / bfloat quantization.
+ *
+ * The library replaces the native extension the reference builds at import time
+ * (mx/custom_extensions.py:11-19 -> mx/cpp/funcs.cpp:234-242).  Each entry point below names the
+ * reference function it stands in for.  Differences from the reference's pybind surface, all of
+ * which keep torch types out of the signatures:
+ *   - tensors are raw device pointers plus a dtype code; shapes arrive collapsed to
+ *     (pre, axis, post) as 64-bit counts, the way mx/cpp/mx.cu:29-46 collapses them;
+ *   - the caller allocates the output (the reference returns empty_like(input));
+ *   - every launch goes to the HIP stream the caller passes (the reference uses the legacy
+ *     default stream, mx/cpp/mx.cu:57);
+ *   - failures return a non-zero status and leave a message for mxq_last_error(); the reference
+ *     prints and calls exit() (mx/cpp/common.cuh:247-255).
+ * Entry points never allocate, never synchronise and keep no state between calls.
+ *
+ * Numerics: results are bit-identical to the reference's pure-PyTorch CPU path
+ * (custom_cuda=False) for fp32 and bf16 tensors, including its floor(log2(x)) rounding just
+ * below powers of two; MXQ_FLAG_EXACT_EXPONENT switches to bit-field exponents, which is what the
+ * reference's own CUDA kernels compute (mx/cpp/common.cuh:146-154).  fp16 tensors are widened to
+ * fp32, quantized, and rounded back to fp16 like the reference's CUDA kernels do
+ * (mx/cpp/mx.cuh:72,88).
+ */
+#ifndef MXQ_H
+#define MXQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype codes */
+#define MXQ_DTYPE_F32 0
+#define MXQ_DTYPE_F16 1
+#define MXQ_DTYPE_BF16 2
+
+/* rounding modes = int(RoundingMode), mx/formats.py:12-19 */
+#define MXQ_ROUND_NEAREST 0 /* half away from zero */
+#define MXQ_ROUND_FLOOR 1   /* toward zero */
+#define MXQ_ROUND_EVEN 2    /* half to even */
+
+/* flags */
+#define MXQ_FLAG_EXACT_EXPONENT 1 /* bit-field exponents instead of torch's floor(log2(x)) */
+
+/* status codes */
+#define MXQ_OK 0
+#define MXQ_ERR_ARGUMENT 1 /* bad dtype / sizes / parameters; nothing was launched */
+#define MXQ_ERR_LAUNCH 2   /* hipGetLastError() reported a failed launch */
+
+/* Message for the last non-zero status returned on the calling thread. */
+const char* mxq_last_error(void);
+
+/* Library version (major * 100 + minor). */
+int mxq_version(void);
+
+/* quantize_mx_by_tile_func_cuda (mx/cpp/funcs.cpp:177-197, mx/cpp/mx.cu:116-287).
+ * MX-quantize `in`, shape (pre, axis_size, post) contiguous, sharing one exponent per
+ * `tile_size` consecutive elements of the middle axis (a shorter last tile is allowed;
+ * tile_size <= 0 means the whole axis).  `out` has the same shape and dtype. */
+int mxq_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre, int64_t axis_size,
+                            int64_t post, int scale_bits, int elem_ebits, int elem_mbits,
+                            float elem_max_norm, int64_t tile_size, int flush_fp32_subnorms,
+                            int rmode, int flags, void* hip_stream);
+
+/* quantize_mx_func_cuda (mx/cpp/funcs.cpp:154-175, mx/cpp/mx.cu:12-110).
+ * As above, but the shared exponent of element (i, k, j) comes from max_values[i * post + j]
+ * (the keepdim abs-max over the middle axis, same dtype as `in`). */
+int mxq_quantize_mx_given_max(const void* in, void* out, const void* max_values, int dtype,
+                              int64_t pre, int64_t axis_size, int64_t post, int scale_bits,
+                              int elem_ebits, int elem_mbits, float elem_max_norm,
+                              int flush_fp32_subnorms, int rmode, int flags, void* hip_stream);
+
+/* quantize_elemwise_func_cuda (mx/cpp/funcs.cpp:199-217, mx/cpp/elemwise.cu:12-94).
+ * Round each of the n elements to a (bits, exp_bits, max_norm) format. */
+int mxq_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int bits, int exp_bits,
+                          float max_norm, int rmode, int saturate_normals, int allow_denorm,
+                          int flags, void* hip_stream);
+
+/* reduce_sum_inner_dim / reduce_max_inner_dim (mx/cpp/funcs.cpp:219-231, mx/cpp/reduce.cu:15-89).
+ * fp32 (rows, inner) -> fp32 (rows).  Unlike the reference there is no restriction on `inner`,
+ * the sum order is fixed (no atomics), and max propagates NaN like torch.max. */
+int mxq_reduce_sum_inner(const float* in, float* out, int64_t rows, int64_t inner,
+                         void* hip_stream);
+int mxq_reduce_max_inner(const float* in, float* out, int64_t rows, int64_t inner,
+                         void* hip_stream);
+
+/* Reductions over the outermost axis: fp32 (outer, inner) -> fp32 (inner).  No counterpart in the
+ * reference's extension (its callers use torch.sum / torch.max for other axes).  `workspace` must
+ * hold mxq_reduce_outer_workspace_bytes(outer, inner) bytes of device memory. */
+int64_t mxq_reduce_outer_workspace_bytes(int64_t outer, int64_t inner);
+int mxq_reduce_sum_outer(const float* in, float* out, void* workspace, int64_t outer,
+                         int64_t inner, void* hip_stream);
+int mxq_reduce_max_outer(const float* in, float* out, void* workspace, int64_t outer,
+                         int64_t inner, void* hip_stream);
+
+/* ---- libmxq_host.so: the same arithmetic compiled for the host ----------------------------------
+ * quantize_mx_func_cpp (mx/cpp/funcs.cpp:23-98) and quantize_elemwise_func_cpp
+ * (mx/cpp/funcs.cpp:117-149) take CPU tensors; these are their stand-ins.  Pointers are host
+ * pointers and the calls run synchronously on the calling thread.  The by-tile variant has no
+ * CPU counterpart in the reference; it mirrors mxq_quantize_mx_by_tile so the kernel arithmetic
+ * can be checked on a machine without a GPU. */
+#define MXQ_HOST_FLAG_ROUND_EVERY_OP 2 /* bf16: round to bf16 after every op, no shortcuts */
+
+const char* mxq_host_last_error(void);
+int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_values, int dtype,
+                                   int64_t pre, int64_t axis_size, int64_t post, int scale_bits,
+                                   int elem_ebits, int elem_mbits, float elem_max_norm,
+                                   int flush_fp32_subnorms, int rmode, int flags);
+int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre,
+                                 int64_t axis_size, int64_t post, int scale_bits, int elem_ebits,
+                                 int elem_mbits, float elem_max_norm, int64_t tile_size,
+                                 int flush_fp32_subnorms, int rmode, int flags);
+int mxq_host_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int bits,
+                               int exp_bits, float max_norm, int rmode, int saturate_normals,
+                               int allow_denorm, int flags);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXQ_H */

@@ -1,0 +1,11 @@
+"""MI355X-native MX / bfloat quantization with the call surface of microsoft/microxcaling.
+
+    from microxcaling_amd.mx_ops import quantize_mx_op, _quantize_mx
+    from microxcaling_amd.elemwise_ops import quantize_elemwise_op, _quantize_elemwise_core
+    from microxcaling_amd import custom_extensions      # .funcs: the native entry points
+"""
+from .specs import (MxSpecs, get_default_mx_specs, get_backwards_mx_specs, apply_mx_specs,
+                    add_mx_args, finalize_mx_specs, get_mx_specs, mx_assert_test)
+from .formats import ElemFormat, RoundingMode
+from .mx_ops import quantize_mx_op
+from .elemwise_ops import quantize_elemwise_op

@@ -1,0 +1,60 @@
+"""Builds the two native libraries in-tree, next to this file.
+
+    libmxq_gfx950.so   HIP kernels for gfx950 + the C ABI of include/mxq.h   (hipcc)
+    libmxq_host.so     the same scalar arithmetic for CPU tensors            (ROCm clang++)
+
+Usage:  python -m microxcaling_amd.build_ext
+hipcc cross-compiles, so no GPU is needed to build.
+"""
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+
+GPU_LIB = os.path.join(PKG, "libmxq_gfx950.so")
+HOST_LIB = os.path.join(PKG, "libmxq_host.so")
+
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-fvisibility=hidden",
+          "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+
+
+def _run(cmd, verbose):
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # the host pass of hipcc does not know the gfx950 target feature below and says so: harmless
+    out = "\n".join(l for l in res.stdout.splitlines()
+                    if "packed-fp32-ops" not in l and l.strip())
+    if res.returncode != 0:
+        raise RuntimeError("build failed (%d): %s\n%s" % (res.returncode, " ".join(cmd), out))
+    if verbose and out:
+        print(out, flush=True)
+
+
+def build_gpu(verbose=True):
+    cmd = [os.path.join(ROCM, "bin", "hipcc"), "--offload-arch=gfx950",
+           # keep fp32 math scalar: packed fp32 instructions are not used by these kernels
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           *COMMON, "-o", GPU_LIB, os.path.join(CSRC, "mxq_capi.hip")]
+    _run(cmd, verbose)
+    return GPU_LIB
+
+
+def build_host(verbose=True):
+    cmd = [os.path.join(ROCM, "lib", "llvm", "bin", "clang++"), *COMMON, "-o", HOST_LIB,
+           os.path.join(CSRC, "mxq_host.cpp")]
+    _run(cmd, verbose)
+    return HOST_LIB
+
+
+def build_all(verbose=True):
+    return build_gpu(verbose), build_host(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    print("built", GPU_LIB, HOST_LIB)

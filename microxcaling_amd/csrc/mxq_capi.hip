@@ -1,0 +1,266 @@
+// C ABI of libmxq_gfx950.so: argument checks, kernel selection and launch geometry.
+// Declarations and the reference functions each entry point replaces are in include/mxq.h.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mxq.h"
+#include "mxq_kernels.h"
+
+namespace {
+
+using namespace mxq_detail;
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(MXQ_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return MXQ_OK;
+}
+
+constexpr int kThreads = 256;
+constexpr int64_t kMaxBlocks = 256 * 8;      // 256 CUs x 8 resident blocks of 256 lanes
+
+int grid_for(int64_t work_items_per_block_iter_total) {
+    int64_t g = work_items_per_block_iter_total;
+    if (g < 1) g = 1;
+    if (g > kMaxBlocks) g = kMaxBlocks;
+    return (int)g;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int elem_size(int dtype) { return dtype == MXQ_DTYPE_F32 ? 4 : 2; }
+
+// ---- dispatch over (dtype, rounding mode, element zone) -----------------------------------------
+// F is a functor template: F<DT, RMODE, ZONE_ELEM>::run(args...)
+template <template <int, int, bool> class F, int DT, typename... A>
+void dispatch_round(int rmode, bool zone_elem, A... a) {
+    if (rmode == MXQ_ROUND_FLOOR) F<DT, MXQ_FLOOR, true>::run(a...);
+    else if (rmode == MXQ_ROUND_NEAREST) {
+        if (zone_elem) F<DT, MXQ_NEAREST, true>::run(a...);
+        else F<DT, MXQ_NEAREST, false>::run(a...);
+    } else {
+        if (zone_elem) F<DT, MXQ_EVEN, true>::run(a...);
+        else F<DT, MXQ_EVEN, false>::run(a...);
+    }
+}
+template <template <int, int, bool> class F, typename... A>
+void dispatch(int dtype, int rmode, bool zone_elem, A... a) {
+    if (dtype == MXQ_DTYPE_F32) dispatch_round<F, MXQ_F32>(rmode, zone_elem, a...);
+    else if (dtype == MXQ_DTYPE_BF16) dispatch_round<F, MXQ_BF16>(rmode, zone_elem, a...);
+    else dispatch_round<F, MXQ_F16>(rmode, zone_elem, a...);
+}
+
+constexpr int kLastAxisUnroll = 4;
+
+template <int DT, int RMODE, bool ZE>
+struct LaunchLastAxis {
+    static void run(const void* in, void* out, int64_t n_vec, int lpt, MxParams p, hipStream_t s) {
+        const int grid = grid_for(ceil_div(n_vec, (int64_t)kThreads * kLastAxisUnroll));
+        const u32x4* i4 = reinterpret_cast<const u32x4*>(in);
+        u32x4* o4 = reinterpret_cast<u32x4*>(out);
+#define MXQ_CASE(L)                                                                               \
+    case L:                                                                                       \
+        mx_lastaxis_kernel<DT, RMODE, L, ZE, kLastAxisUnroll><<<grid, kThreads, 0, s>>>(i4, o4, n_vec, p); \
+        break;
+        switch (lpt) {
+            MXQ_CASE(1) MXQ_CASE(2) MXQ_CASE(4) MXQ_CASE(8) MXQ_CASE(16)
+        }
+#undef MXQ_CASE
+    }
+};
+
+template <int DT, int RMODE, bool ZE>
+struct LaunchStrided {
+    static void run(const void* in, void* out, int64_t pre, int64_t axis, int64_t post, int64_t tile,
+                    bool vec, MxParams p, hipStream_t s) {
+        constexpr int VWV = (DT == MXQ_F32) ? 4 : 8;
+        const int64_t num_tiles = ceil_div(axis, tile);
+        const bool in_regs = tile <= 32;
+        if (vec) {
+            const int64_t items = pre * num_tiles * (post / VWV);
+            const int grid = grid_for(ceil_div(items, kThreads));
+            if (in_regs)
+                mx_strided_kernel<DT, RMODE, VWV, 32, ZE><<<grid, kThreads, 0, s>>>(in, out, pre, axis, post, tile, num_tiles, p);
+            else
+                mx_strided_kernel<DT, RMODE, VWV, 0, ZE><<<grid, kThreads, 0, s>>>(in, out, pre, axis, post, tile, num_tiles, p);
+        } else {
+            const int64_t items = pre * num_tiles * post;
+            const int grid = grid_for(ceil_div(items, kThreads));
+            if (in_regs)
+                mx_strided_kernel<DT, RMODE, 1, 32, ZE><<<grid, kThreads, 0, s>>>(in, out, pre, axis, post, tile, num_tiles, p);
+            else
+                mx_strided_kernel<DT, RMODE, 1, 0, ZE><<<grid, kThreads, 0, s>>>(in, out, pre, axis, post, tile, num_tiles, p);
+        }
+    }
+};
+
+template <int DT, int RMODE, bool ZE>
+struct LaunchGivenMax {
+    static void run(const void* in, void* out, const void* maxv, int64_t total, int64_t axis,
+                    int64_t post, MxParams p, hipStream_t s) {
+        const int grid = grid_for(ceil_div(total, kThreads * 4));
+        mx_given_max_kernel<DT, RMODE, ZE><<<grid, kThreads, 0, s>>>(in, out, maxv, total, axis, post, p);
+    }
+};
+
+constexpr int kElemUnroll = 4;
+
+template <int DT, int RMODE, bool>
+struct LaunchElemwise {
+    static void run(const void* in, void* out, int64_t n, ElemParams p, hipStream_t s) {
+        const int epv = (DT == MXQ_F32) ? 4 : 8;
+        const int grid = grid_for(ceil_div(ceil_div(n, epv), (int64_t)kThreads * kElemUnroll));
+        elemwise_kernel<DT, RMODE, kElemUnroll><<<grid, kThreads, 0, s>>>(in, out, n, p);
+    }
+};
+
+// splits of the outer axis for the two-pass outer reduction
+int64_t outer_splits(int64_t outer, int64_t inner) {
+    const int vw = (inner % 4 == 0) ? 4 : 1;
+    const int64_t col_blocks = ceil_div(ceil_div(inner, vw), kThreads);
+    int64_t s = ceil_div(kMaxBlocks, col_blocks);
+    const int64_t most = ceil_div(outer, 16);          // at least 16 rows per split
+    if (s > most) s = most;
+    if (s < 1) s = 1;
+    if (s > 65535) s = 65535;
+    return s;
+}
+
+template <class OP>
+int reduce_inner(const float* in, float* out, int64_t rows, int64_t inner, void* stream, const char* who) {
+    if (rows < 0 || inner < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (rows == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    hipStream_t s = (hipStream_t)stream;
+    if (inner >= 2048) {
+        const int grid = (int)(rows < 65536 ? rows : 65536);
+        reduce_inner_block_kernel<OP><<<grid, kThreads, 0, s>>>(in, out, rows, inner);
+    } else {
+        const int grid = grid_for(ceil_div(rows, kThreads / 64));
+        reduce_inner_wave_kernel<OP><<<grid, kThreads, 0, s>>>(in, out, rows, inner);
+    }
+    return check_launch(who);
+}
+
+template <class OP>
+int reduce_outer(const float* in, float* out, void* workspace, int64_t outer, int64_t inner,
+                 void* stream, const char* who) {
+    if (outer < 0 || inner < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (inner == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t splits = outer_splits(outer, inner);
+    if (splits > 1 && !workspace) return fail(MXQ_ERR_ARGUMENT, "%s: workspace required", who);
+    const bool vec = (inner % 4 == 0) && aligned16(in) && aligned16(out) && (splits == 1 || aligned16(workspace));
+    const int64_t rows_per_split = ceil_div(outer > 0 ? outer : 1, splits);
+    float* partial = splits == 1 ? out : reinterpret_cast<float*>(workspace);
+    dim3 grid((unsigned)ceil_div(ceil_div(inner, vec ? 4 : 1), kThreads), (unsigned)splits);
+    if (vec) reduce_outer_kernel<OP, 4><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
+    else reduce_outer_kernel<OP, 1><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
+    int rc = check_launch(who);
+    if (rc || splits == 1) return rc;
+    reduce_outer_final_kernel<OP><<<(unsigned)ceil_div(inner, kThreads), kThreads, 0, s>>>(partial, out, splits, inner);
+    return check_launch(who);
+}
+
+}  // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+const char* mxq_last_error(void) { return last_error().c_str(); }
+
+int mxq_version(void) { return 100; }
+
+int mxq_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre, int64_t axis_size,
+                            int64_t post, int scale_bits, int elem_ebits, int elem_mbits,
+                            float elem_max_norm, int64_t tile_size, int flush_fp32_subnorms,
+                            int rmode, int flags, void* hip_stream) {
+    const char* who = "mxq_quantize_mx_by_tile";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    if (pre < 0 || axis_size < 0 || post < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    int64_t total;
+    if (mul_overflows(pre, axis_size, post, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    int64_t tile = (tile_size <= 0 || tile_size > axis_size) ? axis_size : tile_size;
+    hipStream_t s = (hipStream_t)hip_stream;
+
+    const int vec_elems = 16 / elem_size(dtype);
+    const bool ptr_ok = aligned16(in) && aligned16(out);
+    if (post == 1 && ptr_ok && axis_size % tile == 0 && tile % vec_elems == 0) {
+        const int64_t lpt = tile / vec_elems;
+        if (lpt == 1 || lpt == 2 || lpt == 4 || lpt == 8 || lpt == 16) {
+            dispatch<LaunchLastAxis>(dtype, rmode, ze, in, out, total / vec_elems, (int)lpt, p, s);
+            return check_launch(who);
+        }
+    }
+    const bool vec = ptr_ok && post % vec_elems == 0;
+    dispatch<LaunchStrided>(dtype, rmode, ze, in, out, pre, axis_size, post, tile, vec, p, s);
+    return check_launch(who);
+}
+
+int mxq_quantize_mx_given_max(const void* in, void* out, const void* max_values, int dtype,
+                              int64_t pre, int64_t axis_size, int64_t post, int scale_bits,
+                              int elem_ebits, int elem_mbits, float elem_max_norm,
+                              int flush_fp32_subnorms, int rmode, int flags, void* hip_stream) {
+    const char* who = "mxq_quantize_mx_given_max";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    if (pre < 0 || axis_size < 0 || post < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    int64_t total;
+    if (mul_overflows(pre, axis_size, post, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !out || !max_values) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    dispatch<LaunchGivenMax>(dtype, rmode, ze, in, out, max_values, total, axis_size, post, p,
+                             (hipStream_t)hip_stream);
+    return check_launch(who);
+}
+
+int mxq_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int bits, int exp_bits,
+                          float max_norm, int rmode, int saturate_normals, int allow_denorm,
+                          int flags, void* hip_stream) {
+    const char* who = "mxq_quantize_elemwise";
+    ElemParams p;
+    int rc = make_elem_params(dtype, bits, exp_bits, max_norm, rmode, saturate_normals, allow_denorm,
+                              flags, &p, who);
+    if (rc) return rc;
+    if (n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (n == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(in) || !aligned16(out))
+        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    dispatch<LaunchElemwise>(dtype, rmode, true, in, out, n, p, (hipStream_t)hip_stream);
+    return check_launch(who);
+}
+
+int mxq_reduce_sum_inner(const float* in, float* out, int64_t rows, int64_t inner, void* hip_stream) {
+    return reduce_inner<SumOp>(in, out, rows, inner, hip_stream, "mxq_reduce_sum_inner");
+}
+int mxq_reduce_max_inner(const float* in, float* out, int64_t rows, int64_t inner, void* hip_stream) {
+    return reduce_inner<MaxOp>(in, out, rows, inner, hip_stream, "mxq_reduce_max_inner");
+}
+
+int64_t mxq_reduce_outer_workspace_bytes(int64_t outer, int64_t inner) {
+    if (outer <= 0 || inner <= 0) return 0;
+    const int64_t s = outer_splits(outer, inner);
+    return s == 1 ? 0 : s * inner * (int64_t)sizeof(float);
+}
+int mxq_reduce_sum_outer(const float* in, float* out, void* workspace, int64_t outer, int64_t inner,
+                         void* hip_stream) {
+    return reduce_outer<SumOp>(in, out, workspace, outer, inner, hip_stream, "mxq_reduce_sum_outer");
+}
+int mxq_reduce_max_outer(const float* in, float* out, void* workspace, int64_t outer, int64_t inner,
+                         void* hip_stream) {
+    return reduce_outer<MaxOp>(in, out, workspace, outer, inner, hip_stream, "mxq_reduce_max_outer");
+}
+
+}  // extern "C"
+#pragma GCC visibility pop

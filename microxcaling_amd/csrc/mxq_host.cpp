@@ -1,0 +1,149 @@
+// libmxq_host.so: the same scalar arithmetic as the GPU kernels (mxq_core.h), compiled for the
+// host.  It serves the two CPU entry points of the reference's extension
+// (quantize_mx_func_cpp, quantize_elemwise_func_cpp -- mx/cpp/funcs.cpp:23-149) for CPU tensors,
+// and lets the kernel arithmetic be checked exhaustively without a GPU.  GPU tensors never come
+// here: the GPU entry points live in libmxq_gfx950.so and there is no fallback between the two.
+#include <stdint.h>
+#include <string.h>
+
+#include <algorithm>
+
+#include "mxq.h"
+#include "mxq_params.h"
+
+namespace {
+
+using namespace mxq_detail;
+
+const unsigned char kZone[3][MXQ_ZONE_PAD] = {{MXQ_ZONE_ROW_F32}, {MXQ_ZONE_ROW_BF16}, {0}};
+
+float load_as_float(const void* p, int dtype, int64_t i) {
+    if (dtype == MXQ_DTYPE_F32) return reinterpret_cast<const float*>(p)[i];
+    uint16_t h = reinterpret_cast<const uint16_t*>(p)[i];
+    if (dtype == MXQ_DTYPE_BF16) return mxq_float((uint32_t)h << 16);
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+
+void store_from_float(void* p, int dtype, int64_t i, float v) {
+    if (dtype == MXQ_DTYPE_F32) {
+        reinterpret_cast<float*>(p)[i] = v;
+    } else if (dtype == MXQ_DTYPE_BF16) {
+        reinterpret_cast<uint16_t*>(p)[i] = (uint16_t)(mxq_bits(v) >> 16);   // already bf16-exact
+    } else {
+        reinterpret_cast<uint16_t*>(p)[i] = __builtin_bit_cast(uint16_t, (_Float16)v);
+    }
+}
+
+// element kernels selected once per call
+typedef float (*MxElemFn)(float, const MxqScale&, const MxqFmt&, const unsigned char*, int);
+typedef float (*ElemFn)(float, const MxqFmt&, bool, bool, const unsigned char*, int);
+
+template <int DT, bool FULL>
+MxElemFn pick_mx(int rmode, bool ze) {
+    if (rmode == MXQ_ROUND_FLOOR) return mxq_quant_mx_elem<MXQ_FLOOR, DT, true, FULL>;
+    if (rmode == MXQ_ROUND_NEAREST)
+        return ze ? mxq_quant_mx_elem<MXQ_NEAREST, DT, true, FULL> : mxq_quant_mx_elem<MXQ_NEAREST, DT, false, FULL>;
+    return ze ? mxq_quant_mx_elem<MXQ_EVEN, DT, true, FULL> : mxq_quant_mx_elem<MXQ_EVEN, DT, false, FULL>;
+}
+MxElemFn pick_mx(int dtype, int rmode, bool ze, bool full) {
+    if (dtype == MXQ_DTYPE_BF16) return full ? pick_mx<MXQ_BF16, true>(rmode, true) : pick_mx<MXQ_BF16, false>(rmode, ze);
+    return full ? pick_mx<MXQ_F32, true>(rmode, true) : pick_mx<MXQ_F32, false>(rmode, ze);
+}
+template <int DT, bool FULL>
+ElemFn pick_elem(int rmode) {
+    if (rmode == MXQ_ROUND_FLOOR) return mxq_quant_elemwise<MXQ_FLOOR, DT, FULL>;
+    if (rmode == MXQ_ROUND_NEAREST) return mxq_quant_elemwise<MXQ_NEAREST, DT, FULL>;
+    return mxq_quant_elemwise<MXQ_EVEN, DT, FULL>;
+}
+
+}  // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+const char* mxq_host_last_error(void) { return last_error().c_str(); }
+
+int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre, int64_t axis_size,
+                                 int64_t post, int scale_bits, int elem_ebits, int elem_mbits,
+                                 float elem_max_norm, int64_t tile_size, int flush_fp32_subnorms,
+                                 int rmode, int flags) {
+    const char* who = "mxq_host_quantize_mx_by_tile";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    if (pre < 0 || axis_size < 0 || post < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    int64_t total;
+    if (mul_overflows(pre, axis_size, post, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    const int64_t tile = (tile_size <= 0 || tile_size > axis_size) ? axis_size : tile_size;
+    const unsigned char* zone = kZone[p.zone_row];
+    MxElemFn fn = pick_mx(dtype, rmode, ze, (flags & MXQ_HOST_FLAG_ROUND_EVERY_OP) != 0);
+    for (int64_t i = 0; i < pre; ++i)
+        for (int64_t k0 = 0; k0 < axis_size; k0 += tile)
+            for (int64_t j = 0; j < post; ++j) {
+                const int64_t k1 = std::min(k0 + tile, axis_size);
+                uint32_t um = 0;
+                for (int64_t k = k0; k < k1; ++k)
+                    um = std::max(um, mxq_bits(load_as_float(in, dtype, (i * axis_size + k) * post + j)) & 0x7FFFFFFFu);
+                MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+                for (int64_t k = k0; k < k1; ++k) {
+                    const int64_t idx = (i * axis_size + k) * post + j;
+                    store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift));
+                }
+            }
+    return MXQ_OK;
+}
+
+int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_values, int dtype,
+                                   int64_t pre, int64_t axis_size, int64_t post, int scale_bits,
+                                   int elem_ebits, int elem_mbits, float elem_max_norm,
+                                   int flush_fp32_subnorms, int rmode, int flags) {
+    const char* who = "mxq_host_quantize_mx_given_max";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    if (pre < 0 || axis_size < 0 || post < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    int64_t total;
+    if (mul_overflows(pre, axis_size, post, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !out || !max_values) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    const unsigned char* zone = kZone[p.zone_row];
+    MxElemFn fn = pick_mx(dtype, rmode, ze, (flags & MXQ_HOST_FLAG_ROUND_EVERY_OP) != 0);
+    for (int64_t i = 0; i < pre; ++i)
+        for (int64_t j = 0; j < post; ++j) {
+            const uint32_t um = mxq_bits(load_as_float(max_values, dtype, i * post + j)) & 0x7FFFFFFFu;
+            MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+            for (int64_t k = 0; k < axis_size; ++k) {
+                const int64_t idx = (i * axis_size + k) * post + j;
+                store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift));
+            }
+        }
+    return MXQ_OK;
+}
+
+int mxq_host_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int bits, int exp_bits,
+                               float max_norm, int rmode, int saturate_normals, int allow_denorm,
+                               int flags) {
+    const char* who = "mxq_host_quantize_elemwise";
+    ElemParams p;
+    int rc = make_elem_params(dtype, bits, exp_bits, max_norm, rmode, saturate_normals, allow_denorm,
+                              flags, &p, who);
+    if (rc) return rc;
+    if (n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (n == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    const unsigned char* zone = kZone[p.zone_row];
+    ElemFn fn = dtype == MXQ_DTYPE_BF16 ? pick_elem<MXQ_BF16, true>(rmode) : pick_elem<MXQ_F32, true>(rmode);
+    for (int64_t i = 0; i < n; ++i)
+        store_from_float(out, dtype, i,
+                         fn(load_as_float(in, dtype, i), p.fmt, p.saturate != 0, p.allow_denorm != 0, zone, p.zshift));
+    return MXQ_OK;
+}
+
+}  // extern "C"
+#pragma GCC visibility pop

@@ -1,0 +1,494 @@
+// HIP kernels for gfx950 (MI355X): MX block quantization, elementwise quantization, reductions.
+// All of them are HBM-bandwidth bound: 16-byte accesses per lane, grid-sized to the chip, the
+// block maximum taken with DPP lane exchanges (last axis) or held in registers (other axes), and
+// non-temporal stores for the write-once output.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mxq_core.h"
+#include "mxq_log2_tables.h"
+#include "mxq_params.h"
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// round-up zone tables in device memory: [0] fp32, [1] bf16, [2] all zero (bit-field exponents)
+#define ZONE_PAD MXQ_ZONE_PAD
+__device__ const unsigned char g_zone_tables[3][ZONE_PAD] = {
+    {MXQ_ZONE_ROW_F32}, {MXQ_ZONE_ROW_BF16}, {0}};
+
+namespace {
+
+__device__ __forceinline__ void load_zone(unsigned char* lds, const unsigned char* src) {
+    for (int i = threadIdx.x; i < ZONE_PAD / 4; i += blockDim.x)
+        reinterpret_cast<uint32_t*>(lds)[i] = reinterpret_cast<const uint32_t*>(src)[i];
+    __syncthreads();
+}
+
+// ---- dtype packing ----------------------------------------------------------------------------
+template <int DT> struct Pack;
+template <> struct Pack<MXQ_F32> {
+    static constexpr int PER_DWORD = 1;
+    static __device__ __forceinline__ float get(uint32_t w, int) { return mxq_float(w); }
+    static __device__ __forceinline__ uint32_t put(float lo, float) { return mxq_bits(lo); }
+};
+template <> struct Pack<MXQ_BF16> {
+    static constexpr int PER_DWORD = 2;
+    static __device__ __forceinline__ float get(uint32_t w, int half) {
+        return mxq_float(half ? (w & 0xFFFF0000u) : (w << 16));
+    }
+    // values are already bf16-exact: keep the top halves
+    static __device__ __forceinline__ uint32_t put(float lo, float hi) {
+        return (mxq_bits(lo) >> 16) | (mxq_bits(hi) & 0xFFFF0000u);
+    }
+};
+template <> struct Pack<MXQ_F16> {
+    static constexpr int PER_DWORD = 2;
+    static __device__ __forceinline__ float get(uint32_t w, int half) {
+        unsigned short h = half ? (unsigned short)(w >> 16) : (unsigned short)(w & 0xFFFFu);
+        return (float)__builtin_bit_cast(_Float16, h);
+    }
+    static __device__ __forceinline__ uint32_t put(float lo, float hi) {   // RNE, like torch
+        unsigned short l = __builtin_bit_cast(unsigned short, (_Float16)lo);
+        unsigned short h = __builtin_bit_cast(unsigned short, (_Float16)hi);
+        return (uint32_t)l | ((uint32_t)h << 16);
+    }
+};
+
+// dtype whose op-by-op rounding the arithmetic follows (fp16 tensors are computed as fp32)
+template <int DT> struct Arith { static constexpr int DT_ = (DT == MXQ_BF16) ? MXQ_BF16 : MXQ_F32; };
+
+template <int DT>
+__device__ __forceinline__ float load_scalar(const void* p, int64_t i) {
+    if (DT == MXQ_F32) return reinterpret_cast<const float*>(p)[i];
+    unsigned short h = reinterpret_cast<const unsigned short*>(p)[i];
+    if (DT == MXQ_BF16) return mxq_float((uint32_t)h << 16);
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+template <int DT>
+__device__ __forceinline__ void store_scalar(void* p, int64_t i, float v) {
+    if (DT == MXQ_F32) {
+        reinterpret_cast<float*>(p)[i] = v;
+    } else if (DT == MXQ_BF16) {
+        reinterpret_cast<unsigned short*>(p)[i] = (unsigned short)(mxq_bits(v) >> 16);
+    } else {
+        reinterpret_cast<unsigned short*>(p)[i] = __builtin_bit_cast(unsigned short, (_Float16)v);
+    }
+}
+
+__device__ __forceinline__ uint32_t abs_bits(float f) { return mxq_bits(f) & 0x7FFFFFFFu; }
+
+// ---- lane exchange ----------------------------------------------------------------------------
+// max over groups of LANES consecutive lanes (LANES in 1,2,4,8,16), result in every lane
+template <int LANES>
+__device__ __forceinline__ uint32_t group_max(uint32_t v) {
+    if (LANES >= 2)    // quad_perm [1,0,3,2]
+        v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, false));
+    if (LANES >= 4)    // quad_perm [2,3,0,1]
+        v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, false));
+    if (LANES >= 8)    // row_half_mirror: lane i <-> 7-i inside each group of 8
+        v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, false));
+    if (LANES >= 16)   // row_mirror: lane i <-> 15-i inside each row of 16
+        v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, false));
+    return v;
+}
+
+// ================================================================================================
+// MX quantization, shared axis innermost, tile = LPT lanes x 16 bytes, tile-aligned tensor.
+// One lane owns 16 bytes (4 fp32 / 8 16-bit elements); LPT neighbouring lanes share a tile.
+// ================================================================================================
+template <int DT, int RMODE, int LPT, bool ZONE_ELEM, int UNROLL>
+__global__ __launch_bounds__(256) void mx_lastaxis_kernel(const u32x4* __restrict__ in,
+                                                          u32x4* __restrict__ out, int64_t n_vec,
+                                                          MxParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    __shared__ unsigned char zone[ZONE_PAD];
+
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x * UNROLL;
+    int64_t base = (int64_t)blockIdx.x * blockDim.x * UNROLL + threadIdx.x;
+
+    // first batch of loads goes out before the table copy so the two latencies overlap
+    u32x4 v[UNROLL];
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) {
+        int64_t i = base + (int64_t)j * blockDim.x;
+        v[j] = (i < n_vec) ? in[i] : u32x4{0, 0, 0, 0};
+    }
+    load_zone(zone, g_zone_tables[p.zone_row]);
+
+    while (true) {
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            int64_t i = base + (int64_t)j * blockDim.x;
+            float x[4 * PD];
+            uint32_t um = 0;
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    x[d * PD + h] = Pack<DT>::get(v[j][d], h);
+                    um = max(um, abs_bits(x[d * PD + h]));
+                }
+            um = group_max<LPT>(um);
+            MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+            u32x4 o;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                float q[2];
+#pragma unroll
+                for (int h = 0; h < PD; ++h)
+                    q[h] = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, false>(x[d * PD + h], sc, p.fmt,
+                                                                          zone, p.zshift);
+                o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+            }
+            if (i < n_vec) __builtin_nontemporal_store(o, &out[i]);
+        }
+        base += stride;
+        if (base - threadIdx.x >= n_vec) break;     // uniform per block
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            int64_t i = base + (int64_t)j * blockDim.x;
+            v[j] = (i < n_vec) ? in[i] : u32x4{0, 0, 0, 0};
+        }
+    }
+}
+
+// ================================================================================================
+// MX quantization along any axis: tensor (pre, axis, post), tiles of `tile` rows of the middle
+// axis.  One lane owns VW consecutive `post` positions of one tile, so a wave reads 64*VW
+// contiguous elements per row.  ROWS > 0: the tile (<= ROWS rows) stays in registers between the
+// max pass and the rounding pass; ROWS == 0: any tile size, second pass re-reads memory.
+// ================================================================================================
+template <int DT, int VW> struct ColVec;     // VW elements of dtype DT
+template <> struct ColVec<MXQ_F32, 1> { typedef uint32_t T; static constexpr int DW = 1; };
+template <> struct ColVec<MXQ_F32, 4> { typedef u32x4 T; static constexpr int DW = 4; };
+template <> struct ColVec<MXQ_BF16, 1> { typedef unsigned short T; static constexpr int DW = 1; };
+template <> struct ColVec<MXQ_BF16, 8> { typedef u32x4 T; static constexpr int DW = 4; };
+template <> struct ColVec<MXQ_BF16, 4> { typedef u32x2 T; static constexpr int DW = 2; };
+template <> struct ColVec<MXQ_F16, 1> { typedef unsigned short T; static constexpr int DW = 1; };
+template <> struct ColVec<MXQ_F16, 8> { typedef u32x4 T; static constexpr int DW = 4; };
+template <> struct ColVec<MXQ_F16, 4> { typedef u32x2 T; static constexpr int DW = 2; };
+
+template <int DT, int VW>
+__device__ __forceinline__ void unpack_cols(const typename ColVec<DT, VW>::T& raw, float* x) {
+    if constexpr (VW == 1) {
+        if (DT == MXQ_F32) x[0] = mxq_float((uint32_t)raw);
+        else if (DT == MXQ_BF16) x[0] = mxq_float((uint32_t)raw << 16);
+        else x[0] = (float)__builtin_bit_cast(_Float16, (unsigned short)raw);
+    } else {
+        constexpr int PD = Pack<DT>::PER_DWORD;
+#pragma unroll
+        for (int d = 0; d < ColVec<DT, VW>::DW; ++d)
+#pragma unroll
+            for (int h = 0; h < PD; ++h) x[d * PD + h] = Pack<DT>::get(raw[d], h);
+    }
+}
+template <int DT, int VW>
+__device__ __forceinline__ typename ColVec<DT, VW>::T pack_cols(const float* q) {
+    typename ColVec<DT, VW>::T r;
+    if constexpr (VW == 1) {
+        if (DT == MXQ_F32) r = mxq_bits(q[0]);
+        else if (DT == MXQ_BF16) r = (unsigned short)(mxq_bits(q[0]) >> 16);
+        else r = __builtin_bit_cast(unsigned short, (_Float16)q[0]);
+    } else {
+        constexpr int PD = Pack<DT>::PER_DWORD;
+#pragma unroll
+        for (int d = 0; d < ColVec<DT, VW>::DW; ++d) r[d] = Pack<DT>::put(q[d * PD], q[d * PD + PD - 1]);
+    }
+    return r;
+}
+
+template <int DT, int RMODE, int VW, int ROWS, bool ZONE_ELEM>
+__global__ __launch_bounds__(256) void mx_strided_kernel(const void* __restrict__ in_,
+                                                         void* __restrict__ out_, int64_t pre,
+                                                         int64_t axis_size, int64_t post,
+                                                         int64_t tile, int64_t num_tiles,
+                                                         MxParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    typedef typename ColVec<DT, VW>::T V;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.zone_row]);
+
+    const V* in = reinterpret_cast<const V*>(in_);
+    V* out = reinterpret_cast<V*>(out_);
+    const int64_t pv = post / VW;                       // column groups per row
+    const int64_t total = pre * num_tiles * pv;
+    for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total;
+         w += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t c = w % pv;
+        const int64_t ti = (w / pv) % num_tiles;
+        const int64_t pi = w / (pv * num_tiles);
+        const int64_t row0 = ti * tile;
+        const int rows = (int)((row0 + tile > axis_size) ? (axis_size - row0) : tile);
+        const int64_t off0 = (pi * axis_size + row0) * pv + c;   // in units of V
+
+        uint32_t um[VW];
+#pragma unroll
+        for (int k = 0; k < VW; ++k) um[k] = 0;
+
+        if constexpr (ROWS > 0) {
+            V raw[ROWS];
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+                if (r < rows) raw[r] = in[off0 + (int64_t)r * pv];
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+                if (r < rows) {
+                    float x[VW];
+                    unpack_cols<DT, VW>(raw[r], x);
+#pragma unroll
+                    for (int k = 0; k < VW; ++k) um[k] = max(um[k], abs_bits(x[k]));
+                }
+            MxqScale sc[VW];
+#pragma unroll
+            for (int k = 0; k < VW; ++k)
+                sc[k] = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+                if (r < rows) {
+                    float x[VW], q[VW];
+                    unpack_cols<DT, VW>(raw[r], x);
+#pragma unroll
+                    for (int k = 0; k < VW; ++k)
+                        q[k] = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, false>(x[k], sc[k], p.fmt,
+                                                                              zone, p.zshift);
+                    __builtin_nontemporal_store(pack_cols<DT, VW>(q), &out[off0 + (int64_t)r * pv]);
+                }
+        } else {
+            for (int r = 0; r < rows; ++r) {
+                float x[VW];
+                unpack_cols<DT, VW>(in[off0 + (int64_t)r * pv], x);
+#pragma unroll
+                for (int k = 0; k < VW; ++k) um[k] = max(um[k], abs_bits(x[k]));
+            }
+            MxqScale sc[VW];
+#pragma unroll
+            for (int k = 0; k < VW; ++k)
+                sc[k] = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+            for (int r = 0; r < rows; ++r) {
+                float x[VW], q[VW];
+                unpack_cols<DT, VW>(in[off0 + (int64_t)r * pv], x);
+#pragma unroll
+                for (int k = 0; k < VW; ++k)
+                    q[k] = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, false>(x[k], sc[k], p.fmt, zone,
+                                                                          p.zshift);
+                out[off0 + (int64_t)r * pv] = pack_cols<DT, VW>(q);
+            }
+        }
+    }
+}
+
+// ================================================================================================
+// MX quantization with the block maximum supplied by the caller: element (i, k, j) uses
+// max_values[i * post + j].
+// ================================================================================================
+template <int DT, int RMODE, bool ZONE_ELEM>
+__global__ __launch_bounds__(256) void mx_given_max_kernel(const void* __restrict__ in,
+                                                           void* __restrict__ out,
+                                                           const void* __restrict__ maxv,
+                                                           int64_t total, int64_t axis_size,
+                                                           int64_t post, MxParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.zone_row]);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t j = i % post;
+        const int64_t pi = i / (post * axis_size);
+        const uint32_t um = abs_bits(load_scalar<DT>(maxv, pi * post + j));
+        MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+        float q = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, false>(load_scalar<DT>(in, i), sc, p.fmt,
+                                                                 zone, p.zshift);
+        store_scalar<DT>(out, i, q);
+    }
+}
+
+// ================================================================================================
+// Elementwise quantization.  Body: 16 bytes per lane; the (< 16 byte) tail is done per element.
+// ================================================================================================
+template <int DT, int RMODE, int UNROLL>
+__global__ __launch_bounds__(256) void elemwise_kernel(const void* __restrict__ in_,
+                                                       void* __restrict__ out_, int64_t n,
+                                                       ElemParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int EPV = 4 * PD;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.zone_row]);
+
+    const u32x4* in = reinterpret_cast<const u32x4*>(in_);
+    u32x4* out = reinterpret_cast<u32x4*>(out_);
+    const int64_t n_vec = n / EPV;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x * UNROLL;
+    for (int64_t base = (int64_t)blockIdx.x * blockDim.x * UNROLL + threadIdx.x;
+         base - threadIdx.x < n_vec; base += stride) {
+        u32x4 v[UNROLL];
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            int64_t i = base + (int64_t)j * blockDim.x;
+            v[j] = (i < n_vec) ? in[i] : u32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            int64_t i = base + (int64_t)j * blockDim.x;
+            u32x4 o;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                float q[2];
+#pragma unroll
+                for (int h = 0; h < PD; ++h)
+                    q[h] = mxq_quant_elemwise<RMODE, ADT, true>(Pack<DT>::get(v[j][d], h), p.fmt,
+                                                                p.saturate != 0, p.allow_denorm != 0,
+                                                                zone, p.zshift);
+                o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+            }
+            if (i < n_vec) __builtin_nontemporal_store(o, &out[i]);
+        }
+    }
+    // tail
+    const int64_t t0 = n_vec * EPV;
+    const int64_t gi = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gi < n - t0) {
+        float q = mxq_quant_elemwise<RMODE, ADT, true>(load_scalar<DT>(in_, t0 + gi), p.fmt,
+                                                       p.saturate != 0, p.allow_denorm != 0, zone,
+                                                       p.zshift);
+        store_scalar<DT>(out_, t0 + gi, q);
+    }
+}
+
+// ================================================================================================
+// Reductions (fp32).  max propagates NaN like torch.max; sums are accumulated in a fixed order.
+// ================================================================================================
+struct SumOp {
+    static __device__ __forceinline__ float init() { return 0.0f; }
+    static __device__ __forceinline__ float apply(float a, float b) { return a + b; }
+};
+struct MaxOp {
+    static __device__ __forceinline__ float init() { return -__builtin_inff(); }
+    static __device__ __forceinline__ float apply(float a, float b) {
+        return (b > a || b != b) ? b : a;          // NaN sticks once seen
+    }
+};
+
+template <class OP>
+__device__ __forceinline__ float wave_reduce(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = OP::apply(v, __shfl_xor(v, m, 64));
+    return v;
+}
+
+// one block of 256 lanes per row (inner large) ...
+template <class OP>
+__global__ __launch_bounds__(256) void reduce_inner_block_kernel(const float* __restrict__ in,
+                                                                 float* __restrict__ out,
+                                                                 int64_t rows, int64_t inner) {
+    __shared__ float part[4];
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+        const float* row = in + r * inner;
+        float acc = OP::init();
+        const bool vec_ok = (inner % 4 == 0) && ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
+        if (vec_ok) {
+            const u32x4* rv = reinterpret_cast<const u32x4*>(row);
+            for (int64_t i = threadIdx.x; i < inner / 4; i += blockDim.x) {
+                u32x4 w = rv[i];
+#pragma unroll
+                for (int d = 0; d < 4; ++d) acc = OP::apply(acc, mxq_float(w[d]));
+            }
+        } else {
+            for (int64_t i = threadIdx.x; i < inner; i += blockDim.x) acc = OP::apply(acc, row[i]);
+        }
+        acc = wave_reduce<OP>(acc);
+        if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float t = part[0];
+            for (int wv = 1; wv < (int)(blockDim.x >> 6); ++wv) t = OP::apply(t, part[wv]);
+            out[r] = t;
+        }
+        __syncthreads();
+    }
+}
+
+// ... or one wave per row (inner small)
+template <class OP>
+__global__ __launch_bounds__(256) void reduce_inner_wave_kernel(const float* __restrict__ in,
+                                                                float* __restrict__ out,
+                                                                int64_t rows, int64_t inner) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int64_t n_waves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    for (int64_t r = wave; r < rows; r += n_waves) {
+        const float* row = in + r * inner;
+        float acc = OP::init();
+        const bool vec_ok = (inner % 4 == 0) && ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
+        if (vec_ok) {
+            const u32x4* rv = reinterpret_cast<const u32x4*>(row);
+            for (int64_t i = lane; i < inner / 4; i += 64) {
+                u32x4 w = rv[i];
+#pragma unroll
+                for (int d = 0; d < 4; ++d) acc = OP::apply(acc, mxq_float(w[d]));
+            }
+        } else {
+            for (int64_t i = lane; i < inner; i += 64) acc = OP::apply(acc, row[i]);
+        }
+        acc = wave_reduce<OP>(acc);
+        if (lane == 0) out[r] = acc;
+    }
+}
+
+// outer axis: (outer, inner) -> partial (splits, inner); lane owns 4 (or 1) consecutive columns
+template <class OP, int VW>
+__global__ __launch_bounds__(256) void reduce_outer_kernel(const float* __restrict__ in,
+                                                           float* __restrict__ partial,
+                                                           int64_t outer, int64_t inner,
+                                                           int64_t rows_per_split) {
+    const int64_t cg = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // column group
+    if (cg * VW >= inner) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_split;
+    const int64_t r1 = (r0 + rows_per_split < outer) ? r0 + rows_per_split : outer;
+    float acc[VW];
+#pragma unroll
+    for (int k = 0; k < VW; ++k) acc[k] = OP::init();
+    if constexpr (VW == 4) {
+        const u32x4* p = reinterpret_cast<const u32x4*>(in) + cg;
+        const int64_t pv = inner / 4;
+        int64_t r = r0;
+        for (; r + 4 <= r1; r += 4) {                 // four rows in flight
+            u32x4 w0 = p[r * pv], w1 = p[(r + 1) * pv], w2 = p[(r + 2) * pv], w3 = p[(r + 3) * pv];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                acc[k] = OP::apply(acc[k], mxq_float(w0[k]));
+                acc[k] = OP::apply(acc[k], mxq_float(w1[k]));
+                acc[k] = OP::apply(acc[k], mxq_float(w2[k]));
+                acc[k] = OP::apply(acc[k], mxq_float(w3[k]));
+            }
+        }
+        for (; r < r1; ++r) {
+            u32x4 w = p[r * pv];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) acc[k] = OP::apply(acc[k], mxq_float(w[k]));
+        }
+        u32x4 o;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[k] = mxq_bits(acc[k]);
+        reinterpret_cast<u32x4*>(partial + (int64_t)blockIdx.y * inner)[cg] = o;
+    } else {
+        for (int64_t r = r0; r < r1; ++r) acc[0] = OP::apply(acc[0], in[r * inner + cg]);
+        partial[(int64_t)blockIdx.y * inner + cg] = acc[0];
+    }
+}
+
+template <class OP>
+__global__ __launch_bounds__(256) void reduce_outer_final_kernel(const float* __restrict__ partial,
+                                                                 float* __restrict__ out,
+                                                                 int64_t splits, int64_t inner) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= inner) return;
+    float acc = OP::init();
+    for (int64_t s = 0; s < splits; ++s) acc = OP::apply(acc, partial[s * inner + c]);
+    out[c] = acc;
+}
+
+}  // namespace

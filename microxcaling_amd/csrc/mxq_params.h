@@ -1,0 +1,129 @@
+// Host-side parameter preparation shared by the GPU entry points (mxq_capi.hip) and the host
+// build (mxq_host.cpp): argument checks, element-format constants, choice of round-up-zone table.
+#pragma once
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include <string>
+
+#include "mxq.h"
+#include "mxq_core.h"
+#include "mxq_log2_tables.h"
+
+enum { ZONE_ROW_F32 = 0, ZONE_ROW_BF16 = 1, ZONE_ROW_NONE = 2 };
+
+struct MxParams {
+    MxqFmt fmt;
+    int emax;         // exponent of the element format's max_norm
+    int scale_emax;   // 2^(scale_bits-1) - 1
+    int flush;
+    int zone_row;     // which round-up-zone table
+    int zshift;       // 0 for fp32 significands, 16 for bf16
+};
+
+struct ElemParams {
+    MxqFmt fmt;
+    int saturate;
+    int allow_denorm;
+    int zone_row;
+    int zshift;
+};
+
+namespace mxq_detail {
+
+inline std::string& last_error() {
+    static thread_local std::string s;
+    return s;
+}
+
+inline int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+inline int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    last_error() = buf;
+    return code;
+}
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+inline bool mul_overflows(int64_t a, int64_t b, int64_t c, int64_t* out) {
+    __int128 t = (__int128)a * b * c;
+    if (t > (__int128)INT64_MAX) return true;
+    *out = (int64_t)t;
+    return false;
+}
+
+inline int make_fmt(int dtype, int ebits, int mbits, float max_norm, MxqFmt* fmt, const char* who) {
+    if (ebits < 0 || ebits > 8) return fail(MXQ_ERR_ARGUMENT, "%s: exponent bits %d outside [0, 8]", who, ebits);
+    if (mbits < 2 || mbits > 24)
+        return fail(MXQ_ERR_ARGUMENT, "%s: bits %d outside [2, 24] (sign + implicit one + fraction)", who, mbits);
+    if (!(max_norm > 0.0f) || !(max_norm < __builtin_inff()))
+        return fail(MXQ_ERR_ARGUMENT, "%s: max_norm must be positive and finite", who);
+    fmt->ebits = ebits;
+    fmt->t = mbits - 2;
+    fmt->min_exp = ebits ? 2 - (1 << (ebits - 1)) : 0;
+    // torch casts the clamp bound to the tensor dtype (65504 becomes 65536 for a bf16 tensor)
+    fmt->max_bits = mxq_bits(dtype == MXQ_DTYPE_BF16 ? mxq_round_bf16(max_norm) : max_norm);
+    return MXQ_OK;
+}
+
+inline void zone_for(int dtype, int flags, int* row, int* zshift) {
+    *zshift = 0;
+    if ((flags & MXQ_FLAG_EXACT_EXPONENT) || dtype == MXQ_DTYPE_F16) {
+        *row = ZONE_ROW_NONE;
+    } else if (dtype == MXQ_DTYPE_BF16) {
+        *row = ZONE_ROW_BF16;
+        *zshift = 16;
+    } else {
+        *row = ZONE_ROW_F32;
+    }
+}
+
+// Does the round-up zone of the *element* exponent change results?  In nearest / even modes a
+// value in the zone rounds to the next power of two whichever exponent is used, as long as the
+// zone is narrower than half a rounding step: count * 2^t <= 2^(22 - zshift) (largest count 88 for
+// fp32; bf16 has count <= 5 while |exponent| <= 16, i.e. for formats with at most 5 exponent bits).
+inline bool elem_zone_matters(int dtype, int flags, const MxqFmt& f, int rmode) {
+    int row, zs;
+    zone_for(dtype, flags, &row, &zs);
+    if (row == ZONE_ROW_NONE || f.ebits == 0) return false;
+    if (rmode == MXQ_ROUND_FLOOR) return true;
+    if (row == ZONE_ROW_F32) return f.t > 15;
+    return !(f.ebits <= 5 && f.t <= 3);
+}
+
+inline int make_mx_params(int dtype, int scale_bits, int ebits, int mbits, float max_norm, int flush,
+                          int rmode, int flags, MxParams* p, bool* zone_elem, const char* who) {
+    if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
+    if (rmode < 0 || rmode > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown rounding mode %d", who, rmode);
+    if (scale_bits < 1 || scale_bits > 8)
+        return fail(MXQ_ERR_ARGUMENT, "%s: scale_bits %d outside [1, 8]", who, scale_bits);
+    int rc = make_fmt(dtype, ebits, mbits, max_norm, &p->fmt, who);
+    if (rc) return rc;
+    // exponent of max_norm, the way the reference's kernels derive it (mx/cpp/shared_exp.cuh:33)
+    int be = (int)((mxq_bits(max_norm) >> 23) & 0xFF);
+    p->emax = be ? be - 127 : -126;
+    p->scale_emax = (1 << (scale_bits - 1)) - 1;
+    p->flush = flush ? 1 : 0;
+    zone_for(dtype, flags, &p->zone_row, &p->zshift);
+    *zone_elem = elem_zone_matters(dtype, flags, p->fmt, rmode);
+    return MXQ_OK;
+}
+
+inline int make_elem_params(int dtype, int bits, int exp_bits, float max_norm, int rmode,
+                            int saturate, int allow_denorm, int flags, ElemParams* p, const char* who) {
+    if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
+    if (rmode < 0 || rmode > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown rounding mode %d", who, rmode);
+    int rc = make_fmt(dtype, exp_bits, bits, max_norm, &p->fmt, who);
+    if (rc) return rc;
+    p->saturate = saturate ? 1 : 0;
+    p->allow_denorm = allow_denorm ? 1 : 0;
+    zone_for(dtype, flags, &p->zone_row, &p->zshift);
+    return MXQ_OK;
+}
+
+}  // namespace mxq_detail

@@ -1,0 +1,107 @@
+"""Elementwise (bfloat / fp) quantization: the call surface of the reference's mx/elemwise_ops.py,
+served by the native kernels for every supported tensor.
+
+Differences from the reference, on purpose:
+  * there is one implementation per device -- HIP kernels for GPU tensors, the host library for CPU
+    tensors -- and its results are bit-identical to the reference's pure-PyTorch path, so the
+    ``custom_cuda`` switch is accepted but does not change the result;
+  * ``round='dither'`` (stochastic) is not implemented and raises.
+"""
+import torch
+
+from .formats import RoundingMode, _get_format_params, _get_max_norm
+
+
+def _native_round(round):
+    if round not in RoundingMode.string_enums():
+        raise NotImplementedError(
+            "rounding mode %r is not implemented by the native kernels (supported: %s)"
+            % (round, ", ".join(RoundingMode.string_enums())))
+    return int(RoundingMode[round])
+
+
+def _quantize_elemwise_core(A, bits, exp_bits, max_norm, round='nearest',
+                            saturate_normals=False, allow_denorm=True, custom_cuda=False):
+    """Round every element of A to a format with `bits` = sign + implicit one + fraction bits and
+    `exp_bits` exponent bits (0 = integer), overflowing to +-Inf or, if `saturate_normals`,
+    clamping to +-max_norm.  Same contract as mx/elemwise_ops.py:82-170."""
+    rmode = _native_round(round)
+    if A.is_sparse:
+        if A.layout != torch.sparse_coo:
+            raise NotImplementedError("Only COO layout sparse tensors are currently supported.")
+        sp = A.coalesce()
+        vals = _quantize_elemwise_core(sp.values().clone(), bits, exp_bits, max_norm, round=round,
+                                       saturate_normals=saturate_normals,
+                                       allow_denorm=allow_denorm, custom_cuda=custom_cuda)
+        return torch.sparse_coo_tensor(sp.indices(), vals, sp.size(), dtype=sp.dtype,
+                                       device=sp.device, requires_grad=sp.requires_grad)
+
+    from . import custom_extensions
+    A = A.contiguous()
+    if A.device.type == "cuda":
+        return custom_extensions.funcs.quantize_elemwise_func_cuda(
+            A, bits, exp_bits, max_norm, rmode, saturate_normals, allow_denorm)
+    if A.device.type == "cpu":
+        return custom_extensions.funcs.quantize_elemwise_func_cpp(
+            A, bits, exp_bits, max_norm, rmode, saturate_normals, allow_denorm)
+    raise ValueError("Unrecognized device type %s" % A.device.type)
+
+
+def _quantize_elemwise(A, elem_format, round='nearest', custom_cuda=False,
+                       saturate_normals=False, allow_denorm=True):
+    """Quantize to a named element format (mx/elemwise_ops.py:173-188)."""
+    if elem_format is None:
+        return A
+    ebits, mbits, _, max_norm, _ = _get_format_params(elem_format)
+    return _quantize_elemwise_core(A, mbits, ebits, max_norm, round=round,
+                                   allow_denorm=allow_denorm, saturate_normals=saturate_normals,
+                                   custom_cuda=custom_cuda)
+
+
+def _quantize_bfloat(A, bfloat, round='nearest', custom_cuda=False, allow_denorm=True):
+    """bfloatX = 1 sign + 8 exponent + (X - 9) fraction bits (mx/elemwise_ops.py:191-206)."""
+    if bfloat == 0 or bfloat == 32:
+        return A
+    return _quantize_elemwise_core(A, bits=bfloat - 7, exp_bits=8,
+                                   max_norm=_get_max_norm(8, bfloat - 7), round=round,
+                                   allow_denorm=allow_denorm, custom_cuda=custom_cuda)
+
+
+def _quantize_fp(A, exp_bits=None, mantissa_bits=None, round='nearest', custom_cuda=False,
+                 allow_denorm=True):
+    """IEEE-style fpX with Inf/NaN in the top exponent (mx/elemwise_ops.py:209-230)."""
+    if exp_bits is None or mantissa_bits is None:
+        return A
+    return _quantize_elemwise_core(A, bits=mantissa_bits + 2, exp_bits=exp_bits,
+                                   max_norm=_get_max_norm(exp_bits, mantissa_bits + 2),
+                                   round=round, allow_denorm=allow_denorm, custom_cuda=custom_cuda)
+
+
+def quantize_elemwise_op(A, mx_specs, round=None):
+    """Elementwise quantization selected by mx_specs['bfloat'] / ['fp']
+    (mx/elemwise_ops.py:233-267)."""
+    if mx_specs is None:
+        return A
+    if round is None:
+        round = mx_specs['round']
+
+    # torch's own cast is round-to-nearest-even to bfloat16; note it also changes the dtype
+    if mx_specs['bfloat'] == 16 and round == 'even' and torch.cuda.is_bf16_supported() \
+            and mx_specs['bfloat_subnorms'] == True:
+        return A.to(torch.bfloat16)
+
+    if mx_specs['bfloat'] > 0 and mx_specs['fp'] > 0:
+        raise ValueError("Cannot set both [bfloat] and [fp] in mx_specs.")
+    if mx_specs['bfloat'] > 9:
+        return _quantize_bfloat(A, bfloat=mx_specs['bfloat'], round=round,
+                                custom_cuda=mx_specs['custom_cuda'],
+                                allow_denorm=mx_specs['bfloat_subnorms'])
+    if mx_specs['bfloat'] > 0:
+        raise ValueError("Cannot set [bfloat] <= 9 in mx_specs.")
+    if mx_specs['fp'] > 6:
+        return _quantize_fp(A, exp_bits=5, mantissa_bits=mx_specs['fp'] - 6, round=round,
+                            custom_cuda=mx_specs['custom_cuda'],
+                            allow_denorm=mx_specs['bfloat_subnorms'])
+    if mx_specs['fp'] > 0:
+        raise ValueError("Cannot set [fp] <= 6 in mx_specs.")
+    return A

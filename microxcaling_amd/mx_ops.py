@@ -1,0 +1,70 @@
+"""MX block quantization: the call surface of the reference's mx/mx_ops.py, served by the native
+kernels.
+
+One shared 2^k scale per `block_size` consecutive elements along one axis; elements are rounded to
+`elem_format` relative to that scale and returned in the input dtype ("fake quantization").
+
+Differences from the reference, on purpose:
+  * every single-axis case -- any axis, any block size, ragged last block -- is one kernel launch
+    (the reference reshapes, pads and takes a separate max for block sizes above 32 on the last
+    axis, mx/mx_ops.py:226-263); results are bit-identical to its pure-PyTorch path either way,
+    so ``custom_cuda`` is accepted but does not change the result;
+  * sharing an exponent across more than one axis and ``round='dither'`` raise.
+"""
+import torch
+
+from .specs import mx_assert_test
+from .formats import ElemFormat, RoundingMode, _get_format_params
+from .elemwise_ops import _native_round
+
+
+def _quantize_mx(A, scale_bits, elem_format, shared_exp_method="max", axes=None, block_size=0,
+                 round="nearest", flush_fp32_subnorms=False, custom_cuda=False):
+    """Same contract as mx/mx_ops.py:173-298."""
+    if elem_format is None:
+        return A
+    assert scale_bits > 0
+    if axes is None:
+        raise Exception("axes required in order to determine which dimension to apply "
+                        "block size to")
+    axes = [axes] if type(axes) == int else list(axes)
+    axes = [x + A.ndim if x < 0 else x for x in axes]
+    if len(axes) != 1:
+        raise NotImplementedError("the native kernels share exponents along exactly one axis")
+    axis = axes[0]
+    rmode = _native_round(round)
+    ebits, mbits, _, max_norm, _ = _get_format_params(elem_format)
+
+    if shared_exp_method == "none":          # an exponent per element = blocks of one
+        tile = 1
+    elif shared_exp_method == "max":
+        tile = block_size if block_size > 0 else 0      # 0: the whole axis is one block
+    else:
+        raise Exception("Unrecognized shared exponent selection method %s" % shared_exp_method)
+
+    from . import custom_extensions as ce
+    A = A.contiguous()
+    if A.device.type == "cuda":
+        return ce.funcs.quantize_mx_by_tile_func_cuda(
+            A, scale_bits, ebits, mbits, max_norm, tile, axis, flush_fp32_subnorms, rmode)
+    if A.device.type == "cpu":
+        return ce.funcs.quantize_mx_by_tile_func_cpp(
+            A, scale_bits, ebits, mbits, max_norm, tile, axis, flush_fp32_subnorms, rmode)
+    raise ValueError("Unrecognized device type %s" % A.device.type)
+
+
+def quantize_mx_op(A, mx_specs: dict, elem_format=None, block_size=None, axes=None,
+                   round="nearest", expand_and_reshape=False):
+    """Spec-driven entry point used by every MX layer (mx/mx_ops.py:301-331)."""
+    mx_assert_test(mx_specs)
+    if elem_format is None:
+        return A
+    if type(elem_format) is str:
+        elem_format = ElemFormat.from_str(elem_format)
+    if block_size is None:
+        block_size = mx_specs["block_size"]
+    scale_bits = mx_specs["scale_bits"] if mx_specs["scale_bits"] != 0 else 8
+    return _quantize_mx(A, scale_bits, elem_format, block_size=block_size, axes=axes, round=round,
+                        shared_exp_method=mx_specs["shared_exp_method"],
+                        flush_fp32_subnorms=mx_specs["mx_flush_fp32_subnorms"],
+                        custom_cuda=mx_specs["custom_cuda"])

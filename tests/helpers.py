@@ -1,0 +1,68 @@
+"""Shared helpers for the test-suite: bit-pattern comparison and fixture access."""
+import importlib.util
+import json
+import os
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLDEN = os.path.join(HERE, "golden")
+
+
+def canon_bits(t):
+    """Integer bit patterns of a float tensor with every NaN mapped to the canonical quiet NaN
+    (NaN payloads are not part of the parity contract; the sign of zero is)."""
+    t = t.detach().cpu().contiguous()
+    if t.dtype == torch.float32:
+        b = t.view(torch.int32).numpy()
+        return np.where(np.isnan(t.numpy()), np.int32(0x7FC00000), b)
+    if t.dtype == torch.bfloat16:
+        b = t.view(torch.int16).numpy()
+        return np.where(np.isnan(t.float().numpy()), np.int16(0x7FC0), b)
+    if t.dtype == torch.float16:
+        b = t.view(torch.int16).numpy()
+        return np.where(np.isnan(t.float().numpy()), np.int16(0x7E00), b)
+    raise TypeError(t.dtype)
+
+
+def assert_bits_equal(got, want, what=""):
+    g, w = canon_bits(got), canon_bits(want)
+    assert g.shape == w.shape, (what, g.shape, w.shape)
+    bad = np.flatnonzero(g.reshape(-1) != w.reshape(-1))
+    if bad.size:
+        i = int(bad[0])
+        gf = got.detach().cpu().reshape(-1)[i].item()
+        wf = want.detach().cpu().reshape(-1)[i].item()
+        raise AssertionError("%s: %d of %d elements differ; first at flat index %d: got %r (0x%x) "
+                             "want %r (0x%x)" % (what, bad.size, g.size, i, gf,
+                                                 int(g.reshape(-1)[i]) & 0xFFFFFFFF, wf,
+                                                 int(w.reshape(-1)[i]) & 0xFFFFFFFF))
+
+
+def from_bits(a, dtype):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    return t.view(dtype)
+
+
+_golden = None
+
+
+def golden():
+    """(npz arrays, json meta) written by tests/golden/gen_reference_vectors.py."""
+    global _golden
+    if _golden is None:
+        z = np.load(os.path.join(GOLDEN, "reference_vectors.npz"))
+        with open(os.path.join(GOLDEN, "reference_vectors.json")) as f:
+            meta = json.load(f)
+        _golden = (z, meta)
+    return _golden
+
+
+def golden_inputs_module():
+    """The fixture generator, imported for its seeded input builders (its main() is not run)."""
+    spec = importlib.util.spec_from_file_location(
+        "gen_reference_vectors", os.path.join(GOLDEN, "gen_reference_vectors.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
