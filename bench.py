@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of the MX quantization hot path on one MI355X.
+
+One "step" = one `_quantize_mx` pass (MXFP8 e4m3, block 32 along the last axis, scale_bits 8,
+round 'nearest') over a seeded fp32 [8192, 8192] tensor that is already resident in HBM.
+Prints ONE JSON line: whole-job throughput in GB/s of algorithmic bytes (8 B per element: fp32 in,
+fp32 out), the roofline position of the kernel from HIP events around every launch, and the CPU
+baseline (the torch op-sequence oracle timed on this box's host cores on a bounded row sample).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+Workloads (all sizes from BASELINE.json):
+    mxfp8_fp32_8192      headline (default)
+    mxfp8_fp32_4096      config 1 (fits in the 256 MB Infinity Cache -- not an HBM figure)
+    mxfp6_e3m2_bf16_m1 / mxfp6_e2m3_bf16_m1 / mxfp4_bf16_m1      config 2, axis -1
+    mxfp6_e3m2_bf16_m2 / mxfp6_e2m3_bf16_m2 / mxfp4_bf16_m2      config 2, axis -2
+    elem_bf16_fp32 / elem_fp16_fp32                              config 3, elementwise
+    reduce_sum_m1 / reduce_max_m1 / reduce_sum_0 / reduce_max_0  config 3, reductions
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E peak
+
+
+def outlier_bf16(rows, cols, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, cols, generator=g)
+    idx = torch.randperm(cols, generator=g)[: cols // 100]
+    scale = torch.ones(cols)
+    scale[idx] = torch.exp(2.0 * torch.randn(idx.numel(), generator=g))
+    return (x * scale).to(torch.bfloat16)
+
+
+def wide_fp32(rows, cols, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, cols, generator=g) .double()
+    x = x * 10.0 ** (torch.rand(rows, cols, generator=g).double() * 80 - 40)
+    x = x.to(torch.float32).reshape(-1)
+    n = x.numel()
+    sp = torch.randperm(n, generator=g)
+    k = n // 1000
+    x[sp[:k]] = torch.tensor([float("inf"), -float("inf"), float("nan")]).repeat(k // 3 + 1)[:k]
+    m = n // 100
+    sub = torch.randint(1, 1 << 23, (m,), generator=g, dtype=torch.int32)
+    sub |= torch.randint(0, 2, (m,), generator=g, dtype=torch.int32) << 31
+    x[sp[k:k + m]] = sub.view(torch.float32)
+    return x.reshape(rows, cols)
+
+
+def make_workload(name):
+    """-> dict(x=cpu tensor, gpu=callable(xd), cpu=callable(x_rows), bytes=algorithmic bytes per
+    step, dtype=..., desc=...)"""
+    from microxcaling_amd.mx_ops import _quantize_mx
+    from microxcaling_amd.elemwise_ops import _quantize_elemwise_core
+    from microxcaling_amd.custom_extensions import funcs
+    from oracle import mx_oracle as O
+
+    def mx(fmt, axis, rnd="nearest"):
+        return (lambda t: _quantize_mx(t, 8, fmt, axes=[axis], block_size=32, round=rnd),
+                lambda t: O.quantize_mx(t, 8, fmt, axes=[axis], block_size=32, round=rnd))
+
+    if name in ("mxfp8_fp32_8192", "mxfp8_fp32_4096"):
+        n = 8192 if name.endswith("8192") else 4096
+        x = torch.randn(n, n, generator=torch.Generator().manual_seed(0))
+        g, c = mx("fp8_e4m3", -1)
+        return dict(x=x, gpu=g, cpu=c, bytes=x.numel() * 8, dtype="f32", sample_axis=0,
+                    desc="_quantize_mx fp8_e4m3 block 32 axis -1 nearest, fp32 [%d,%d] N(0,1)" % (n, n))
+    if name.startswith("mxfp") and "_bf16_m" in name:
+        fmt = {"mxfp6_e3m2": "fp6_e3m2", "mxfp6_e2m3": "fp6_e2m3", "mxfp4": "fp4_e2m1"}[name.split("_bf16_")[0]]
+        axis = -1 if name.endswith("m1") else -2
+        x = outlier_bf16(8192, 8192, 7)
+        g, c = mx(fmt, axis)
+        return dict(x=x, gpu=g, cpu=c, bytes=x.numel() * 4, dtype="bf16", sample_axis=0 if axis == -1 else 1,
+                    desc="_quantize_mx %s block 32 axis %d nearest, bf16 [8192,8192] with outlier columns" % (fmt, axis))
+    if name in ("elem_bf16_fp32", "elem_fp16_fp32"):
+        bits, eb, mn = (9, 8, 2 ** 127 * 255 / 128) if "bf16" in name else (12, 5, 65504.0)
+        x = wide_fp32(16384, 8192, 11)
+        return dict(x=x, gpu=lambda t: _quantize_elemwise_core(t, bits, eb, mn, round="nearest"),
+                    cpu=lambda t: O.quantize_elemwise_core(t, bits, eb, mn, round="nearest"),
+                    bytes=x.numel() * 8, dtype="f32", sample_axis=0,
+                    desc="_quantize_elemwise_core bits=%d exp_bits=%d nearest, fp32 [16384,8192] wide range" % (bits, eb))
+    if name.startswith("reduce_"):
+        x = wide_fp32(16384, 8192, 13)
+        x[~torch.isfinite(x)] = 1.0
+        op, ax = name.split("_")[1], name.split("_")[2]
+        fn = {("sum", "m1"): funcs.reduce_sum_inner_dim, ("max", "m1"): funcs.reduce_max_inner_dim,
+              ("sum", "0"): funcs.reduce_sum_outer_dim, ("max", "0"): funcs.reduce_max_outer_dim}[(op, ax)]
+        dim = -1 if ax == "m1" else 0
+        cpu = (lambda t: t.sum(dim)) if op == "sum" else (lambda t: t.max(dim).values)
+        return dict(x=x, gpu=fn, cpu=cpu, bytes=x.numel() * 4, dtype="f32", sample_axis=0 if dim == -1 else 1,
+                    desc="reduce %s over axis %d, fp32 [16384,8192]" % (op, dim))
+    raise SystemExit("unknown workload %r" % name)
+
+
+def cpu_baseline(wl, budget_s=15.0):
+    """Time the oracle on the host cores: repeated passes over the FULL workload tensor (so caches
+    do not flatter it) until about `budget_s` seconds of CPU work are spent; median pass."""
+    x = wl["x"]
+    cores = min(os.cpu_count() or 1, 16)      # the box's CPU share for one GPU
+    torch.set_num_threads(cores)
+    wl["cpu"](x[:64, :64].contiguous())       # warm up the op sequence
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_all < budget_s and len(times) < 25):
+        t0 = time.perf_counter()
+        wl["cpu"](x)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_all > 4 * budget_s:
+            break
+    times.sort()
+    t = times[len(times) // 2]
+    return {"value": round(wl["bytes"] / t / 1e9, 4), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "the full workload tensor (%s), %d passes in %.1f s, median pass %.3f s; torch %s "
+                      "op-by-op oracle (oracle/mx_oracle.py), %d threads"
+                      % ("x".join(str(n) for n in x.shape), len(times), time.perf_counter() - t_all, t,
+                         torch.__version__, cores)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="mxfp8_fp32_8192")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: the quantization path has no multi-GPU part "
+                         "(blocks are independent; see DESIGN.md); run with --gpus 1")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
+
+    wl = make_workload(args.workload)
+    dev = torch.device("cuda:0")
+    xd = wl["x"].to(dev)
+    torch.cuda.synchronize()
+
+    for _ in range(args.warmup):
+        wl["gpu"](xd)
+    torch.cuda.synchronize()
+
+    # timed region: K steps, HIP events around every launch on the stream the kernels run on
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record()
+        y = wl["gpu"](xd)
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    del y
+
+    ms_per_step = wall * 1e3 / args.steps
+    kern_ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
+    kern_avg_ms = sum(kern_ms) / len(kern_ms)
+    value = wl["bytes"] / (ms_per_step * 1e-3) / 1e9
+    achieved = wl["bytes"] / (kern_avg_ms * 1e-3) / 1e9
+
+    traffic = None
+    tfile = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
+    if os.path.exists(tfile):
+        with open(tfile) as f:
+            traffic = json.load(f).get(args.workload)
+
+    out = {
+        "metric": "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"], "data": "synthetic",
+        "config": {"workload": args.workload, "detail": wl["desc"],
+                   "algorithmic_bytes_per_step": wl["bytes"],
+                   "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "kernel_ms_avg": round(kern_avg_ms, 5), "kernel_ms_median": round(kern_ms[len(kern_ms) // 2], 5),
+                     "kernel_ms_min": round(kern_ms[0], 5)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(out, ensure_ascii=False), flush=True)
+
+
+if __name__ == "__main__":
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    main()

@@ -1,0 +1,57 @@
+"""ctypes access to the C restatement (libmxq_oracle.so).  TEST INFRASTRUCTURE ONLY."""
+import ctypes
+import os
+
+import torch
+
+from . import build_oracle
+from .mx_oracle import format_params
+
+_lib = None
+_DT = {torch.float32: 0, torch.bfloat16: 2}
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(build_oracle.LIB):
+            build_oracle.build(verbose=False)
+        _lib = ctypes.CDLL(build_oracle.LIB)
+        i64, ci, cf, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+        _lib.oracle_quantize_elemwise.argtypes = [vp, vp, ci, i64, ci, ci, cf, ci, ci, ci]
+        _lib.oracle_quantize_elemwise.restype = None
+        _lib.oracle_quantize_mx.argtypes = [vp, vp, ci, i64, i64, i64, ci, ci, ci, ci, cf, i64, ci, ci]
+        _lib.oracle_quantize_mx.restype = None
+    return _lib
+
+
+_RMODE = {"nearest": 0, "floor": 1, "even": 2}
+
+
+def quantize_elemwise_core(A, bits, exp_bits, max_norm, round="nearest", saturate_normals=False,
+                           allow_denorm=True):
+    A = A.contiguous()
+    out = torch.empty_like(A)
+    lib().oracle_quantize_elemwise(A.data_ptr(), out.data_ptr(), _DT[A.dtype], A.numel(), bits,
+                                   exp_bits, max_norm, _RMODE[round], int(saturate_normals),
+                                   int(allow_denorm))
+    return out
+
+
+def quantize_mx(A, scale_bits, elem_format, axes, block_size=0, round="nearest",
+                flush_fp32_subnorms=False):
+    A = A.contiguous()
+    (axis,) = [axes] if isinstance(axes, int) else axes
+    axis = axis + A.ndim if axis < 0 else axis
+    pre = 1
+    for n in A.shape[:axis]:
+        pre *= n
+    post = 1
+    for n in A.shape[axis + 1:]:
+        post *= n
+    ebits, mbits, emax, max_norm, _ = format_params(elem_format)
+    out = torch.empty_like(A)
+    lib().oracle_quantize_mx(A.data_ptr(), out.data_ptr(), _DT[A.dtype], pre, A.shape[axis], post,
+                             scale_bits, ebits, mbits, emax, max_norm, block_size,
+                             int(flush_fp32_subnorms), _RMODE[round])
+    return out
