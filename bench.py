@@ -183,7 +183,7 @@ def main():
     tfile = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
     if os.path.exists(tfile):
         with open(tfile) as f:
-            traffic = json.load(f).get(args.workload)
+            traffic = json.load(f).get(args.workload)       # measured separately with rocprofv3 --pmc
 
     out = {
         "metric": "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s",

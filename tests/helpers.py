@@ -8,6 +8,7 @@ import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 GOLDEN = os.path.join(HERE, "golden")
+ROOT_DIR = os.path.dirname(HERE)
 
 
 def canon_bits(t):

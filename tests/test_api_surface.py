@@ -1,0 +1,87 @@
+"""The host-side mirror of the reference's interface: formats, specs, spec-driven entry points."""
+import argparse
+
+import pytest
+import torch
+
+from helpers import assert_bits_equal
+from oracle import mx_oracle as O
+import microxcaling_amd as mx
+from microxcaling_amd.formats import ElemFormat, RoundingMode, _get_format_params
+from microxcaling_amd.specs import (MxSpecs, add_mx_args, apply_mx_specs, finalize_mx_specs,
+                                    get_backwards_mx_specs, get_default_mx_specs, get_mx_specs)
+from microxcaling_amd.mx_ops import quantize_mx_op
+from microxcaling_amd.elemwise_ops import quantize_elemwise_op, _quantize_bfloat, _quantize_fp
+
+
+def test_format_params_match_closed_forms():
+    """mx/tests/test_formats.py:12-95."""
+    for name in ("float16", "fp16", "bfloat16", "bf16", "fp8_e5m2", "fp8_e4m3", "fp6_e3m2",
+                 "fp6_e2m3", "fp4_e2m1", "fp4", "int8", "int4", "int2"):
+        assert _get_format_params(name) == O.format_params(name), name
+    assert _get_format_params(ElemFormat.fp8_e4m3)[3] == 448.0
+    assert [int(m) for m in RoundingMode] == [0, 1, 2]
+    assert RoundingMode.string_enums() == ["nearest", "floor", "even"]
+    assert ElemFormat.from_str("FP4") is ElemFormat.fp4_e2m1
+    with pytest.raises(Exception):
+        ElemFormat.from_str("fp5")
+
+
+def test_specs_defaults_and_dependencies():
+    d = get_default_mx_specs()
+    assert d["scale_bits"] == 0 and d["round"] == "nearest" and d["custom_cuda"] is False
+    assert d["bfloat_subnorms"] is True and d["shared_exp_method"] == "max"
+    assert finalize_mx_specs({}) is None
+    s = finalize_mx_specs({"w_elem_format": "fp8_e4m3", "a_elem_format": "fp6_e2m3",
+                           "a_elem_format_bp_os": "fp4_e2m1", "round": "even", "block_size": 32})
+    assert s["w_elem_format_bp"] == "fp8_e4m3" and s["a_elem_format_bp_ex"] == "fp6_e2m3"
+    assert s["a_elem_format_bp_os"] == "fp4_e2m1"
+    assert s["round_mx_output"] == "even" and s["round_mx_input_grad_input"] == "even"
+    with pytest.raises(KeyError):
+        apply_mx_specs({"no_such_key": 1})
+    with pytest.raises(AssertionError):
+        MxSpecs({"no_such_key": 1})
+    b = get_backwards_mx_specs(MxSpecs({"quantize_backprop": False, "bfloat": 16, "block_size": 32}))
+    assert b["bfloat"] == 0 and b["block_size"] == 0
+
+
+def test_specs_argparse_round_trip():
+    """mx/tests/test_finalize_mxfp.py:17-43 and the self-test at mx/specs.py:366-388."""
+    p = add_mx_args(argparse.ArgumentParser())
+    assert get_mx_specs(p.parse_args([])) is None
+    s = get_mx_specs(p.parse_args(["--bfloat", "16", "--no_quantize_backprop", "--custom_cuda"]
+                                  if torch.cuda.is_available() else ["--bfloat", "16", "--no_quantize_backprop"]))
+    assert s["bfloat"] == 16 and s["quantize_backprop"] is False
+    for k, v in get_default_mx_specs().items():
+        if k not in ("bfloat", "quantize_backprop", "custom_cuda"):
+            assert s[k] == v, k
+    s = get_mx_specs(p.parse_args(["--w_elem_format", "fp6_e3m2", "--block_size", "32", "--skip_early_exit"]))
+    assert s["w_elem_format_bp"] == "fp6_e3m2" and s["block_size"] == 32
+
+
+def test_spec_driven_ops_on_cpu_tensors():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(8, 64, generator=g)
+    specs = finalize_mx_specs({"a_elem_format": "fp8_e4m3", "block_size": 32, "bfloat": 16})
+    y = quantize_mx_op(x, specs, elem_format=specs["a_elem_format"], axes=[-1], round="floor")
+    assert_bits_equal(y, O.quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=32, round="floor"))
+    assert quantize_mx_op(x, specs, elem_format=None) is x
+    y = quantize_elemwise_op(x, specs)
+    assert_bits_equal(y, O.quantize_bfloat(x, 16))
+    specs["round"] = "even"
+    assert quantize_elemwise_op(x, specs).dtype == torch.bfloat16          # torch cast shortcut
+    assert quantize_elemwise_op(x, None) is x
+    bad = get_default_mx_specs()
+    bad["bfloat"], bad["fp"] = 16, 16
+    with pytest.raises(ValueError):
+        quantize_elemwise_op(x, bad)
+    assert _quantize_bfloat(x, 32) is x and _quantize_fp(x) is x
+    assert_bits_equal(_quantize_fp(x, exp_bits=5, mantissa_bits=10, round="even"), x.half().float())
+
+
+def test_sparse_coo_values_are_quantized():
+    from microxcaling_amd.elemwise_ops import _quantize_elemwise_core
+    x = torch.tensor([[0.0, 1.2345], [3.21, 0.0]]).to_sparse()
+    y = _quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128, round="even")
+    assert y.is_sparse
+    assert_bits_equal(y.to_dense(), x.to_dense().to(torch.bfloat16).float())

@@ -1,0 +1,257 @@
+"""CPU-side checks of the native code: both shared libraries load and export every symbol that
+include/mxq.h declares; the kernels' scalar arithmetic (mxq_core.h, compiled for the host in
+libmxq_host.so) is bit-identical to the oracle on exhaustive sweeps; the round-up-zone tables
+agree with torch's CPU log2 on this machine.  No GPU compute happens here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import ROOT_DIR, assert_bits_equal, golden_inputs_module
+from oracle import mx_oracle as O
+from microxcaling_amd import _lib
+from microxcaling_amd.custom_extensions import funcs
+from microxcaling_amd.formats import _get_format_params
+from microxcaling_amd.mx_ops import _quantize_mx
+from microxcaling_amd.elemwise_ops import _quantize_elemwise_core
+
+ROUNDS = ["nearest", "floor", "even"]
+RMODE = {"nearest": 0, "floor": 1, "even": 2}
+MX_FORMATS = ["fp8_e4m3", "fp8_e5m2", "fp6_e3m2", "fp6_e2m3", "fp4_e2m1", "int8", "int4", "int2"]
+
+
+# ---- the C ABI ----------------------------------------------------------------------------------
+def declared_symbols():
+    text = open(os.path.join(ROOT_DIR, "include", "mxq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mxq_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_symbols()
+    for must in ("mxq_quantize_mx_by_tile", "mxq_quantize_mx_given_max", "mxq_quantize_elemwise",
+                 "mxq_reduce_sum_inner", "mxq_reduce_max_inner", "mxq_last_error",
+                 "mxq_host_quantize_mx_given_max", "mxq_host_quantize_elemwise"):
+        assert must in names
+
+
+def test_libraries_export_every_declared_symbol():
+    assert os.path.exists(_lib.GPU_LIB_PATH), "run python -m microxcaling_amd.build_ext"
+    gpu = ctypes.CDLL(_lib.GPU_LIB_PATH)          # loads without a GPU; nothing is launched
+    host = ctypes.CDLL(_lib.HOST_LIB_PATH)
+    for name in declared_symbols():
+        lib = host if name.startswith("mxq_host_") else gpu
+        assert hasattr(lib, name), "%s is declared in include/mxq.h but not exported" % name
+    assert set(_lib.GPU_SYMBOLS) | set(_lib.HOST_SYMBOLS) == set(declared_symbols())
+
+
+def test_gpu_entry_points_reject_bad_arguments_without_a_gpu():
+    lib = _lib.gpu()
+    assert lib.mxq_version() >= 100
+    # argument errors are detected before anything touches the device
+    rc = lib.mxq_quantize_mx_by_tile(None, None, 7, 1, 32, 1, 8, 4, 5, 448.0, 32, 0, 0, 0, None)
+    assert rc == 1 and b"dtype" in lib.mxq_last_error()
+    rc = lib.mxq_quantize_mx_by_tile(None, None, 0, 1, 32, 1, 9, 4, 5, 448.0, 32, 0, 0, 0, None)
+    assert rc == 1 and b"scale_bits" in lib.mxq_last_error()
+    rc = lib.mxq_quantize_elemwise(None, None, 0, 16, 30, 8, 1.0, 0, 0, 1, 0, None)
+    assert rc == 1 and b"bits" in lib.mxq_last_error()
+    rc = lib.mxq_quantize_elemwise(None, None, 0, 16, 9, 8, 1.0, 5, 0, 1, 0, None)
+    assert rc == 1 and b"rounding" in lib.mxq_last_error()
+    rc = lib.mxq_quantize_mx_by_tile(None, None, 0, 1, 32, 1, 8, 4, 5, 448.0, 32, 0, 0, 0, None)
+    assert rc == 1 and b"null" in lib.mxq_last_error()
+    assert lib.mxq_quantize_mx_by_tile(None, None, 0, 0, 32, 1, 8, 4, 5, 448.0, 32, 0, 0, 0, None) == 0
+    assert lib.mxq_reduce_outer_workspace_bytes(16384, 8192) > 0
+
+
+def test_host_functions_reject_gpu_only_misuse():
+    x = torch.zeros(4, 4)
+    with pytest.raises(RuntimeError):
+        funcs.quantize_mx_by_tile_func_cuda(x, 8, 4, 5, 448.0, 32, 1)        # CPU tensor
+    with pytest.raises(RuntimeError):
+        funcs.quantize_elemwise_func_cuda(x, 9, 8, 1.0)
+    with pytest.raises(RuntimeError):
+        funcs.reduce_sum_inner_dim(x)
+    with pytest.raises(RuntimeError):
+        funcs.quantize_mx_func_cpp(torch.zeros(2, 2, 2, 2, 2, 2), 8, 4, 5, 448.0,
+                                   torch.zeros(1), 0, False)                  # ndim > 5
+    with pytest.raises(NotImplementedError):
+        _quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=2, round="dither")
+    with pytest.raises(NotImplementedError):
+        _quantize_mx(x, 8, "fp8_e4m3", axes=[0, 1], block_size=2)
+
+
+# ---- round-up zones against torch's own log2 ----------------------------------------------------
+def test_zone_tables_match_torch_log2_bf16():
+    codes = torch.arange(1, 0x7F80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    want = torch.floor(torch.log2(codes)).float()
+    # Read the kernels' floor(log2|x|) back through the quantizer: a block holding just x, int2
+    # elements (values {0, +-1} x 2**E), floor rounding.
+    y = _quantize_mx(codes.view(-1, 1), 8, "int2", axes=[1], block_size=1, round="floor").float()
+    # int2 with shared exponent E: x / 2**E in [1, 2) floors to 1 when E is the true exponent, and
+    # x / 2**(E+1) in [0.5, 1) floors to 0 when the zone pushed E up.
+    true_k = torch.floor(torch.log2(codes.double())).float()
+    got = torch.where(y.view(-1) == 0, true_k + 1, true_k)
+    inrange = (want - 0).abs() <= 127                          # scale exponent clamps at +-127
+    assert torch.equal(got[inrange], want[inrange])
+
+
+def test_zone_tables_match_torch_log2_fp32():
+    parts = []
+    for be in range(1, 255):
+        parts.append(((be << 23) + (1 << 23) - 1 - torch.arange(0, 128, dtype=torch.int64)))
+    for k in range(-149, -126):                                  # subnormal binades, top codes
+        hi = (1 << (k + 150)) - 1
+        c = hi - torch.arange(0, 128, dtype=torch.int64)
+        parts.append(c[c >= (1 << (k + 149))])
+    x = torch.cat(parts).to(torch.int32).view(torch.float32)
+    want = torch.floor(torch.log2(x))
+    y = _quantize_mx(x.view(-1, 1), 8, "int2", axes=[1], block_size=1, round="floor")
+    true_k = torch.floor(torch.log2(x.double())).float()
+    got = torch.where(y.view(-1) == 0, true_k + 1, true_k)
+    inrange = want.abs() <= 127
+    assert inrange.sum() > 30000
+    assert torch.equal(got[inrange], want[inrange])
+
+
+# ---- exhaustive sweeps: host build of the kernel arithmetic vs the torch oracle ------------------
+def all_bf16():
+    return torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+
+
+@pytest.mark.parametrize("bits,ebits,max_norm", [(9, 8, 2 ** 127 * 255 / 128), (12, 5, 65504.0),
+                                                 (5, 4, 448.0), (4, 5, 57344.0), (3, 2, 6.0),
+                                                 (8, 0, 127 / 64), (5, 8, 2 ** 127 * 15 / 8)])
+@pytest.mark.parametrize("rnd", ROUNDS)
+def test_elementwise_every_bf16_code(bits, ebits, max_norm, rnd):
+    x = all_bf16()
+    for sat in (False, True):
+        for den in (True, False):
+            want = O.quantize_elemwise_core(x.clone(), bits, ebits, max_norm, round=rnd,
+                                            saturate_normals=sat, allow_denorm=den)
+            got = _quantize_elemwise_core(x.clone(), bits, ebits, max_norm, round=rnd,
+                                          saturate_normals=sat, allow_denorm=den)
+            assert_bits_equal(got, want, "sat=%s den=%s" % (sat, den))
+
+
+def fp32_probe_values():
+    """Every (8 exponent, 9 mantissa)-bit value (the sweep of mx/tests/test_quantize_mx.py:52),
+    the top 96 codes of every binade, specials and seeded random bit patterns."""
+    e = torch.arange(0, 256, dtype=torch.int64).view(-1, 1)
+    m = torch.arange(0, 512, dtype=torch.int64).view(1, -1)
+    a = ((e << 23) | (m << 14)).reshape(-1)
+    tops = ((torch.arange(0, 255, dtype=torch.int64).view(-1, 1) << 23) + (1 << 23) - 1
+            - torch.arange(0, 96, dtype=torch.int64).view(1, -1)).reshape(-1)
+    g = torch.Generator().manual_seed(5)
+    r = torch.randint(0, 2 ** 31 - 1, (100000,), generator=g, dtype=torch.int64)
+    c = torch.cat([a, tops[tops > 0], r])
+    c = torch.cat([c, c | (1 << 31)])
+    return c.to(torch.int32).view(torch.float32)
+
+
+@pytest.mark.parametrize("bits,ebits,max_norm", [(9, 8, 2 ** 127 * 255 / 128), (12, 5, 65504.0),
+                                                 (5, 4, 448.0), (8, 0, 127 / 64), (24, 8, 3.4028234663852886e38)])
+@pytest.mark.parametrize("rnd", ROUNDS)
+def test_elementwise_fp32_probes(bits, ebits, max_norm, rnd):
+    x = fp32_probe_values()
+    for sat, den in ((False, True), (True, False)):
+        want = O.quantize_elemwise_core(x.clone(), bits, ebits, max_norm, round=rnd,
+                                        saturate_normals=sat, allow_denorm=den)
+        got = _quantize_elemwise_core(x.clone(), bits, ebits, max_norm, round=rnd,
+                                      saturate_normals=sat, allow_denorm=den)
+        assert_bits_equal(got, want, "sat=%s den=%s" % (sat, den))
+
+
+def bf16_blocks(Mcode):
+    """[n, 32] bf16 blocks: column 0 is the block maximum, the other 31 columns sweep every finite
+    bf16 code whose magnitude does not exceed it."""
+    codes = all_bf16()
+    M = torch.tensor([Mcode], dtype=torch.int16).view(torch.bfloat16)
+    sel = codes[torch.isfinite(codes.float()) & (codes.float().abs() <= M.float())]
+    n = (sel.numel() + 30) // 31 * 31
+    body = torch.cat([sel, torch.zeros(n - sel.numel(), dtype=torch.bfloat16)]).view(-1, 31)
+    return torch.cat([M.expand(body.shape[0], 1), body], dim=1).contiguous()
+
+
+# block maxima: powers of two and zone / top-of-binade mantissas across the whole exponent range
+_MCODES = [(be << 7) | man for be in (0, 1, 2, 60, 110, 120, 124, 126, 127, 128, 130, 133, 140, 200,
+                                      250, 254) for man in (0, 0x58, 0x7B, 0x7F)] + [1, 3, 0x40]
+
+
+@pytest.mark.parametrize("fmt", MX_FORMATS)
+@pytest.mark.parametrize("rnd", ROUNDS)
+def test_mx_every_bf16_code_under_many_scales(fmt, rnd):
+    ebits, mbits, _, max_norm, _ = _get_format_params(fmt)
+    for Mcode in _MCODES:
+        if Mcode == 0:
+            continue
+        x = bf16_blocks(Mcode)
+        want = O.quantize_mx(x.clone(), 8, fmt, axes=[-1], block_size=32, round=rnd)
+        got = _quantize_mx(x.clone(), 8, fmt, axes=[-1], block_size=32, round=rnd)
+        assert_bits_equal(got, want, "max code 0x%04x" % Mcode)
+        # the variant that rounds to bf16 after every op must agree with the lean one
+        full = funcs.quantize_mx_by_tile_func_cpp(x.clone(), 8, ebits, mbits, max_norm, 32, 1, False,
+                                                  RMODE[rnd], round_every_op=True)
+        assert_bits_equal(full, want, "every-op variant, max code 0x%04x" % Mcode)
+
+
+@pytest.mark.parametrize("fmt", ["fp8_e4m3", "fp4_e2m1", "int4"])
+@pytest.mark.parametrize("rnd", ROUNDS)
+@pytest.mark.parametrize("scale_bits,flush", [(8, False), (5, True), (5, False), (8, True)])
+def test_mx_fp32_encoding_sweep(fmt, rnd, scale_bits, flush):
+    """The reference's own sweep (mx/tests/test_quantize_mx.py:47-74): all 2^18 (8, 9)-bit values,
+    block sizes 8 / 9 / 64."""
+    e = torch.arange(0, 255, dtype=torch.int64).view(-1, 1)
+    m = torch.arange(0, 512, dtype=torch.int64).view(1, -1)
+    c = ((e << 23) | (m << 14)).reshape(-1)
+    x = torch.cat([c, c | (1 << 31)]).to(torch.int32).view(torch.float32)
+    for bs in (8, 9, 64):
+        want = O.quantize_mx(x.clone(), scale_bits, fmt, axes=[-1], block_size=bs, round=rnd,
+                             flush_fp32_subnorms=flush)
+        got = _quantize_mx(x.clone(), scale_bits, fmt, axes=[-1], block_size=bs, round=rnd,
+                           flush_fp32_subnorms=flush)
+        assert_bits_equal(got, want, "block %d" % bs)
+
+
+@pytest.mark.parametrize("fmt", MX_FORMATS)
+@pytest.mark.parametrize("rnd", ROUNDS)
+def test_mx_fp32_zone_blocks(fmt, rnd):
+    gen = golden_inputs_module()
+    x = gen.fp32_zone_cases()
+    want = O.quantize_mx(x.clone(), 8, fmt, axes=[-1], block_size=32, round=rnd)
+    got = _quantize_mx(x.clone(), 8, fmt, axes=[-1], block_size=32, round=rnd)
+    assert_bits_equal(got, want)
+
+
+def test_cpp_entry_points_follow_the_reference_call_pattern():
+    """quantize_mx_func_cpp is called with the blocked view and its abs-max
+    (mx/mx_ops.py:244-263)."""
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(6, 128, generator=g)
+    ebits, mbits, _, max_norm, _ = _get_format_params("fp6_e3m2")
+    xb = x.view(6, 4, 32)
+    mv = xb.abs().max(dim=2, keepdim=True).values
+    got = funcs.quantize_mx_func_cpp(xb.contiguous(), 8, ebits, mbits, max_norm, mv, 2, False, 0)
+    want = O.quantize_mx(x, 8, "fp6_e3m2", axes=[-1], block_size=32)
+    assert_bits_equal(got.view(6, 128), want)
+    got = funcs.quantize_elemwise_func_cpp(x, 9, 8, 2 ** 127 * 255 / 128, 2, False, True)
+    assert_bits_equal(got, x.to(torch.bfloat16).float())
+
+
+@pytest.mark.parametrize("shape,axis,bs", [((3, 70, 5), 1, 32), ((4, 64), 0, 32), ((7, 90), 1, 9),
+                                           ((6, 33), 1, 0), ((2, 40, 3, 4), 1, 32), ((65, 7), 0, 10)])
+def test_mx_shapes_on_host(shape, axis, bs):
+    g = torch.Generator().manual_seed(sum(shape))
+    for dtype in (torch.float32, torch.bfloat16):
+        x = (torch.randn(*shape, generator=g) * torch.exp(torch.randn(*shape, generator=g))).to(dtype)
+        want = O.quantize_mx(x, 8, "fp8_e4m3", axes=[axis], block_size=bs)
+        assert_bits_equal(_quantize_mx(x, 8, "fp8_e4m3", axes=[axis], block_size=bs), want)
+
+
+def test_shared_exp_method_none_is_block_of_one():
+    x = torch.randn(5, 16, generator=torch.Generator().manual_seed(2))
+    a = _quantize_mx(x, 8, "fp8_e4m3", shared_exp_method="none", axes=[-1], block_size=4)
+    b = O.quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=1)
+    assert_bits_equal(a, b)

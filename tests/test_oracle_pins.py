@@ -1,0 +1,380 @@
+"""Pins the CPU oracle (oracle/mx_oracle.py and the C restatement) to facts it did not produce
+itself: the literal known-answer vectors of the reference's own tests, library special cases
+(torch's bf16 / fp16 / fp8 casts), closed-form format constants, an exact-rational brute force,
+and the golden vectors written from the reference's pure path (tests/golden/)."""
+import hashlib
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_bits_equal, canon_bits, from_bits, golden, golden_inputs_module
+from oracle import c_oracle as C
+from oracle import mx_oracle as O
+
+inf, nan = float("inf"), float("nan")
+ROUNDS = ["nearest", "floor", "even"]
+MX_FORMATS = ["fp8_e4m3", "fp8_e5m2", "fp6_e3m2", "fp6_e2m3", "fp4_e2m1", "int8", "int4"]
+ORACLES = [pytest.param(O, id="torch"), pytest.param(C, id="c")]
+
+
+def same_values(got, want):
+    """The reference's own comparison (mx/tests/common_lib.py:91-134): NaN and Inf positions must
+    coincide (they are interchangeable there), everything else must be equal."""
+    got, want = got.float(), torch.as_tensor(want, dtype=torch.float32)
+    bad_g, bad_w = ~torch.isfinite(got), ~torch.isfinite(want)
+    assert torch.equal(bad_g, bad_w), (got, want)
+    assert torch.equal(torch.where(bad_g, torch.zeros_like(got), got),
+                       torch.where(bad_w, torch.zeros_like(want), want)), (got, want)
+
+
+# ---- format constants: mx/tests/test_formats.py:12-95 -------------------------------------------
+def test_format_constants():
+    assert O.format_params("fp16") == (5, 12, 15, 2 ** 15 * (1 + 1023 / 1024), 2 ** -14)
+    assert O.format_params("float16") == O.format_params("fp16")
+    assert O.format_params("bf16") == (8, 9, 127, 2 ** 127 * (1 + 127 / 128), 2 ** -126)
+    assert O.format_params("bfloat16") == O.format_params("bf16")
+    assert O.format_params("fp8_e5m2") == (5, 4, 15, 2 ** 15 * 1.75, 2 ** -14)
+    assert O.format_params("fp8_e4m3") == (4, 5, 8, 2 ** 8 * 1.75, 2 ** -6)
+    assert O.format_params("fp6_e3m2") == (3, 4, 4, 2 ** 4 * 1.75, 2 ** -2)
+    assert O.format_params("fp6_e2m3") == (2, 5, 2, 2 ** 2 * 1.875, 1)
+    assert O.format_params("fp4_e2m1") == (2, 3, 2, 2 ** 2 * 1.5, 1)
+    assert O.format_params("fp4") == O.format_params("fp4_e2m1")
+    assert O.format_params("int8") == (0, 8, 0, 1 + 63 / 64, 0)
+    assert O.format_params("int4") == (0, 4, 0, 1.75, 0)
+
+
+# ---- MX literal vectors -------------------------------------------------------------------------
+@pytest.mark.parametrize("orc", ORACLES)
+def test_e4m3_saturation(orc):
+    """mx/tests/test_fp8_e4m3_fix.py:17-18."""
+    x = torch.tensor([485, 475, 400, -485, -475, -450, 2 ** -6, -(2 ** -6)], dtype=torch.float32)
+    t = [448, 448, 416, -448, -448, -448, 2 ** -6, -(2 ** -6)]
+    same_values(orc.quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=8), t)
+
+
+_MXFP8_X = [-0.582733273506, -0.256973713636, 0.506033003330, 0.400039970875,
+            -0.437093466520, 1.275019764900, -2.123294353485, 1.514909625053,
+            -2.660086154938, -0.200791791081, -0.060985822231, -0.209203109145,
+            2.385987281799, 0.062245476991, 0.217003762722, -0.857734560966,
+            0.507945835590, 0.896152675152, -0.751049160957, -0.488164335489,
+            0.805381953716, -0.172028362751, 0.271137863398, -0.503807783127,
+            1.879478693008, -0.294227510691, 0.968807995319, 0.670037031174,
+            -0.871595799923, 0.304561793804, -0.567594051361, -1.265962004662]
+_MXFP8_T = [-0.5625, -0.25, 0.5, 0.40625, -0.4375, 1.25, -2.0, 1.5, -2.75, -0.203125, -0.0625,
+            -0.203125, 2.5, 0.0625, 0.21875, -0.875, 0.5, 0.875, -0.75, -0.5, 0.8125, -0.171875,
+            0.28125, -0.5, 1.875, -0.28125, 1.0, 0.6875, -0.875, 0.3125, -0.5625, -1.25]
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+@pytest.mark.parametrize("rnd", ["nearest", "even"])
+def test_mxfp8_block_known_answer(orc, rnd):
+    """mx/tests/test_fp8_e4m3_fix.py:89-119."""
+    x = torch.tensor(_MXFP8_X, dtype=torch.float32)
+    same_values(orc.quantize_mx(x, 8, "fp8_e4m3", axes=[0], block_size=32, round=rnd), _MXFP8_T)
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+def test_five_bit_scale(orc):
+    """mx/tests/test_e5m0_scale.py:23-27: scale overflow -> NaN/Inf block, underflow clamps."""
+    firsts = [2 ** 16, 2 ** 15, 2 ** -16, 2 ** -17, 2 ** -15, 2 ** -14, 1, 0]
+    wants = [inf, 2 ** 15, 2 ** -15, 0, 2 ** -15, 2 ** -14, 1, 0]
+    x = torch.tensor([[e] + 7 * [0] for e in firsts], dtype=torch.float32)
+    t = torch.tensor([[e] + 7 * [inf if e == inf else 0] for e in wants], dtype=torch.float32)
+    same_values(orc.quantize_mx(x, 5, "int2", axes=[-1], block_size=8), t)
+    same_values(orc.quantize_mx(-x, 5, "int2", axes=[-1], block_size=8), -t)
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+@pytest.mark.parametrize("val", [nan, inf, -inf])
+@pytest.mark.parametrize("fmt", ["fp8_e4m3", "fp4_e2m1", "int4"])
+def test_nonfinite_poisons_block(orc, val, fmt):
+    """mx/tests/test_corners_mx.py:27-56."""
+    x = torch.tensor([val, 0, 2.0 ** 127, 0], dtype=torch.float32)
+    y = orc.quantize_mx(x, 8, fmt, axes=[-1], block_size=4, round="floor")
+    assert torch.isnan(y).all()
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+def test_int4_never_minus_two(orc):
+    """mx/tests/test_corners_mx.py:59-79."""
+    x = torch.tensor([[-1.0, -1.75, -1.99, 1.99], [1.0, -1.75, -1.99, 1.99]])
+    t = [[-1.0, -1.75, -1.75, 1.75], [1.0, -1.75, -1.75, 1.75]]
+    same_values(orc.quantize_mx(x, 8, "int4", axes=[1], block_size=0), t)
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+def test_int8_hardware_matrix(orc):
+    """mx/tests/test_corners_mx.py:83-124 (block of 10 along axis 1)."""
+    x = torch.tensor([
+        [1.0] * 10,
+        [1.0] * 5 + [2.0] * 5,
+        [-1.0] * 5 + [-2.0] * 5,
+        [1.0] * 5 + [-2.0] * 5,
+        [1.015625, 1.0234375, 1.03125, 1.0390625, 1.25, 1.2578125, 1.9375, 1.9453125, 1.984375,
+         1.9921875],
+        [-1.984375, -1.9765625, -1.96875, -1.9609375, -1.9375, -1.9296875, -1.75, -1.7421875, -1.0,
+         -1.9921875],
+        [1.99609375, 1.98828125, 0.0, 0.00390625, 0.0078125, 0.01171875, -0.015625, -0.01171875,
+         -0.0078125, -0.00390625]])
+    t = [
+        [1.0] * 10,
+        [1.0] * 5 + [2.0] * 5,
+        [-1.0] * 5 + [-2.0] * 5,
+        [1.0] * 5 + [-2.0] * 5,
+        [1.015625, 1.03125, 1.03125, 1.046875, 1.25, 1.265625, 1.9375, 1.953125, 1.984375, 1.984375],
+        [-1.984375, -1.984375, -1.96875, -1.96875, -1.9375, -1.9375, -1.75, -1.75, -1.0, -1.984375],
+        [1.984375, 1.984375, 0.0, 0.0, 0.015625, 0.015625, -0.015625, -0.015625, -0.015625, 0.0]]
+    same_values(orc.quantize_mx(x, 8, "int8", axes=[1], block_size=10), t)
+
+
+# ---- elementwise literal vectors ----------------------------------------------------------------
+BF16_MAX = 2 ** 127 * 255 / 128
+
+
+def q_bf16(orc, x, rnd="nearest", den=True):
+    return orc.quantize_elemwise_core(torch.tensor(x, dtype=torch.float32), 9, 8, BF16_MAX,
+                                      round=rnd, allow_denorm=den)
+
+
+def q_fp16(orc, x, rnd="nearest", den=True):
+    return orc.quantize_elemwise_core(torch.tensor(x, dtype=torch.float32), 12, 5, 65504.0,
+                                      round=rnd, allow_denorm=den)
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+@pytest.mark.parametrize("den", [True, False])
+def test_bf16_rne_vector(orc, den):
+    """mx/tests/test_quantize_elemwise.py:54-69 (tolerance 1e-8 there: the expected values are
+    printed with 8 significant digits)."""
+    x = [65535., -65535., -1.9985847, 0.4999000132083893, -0.49968934059143066, -0.0018959,
+         0.0018959, -2.52075195e-02, 0.0156078, 0.00780624, -0.00048747, -0.01561374, -0.00780595,
+         -0.0039039, 0.01557725, -0.0077924, 0.00389144, -0.00779678, -0.01556631, -0.00194835]
+    t = [65536., -65536., -2.0, 0.5, -0.5, -0.00189209, 0.00189209, -2.51464844e-02, 0.015625,
+         0.0078125, -0.00048828, -0.015625, -0.0078125, -0.00390625, 0.01556396, -0.00778198,
+         0.00389099, -0.00778198, -0.01556396, -0.0019455]
+    y = q_bf16(orc, x, "even", den)
+    assert (y - torch.tensor(t)).abs().max() <= 1e-8
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+def test_overflow_thresholds(orc):
+    """mx/tests/test_corners_elemwise.py:28-79, 172-184."""
+    m = 2.0 ** 127
+    y = q_bf16(orc, [m * 255 / 128, -m * 255 / 128, m * 1021 / 512, -m * 1021 / 512,
+                     m * 1023 / 512, -m * 1023 / 512])
+    assert torch.isfinite(y).tolist() == [True, True, True, True, False, False]
+    y = q_fp16(orc, [65504., -65504., 65519., -65519., 65520., -65520.])
+    same_values(y, [65504., -65504., 65504., -65504., inf, -inf])
+    y = q_bf16(orc, [m * 1.9921875, m * 1.9921874, -m * 1.9921875, m * 1.99609375, -m * 1.99609375])
+    same_values(y, [m * 1.9921875, m * 1.9921875, -m * 1.9921875, inf, -inf])
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+@pytest.mark.parametrize("rnd", ROUNDS)
+def test_nan_inf_preserved(orc, rnd):
+    """mx/tests/test_corners_elemwise.py:82-109."""
+    y = q_bf16(orc, [0., nan, inf, 0.], rnd)
+    assert y[0] == 0 and torch.isnan(y[1]) and y[2] == inf and y[3] == 0
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+def test_bf16_nearest_and_large_shifts(orc):
+    """mx/tests/test_corners_elemwise.py:114-145."""
+    same_values(q_bf16(orc, [65535., -65535., -1.9985847, 0.4999000132083893, -0.49968934059143066]),
+                [65536., -65536., -2.0, 0.5, -0.5])
+    x = [65535., 65536., 131072., 262144., 524288.]
+    same_values(q_bf16(orc, x), [65536., 65536., 131072., 262144., 524288.])
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+@pytest.mark.parametrize("den", [False, True])
+def test_subnormals(orc, den):
+    """mx/tests/test_corners_elemwise.py:147-225."""
+    s = 2.0 ** -14
+    x = [s, s * 0.5, s * 2 ** -10, s * 2 ** -11, s * 2 ** -12, s * 1023 / 1024, s * 2047 / 2048]
+    t = [s, s * 0.5, s * 2 ** -10, s * 2 ** -10, 0, s * 1023 / 1024, s] if den else [s] + [0.0] * 6
+    same_values(q_fp16(orc, x, den=den), t)
+    s = 2.0 ** -126
+    x = [s, s * 0.5, s * 2 ** -7, s * 2 ** -8, s * 2 ** -9, s * 127 / 128, s * 255 / 256]
+    t = [s, s * 0.5, s * 2 ** -7, s * 2 ** -7, 0, s * 127 / 128, s] if den else [s] + [0.0] * 6
+    same_values(q_bf16(orc, x, den=den), t)
+    if den:
+        same_values(q_bf16(orc, [s * 253 / 256, s * 251 / 256], "even"), [s * 126 / 128] * 2)
+
+
+# ---- library special cases ----------------------------------------------------------------------
+def all_encodings(ebits, mbits, encodes_infs=True):
+    """Every value of a small eXmY format (the enumeration of mx/tests/common_lib.py:142-180)."""
+    vals = []
+    for code in range(2 ** (ebits + mbits)):
+        if ebits > 0:
+            e, m = code >> mbits, code & (2 ** mbits - 1)
+            if encodes_infs and e == 2 ** ebits - 1:
+                continue
+            bias = 2 ** (ebits - 1) - 1
+            v = 2.0 ** (1 - bias) * (m / 2 ** mbits) if e == 0 else 2.0 ** (e - bias) * (1 + m / 2 ** mbits)
+            if ebits == 4 and mbits == 3 and e - bias == 8 and m == 7:
+                v = 0.0                                     # S.1111.111 is NaN in e4m3
+        else:
+            v = code / 2 ** (mbits - 1)
+        vals += [v, -v]
+    return torch.tensor(vals, dtype=torch.float32)
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+def test_even_rounding_is_torch_cast(orc):
+    """round='even' to bf16 / fp16 must equal torch's own casts wherever those stay finite
+    (mx/tests/test_quantize_elemwise.py:111-125 for bf16; fp16 by the same argument)."""
+    x = all_encodings(8, 9)
+    y = orc.quantize_elemwise_core(x.clone(), 9, 8, BF16_MAX, round="even")
+    t = x.to(torch.bfloat16).float()
+    keep = torch.isfinite(t) & (x != 0)                     # the reference maps -0.0 to +0.0
+    assert_bits_equal(y[keep], t[keep], "bf16 cast")
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(20000, generator=g) * torch.exp(4 * torch.randn(20000, generator=g))
+    y = orc.quantize_elemwise_core(x.clone(), 12, 5, 65504.0, round="even")
+    t = x.half().float()
+    keep = torch.isfinite(t) & (t != 0)                    # sign of an underflowed zero differs
+    assert_bits_equal(y[keep], t[keep], "fp16 cast")
+    y = orc.quantize_elemwise_core(x.clone(), 9, 8, BF16_MAX, round="even")
+    assert_bits_equal(y, x.to(torch.bfloat16).float(), "bf16 cast, random")
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+def test_fp8_casts(orc):
+    """In-range e4m3 / e5m2 rounding with round='even' equals torch's float8 casts."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(20000, generator=g) * torch.exp(2 * torch.randn(20000, generator=g))
+    x = x[(x.abs() < 400) & (x.abs() > 2 ** -5)]
+    y = orc.quantize_elemwise_core(x.clone(), 5, 4, 448.0, round="even", saturate_normals=True)
+    assert_bits_equal(y, x.to(torch.float8_e4m3fn).float(), "e4m3fn")
+    y = orc.quantize_elemwise_core(x.clone(), 4, 5, 57344.0, round="even", saturate_normals=True)
+    assert_bits_equal(y, x.to(torch.float8_e5m2).float(), "e5m2")
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+@pytest.mark.parametrize("fmt,infs", [("int8", False), ("fp8_e4m3", False), ("fp8_e5m2", True),
+                                      ("fp6_e3m2", False), ("fp6_e2m3", False),
+                                      ("fp4_e2m1", False), ("bf16", True), ("fp16", True)])
+@pytest.mark.parametrize("rnd", ROUNDS)
+def test_representable_values_are_fixed_points(orc, fmt, infs, rnd):
+    """mx/tests/test_quantize_elemwise.py:191-224."""
+    ebits, mbits, _, max_norm, _ = O.format_params(fmt)
+    x = all_encodings(ebits, mbits - 1 if ebits == 0 else mbits - 2, infs)
+    y = orc.quantize_elemwise_core(x.clone(), mbits, ebits, max_norm, round=rnd)
+    assert torch.equal(y, x)
+
+
+# ---- exact-rational brute force -----------------------------------------------------------------
+def exact_quantize(v, mbits, ebits, max_norm, rnd, saturate):
+    """Value-level definition with exact rationals: clip the exponent, scale, round, clamp."""
+    if v == 0:
+        return Fraction(0)
+    a = abs(Fraction(v))
+    if ebits:
+        e = math.floor(math.log2(a)) if a.numerator else 0
+        while Fraction(2) ** e > a:
+            e -= 1
+        while Fraction(2) ** (e + 1) <= a:
+            e += 1
+        e = max(e, 2 - 2 ** (ebits - 1))
+    else:
+        e = 0
+    step = Fraction(2) ** (e - (mbits - 2))
+    s = a / step
+    fl = s.numerator // s.denominator
+    rem = s - fl
+    if rnd == "floor":
+        q = fl
+    elif rnd == "nearest":
+        q = fl + (1 if rem >= Fraction(1, 2) else 0)
+    else:
+        q = fl + (1 if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2) else 0)
+    y = q * step
+    if y > Fraction(max_norm):
+        y = Fraction(max_norm) if saturate else None
+    return None if y is None else (y if v > 0 else -y)
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+@pytest.mark.parametrize("fmt", ["fp8_e4m3", "fp8_e5m2", "fp6_e3m2", "fp6_e2m3", "fp4_e2m1", "int8"])
+@pytest.mark.parametrize("rnd", ROUNDS)
+def test_against_exact_rationals(orc, fmt, rnd):
+    """Inputs with two extra fraction bits (all quarter-step cases) plus random values, away from
+    the few-ulp zone below powers of two where torch's floor(log2) differs by design."""
+    ebits, mbits, _, max_norm, _ = O.format_params(fmt)
+    x = all_encodings(ebits, mbits + 1 if ebits == 0 else mbits, ebits >= 5)
+    g = torch.Generator().manual_seed(17)
+    r = (torch.randn(300, generator=g) * max_norm / 2).to(torch.bfloat16).float()
+    x = torch.cat([x, r])
+    y = orc.quantize_elemwise_core(x.clone(), mbits, ebits, max_norm, round=rnd,
+                                   saturate_normals=True)
+    for xi, yi in zip(x.tolist(), y.tolist()):
+        assert Fraction(yi) == exact_quantize(xi, mbits, ebits, max_norm, rnd, True), (xi, yi)
+
+
+# ---- golden vectors from the reference's pure path ----------------------------------------------
+@pytest.mark.parametrize("orc", ORACLES)
+def test_golden_mx(orc):
+    z, _ = golden()
+    xb = from_bits(z["mx_bf16_x"], torch.bfloat16)
+    xz = from_bits(z["mx_fp32_zone_x"], torch.float32)
+    for fmt in MX_FORMATS:
+        for rnd in ROUNDS:
+            y = orc.quantize_mx(xb.clone(), 8, fmt, axes=[-1], block_size=32, round=rnd)
+            assert_bits_equal(y, from_bits(z["mx_bf16_y.%s.%s" % (fmt, rnd)], torch.bfloat16), fmt + rnd)
+            y = orc.quantize_mx(xz.clone(), 8, fmt, axes=[-1], block_size=32, round=rnd)
+            assert_bits_equal(y, from_bits(z["mx_fp32_zone_y.%s.%s" % (fmt, rnd)], torch.float32), fmt + rnd)
+    y = orc.quantize_mx(xb.t().contiguous(), 5, "fp8_e4m3", axes=[0], block_size=32, round="even",
+                        flush_fp32_subnorms=True)
+    assert_bits_equal(y, from_bits(z["mx_bf16_y.t.fp8_e4m3.even.sb5.flush"], torch.bfloat16))
+
+
+def _digest(t):
+    return hashlib.sha256(np.ascontiguousarray(canon_bits(t)).tobytes()).hexdigest()
+
+
+ELEM_CFG = {"bf16": (9, 8, BF16_MAX), "fp16": (12, 5, 65504.0), "bf12": (5, 8, 2 ** 127 * 15 / 8),
+            "e4m3": (5, 4, 448.0)}
+
+
+@pytest.mark.parametrize("orc", ORACLES)
+def test_golden_elementwise_digests(orc):
+    z, meta = golden()
+    xe = from_bits(z["elem_fp32_x"], torch.float32)
+    xb = from_bits(z["elem_bf16_x"], torch.bfloat16)
+    n = 0
+    for key, want in meta["digests"].items():
+        parts = key.split(".")
+        b, e, m = ELEM_CFG[parts[1]]
+        if parts[0] == "elem_fp32_y":
+            y = orc.quantize_elemwise_core(xe.clone(), b, e, m, round=parts[2],
+                                           saturate_normals=bool(int(parts[3])),
+                                           allow_denorm=bool(int(parts[4])))
+        else:
+            y = orc.quantize_elemwise_core(xb.clone(), b, e, m, round=parts[2],
+                                           saturate_normals=bool(int(parts[3])))
+        assert _digest(y) == want, key
+        n += 1
+    assert n == 54
+
+
+def test_golden_exhaustive_bf16_digests():
+    """Every finite bf16 code as an element under ten block maxima x 7 formats x 3 roundings."""
+    _, meta = golden()
+    gen = golden_inputs_module()
+    codes = gen.all_bf16_codes()
+    finite = codes[torch.isfinite(codes.float())]
+    for Mexp in (-130, -126, -100, -3, 0, 1, 5, 60, 120, 127):
+        M = 2.0 ** Mexp
+        sel = finite[finite.float().abs() <= M]
+        n = (sel.numel() + 30) // 31 * 31
+        body = torch.cat([sel, torch.zeros(n - sel.numel(), dtype=torch.bfloat16)]).view(-1, 31)
+        blk = torch.cat([torch.full((body.shape[0], 1), M, dtype=torch.bfloat16), body], dim=1)
+        for fmt in MX_FORMATS:
+            for rnd in ROUNDS:
+                y = O.quantize_mx(blk.clone(), 8, fmt, axes=[-1], block_size=32, round=rnd)
+                assert _digest(y) == meta["bf16_exhaustive_digests"]["%d.%s.%s" % (Mexp, fmt, rnd)]
