@@ -30,29 +30,38 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 int elem_size(int dtype) { return dtype == MXQ_DTYPE_F32 ? 4 : 2; }
 
-// ---- dispatch over (dtype, rounding mode, element zone) -----------------------------------------
-// F is a functor template: F<DT, RMODE, ZONE_ELEM>::run(args...)
-template <template <int, int, bool> class F, int DT, typename... A>
-void dispatch_round(int rmode, bool zone_elem, A... a) {
-    if (rmode == MXQ_ROUND_FLOOR) F<DT, MXQ_FLOOR, true>::run(a...);
-    else if (rmode == MXQ_ROUND_NEAREST) {
-        if (zone_elem) F<DT, MXQ_NEAREST, true>::run(a...);
-        else F<DT, MXQ_NEAREST, false>::run(a...);
+// ---- dispatch over (dtype, rounding mode, element zone, lean) ------------------------------------
+// F is a functor template: F<DT, RMODE, ZONE_ELEM, LEAN>::run(args...).  The op-by-op form always
+// consults the zone table, so it exists once per rounding mode, and only bf16 tensors need it.
+template <template <int, int, bool, bool> class F, int DT, typename... A>
+void dispatch_round(int rmode, bool zone_elem, bool lean, A... a) {
+    if (DT == MXQ_BF16 && !lean) {
+        if (rmode == MXQ_ROUND_FLOOR) F<MXQ_BF16, MXQ_FLOOR, true, false>::run(a...);
+        else if (rmode == MXQ_ROUND_NEAREST) F<MXQ_BF16, MXQ_NEAREST, true, false>::run(a...);
+        else F<MXQ_BF16, MXQ_EVEN, true, false>::run(a...);
+        return;
+    }
+    if (rmode == MXQ_ROUND_FLOOR) {
+        if (zone_elem) F<DT, MXQ_FLOOR, true, true>::run(a...);
+        else F<DT, MXQ_FLOOR, false, true>::run(a...);
+    } else if (rmode == MXQ_ROUND_NEAREST) {
+        if (zone_elem) F<DT, MXQ_NEAREST, true, true>::run(a...);
+        else F<DT, MXQ_NEAREST, false, true>::run(a...);
     } else {
-        if (zone_elem) F<DT, MXQ_EVEN, true>::run(a...);
-        else F<DT, MXQ_EVEN, false>::run(a...);
+        if (zone_elem) F<DT, MXQ_EVEN, true, true>::run(a...);
+        else F<DT, MXQ_EVEN, false, true>::run(a...);
     }
 }
-template <template <int, int, bool> class F, typename... A>
-void dispatch(int dtype, int rmode, bool zone_elem, A... a) {
-    if (dtype == MXQ_DTYPE_F32) dispatch_round<F, MXQ_F32>(rmode, zone_elem, a...);
-    else if (dtype == MXQ_DTYPE_BF16) dispatch_round<F, MXQ_BF16>(rmode, zone_elem, a...);
-    else dispatch_round<F, MXQ_F16>(rmode, zone_elem, a...);
+template <template <int, int, bool, bool> class F, typename... A>
+void dispatch(int dtype, int rmode, bool zone_elem, bool lean, A... a) {
+    if (dtype == MXQ_DTYPE_F32) dispatch_round<F, MXQ_F32>(rmode, zone_elem, lean, a...);
+    else if (dtype == MXQ_DTYPE_BF16) dispatch_round<F, MXQ_BF16>(rmode, zone_elem, lean, a...);
+    else dispatch_round<F, MXQ_F16>(rmode, zone_elem, lean, a...);
 }
 
 constexpr int kLastAxisUnroll = 4;
 
-template <int DT, int RMODE, bool ZE>
+template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchLastAxis {
     static void run(const void* in, void* out, int64_t n_vec, int lpt, MxParams p, hipStream_t s) {
         const int grid = grid_for(ceil_div(n_vec, (int64_t)kThreads * kLastAxisUnroll));
@@ -60,7 +69,7 @@ struct LaunchLastAxis {
         u32x4* o4 = reinterpret_cast<u32x4*>(out);
 #define MXQ_CASE(L)                                                                               \
     case L:                                                                                       \
-        mx_lastaxis_kernel<DT, RMODE, L, ZE, kLastAxisUnroll><<<grid, kThreads, 0, s>>>(i4, o4, n_vec, p); \
+        mx_lastaxis_kernel<DT, RMODE, ZE, LEAN, L, kLastAxisUnroll><<<grid, kThreads, 0, s>>>(i4, o4, n_vec, p); \
         break;
         switch (lpt) {
             MXQ_CASE(1) MXQ_CASE(2) MXQ_CASE(4) MXQ_CASE(8) MXQ_CASE(16)
@@ -69,48 +78,52 @@ struct LaunchLastAxis {
     }
 };
 
-template <int DT, int RMODE, bool ZE>
+template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchStrided {
     static void run(const void* in, void* out, int64_t pre, int64_t axis, int64_t post, int64_t tile,
-                    bool vec, MxParams p, hipStream_t s) {
-        constexpr int VWV = (DT == MXQ_F32) ? 4 : 8;
+                    bool aligned, MxParams p, hipStream_t s) {
+        constexpr int VW8 = (DT == MXQ_F32) ? 2 : 4;        // elements in 8 bytes
+        constexpr int VW16 = (DT == MXQ_F32) ? 4 : 8;       // elements in 16 bytes
         const int64_t num_tiles = ceil_div(axis, tile);
-        const bool in_regs = tile <= 32;
-        if (vec) {
-            const int64_t items = pre * num_tiles * (post / VWV);
-            const int grid = grid_for(ceil_div(items, kThreads));
-            if (in_regs)
-                mx_strided_kernel<DT, RMODE, VWV, 32, ZE><<<grid, kThreads, 0, s>>>(in, out, pre, axis, post, tile, num_tiles, p);
-            else
-                mx_strided_kernel<DT, RMODE, VWV, 0, ZE><<<grid, kThreads, 0, s>>>(in, out, pre, axis, post, tile, num_tiles, p);
+        if (aligned && tile == 32 && axis % 32 == 0 && post % VW8 == 0) {
+            const int64_t pv = post / VW8;
+            const int64_t items = pre * num_tiles * pv;
+            const int64_t blocks = ceil_div(items, kThreads);
+            if (blocks <= 0x7FFFFFFF) {
+                mx_strided_tile_kernel<DT, RMODE, ZE, LEAN, 32><<<(unsigned)blocks, kThreads, 0, s>>>(
+                    reinterpret_cast<const u32x2*>(in), reinterpret_cast<u32x2*>(out), items, num_tiles, pv, p);
+                return;
+            }
+        }
+        if (aligned && post % VW16 == 0) {
+            const int64_t items = pre * num_tiles * (post / VW16);
+            mx_strided_kernel<DT, RMODE, ZE, LEAN, VW16><<<grid_for(ceil_div(items, kThreads)), kThreads, 0, s>>>(
+                in, out, pre, axis, post, tile, num_tiles, p);
         } else {
             const int64_t items = pre * num_tiles * post;
-            const int grid = grid_for(ceil_div(items, kThreads));
-            if (in_regs)
-                mx_strided_kernel<DT, RMODE, 1, 32, ZE><<<grid, kThreads, 0, s>>>(in, out, pre, axis, post, tile, num_tiles, p);
-            else
-                mx_strided_kernel<DT, RMODE, 1, 0, ZE><<<grid, kThreads, 0, s>>>(in, out, pre, axis, post, tile, num_tiles, p);
+            mx_strided_kernel<DT, RMODE, ZE, LEAN, 1><<<grid_for(ceil_div(items, kThreads)), kThreads, 0, s>>>(
+                in, out, pre, axis, post, tile, num_tiles, p);
         }
     }
 };
 
-template <int DT, int RMODE, bool ZE>
+template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchGivenMax {
     static void run(const void* in, void* out, const void* maxv, int64_t total, int64_t axis,
                     int64_t post, MxParams p, hipStream_t s) {
         const int grid = grid_for(ceil_div(total, kThreads * 4));
-        mx_given_max_kernel<DT, RMODE, ZE><<<grid, kThreads, 0, s>>>(in, out, maxv, total, axis, post, p);
+        mx_given_max_kernel<DT, RMODE, ZE, LEAN><<<grid, kThreads, 0, s>>>(in, out, maxv, total, axis, post, p);
     }
 };
 
 constexpr int kElemUnroll = 4;
 
-template <int DT, int RMODE, bool>
+template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchElemwise {
     static void run(const void* in, void* out, int64_t n, ElemParams p, hipStream_t s) {
         const int epv = (DT == MXQ_F32) ? 4 : 8;
         const int grid = grid_for(ceil_div(ceil_div(n, epv), (int64_t)kThreads * kElemUnroll));
-        elemwise_kernel<DT, RMODE, kElemUnroll><<<grid, kThreads, 0, s>>>(in, out, n, p);
+        elemwise_kernel<DT, RMODE, ZE, LEAN, kElemUnroll><<<grid, kThreads, 0, s>>>(in, out, n, p);
     }
 };
 
@@ -195,12 +208,11 @@ int mxq_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre, i
     if (post == 1 && ptr_ok && axis_size % tile == 0 && tile % vec_elems == 0) {
         const int64_t lpt = tile / vec_elems;
         if (lpt == 1 || lpt == 2 || lpt == 4 || lpt == 8 || lpt == 16) {
-            dispatch<LaunchLastAxis>(dtype, rmode, ze, in, out, total / vec_elems, (int)lpt, p, s);
+            dispatch<LaunchLastAxis>(dtype, rmode, ze, lean_ok(dtype, p.fmt), in, out, total / vec_elems, (int)lpt, p, s);
             return check_launch(who);
         }
     }
-    const bool vec = ptr_ok && post % vec_elems == 0;
-    dispatch<LaunchStrided>(dtype, rmode, ze, in, out, pre, axis_size, post, tile, vec, p, s);
+    dispatch<LaunchStrided>(dtype, rmode, ze, lean_ok(dtype, p.fmt), in, out, pre, axis_size, post, tile, ptr_ok, p, s);
     return check_launch(who);
 }
 
@@ -219,7 +231,7 @@ int mxq_quantize_mx_given_max(const void* in, void* out, const void* max_values,
     if (mul_overflows(pre, axis_size, post, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
     if (total == 0) return MXQ_OK;
     if (!in || !out || !max_values) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
-    dispatch<LaunchGivenMax>(dtype, rmode, ze, in, out, max_values, total, axis_size, post, p,
+    dispatch<LaunchGivenMax>(dtype, rmode, ze, lean_ok(dtype, p.fmt), in, out, max_values, total, axis_size, post, p,
                              (hipStream_t)hip_stream);
     return check_launch(who);
 }
@@ -237,7 +249,7 @@ int mxq_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int b
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     if (!aligned16(in) || !aligned16(out))
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
-    dispatch<LaunchElemwise>(dtype, rmode, true, in, out, n, p, (hipStream_t)hip_stream);
+    dispatch<LaunchElemwise>(dtype, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode), lean_ok(dtype, p.fmt), in, out, n, p, (hipStream_t)hip_stream);
     return check_launch(who);
 }
 

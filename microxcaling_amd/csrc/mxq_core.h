@@ -56,132 +56,172 @@ struct MxqFmt {
     int t;              // fraction bits kept = mbits - 2 (mbits counts sign and implicit one)
     int min_exp;        // 2 - 2^(ebits-1): exponent of the smallest normal (mx/elemwise_ops.py:139)
     uint32_t max_bits;  // bit pattern of max_norm (already rounded to the tensor dtype)
+    // derived, for the lean path
+    uint32_t min_eb;    // min_exp + 127, or 127 for integer formats (their exponent is fixed at 0)
+    int t127;           // t + 127
+    float half;         // what "+ 0.5" must add so that floor() sees the dtype-rounded sum
+    float tie_fix;      // the one input of the scaled domain whose "+ 0.5" rounds up to 1.0
+    uint32_t nan_from;  // elementwise only: |x| bit pattern from which floor(log2|x|) is 128
 };
 
 // ---- floor(log2(x)) in the tensor dtype --------------------------------------------------------
-// ua: |x| in fp32 layout, finite and non-zero.  zone[k+149] / zshift: see gen_log2_tables.py.
-MXQ_HD int mxq_floor_log2(uint32_t ua, const unsigned char* zone, int zshift) {
-    int be = (int)(ua >> 23);
-    uint32_t man = ua & 0x7FFFFFu;
-    int k;
-    uint32_t sig;
-    if (be != 0) {
-        k = be - 127;
-        sig = man | 0x800000u;
-    } else {                                    // fp32 subnormal: normalise
-        int lz = __builtin_clz(man);            // man != 0
-        sig = man << (lz - 8);
-        k = -118 - lz;
-    }
-    uint32_t gap = 0x1000000u - sig;
+// m: positive and finite.  zone[k+149] / zshift: see gen_log2_tables.py.
+MXQ_HD int mxq_floor_log2(float m, const unsigned char* zone, int zshift) {
+    int ex;
+    const float fr = frexpf(m, &ex);            // m = fr * 2^ex, fr in [0.5, 1); handles subnormals
+    const int k = ex - 1;
+    const uint32_t gap = 0x800000u - (mxq_bits(fr) & 0x7FFFFFu);   // 2^24 - normalised significand
     return k + (gap <= ((uint32_t)zone[k + 149] << zshift) ? 1 : 0);
 }
 
-// 2^n as fp32 for n in [-149, 127]
-MXQ_HD float mxq_pow2(int n) {
-    return mxq_float(n >= -126 ? (uint32_t)(n + 127) << 23 : 0x00400000u >> (-127 - n));
-}
-
 // ---- shared exponent of one block (mx/mx_ops.py:269-283) ---------------------------------------
+// A block that must become NaN (Inf/NaN seen, or scale exponent overflow) gets scale = NaN; a
+// block that must be flushed gets inv_scale = 0: the element code then needs no special cases.
 struct MxqScale {
     float scale;      // 2^se
     float inv_scale;  // 2^-se
-    bool nan;         // block becomes NaN: max is Inf/NaN or the scale exponent overflows
-    bool flush;       // block becomes +0: max is an fp32 subnormal and flushing was requested
 };
 
 // um: max |x| of the block as an fp32-layout bit pattern (0x7F800000 and above = Inf/NaN seen).
+// emax = exponent of the element format's max_norm; scale_emax = 2^(scale_bits-1) - 1.
 MXQ_HD MxqScale mxq_block_scale(uint32_t um, int emax, int scale_emax, bool flush_subnorms,
                                 const unsigned char* zone, int zshift) {
-    MxqScale r;
-    r.nan = um >= MXQ_INF_BITS;
-    int E = (um == 0u || r.nan) ? -126 : mxq_floor_log2(um, zone, zshift);
-    r.flush = flush_subnorms && E <= -127;
+    const uint32_t eb = um >> 23;
+    // normal maximum (also Inf/NaN, overwritten below): exponent field plus the round-up zone
+    const uint32_t gap = 0x800000u - (um & 0x7FFFFFu);
+    int E = (int)eb - 127 + (gap <= ((uint32_t)zone[eb + 22] << zshift) ? 1 : 0);
+    if (eb == 0u)                                // rare: zero -> log2(2^-126); fp32 subnormal
+        E = (um == 0u) ? -126 : mxq_floor_log2(mxq_float(um), zone, zshift);
     int se = E - emax;
-    if (se > scale_emax) r.nan = true;
-    if (se < -scale_emax) se = -scale_emax;
-    if (r.nan) se = 0;
-    r.scale = mxq_pow2(se);
-    r.inv_scale = mxq_pow2(-se);
+    const bool nan = um >= MXQ_INF_BITS || se > scale_emax;
+    se = se < -scale_emax ? -scale_emax : se;
+    se = se > 127 ? 127 : se;
+    MxqScale r;
+    r.scale = nan ? mxq_float(MXQ_QNAN_BITS) : ldexpf(1.0f, se);
+    r.inv_scale = (flush_subnorms && E <= -127) ? 0.0f : ldexpf(1.0f, -se);
     return r;
 }
 
-// ---- element rounding (mx/elemwise_ops.py:134-157) ---------------------------------------------
-// a: finite input already in the tensor dtype.  Returns the quantized value before any block
-// scale is re-applied.  FULL = round to the dtype after every op like torch does; !FULL drops the
-// roundings that provably never change a bf16 result when t <= 6 (checked exhaustively on the
-// host against the FULL variant and the torch oracle).
-template <int RMODE, int DT, bool ZONE, bool FULL>
-MXQ_HD float mxq_quant_finite(float a, const MxqFmt& f, bool saturate,
-                              const unsigned char* zone, int zshift) {
+// ---- element rounding, lean form ----------------------------------------------------------------
+// a: input in the tensor dtype, already divided by the block scale.  Valid for fp32 tensors with
+// any t <= 22 and for bf16 tensors with t <= 6: there the only place where the dtype rounding of
+// an intermediate changes a result is "s + 0.5" for s just below one half (0.5 - 2^-25 in fp32,
+// which the fp32 add reproduces by itself; 0.5 - 2^-9 in bf16, reproduced by adding 2^-9 more),
+// and torch's even-mode emulation equals round-half-even except for that same input.
+// Inf/NaN inputs give unspecified results here; callers overwrite them.
+// sign_src: a value with the sign the result must carry (+0.0 when the result must be +0).
+template <int RMODE, bool ZONE>
+MXQ_HD float mxq_round_lean(float a, float sign_src, const MxqFmt& f, bool saturate,
+                            const unsigned char* zone, int zshift) {
+    const uint32_t ua = mxq_bits(a) & 0x7FFFFFFFu;
+    uint32_t eb = (mxq_bits(a) >> 23) & 0xFFu;  // biased exponent; 0 for subnormals and zero
+    if (ZONE) {                                 // eb + 22 == k + 149; rows are zero-padded past 276
+        const uint32_t gap = 0x1000000u - ((ua & 0x7FFFFFu) | 0x800000u);
+        eb += (gap <= ((uint32_t)zone[eb + 22] << zshift)) ? 1u : 0u;
+    }
+    // integer formats: min_eb = 127 pins the exponent at 0 for |a| < 2; larger |a| end above
+    // max_norm with either exponent and are clamped to it
+    const uint32_t ebc = eb > f.min_eb ? eb : f.min_eb;
+    const int n = f.t127 - (int)ebc;
+    const float s = ldexpf(mxq_float(ua), n);   // exact
+    float r;
+    if (RMODE == MXQ_FLOOR) {
+        r = floorf(s);
+    } else if (RMODE == MXQ_NEAREST) {
+        r = floorf(s + f.half);
+    } else {
+        r = __builtin_rintf(s);                 // ties to even (default rounding mode)
+        r = (s == f.tie_fix) ? 1.0f : r;
+    }
+    const float y = ldexpf(r, -n);              // exact
+    uint32_t uy = mxq_bits(y);
+    if (saturate) uy = uy < f.max_bits ? uy : f.max_bits;
+    else uy = uy > f.max_bits ? MXQ_INF_BITS : uy;
+    return mxq_float(uy | (mxq_bits(sign_src) & 0x80000000u));
+}
+
+// sign(a) * r gives -0.0 when a negative value rounds to zero but +0.0 for a = +-0: a + 0.0 has
+// exactly that sign.  For bf16 tensors a was first rounded to bf16, where |a| <= 2^-134 becomes
+// +-0: a * 2^-16 rounds to +-0 in fp32 for exactly those values.
+template <int DT>
+MXQ_HD float mxq_sign_source(float a) {
+    if (DT == MXQ_BF16) return a * 1.52587890625e-05f + 0.0f;
+    return a + 0.0f;
+}
+
+// ---- element rounding, op-by-op form (mx/elemwise_ops.py:134-157) -------------------------------
+// Rounds to the tensor dtype after every op exactly like torch's CPU kernels do.  Used for bf16
+// tensors with wide element formats (t >= 7) and, on the host, to cross-check the lean form.
+template <int RMODE, int DT>
+MXQ_HD float mxq_round_every_op(float a, const MxqFmt& f, bool saturate, const unsigned char* zone,
+                                int zshift) {
     const uint32_t ba = mxq_bits(a);
     const uint32_t ua = ba & 0x7FFFFFFFu;
     int e = 0;
     if (f.ebits != 0) {
         int k = (int)(ua >> 23) - 127;          // subnormal or zero: below every min_exp
-        if (ZONE && ua >= 0x00800000u) {
+        if (ua >= 0x00800000u) {
             uint32_t gap = 0x1000000u - ((ua & 0x7FFFFFu) | 0x800000u);
             k += (gap <= ((uint32_t)zone[k + 149] << zshift)) ? 1 : 0;
         }
         e = k > f.min_exp ? k : f.min_exp;
         if (e >= 128) return mxq_float(MXQ_QNAN_BITS);    // 2**128 = inf -> 0 * inf
     }
-    const float mag = mxq_float(ua);
-    float s;
-    if (FULL) {
-        s = mxq_round_dt<DT>(ldexpf(mag, -e));             // out / 2**e
-        s = mxq_round_dt<DT>(ldexpf(s, f.t));              // * 2**(bits-2)
-    } else {
-        s = ldexpf(mag, f.t - e);
-    }
+    float s = mxq_round_dt<DT>(ldexpf(mxq_float(ua), -e));  // out / 2**e
+    s = mxq_round_dt<DT>(ldexpf(s, f.t));                   // * 2**(bits-2)
     float r;
     if (RMODE == MXQ_FLOOR) {
         r = floorf(s);
     } else if (RMODE == MXQ_NEAREST) {
         r = floorf(mxq_round_dt<DT>(s + 0.5f));
     } else {
-        float d = s - 0.5f;
-        if (FULL) d = mxq_round_dt<DT>(d);
+        float d = mxq_round_dt<DT>(s - 0.5f);
         float h = d * 0.5f;
-        float tie = (h == floorf(h)) ? 1.0f : 0.0f;        // (|v| - 0.5) % 2 == 0
+        float tie = (h == floorf(h)) ? 1.0f : 0.0f;         // (|v| - 0.5) % 2 == 0
         r = floorf(mxq_round_dt<DT>(s + 0.5f)) - tie;
     }
-    float y;
-    if (FULL) {
-        y = mxq_round_dt<DT>(ldexpf(r, -f.t));
-        y = mxq_round_dt<DT>(ldexpf(y, e));
-    } else {
-        y = ldexpf(r, e - f.t);
-    }
+    float y = mxq_round_dt<DT>(ldexpf(r, -f.t));
+    y = mxq_round_dt<DT>(ldexpf(y, e));
     uint32_t uy = mxq_bits(y) & 0x7FFFFFFFu;
     if (uy > f.max_bits) uy = (saturate || f.ebits == 0) ? f.max_bits : MXQ_INF_BITS;
-    // sign(a) * r: -0.0 when a negative value rounds to zero, +0.0 for a = +-0
     return mxq_float(uy | (ua != 0u ? (ba & 0x80000000u) : 0u));
 }
 
-// One element of an MX block: x / 2^se -> round -> * 2^se  (mx/mx_ops.py:285-292).
-template <int RMODE, int DT, bool ZONE, bool FULL>
+// One element of an MX block: x / 2^se -> round -> * 2^se  (mx/mx_ops.py:285-292).  The result
+// still has to be rounded to the tensor dtype (mxq_round_dt, or the packing conversion).
+// LEAN: see mxq_round_lean for when it may be used.
+template <int RMODE, int DT, bool ZONE, bool LEAN>
+MXQ_HD float mxq_quant_mx_elem_raw(float x, const MxqScale& sc, const MxqFmt& f,
+                                   const unsigned char* zone, int zshift) {
+    const float a = x * sc.inv_scale;
+    float y;
+    if (LEAN) {
+        // a bf16-subnormal quotient is not rounded to bf16 here: it rounds to zero in the element
+        // format either way, only its sign needs the bf16 view (mxq_sign_source)
+        y = mxq_round_lean<RMODE, ZONE>(a, mxq_sign_source<DT>(a), f, true, zone, zshift);
+    } else {
+        y = mxq_round_every_op<RMODE, DT>(mxq_round_dt<DT>(a), f, true, zone, zshift);
+    }
+    return y * sc.scale;
+}
+template <int RMODE, int DT, bool ZONE, bool LEAN>
 MXQ_HD float mxq_quant_mx_elem(float x, const MxqScale& sc, const MxqFmt& f,
                                const unsigned char* zone, int zshift) {
-    if (sc.nan) return mxq_float(MXQ_QNAN_BITS);
-    if (sc.flush) return 0.0f;
-    float a = mxq_round_dt<DT>(x * sc.inv_scale);
-    float y = mxq_quant_finite<RMODE, DT, ZONE, FULL>(a, f, true, zone, zshift);
-    return mxq_round_dt<DT>(y * sc.scale);
+    return mxq_round_dt<DT>(mxq_quant_mx_elem_raw<RMODE, DT, ZONE, LEAN>(x, sc, f, zone, zshift));
 }
 
 // One element of the elementwise quantizer (mx/elemwise_ops.py:127-163).
-template <int RMODE, int DT, bool FULL>
+template <int RMODE, int DT, bool ZONE, bool LEAN>
 MXQ_HD float mxq_quant_elemwise(float x, const MxqFmt& f, bool saturate, bool allow_denorm,
                                 const unsigned char* zone, int zshift) {
-    const uint32_t bx = mxq_bits(x);
-    const uint32_t ux = bx & 0x7FFFFFFFu;
-    if (ux > MXQ_INF_BITS) return mxq_float(MXQ_QNAN_BITS);   // NaN propagates
-    if (ux == MXQ_INF_BITS) return x;                          // +-Inf restored (161-162)
-    if (!allow_denorm && f.ebits > 0 && (int)(ux >> 23) - 127 < f.min_exp) {
-        // (|A| >= min_norm) * A gives +-0, whose sign() is 0; but the exponent still comes from A,
-        // and 2**128 = inf turns the zero into NaN for values in the top round-up zone.
-        return 0.0f;
-    }
-    return mxq_quant_finite<RMODE, DT, true, FULL>(x, f, saturate, zone, zshift);
+    const uint32_t ux = mxq_bits(x) & 0x7FFFFFFFu;
+    float y;
+    if (LEAN) y = mxq_round_lean<RMODE, ZONE>(x, x + 0.0f, f, saturate || f.ebits == 0, zone, zshift);
+    else y = mxq_round_every_op<RMODE, DT>(ux < MXQ_INF_BITS ? x : 0.0f, f, saturate, zone, zshift);
+    // (|A| >= min_norm) * A is +-0, and sign(+-0) is 0
+    if (!allow_denorm && f.ebits > 0 && (ux >> 23) < f.min_eb) y = 0.0f;
+    // exponent 128: 2**128 = inf and the value turns into 0 * inf.  +-Inf is restored after the
+    // clamp (161-162); NaN propagates
+    if (ux >= f.nan_from) y = (ux == MXQ_INF_BITS) ? x : mxq_float(MXQ_QNAN_BITS);
+    return y;
 }

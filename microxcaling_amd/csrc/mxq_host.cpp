@@ -38,22 +38,27 @@ void store_from_float(void* p, int dtype, int64_t i, float v) {
 typedef float (*MxElemFn)(float, const MxqScale&, const MxqFmt&, const unsigned char*, int);
 typedef float (*ElemFn)(float, const MxqFmt&, bool, bool, const unsigned char*, int);
 
-template <int DT, bool FULL>
+template <int DT, bool LEAN>
 MxElemFn pick_mx(int rmode, bool ze) {
-    if (rmode == MXQ_ROUND_FLOOR) return mxq_quant_mx_elem<MXQ_FLOOR, DT, true, FULL>;
+    if (rmode == MXQ_ROUND_FLOOR) return ze ? mxq_quant_mx_elem<MXQ_FLOOR, DT, true, LEAN> : mxq_quant_mx_elem<MXQ_FLOOR, DT, false, LEAN>;
     if (rmode == MXQ_ROUND_NEAREST)
-        return ze ? mxq_quant_mx_elem<MXQ_NEAREST, DT, true, FULL> : mxq_quant_mx_elem<MXQ_NEAREST, DT, false, FULL>;
-    return ze ? mxq_quant_mx_elem<MXQ_EVEN, DT, true, FULL> : mxq_quant_mx_elem<MXQ_EVEN, DT, false, FULL>;
+        return ze ? mxq_quant_mx_elem<MXQ_NEAREST, DT, true, LEAN> : mxq_quant_mx_elem<MXQ_NEAREST, DT, false, LEAN>;
+    return ze ? mxq_quant_mx_elem<MXQ_EVEN, DT, true, LEAN> : mxq_quant_mx_elem<MXQ_EVEN, DT, false, LEAN>;
 }
-MxElemFn pick_mx(int dtype, int rmode, bool ze, bool full) {
-    if (dtype == MXQ_DTYPE_BF16) return full ? pick_mx<MXQ_BF16, true>(rmode, true) : pick_mx<MXQ_BF16, false>(rmode, ze);
-    return full ? pick_mx<MXQ_F32, true>(rmode, true) : pick_mx<MXQ_F32, false>(rmode, ze);
+// lean = false selects the op-by-op form, which always consults the zone table
+MxElemFn pick_mx(int dtype, int rmode, bool ze, bool lean) {
+    if (dtype == MXQ_DTYPE_BF16) return lean ? pick_mx<MXQ_BF16, true>(rmode, ze) : pick_mx<MXQ_BF16, false>(rmode, true);
+    return lean ? pick_mx<MXQ_F32, true>(rmode, ze) : pick_mx<MXQ_F32, false>(rmode, true);
 }
-template <int DT, bool FULL>
-ElemFn pick_elem(int rmode) {
-    if (rmode == MXQ_ROUND_FLOOR) return mxq_quant_elemwise<MXQ_FLOOR, DT, FULL>;
-    if (rmode == MXQ_ROUND_NEAREST) return mxq_quant_elemwise<MXQ_NEAREST, DT, FULL>;
-    return mxq_quant_elemwise<MXQ_EVEN, DT, FULL>;
+template <int DT, bool LEAN>
+ElemFn pick_elem(int rmode, bool ze) {
+    if (rmode == MXQ_ROUND_FLOOR) return ze ? mxq_quant_elemwise<MXQ_FLOOR, DT, true, LEAN> : mxq_quant_elemwise<MXQ_FLOOR, DT, false, LEAN>;
+    if (rmode == MXQ_ROUND_NEAREST) return ze ? mxq_quant_elemwise<MXQ_NEAREST, DT, true, LEAN> : mxq_quant_elemwise<MXQ_NEAREST, DT, false, LEAN>;
+    return ze ? mxq_quant_elemwise<MXQ_EVEN, DT, true, LEAN> : mxq_quant_elemwise<MXQ_EVEN, DT, false, LEAN>;
+}
+ElemFn pick_elem(int dtype, int rmode, bool ze, bool lean) {
+    if (dtype == MXQ_DTYPE_BF16) return lean ? pick_elem<MXQ_BF16, true>(rmode, ze) : pick_elem<MXQ_BF16, false>(rmode, true);
+    return lean ? pick_elem<MXQ_F32, true>(rmode, ze) : pick_elem<MXQ_F32, false>(rmode, true);
 }
 
 }  // namespace
@@ -80,7 +85,7 @@ int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t p
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const int64_t tile = (tile_size <= 0 || tile_size > axis_size) ? axis_size : tile_size;
     const unsigned char* zone = kZone[p.zone_row];
-    MxElemFn fn = pick_mx(dtype, rmode, ze, (flags & MXQ_HOST_FLAG_ROUND_EVERY_OP) != 0);
+    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < pre; ++i)
         for (int64_t k0 = 0; k0 < axis_size; k0 += tile)
             for (int64_t j = 0; j < post; ++j) {
@@ -113,7 +118,7 @@ int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_va
     if (total == 0) return MXQ_OK;
     if (!in || !out || !max_values) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const unsigned char* zone = kZone[p.zone_row];
-    MxElemFn fn = pick_mx(dtype, rmode, ze, (flags & MXQ_HOST_FLAG_ROUND_EVERY_OP) != 0);
+    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < pre; ++i)
         for (int64_t j = 0; j < post; ++j) {
             const uint32_t um = mxq_bits(load_as_float(max_values, dtype, i * post + j)) & 0x7FFFFFFFu;
@@ -138,7 +143,8 @@ int mxq_host_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, 
     if (n == 0) return MXQ_OK;
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const unsigned char* zone = kZone[p.zone_row];
-    ElemFn fn = dtype == MXQ_DTYPE_BF16 ? pick_elem<MXQ_BF16, true>(rmode) : pick_elem<MXQ_F32, true>(rmode);
+    ElemFn fn = pick_elem(dtype, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode),
+                           lean_ok(dtype, p.fmt) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < n; ++i)
         store_from_float(out, dtype, i,
                          fn(load_as_float(in, dtype, i), p.fmt, p.saturate != 0, p.allow_denorm != 0, zone, p.zshift));

@@ -20,8 +20,10 @@ __device__ const unsigned char g_zone_tables[3][ZONE_PAD] = {
 
 namespace {
 
+constexpr int TPB = 256;                 // lanes per workgroup (4 wave64), fixed for every kernel
+
 __device__ __forceinline__ void load_zone(unsigned char* lds, const unsigned char* src) {
-    for (int i = threadIdx.x; i < ZONE_PAD / 4; i += blockDim.x)
+    for (int i = threadIdx.x; i < ZONE_PAD / 4; i += TPB)
         reinterpret_cast<uint32_t*>(lds)[i] = reinterpret_cast<const uint32_t*>(src)[i];
     __syncthreads();
 }
@@ -38,9 +40,11 @@ template <> struct Pack<MXQ_BF16> {
     static __device__ __forceinline__ float get(uint32_t w, int half) {
         return mxq_float(half ? (w & 0xFFFF0000u) : (w << 16));
     }
-    // values are already bf16-exact: keep the top halves
+    // round to nearest even and pack: one v_cvt_pk_bf16_f32 per pair
     static __device__ __forceinline__ uint32_t put(float lo, float hi) {
-        return (mxq_bits(lo) >> 16) | (mxq_bits(hi) & 0xFFFF0000u);
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
     }
 };
 template <> struct Pack<MXQ_F16> {
@@ -79,6 +83,25 @@ __device__ __forceinline__ void store_scalar(void* p, int64_t i, float v) {
 
 __device__ __forceinline__ uint32_t abs_bits(float f) { return mxq_bits(f) & 0x7FFFFFFFu; }
 
+// max |x| over the 16 bytes a lane holds, as an fp32-layout bit pattern.  Magnitude bit patterns
+// order like unsigned integers, and Inf/NaN patterns sit above every finite one, so an integer
+// max both finds the maximum and propagates Inf/NaN.  16-bit dtypes are reduced two per dword.
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+template <int DT>
+__device__ __forceinline__ uint32_t vec_abs_max(const u32x4& v) {
+    if (DT == MXQ_F32) {
+        return max(max(v[0] & 0x7FFFFFFFu, v[1] & 0x7FFFFFFFu),
+                   max(v[2] & 0x7FFFFFFFu, v[3] & 0x7FFFFFFFu));
+    }
+    u16x2 m = __builtin_bit_cast(u16x2, v[0] & 0x7FFF7FFFu);
+#pragma unroll
+    for (int d = 1; d < 4; ++d)
+        m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, v[d] & 0x7FFF7FFFu));
+    const unsigned short h = m[0] > m[1] ? m[0] : m[1];
+    if (DT == MXQ_BF16) return (uint32_t)h << 16;
+    return abs_bits((float)__builtin_bit_cast(_Float16, h));
+}
+
 // ---- lane exchange ----------------------------------------------------------------------------
 // max over groups of LANES consecutive lanes (LANES in 1,2,4,8,16), result in every lane
 template <int LANES>
@@ -98,22 +121,24 @@ __device__ __forceinline__ uint32_t group_max(uint32_t v) {
 // MX quantization, shared axis innermost, tile = LPT lanes x 16 bytes, tile-aligned tensor.
 // One lane owns 16 bytes (4 fp32 / 8 16-bit elements); LPT neighbouring lanes share a tile.
 // ================================================================================================
-template <int DT, int RMODE, int LPT, bool ZONE_ELEM, int UNROLL>
-__global__ __launch_bounds__(256) void mx_lastaxis_kernel(const u32x4* __restrict__ in,
+template <int DT, int RMODE, bool ZONE_ELEM, bool LEAN, int LPT, int UNROLL>
+__global__ __launch_bounds__(TPB) void mx_lastaxis_kernel(const u32x4* __restrict__ in,
                                                           u32x4* __restrict__ out, int64_t n_vec,
                                                           MxParams p) {
     constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
     constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int64_t CHUNK = (int64_t)TPB * UNROLL;      // vectors per block and iteration
     __shared__ unsigned char zone[ZONE_PAD];
 
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x * UNROLL;
-    int64_t base = (int64_t)blockIdx.x * blockDim.x * UNROLL + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * CHUNK;
+    int64_t base = (int64_t)blockIdx.x * CHUNK + threadIdx.x;
 
     // first batch of loads goes out before the table copy so the two latencies overlap
     u32x4 v[UNROLL];
 #pragma unroll
     for (int j = 0; j < UNROLL; ++j) {
-        int64_t i = base + (int64_t)j * blockDim.x;
+        const int64_t i = base + j * TPB;
         v[j] = (i < n_vec) ? in[i] : u32x4{0, 0, 0, 0};
     }
     load_zone(zone, g_zone_tables[p.zone_row]);
@@ -121,26 +146,17 @@ __global__ __launch_bounds__(256) void mx_lastaxis_kernel(const u32x4* __restric
     while (true) {
 #pragma unroll
         for (int j = 0; j < UNROLL; ++j) {
-            int64_t i = base + (int64_t)j * blockDim.x;
-            float x[4 * PD];
-            uint32_t um = 0;
-#pragma unroll
-            for (int d = 0; d < 4; ++d)
-#pragma unroll
-                for (int h = 0; h < PD; ++h) {
-                    x[d * PD + h] = Pack<DT>::get(v[j][d], h);
-                    um = max(um, abs_bits(x[d * PD + h]));
-                }
-            um = group_max<LPT>(um);
-            MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+            const int64_t i = base + j * TPB;
+            const uint32_t um = group_max<LPT>(vec_abs_max<DT>(v[j]));
+            const MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, ZS);
             u32x4 o;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
                 float q[2];
 #pragma unroll
                 for (int h = 0; h < PD; ++h)
-                    q[h] = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, false>(x[d * PD + h], sc, p.fmt,
-                                                                          zone, p.zshift);
+                    q[h] = mxq_quant_mx_elem_raw<RMODE, ADT, ZONE_ELEM, LEAN>(Pack<DT>::get(v[j][d], h),
+                                                                             sc, p.fmt, zone, ZS);
                 o[d] = Pack<DT>::put(q[0], q[PD - 1]);
             }
             if (i < n_vec) __builtin_nontemporal_store(o, &out[i]);
@@ -149,7 +165,7 @@ __global__ __launch_bounds__(256) void mx_lastaxis_kernel(const u32x4* __restric
         if (base - threadIdx.x >= n_vec) break;     // uniform per block
 #pragma unroll
         for (int j = 0; j < UNROLL; ++j) {
-            int64_t i = base + (int64_t)j * blockDim.x;
+            const int64_t i = base + j * TPB;
             v[j] = (i < n_vec) ? in[i] : u32x4{0, 0, 0, 0};
         }
     }
@@ -158,18 +174,90 @@ __global__ __launch_bounds__(256) void mx_lastaxis_kernel(const u32x4* __restric
 // ================================================================================================
 // MX quantization along any axis: tensor (pre, axis, post), tiles of `tile` rows of the middle
 // axis.  One lane owns VW consecutive `post` positions of one tile, so a wave reads 64*VW
-// contiguous elements per row.  ROWS > 0: the tile (<= ROWS rows) stays in registers between the
-// max pass and the rounding pass; ROWS == 0: any tile size, second pass re-reads memory.
+// contiguous elements per row.
+//   mx_strided_tile_kernel  tile == ROWS exactly and axis % ROWS == 0, post % VW == 0: the tile
+//                           stays in registers between the max pass and the rounding pass (one
+//                           read of the input), 8-byte accesses per lane.
+//   mx_strided_kernel       anything else (ragged last tile, odd sizes, VW = 1): the rounding pass
+//                           re-reads the tile.
 // ================================================================================================
+template <int DT> struct Col8 {                      // the 8 bytes a lane owns per row
+    static constexpr int VW = (DT == MXQ_F32) ? 2 : 4;
+};
+
+template <int DT, int RMODE, bool ZONE_ELEM, bool LEAN, int ROWS>
+__global__ __launch_bounds__(TPB) void mx_strided_tile_kernel(const u32x2* __restrict__ in,
+                                                              u32x2* __restrict__ out,
+                                                              int64_t items, int64_t n_tiles,
+                                                              int64_t pv, MxParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
+    constexpr int VW = Col8<DT>::VW;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    __shared__ unsigned char zone[ZONE_PAD];
+
+    const int64_t w = (int64_t)blockIdx.x * TPB + threadIdx.x;     // (pre_i, tile_i, column group)
+    const bool live = w < items;
+    const int64_t c = live ? w % pv : 0;
+    const int64_t pt = live ? w / pv : 0;                           // pre_i * n_tiles + tile_i
+    const int64_t off0 = pt * ROWS * pv + c;                        // in units of 8 bytes
+
+    u32x2 raw[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) raw[r] = live ? in[off0 + (int64_t)r * pv] : u32x2{0, 0};
+    load_zone(zone, g_zone_tables[p.zone_row]);
+
+    // column maxima as fp32-layout magnitude patterns
+    uint32_t um[VW];
+    if (DT == MXQ_F32) {
+        um[0] = um[1] = 0;
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            um[0] = max(um[0], raw[r][0] & 0x7FFFFFFFu);
+            um[1] = max(um[1], raw[r][1] & 0x7FFFFFFFu);
+        }
+    } else {
+        u16x2 m0 = {0, 0}, m1 = {0, 0};
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            m0 = __builtin_elementwise_max(m0, __builtin_bit_cast(u16x2, raw[r][0] & 0x7FFF7FFFu));
+            m1 = __builtin_elementwise_max(m1, __builtin_bit_cast(u16x2, raw[r][1] & 0x7FFF7FFFu));
+        }
+        const unsigned short h[4] = {m0[0], m0[1], m1[0], m1[1]};
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            um[k % VW] = (DT == MXQ_BF16) ? (uint32_t)h[k] << 16
+                                          : abs_bits((float)__builtin_bit_cast(_Float16, h[k]));
+    }
+    MxqScale sc[VW];
+#pragma unroll
+    for (int k = 0; k < VW; ++k)
+        sc[k] = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        u32x2 o;
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+            float q[2];
+#pragma unroll
+            for (int h = 0; h < PD; ++h)
+                q[h] = mxq_quant_mx_elem_raw<RMODE, ADT, ZONE_ELEM, LEAN>(Pack<DT>::get(raw[r][d], h),
+                                                                         sc[d * PD + h], p.fmt, zone,
+                                                                         ZS);
+            o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+        }
+        if (live) __builtin_nontemporal_store(o, &out[off0 + (int64_t)r * pv]);
+    }
+}
+
 template <int DT, int VW> struct ColVec;     // VW elements of dtype DT
 template <> struct ColVec<MXQ_F32, 1> { typedef uint32_t T; static constexpr int DW = 1; };
 template <> struct ColVec<MXQ_F32, 4> { typedef u32x4 T; static constexpr int DW = 4; };
 template <> struct ColVec<MXQ_BF16, 1> { typedef unsigned short T; static constexpr int DW = 1; };
 template <> struct ColVec<MXQ_BF16, 8> { typedef u32x4 T; static constexpr int DW = 4; };
-template <> struct ColVec<MXQ_BF16, 4> { typedef u32x2 T; static constexpr int DW = 2; };
 template <> struct ColVec<MXQ_F16, 1> { typedef unsigned short T; static constexpr int DW = 1; };
 template <> struct ColVec<MXQ_F16, 8> { typedef u32x4 T; static constexpr int DW = 4; };
-template <> struct ColVec<MXQ_F16, 4> { typedef u32x2 T; static constexpr int DW = 2; };
 
 template <int DT, int VW>
 __device__ __forceinline__ void unpack_cols(const typename ColVec<DT, VW>::T& raw, float* x) {
@@ -200,13 +288,14 @@ __device__ __forceinline__ typename ColVec<DT, VW>::T pack_cols(const float* q) 
     return r;
 }
 
-template <int DT, int RMODE, int VW, int ROWS, bool ZONE_ELEM>
-__global__ __launch_bounds__(256) void mx_strided_kernel(const void* __restrict__ in_,
+template <int DT, int RMODE, bool ZONE_ELEM, bool LEAN, int VW>
+__global__ __launch_bounds__(TPB) void mx_strided_kernel(const void* __restrict__ in_,
                                                          void* __restrict__ out_, int64_t pre,
                                                          int64_t axis_size, int64_t post,
                                                          int64_t tile, int64_t num_tiles,
                                                          MxParams p) {
     constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
     typedef typename ColVec<DT, VW>::T V;
     __shared__ unsigned char zone[ZONE_PAD];
     load_zone(zone, g_zone_tables[p.zone_row]);
@@ -215,67 +304,35 @@ __global__ __launch_bounds__(256) void mx_strided_kernel(const void* __restrict_
     V* out = reinterpret_cast<V*>(out_);
     const int64_t pv = post / VW;                       // column groups per row
     const int64_t total = pre * num_tiles * pv;
-    for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total;
-         w += (int64_t)gridDim.x * blockDim.x) {
+    for (int64_t w = (int64_t)blockIdx.x * TPB + threadIdx.x; w < total;
+         w += (int64_t)gridDim.x * TPB) {
         const int64_t c = w % pv;
         const int64_t ti = (w / pv) % num_tiles;
         const int64_t pi = w / (pv * num_tiles);
         const int64_t row0 = ti * tile;
-        const int rows = (int)((row0 + tile > axis_size) ? (axis_size - row0) : tile);
+        const int64_t rows = (row0 + tile > axis_size) ? (axis_size - row0) : tile;
         const int64_t off0 = (pi * axis_size + row0) * pv + c;   // in units of V
 
         uint32_t um[VW];
 #pragma unroll
         for (int k = 0; k < VW; ++k) um[k] = 0;
-
-        if constexpr (ROWS > 0) {
-            V raw[ROWS];
+        for (int64_t r = 0; r < rows; ++r) {
+            float x[VW];
+            unpack_cols<DT, VW>(in[off0 + r * pv], x);
 #pragma unroll
-            for (int r = 0; r < ROWS; ++r)
-                if (r < rows) raw[r] = in[off0 + (int64_t)r * pv];
+            for (int k = 0; k < VW; ++k) um[k] = max(um[k], abs_bits(x[k]));
+        }
+        MxqScale sc[VW];
 #pragma unroll
-            for (int r = 0; r < ROWS; ++r)
-                if (r < rows) {
-                    float x[VW];
-                    unpack_cols<DT, VW>(raw[r], x);
-#pragma unroll
-                    for (int k = 0; k < VW; ++k) um[k] = max(um[k], abs_bits(x[k]));
-                }
-            MxqScale sc[VW];
+        for (int k = 0; k < VW; ++k)
+            sc[k] = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+        for (int64_t r = 0; r < rows; ++r) {
+            float x[VW], q[VW];
+            unpack_cols<DT, VW>(in[off0 + r * pv], x);
 #pragma unroll
             for (int k = 0; k < VW; ++k)
-                sc[k] = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
-#pragma unroll
-            for (int r = 0; r < ROWS; ++r)
-                if (r < rows) {
-                    float x[VW], q[VW];
-                    unpack_cols<DT, VW>(raw[r], x);
-#pragma unroll
-                    for (int k = 0; k < VW; ++k)
-                        q[k] = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, false>(x[k], sc[k], p.fmt,
-                                                                              zone, p.zshift);
-                    __builtin_nontemporal_store(pack_cols<DT, VW>(q), &out[off0 + (int64_t)r * pv]);
-                }
-        } else {
-            for (int r = 0; r < rows; ++r) {
-                float x[VW];
-                unpack_cols<DT, VW>(in[off0 + (int64_t)r * pv], x);
-#pragma unroll
-                for (int k = 0; k < VW; ++k) um[k] = max(um[k], abs_bits(x[k]));
-            }
-            MxqScale sc[VW];
-#pragma unroll
-            for (int k = 0; k < VW; ++k)
-                sc[k] = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
-            for (int r = 0; r < rows; ++r) {
-                float x[VW], q[VW];
-                unpack_cols<DT, VW>(in[off0 + (int64_t)r * pv], x);
-#pragma unroll
-                for (int k = 0; k < VW; ++k)
-                    q[k] = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, false>(x[k], sc[k], p.fmt, zone,
-                                                                          p.zshift);
-                out[off0 + (int64_t)r * pv] = pack_cols<DT, VW>(q);
-            }
+                q[k] = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, LEAN>(x[k], sc[k], p.fmt, zone, ZS);
+            out[off0 + r * pv] = pack_cols<DT, VW>(q);
         }
     }
 }
@@ -284,23 +341,24 @@ __global__ __launch_bounds__(256) void mx_strided_kernel(const void* __restrict_
 // MX quantization with the block maximum supplied by the caller: element (i, k, j) uses
 // max_values[i * post + j].
 // ================================================================================================
-template <int DT, int RMODE, bool ZONE_ELEM>
-__global__ __launch_bounds__(256) void mx_given_max_kernel(const void* __restrict__ in,
+template <int DT, int RMODE, bool ZONE_ELEM, bool LEAN>
+__global__ __launch_bounds__(TPB) void mx_given_max_kernel(const void* __restrict__ in,
                                                            void* __restrict__ out,
                                                            const void* __restrict__ maxv,
                                                            int64_t total, int64_t axis_size,
                                                            int64_t post, MxParams p) {
     constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
     __shared__ unsigned char zone[ZONE_PAD];
     load_zone(zone, g_zone_tables[p.zone_row]);
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-         i += (int64_t)gridDim.x * blockDim.x) {
+    for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * TPB) {
         const int64_t j = i % post;
         const int64_t pi = i / (post * axis_size);
         const uint32_t um = abs_bits(load_scalar<DT>(maxv, pi * post + j));
-        MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
-        float q = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, false>(load_scalar<DT>(in, i), sc, p.fmt,
-                                                                 zone, p.zshift);
+        MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+        float q = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, LEAN>(load_scalar<DT>(in, i), sc, p.fmt,
+                                                                 zone, ZS);
         store_scalar<DT>(out, i, q);
     }
 }
@@ -308,11 +366,12 @@ __global__ __launch_bounds__(256) void mx_given_max_kernel(const void* __restric
 // ================================================================================================
 // Elementwise quantization.  Body: 16 bytes per lane; the (< 16 byte) tail is done per element.
 // ================================================================================================
-template <int DT, int RMODE, int UNROLL>
-__global__ __launch_bounds__(256) void elemwise_kernel(const void* __restrict__ in_,
+template <int DT, int RMODE, bool ZONE_ELEM, bool LEAN, int UNROLL>
+__global__ __launch_bounds__(TPB) void elemwise_kernel(const void* __restrict__ in_,
                                                        void* __restrict__ out_, int64_t n,
                                                        ElemParams p) {
     constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
     constexpr int PD = Pack<DT>::PER_DWORD;
     constexpr int EPV = 4 * PD;
     __shared__ unsigned char zone[ZONE_PAD];
@@ -321,27 +380,27 @@ __global__ __launch_bounds__(256) void elemwise_kernel(const void* __restrict__ 
     const u32x4* in = reinterpret_cast<const u32x4*>(in_);
     u32x4* out = reinterpret_cast<u32x4*>(out_);
     const int64_t n_vec = n / EPV;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x * UNROLL;
-    for (int64_t base = (int64_t)blockIdx.x * blockDim.x * UNROLL + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * TPB * UNROLL;
+    for (int64_t base = (int64_t)blockIdx.x * TPB * UNROLL + threadIdx.x;
          base - threadIdx.x < n_vec; base += stride) {
         u32x4 v[UNROLL];
 #pragma unroll
         for (int j = 0; j < UNROLL; ++j) {
-            int64_t i = base + (int64_t)j * blockDim.x;
+            int64_t i = base + (int64_t)j * TPB;
             v[j] = (i < n_vec) ? in[i] : u32x4{0, 0, 0, 0};
         }
 #pragma unroll
         for (int j = 0; j < UNROLL; ++j) {
-            int64_t i = base + (int64_t)j * blockDim.x;
+            int64_t i = base + (int64_t)j * TPB;
             u32x4 o;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
                 float q[2];
 #pragma unroll
                 for (int h = 0; h < PD; ++h)
-                    q[h] = mxq_quant_elemwise<RMODE, ADT, true>(Pack<DT>::get(v[j][d], h), p.fmt,
-                                                                p.saturate != 0, p.allow_denorm != 0,
-                                                                zone, p.zshift);
+                    q[h] = mxq_quant_elemwise<RMODE, ADT, ZONE_ELEM, LEAN>(Pack<DT>::get(v[j][d], h), p.fmt,
+                                                                           p.saturate != 0,
+                                                                           p.allow_denorm != 0, zone, ZS);
                 o[d] = Pack<DT>::put(q[0], q[PD - 1]);
             }
             if (i < n_vec) __builtin_nontemporal_store(o, &out[i]);
@@ -349,11 +408,11 @@ __global__ __launch_bounds__(256) void elemwise_kernel(const void* __restrict__ 
     }
     // tail
     const int64_t t0 = n_vec * EPV;
-    const int64_t gi = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t gi = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (gi < n - t0) {
-        float q = mxq_quant_elemwise<RMODE, ADT, true>(load_scalar<DT>(in_, t0 + gi), p.fmt,
-                                                       p.saturate != 0, p.allow_denorm != 0, zone,
-                                                       p.zshift);
+        float q = mxq_quant_elemwise<RMODE, ADT, ZONE_ELEM, LEAN>(load_scalar<DT>(in_, t0 + gi), p.fmt,
+                                                                  p.saturate != 0, p.allow_denorm != 0,
+                                                                  zone, ZS);
         store_scalar<DT>(out_, t0 + gi, q);
     }
 }
@@ -381,7 +440,7 @@ __device__ __forceinline__ float wave_reduce(float v) {
 
 // one block of 256 lanes per row (inner large) ...
 template <class OP>
-__global__ __launch_bounds__(256) void reduce_inner_block_kernel(const float* __restrict__ in,
+__global__ __launch_bounds__(TPB) void reduce_inner_block_kernel(const float* __restrict__ in,
                                                                  float* __restrict__ out,
                                                                  int64_t rows, int64_t inner) {
     __shared__ float part[4];
@@ -391,20 +450,20 @@ __global__ __launch_bounds__(256) void reduce_inner_block_kernel(const float* __
         const bool vec_ok = (inner % 4 == 0) && ((reinterpret_cast<uintptr_t>(row) & 15) == 0);
         if (vec_ok) {
             const u32x4* rv = reinterpret_cast<const u32x4*>(row);
-            for (int64_t i = threadIdx.x; i < inner / 4; i += blockDim.x) {
+            for (int64_t i = threadIdx.x; i < inner / 4; i += TPB) {
                 u32x4 w = rv[i];
 #pragma unroll
                 for (int d = 0; d < 4; ++d) acc = OP::apply(acc, mxq_float(w[d]));
             }
         } else {
-            for (int64_t i = threadIdx.x; i < inner; i += blockDim.x) acc = OP::apply(acc, row[i]);
+            for (int64_t i = threadIdx.x; i < inner; i += TPB) acc = OP::apply(acc, row[i]);
         }
         acc = wave_reduce<OP>(acc);
         if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
         __syncthreads();
         if (threadIdx.x == 0) {
             float t = part[0];
-            for (int wv = 1; wv < (int)(blockDim.x >> 6); ++wv) t = OP::apply(t, part[wv]);
+            for (int wv = 1; wv < (int)(TPB >> 6); ++wv) t = OP::apply(t, part[wv]);
             out[r] = t;
         }
         __syncthreads();
@@ -413,12 +472,12 @@ __global__ __launch_bounds__(256) void reduce_inner_block_kernel(const float* __
 
 // ... or one wave per row (inner small)
 template <class OP>
-__global__ __launch_bounds__(256) void reduce_inner_wave_kernel(const float* __restrict__ in,
+__global__ __launch_bounds__(TPB) void reduce_inner_wave_kernel(const float* __restrict__ in,
                                                                 float* __restrict__ out,
                                                                 int64_t rows, int64_t inner) {
     const int lane = threadIdx.x & 63;
-    const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const int64_t n_waves = ((int64_t)gridDim.x * blockDim.x) >> 6;
+    const int64_t wave = ((int64_t)blockIdx.x * TPB + threadIdx.x) >> 6;
+    const int64_t n_waves = ((int64_t)gridDim.x * TPB) >> 6;
     for (int64_t r = wave; r < rows; r += n_waves) {
         const float* row = in + r * inner;
         float acc = OP::init();
@@ -440,11 +499,11 @@ __global__ __launch_bounds__(256) void reduce_inner_wave_kernel(const float* __r
 
 // outer axis: (outer, inner) -> partial (splits, inner); lane owns 4 (or 1) consecutive columns
 template <class OP, int VW>
-__global__ __launch_bounds__(256) void reduce_outer_kernel(const float* __restrict__ in,
+__global__ __launch_bounds__(TPB) void reduce_outer_kernel(const float* __restrict__ in,
                                                            float* __restrict__ partial,
                                                            int64_t outer, int64_t inner,
                                                            int64_t rows_per_split) {
-    const int64_t cg = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // column group
+    const int64_t cg = (int64_t)blockIdx.x * TPB + threadIdx.x;   // column group
     if (cg * VW >= inner) return;
     const int64_t r0 = (int64_t)blockIdx.y * rows_per_split;
     const int64_t r1 = (r0 + rows_per_split < outer) ? r0 + rows_per_split : outer;
@@ -481,10 +540,10 @@ __global__ __launch_bounds__(256) void reduce_outer_kernel(const float* __restri
 }
 
 template <class OP>
-__global__ __launch_bounds__(256) void reduce_outer_final_kernel(const float* __restrict__ partial,
+__global__ __launch_bounds__(TPB) void reduce_outer_final_kernel(const float* __restrict__ partial,
                                                                  float* __restrict__ out,
                                                                  int64_t splits, int64_t inner) {
-    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t c = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (c >= inner) return;
     float acc = OP::init();
     for (int64_t s = 0; s < splits; ++s) acc = OP::apply(acc, partial[s * inner + c]);

@@ -32,6 +32,9 @@ struct ElemParams {
 
 namespace mxq_detail {
 
+// host copy of the round-up-zone tables (the kernels read theirs from device memory)
+static const unsigned char zone_rows[2][MXQ_ZONE_PAD] = {{MXQ_ZONE_ROW_F32}, {MXQ_ZONE_ROW_BF16}};
+
 inline std::string& last_error() {
     static thread_local std::string s;
     return s;
@@ -68,6 +71,13 @@ inline int make_fmt(int dtype, int ebits, int mbits, float max_norm, MxqFmt* fmt
     fmt->min_exp = ebits ? 2 - (1 << (ebits - 1)) : 0;
     // torch casts the clamp bound to the tensor dtype (65504 becomes 65536 for a bf16 tensor)
     fmt->max_bits = mxq_bits(dtype == MXQ_DTYPE_BF16 ? mxq_round_bf16(max_norm) : max_norm);
+    fmt->min_eb = ebits ? (uint32_t)(fmt->min_exp + 127) : 127u;
+    fmt->t127 = fmt->t + 127;
+    // "s + 0.5" is rounded to the tensor dtype before the floor: in bf16 that turns 1 - 2^-9 into
+    // 1.0, which adding 2^-9 more reproduces (all other sums keep their integer part)
+    fmt->half = dtype == MXQ_DTYPE_BF16 ? 0.5f + 0.001953125f : 0.5f;
+    fmt->tie_fix = dtype == MXQ_DTYPE_BF16 ? 0.5f - 0.001953125f : 0.5f - 2.98023223876953125e-8f;
+    fmt->nan_from = MXQ_INF_BITS;
     return MXQ_OK;
 }
 
@@ -82,6 +92,10 @@ inline void zone_for(int dtype, int flags, int* row, int* zshift) {
         *row = ZONE_ROW_F32;
     }
 }
+
+// May the lean element rounding be used (see mxq_round_lean)?  bf16 tensors with 7 or more
+// fraction bits need the op-by-op form: there "s + 0.5" itself ties in bf16.
+inline bool lean_ok(int dtype, const MxqFmt& f) { return dtype != MXQ_DTYPE_BF16 || f.t <= 6; }
 
 // Does the round-up zone of the *element* exponent change results?  In nearest / even modes a
 // value in the zone rounds to the next power of two whichever exponent is used, as long as the
@@ -123,6 +137,10 @@ inline int make_elem_params(int dtype, int bits, int exp_bits, float max_norm, i
     p->saturate = saturate ? 1 : 0;
     p->allow_denorm = allow_denorm ? 1 : 0;
     zone_for(dtype, flags, &p->zone_row, &p->zshift);
+    // the top binade's round-up zone: floor(log2|x|) = 128 there
+    static const unsigned char top_count[3] = {zone_rows[0][276], zone_rows[1][276], 0};
+    p->fmt.nan_from = exp_bits ? MXQ_INF_BITS - ((uint32_t)top_count[p->zone_row] << p->zshift)
+                               : MXQ_INF_BITS;
     return MXQ_OK;
 }
 
