@@ -93,6 +93,24 @@ int mxq_reduce_sum_outer(const float* in, float* out, void* workspace, int64_t o
 int mxq_reduce_max_outer(const float* in, float* out, void* workspace, int64_t outer,
                          int64_t inner, void* hip_stream);
 
+/* ---- packed MX tensors and the fused GEMM (no counterpart in the reference, which only ever
+ * fake-quantizes and then calls a dense GEMM: mx/linear.py:62-86, mx/bmm.py:40-59) ---------------
+ * Packed form of a (rows, K) tensor quantized along K in blocks of 32:
+ *   codes  uint8 (rows, K)     OCP e4m3 for fp8_e4m3 / fp6_e3m2 / fp6_e2m3 / fp4_e2m1 elements (e4m3
+ *                              holds all their values exactly), OCP e5m2 for fp8_e5m2 elements
+ *   scales uint8 (rows, K/32)  E8M0 (shared exponent + 127; 255 = the block is NaN)
+ * value = code * 2^(scale - 127), identical to what mxq_quantize_mx_by_tile returns. */
+int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t rows, int64_t K,
+                int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                int flush_fp32_subnorms, int rmode, int flags, void* hip_stream);
+int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, void* out, int dtype,
+                  int64_t rows, int64_t K, void* hip_stream);
+/* C[b] (M, N) = A[b] (M, K) x B[b] (N, K)^T for b < batch, all tensors contiguous, fp32
+ * accumulation on the scaled MFMA units; c_dtype is a MXQ_DTYPE_* code.  K % 128 == 0. */
+int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, const void* b_codes,
+                   const void* b_scales, int b_is_e5m2, void* c, int c_dtype, int64_t batch,
+                   int64_t M, int64_t N, int64_t K, void* hip_stream);
+
 /* ---- libmxq_host.so: the same arithmetic compiled for the host ----------------------------------
  * quantize_mx_func_cpp (mx/cpp/funcs.cpp:23-98) and quantize_elemwise_func_cpp
  * (mx/cpp/funcs.cpp:117-149) take CPU tensors; these are their stand-ins.  Pointers are host

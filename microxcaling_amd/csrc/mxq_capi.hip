@@ -5,6 +5,7 @@
 
 #include "mxq.h"
 #include "mxq_kernels.h"
+#include "mxq_gemm.h"
 
 namespace {
 
@@ -127,12 +128,31 @@ struct LaunchElemwise {
     }
 };
 
+template <int DT, int RMODE, bool ZE, bool LEAN>
+struct LaunchPack {
+    static void run(const void* in, void* codes, void* scales, int64_t n_vec, bool bf8, MxParams p,
+                    hipStream_t s) {
+        const int grid = grid_for(ceil_div(n_vec, (int64_t)kThreads * 4));
+        const u32x4* i4 = reinterpret_cast<const u32x4*>(in);
+        unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
+        if (bf8) mx_pack_kernel<DT, RMODE, ZE, true, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+        else mx_pack_kernel<DT, RMODE, ZE, false, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+    }
+};
+
+template <int CB, int BL>
+void launch_gemm(int c_dtype, dim3 grid, const GemmArgs& g, hipStream_t s) {
+    if (c_dtype == MXQ_DTYPE_F32) mx_gemm_nt_kernel<CB, BL, MXQ_F32><<<grid, kThreads, 0, s>>>(g);
+    else if (c_dtype == MXQ_DTYPE_BF16) mx_gemm_nt_kernel<CB, BL, MXQ_BF16><<<grid, kThreads, 0, s>>>(g);
+    else mx_gemm_nt_kernel<CB, BL, MXQ_F16><<<grid, kThreads, 0, s>>>(g);
+}
+
 // splits of the outer axis for the two-pass outer reduction
 int64_t outer_splits(int64_t outer, int64_t inner) {
     const int vw = (inner % 4 == 0) ? 4 : 1;
     const int64_t col_blocks = ceil_div(ceil_div(inner, vw), kThreads);
-    int64_t s = ceil_div(kMaxBlocks, col_blocks);
-    const int64_t most = ceil_div(outer, 16);          // at least 16 rows per split
+    int64_t s = ceil_div(2 * kMaxBlocks, col_blocks);
+    const int64_t most = ceil_div(outer, 32);          // at least 32 rows per split
     if (s > most) s = most;
     if (s < 1) s = 1;
     if (s > 65535) s = 65535;
@@ -172,7 +192,7 @@ int reduce_outer(const float* in, float* out, void* workspace, int64_t outer, in
     else reduce_outer_kernel<OP, 1><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
     int rc = check_launch(who);
     if (rc || splits == 1) return rc;
-    reduce_outer_final_kernel<OP><<<(unsigned)ceil_div(inner, kThreads), kThreads, 0, s>>>(partial, out, splits, inner);
+    reduce_outer_final_kernel<OP><<<(unsigned)ceil_div(inner, 64), kThreads, 0, s>>>(partial, out, splits, inner);
     return check_launch(who);
 }
 
@@ -250,6 +270,88 @@ int mxq_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int b
     if (!aligned16(in) || !aligned16(out))
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
     dispatch<LaunchElemwise>(dtype, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode), lean_ok(dtype, p.fmt), in, out, n, p, (hipStream_t)hip_stream);
+    return check_launch(who);
+}
+
+int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t rows, int64_t K,
+                int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                int flush_fp32_subnorms, int rmode, int flags, void* hip_stream) {
+    const char* who = "mxq_pack_mx";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    const bool bf8 = elem_ebits == 5 && elem_mbits <= 4;
+    if (!bf8 && !(elem_ebits >= 2 && elem_ebits <= 4 && elem_mbits <= 5))
+        return fail(MXQ_ERR_ARGUMENT, "%s: element format e%dm%d has no 8-bit float code "
+                    "(supported: up to e4m3, and e5m2)", who, elem_ebits, elem_mbits - 2);
+    if (rows < 0 || K < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (K % 32 != 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be a multiple of the block size 32", who);
+    int64_t total;
+    if (mul_overflows(rows, K, 1, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !codes || !scales) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(in) || !aligned16(codes))
+        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    dispatch<LaunchPack>(dtype, rmode, ze, true, in, codes, scales, total / (16 / elem_size(dtype)), bf8,
+                         p, (hipStream_t)hip_stream);
+    return check_launch(who);
+}
+
+int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, void* out, int dtype,
+                  int64_t rows, int64_t K, void* hip_stream) {
+    const char* who = "mxq_unpack_mx";
+    if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
+    if (rows < 0 || K < 0 || K % 32 != 0) return fail(MXQ_ERR_ARGUMENT, "%s: bad size", who);
+    const int64_t n = rows * K;
+    if (n == 0) return MXQ_OK;
+    if (!codes || !scales || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    const unsigned char* cd = reinterpret_cast<const unsigned char*>(codes);
+    const unsigned char* sc = reinterpret_cast<const unsigned char*>(scales);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int grid = grid_for(ceil_div(n, kThreads * 4));
+#define MXQ_UNPACK(DT)                                                                       \
+    if (codes_are_e5m2) mx_unpack_kernel<DT, true><<<grid, kThreads, 0, s>>>(cd, sc, out, n); \
+    else mx_unpack_kernel<DT, false><<<grid, kThreads, 0, s>>>(cd, sc, out, n);
+    if (dtype == MXQ_DTYPE_F32) { MXQ_UNPACK(MXQ_F32) }
+    else if (dtype == MXQ_DTYPE_BF16) { MXQ_UNPACK(MXQ_BF16) }
+    else { MXQ_UNPACK(MXQ_F16) }
+#undef MXQ_UNPACK
+    return check_launch(who);
+}
+
+int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, const void* b_codes,
+                   const void* b_scales, int b_is_e5m2, void* c, int c_dtype, int64_t batch,
+                   int64_t M, int64_t N, int64_t K, void* hip_stream) {
+    const char* who = "mxq_gemm_mx_nt";
+    if (c_dtype < 0 || c_dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, c_dtype);
+    if (batch < 0 || M < 0 || N < 0 || K < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (K % GEMM_BK != 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be a multiple of %d", who, GEMM_BK);
+    if (batch == 0 || M == 0 || N == 0) return MXQ_OK;
+    if (K == 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be positive", who);
+    if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF || batch > 65535)
+        return fail(MXQ_ERR_ARGUMENT, "%s: size too large", who);
+    if (!a_codes || !a_scales || !b_codes || !b_scales || !c) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(a_codes) || !aligned16(b_codes) || (reinterpret_cast<uintptr_t>(a_scales) & 3) ||
+        (reinterpret_cast<uintptr_t>(b_scales) & 3))
+        return fail(MXQ_ERR_ARGUMENT, "%s: codes must be 16-byte and scales 4-byte aligned", who);
+    GemmArgs g;
+    g.a = reinterpret_cast<const unsigned char*>(a_codes);
+    g.sa = reinterpret_cast<const unsigned char*>(a_scales);
+    g.b = reinterpret_cast<const unsigned char*>(b_codes);
+    g.sb = reinterpret_cast<const unsigned char*>(b_scales);
+    g.c = c;
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.batch_a = M * K; g.batch_sa = M * (K / 32);
+    g.batch_b = N * K; g.batch_sb = N * (K / 32);
+    g.batch_c = M * N;
+    dim3 grid((unsigned)ceil_div(N, GEMM_BN), (unsigned)ceil_div(M, GEMM_BM), (unsigned)batch);
+    hipStream_t s = (hipStream_t)hip_stream;
+    if (!a_is_e5m2 && !b_is_e5m2) launch_gemm<0, 0>(c_dtype, grid, g, s);
+    else if (a_is_e5m2 && !b_is_e5m2) launch_gemm<1, 0>(c_dtype, grid, g, s);
+    else if (!a_is_e5m2 && b_is_e5m2) launch_gemm<0, 1>(c_dtype, grid, g, s);
+    else launch_gemm<1, 1>(c_dtype, grid, g, s);
     return check_launch(who);
 }
 

@@ -210,6 +210,49 @@ MXQ_HD float mxq_quant_mx_elem(float x, const MxqScale& sc, const MxqFmt& f,
     return mxq_round_dt<DT>(mxq_quant_mx_elem_raw<RMODE, DT, ZONE, LEAN>(x, sc, f, zone, zshift));
 }
 
+// The same element, but as (value relative to the block scale): what a packed MX tensor stores.
+// Only element formats with at most 6 fraction bits exist in packed form, so the lean rounding
+// always applies.
+template <int RMODE, int DT, bool ZONE>
+MXQ_HD float mxq_quant_mx_elem_unscaled(float x, const MxqScale& sc, const MxqFmt& f,
+                                        const unsigned char* zone, int zshift) {
+    const float a = x * sc.inv_scale;
+    return mxq_round_lean<RMODE, ZONE>(a, mxq_sign_source<DT>(a), f, true, zone, zshift);
+}
+
+// OCP 8-bit float codes of a value that is exactly representable in the format (no rounding
+// happens here).  e4m3 is the "fn" variant: bias 7, subnormals m * 2^-9, no infinities.
+MXQ_HD uint32_t mxq_encode_e4m3(float y) {
+    const uint32_t u = mxq_bits(y), ua = u & 0x7FFFFFFFu;
+    const uint32_t normal = (ua >> 20) - (120u << 3);               // ((e + 7) << 3) | mantissa
+    const uint32_t subnormal = (uint32_t)(mxq_float(ua) * 512.0f);  // |y| / 2^-9
+    return ((u >> 24) & 0x80u) | ((ua >> 23) >= 121u ? normal : subnormal);
+}
+// e5m2: bias 15, subnormals m * 2^-16
+MXQ_HD uint32_t mxq_encode_e5m2(float y) {
+    const uint32_t u = mxq_bits(y), ua = u & 0x7FFFFFFFu;
+    const uint32_t normal = (ua >> 21) - (112u << 2);
+    const uint32_t subnormal = (uint32_t)(mxq_float(ua) * 65536.0f);
+    return ((u >> 24) & 0x80u) | ((ua >> 23) >= 113u ? normal : subnormal);
+}
+MXQ_HD float mxq_decode_e4m3(uint32_t c) {
+    const uint32_t e = (c >> 3) & 15u, m = c & 7u;
+    const float v = e ? ldexpf((float)(8u + m), (int)e - 10) : ldexpf((float)m, -9);
+    return (c & 0x80u) ? -v : v;
+}
+MXQ_HD float mxq_decode_e5m2(uint32_t c) {
+    const uint32_t e = (c >> 2) & 31u, m = c & 3u;
+    const float v = e ? ldexpf((float)(4u + m), (int)e - 17) : ldexpf((float)m, -16);
+    return (c & 0x80u) ? -v : v;
+}
+
+// E8M0 byte of a block scale: exponent + 127, 255 for a NaN block (MxqScale.scale is NaN)
+MXQ_HD uint32_t mxq_encode_e8m0(float scale) {
+    const uint32_t u = mxq_bits(scale);
+    if (u > MXQ_INF_BITS) return 255u;
+    return (u >> 23) ? (u >> 23) : 0u;            // 2^-127 is the fp32 subnormal 0x00400000 -> 0
+}
+
 // One element of the elementwise quantizer (mx/elemwise_ops.py:127-163).
 template <int RMODE, int DT, bool ZONE, bool LEAN>
 MXQ_HD float mxq_quant_elemwise(float x, const MxqFmt& f, bool saturate, bool allow_denorm,

@@ -514,15 +514,14 @@ __global__ __launch_bounds__(TPB) void reduce_outer_kernel(const float* __restri
         const u32x4* p = reinterpret_cast<const u32x4*>(in) + cg;
         const int64_t pv = inner / 4;
         int64_t r = r0;
-        for (; r + 4 <= r1; r += 4) {                 // four rows in flight
-            u32x4 w0 = p[r * pv], w1 = p[(r + 1) * pv], w2 = p[(r + 2) * pv], w3 = p[(r + 3) * pv];
+        for (; r + 8 <= r1; r += 8) {                 // eight rows (128 bytes per lane) in flight
+            u32x4 w[8];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                acc[k] = OP::apply(acc[k], mxq_float(w0[k]));
-                acc[k] = OP::apply(acc[k], mxq_float(w1[k]));
-                acc[k] = OP::apply(acc[k], mxq_float(w2[k]));
-                acc[k] = OP::apply(acc[k], mxq_float(w3[k]));
-            }
+            for (int u = 0; u < 8; ++u) w[u] = p[(r + u) * pv];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) acc[k] = OP::apply(acc[k], mxq_float(w[u][k]));
         }
         for (; r < r1; ++r) {
             u32x4 w = p[r * pv];
@@ -539,15 +538,35 @@ __global__ __launch_bounds__(TPB) void reduce_outer_kernel(const float* __restri
     }
 }
 
+// second pass: (splits, inner) -> (inner).  A block owns 64 columns; its four waves each reduce
+// every fourth split (eight loads in flight), then the four partials are combined in split order.
 template <class OP>
 __global__ __launch_bounds__(TPB) void reduce_outer_final_kernel(const float* __restrict__ partial,
                                                                  float* __restrict__ out,
                                                                  int64_t splits, int64_t inner) {
-    const int64_t c = (int64_t)blockIdx.x * TPB + threadIdx.x;
-    if (c >= inner) return;
+    __shared__ float part[4][64];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t c = (int64_t)blockIdx.x * 64 + lane;
     float acc = OP::init();
-    for (int64_t s = 0; s < splits; ++s) acc = OP::apply(acc, partial[s * inner + c]);
-    out[c] = acc;
+    if (c < inner) {
+        int64_t s = wv;
+        for (; s + 28 < splits; s += 32) {
+            float w[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) w[u] = partial[(s + 4 * u) * inner + c];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc = OP::apply(acc, w[u]);
+        }
+        for (; s < splits; s += 4) acc = OP::apply(acc, partial[s * inner + c]);
+    }
+    part[wv][lane] = acc;
+    __syncthreads();
+    if (wv == 0 && c < inner) {
+        float t = part[0][lane];
+#pragma unroll
+        for (int g = 1; g < 4; ++g) t = OP::apply(t, part[g][lane]);
+        out[c] = t;
+    }
 }
 
 }  // namespace

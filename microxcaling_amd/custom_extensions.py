@@ -31,6 +31,10 @@ def set_exponent_mode(mode):
         raise ValueError("exponent mode must be 'torch' or 'exact'")
 
 
+def _flags_value():
+    return _flags
+
+
 def _dtype_code(t, who):
     if t.dtype not in _DTYPE:
         raise RuntimeError("%s: Tensor dtype not supported (%s)" % (who, t.dtype))

@@ -1,0 +1,125 @@
+"""Fused MX GEMM: operands are quantized straight into packed element codes + E8M0 block scales
+and multiplied by the gfx950 scaled-MFMA kernel (include/mxq.h: mxq_pack_mx, mxq_gemm_mx_nt).
+
+Compared with fake-quantizing and calling a dense GEMM (the reference's way, mx/linear.py:62-86)
+the products are the same numbers -- code x code x 2^(scale_a + scale_b) -- accumulated in fp32 in
+a different order, so results agree to accumulation tolerance, not bit for bit.
+"""
+import torch
+
+from . import _lib
+from .custom_extensions import _DTYPE, _check_gpu_input, _flags_value, _stream
+from .formats import ElemFormat, RoundingMode, _get_format_params
+
+_PACKABLE = (ElemFormat.fp8_e4m3, ElemFormat.fp8_e5m2, ElemFormat.fp6_e3m2, ElemFormat.fp6_e2m3,
+             ElemFormat.fp4)
+GEMM_K_MULTIPLE = 128
+
+
+def _as_format(fmt):
+    if fmt is None:
+        return None
+    return ElemFormat.from_str(fmt) if type(fmt) is str else fmt
+
+
+def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=False):
+    """MX-quantize A along its last axis (block 32) into (codes, scales, codes_are_e5m2):
+    codes uint8 of A's shape, scales uint8 with the last axis divided by 32."""
+    who = "pack_mx"
+    fmt = _as_format(elem_format)
+    if fmt not in _PACKABLE:
+        raise RuntimeError("%s: element format %s has no packed form" % (who, fmt))
+    _check_gpu_input(A, "A", who)
+    if A.dtype not in _DTYPE:
+        raise RuntimeError("%s: Tensor dtype not supported (%s)" % (who, A.dtype))
+    K = A.shape[-1]
+    if A.dim() < 1 or K % 32 != 0:
+        raise RuntimeError("%s: the last axis must be a multiple of 32" % who)
+    ebits, mbits, _, max_norm, _ = _get_format_params(fmt)
+    rows = A.numel() // K if K else 0
+    codes = torch.empty(A.shape, dtype=torch.uint8, device=A.device)
+    scales = torch.empty(A.shape[:-1] + (K // 32,), dtype=torch.uint8, device=A.device)
+    lib = _lib.gpu()
+    with torch.cuda.device(A.device):
+        rc = lib.mxq_pack_mx(A.data_ptr(), codes.data_ptr(), scales.data_ptr(), _DTYPE[A.dtype],
+                             rows, K, scale_bits, ebits, mbits, max_norm,
+                             int(bool(flush_fp32_subnorms)), int(RoundingMode[round]),
+                             _flags_value(), _stream(A))
+    _lib.check(rc, lib)
+    return codes, scales, fmt == ElemFormat.fp8_e5m2
+
+
+def unpack_mx(codes, scales, codes_are_e5m2, dtype=torch.float32):
+    """codes * 2^(scales - 127) as a tensor of `dtype` (255 in scales -> NaN block)."""
+    who = "unpack_mx"
+    _check_gpu_input(codes, "codes", who)
+    _check_gpu_input(scales, "scales", who)
+    K = codes.shape[-1]
+    out = torch.empty(codes.shape, dtype=dtype, device=codes.device)
+    lib = _lib.gpu()
+    with torch.cuda.device(codes.device):
+        rc = lib.mxq_unpack_mx(codes.data_ptr(), scales.data_ptr(), int(codes_are_e5m2),
+                               out.data_ptr(), _DTYPE[dtype], codes.numel() // K if K else 0, K,
+                               _stream(codes))
+    _lib.check(rc, lib)
+    return out
+
+
+def gemm_nt(a_packed, b_packed, out_dtype=torch.float32):
+    """C[b] = A[b] x B[b]^T.  a_packed / b_packed = (codes, scales, is_e5m2) with codes of shape
+    (batch, M, K) / (batch, N, K) or (M, K) / (N, K)."""
+    who = "gemm_nt"
+    (ac, asc, ae), (bc, bsc, be) = a_packed, b_packed
+    for t, n in ((ac, "a codes"), (asc, "a scales"), (bc, "b codes"), (bsc, "b scales")):
+        _check_gpu_input(t, n, who)
+    if ac.dim() != bc.dim() or ac.dim() not in (2, 3) or ac.shape[-1] != bc.shape[-1] \
+            or ac.shape[:-2] != bc.shape[:-2]:
+        raise RuntimeError("%s: operand shapes %s and %s do not match" % (who, tuple(ac.shape),
+                                                                          tuple(bc.shape)))
+    batch = ac.shape[0] if ac.dim() == 3 else 1
+    M, N, K = ac.shape[-2], bc.shape[-2], ac.shape[-1]
+    out = torch.empty(ac.shape[:-2] + (M, N), dtype=out_dtype, device=ac.device)
+    lib = _lib.gpu()
+    with torch.cuda.device(ac.device):
+        rc = lib.mxq_gemm_mx_nt(ac.data_ptr(), asc.data_ptr(), int(ae), bc.data_ptr(),
+                                bsc.data_ptr(), int(be), out.data_ptr(), _DTYPE[out_dtype], batch, M,
+                                N, K, _stream(ac))
+    _lib.check(rc, lib)
+    return out
+
+
+def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round):
+    """a (..., M, K) x b_kmajor (N, K) or (..., N, K), both MX-quantized along K: the fused
+    equivalent of quantize_mx_op(a, axes=[-1]) @ quantize_mx_op(b, axes=[-1]).T.
+    Returns None when the operands do not qualify (the caller then takes the unfused path)."""
+    fa, fb = _as_format(a_fmt), _as_format(b_fmt)
+    if fa not in _PACKABLE or fb not in _PACKABLE:
+        return None
+    if mx_specs["block_size"] != 32 or mx_specs["shared_exp_method"] != "max":
+        return None
+    if round not in RoundingMode.string_enums():
+        return None
+    if not (a.is_cuda and b_kmajor.is_cuda) or a.dtype not in _DTYPE or b_kmajor.dtype not in _DTYPE:
+        return None
+    if a.dim() < 2 or b_kmajor.dim() < 2 or a.shape[-1] != b_kmajor.shape[-1]:
+        return None
+    K = a.shape[-1]
+    if K == 0 or K % GEMM_K_MULTIPLE != 0 or a.numel() == 0 or b_kmajor.numel() == 0:
+        return None
+    if b_kmajor.dim() == 2:
+        a2 = a.contiguous().reshape(-1, K)              # fold every leading axis into M
+        b2 = b_kmajor.contiguous()
+        out_shape = a.shape[:-1] + (b2.shape[0],)
+    elif b_kmajor.shape[:-2] == a.shape[:-2]:
+        a2 = a.contiguous().reshape(-1, a.shape[-2], K)
+        b2 = b_kmajor.contiguous().reshape(-1, b_kmajor.shape[-2], K)
+        out_shape = a.shape[:-1] + (b_kmajor.shape[-2],)
+        if a2.shape[0] > 65535:
+            return None
+    else:
+        return None                                      # broadcast batch axes
+    scale_bits = mx_specs["scale_bits"] if mx_specs["scale_bits"] != 0 else 8
+    flush = mx_specs["mx_flush_fp32_subnorms"]
+    pa = pack_mx(a2, fa, scale_bits, round, flush)
+    pb = pack_mx(b2, fb, scale_bits, round, flush)
+    return gemm_nt(pa, pb, out_dtype=a.dtype).reshape(out_shape)

@@ -1,0 +1,135 @@
+"""MX linear layer: same interface as the reference's mx/linear.py."""
+import torch
+import torch.nn.functional as F
+
+from .elemwise_ops import quantize_elemwise_op
+from .gemm import mx_linear_contract, mx_matmul_contract
+from .mx_ops import quantize_mx_op
+from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
+
+f_linear = F.linear
+
+
+class LinearFunction(torch.autograd.Function):
+    """Forward (mx/linear.py:20-101): bfloat-quantize input / weight / bias, MX-quantize both
+    operands along the input-feature axis, multiply, bfloat-quantize, add the bias, bfloat-quantize.
+    Backward (mx/linear.py:103-200): the two gradient products with their operands MX-quantized
+    along the axis being contracted."""
+
+    @staticmethod
+    def forward(ctx, input, weight, bias=None, mx_specs=None, prequantized_weights=False,
+                name=None):
+        bf_in = quantize_elemwise_op(input, mx_specs=mx_specs, round=mx_specs["round_output"])
+        if prequantized_weights:
+            assert weight.dtype == torch.bfloat16
+            assert bias is None or bias.dtype == torch.bfloat16
+            bf_weight, bf_bias = weight, bias
+        else:
+            bf_weight = quantize_elemwise_op(weight, mx_specs=mx_specs,
+                                             round=mx_specs["round_weight"])
+            bf_bias = None if bias is None else quantize_elemwise_op(
+                bias, mx_specs=mx_specs, round=mx_specs["round_weight"])
+        ctx.has_bias = bias is not None
+        if mx_specs["quantize_backprop"]:
+            ctx.save_for_backward(bf_in, bf_weight)
+        else:
+            ctx.save_for_backward(input, weight)
+
+        output = mx_linear_contract(bf_in, bf_weight, mx_specs["a_elem_format"],
+                                    mx_specs["w_elem_format"], mx_specs,
+                                    mx_specs["round_mx_output"])
+        output = quantize_elemwise_op(output, mx_specs=mx_specs, round=mx_specs["round_output"])
+        if bias is not None:
+            output = quantize_elemwise_op(output + bf_bias, mx_specs=mx_specs,
+                                          round=mx_specs["round_output"])
+        ctx.mx_specs = get_backwards_mx_specs(mx_specs)
+        ctx.prequantized_weights = prequantized_weights
+        ctx.name = name
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert ctx.prequantized_weights == False, "Cannot use prequantized weights when training!"
+        input, weight = ctx.saved_tensors
+        specs = ctx.mx_specs
+        out_dim, in_dim = weight.shape
+        grad_output = quantize_elemwise_op(grad_output, mx_specs=specs,
+                                           round=specs["round_grad_input"])
+
+        # grad_weight = grad_output^T x input, contracted over the example axis
+        q_in = quantize_mx_op(input, specs, elem_format=specs["a_elem_format_bp"], axes=[-2],
+                              round=specs["round_mx_input_grad_weight"])
+        q_go = quantize_mx_op(grad_output, specs, elem_format=specs["a_elem_format_bp_ex"],
+                              axes=[-2], round=specs["round_mx_grad_output_grad_weight"])
+        grad_weight = torch.matmul(q_go.reshape(-1, out_dim).transpose(0, 1),
+                                   q_in.reshape(-1, in_dim))
+        grad_weight = quantize_elemwise_op(grad_weight, mx_specs=specs,
+                                           round=specs["round_grad_weight"])
+
+        # grad_input = grad_output x weight, contracted over the output-feature axis
+        q_w = quantize_mx_op(weight, specs, elem_format=specs["w_elem_format_bp"], axes=[0],
+                             round=specs["round_mx_weight_grad_input"])
+        q_go = quantize_mx_op(grad_output, specs, elem_format=specs["a_elem_format_bp_os"],
+                              axes=[-1], round=specs["round_mx_grad_output_grad_input"])
+        grad_input = quantize_elemwise_op(torch.matmul(q_go, q_w), mx_specs=specs,
+                                          round=specs["round_grad_input"])
+
+        grad_bias = None
+        if ctx.has_bias:
+            grad_bias = quantize_elemwise_op(grad_output.reshape(-1, out_dim).sum(0),
+                                             mx_specs=specs, round=specs["round_grad_weight"])
+        return (grad_input, grad_weight, grad_bias, None, None, None)
+
+
+def linear(input, weight, bias=None, mx_specs=None, prequantized_weights=False, name=None):
+    mx_assert_test(mx_specs)
+    if mx_specs is None:
+        return f_linear(input, weight, bias=bias)
+    mx_specs = apply_mx_specs(mx_specs)
+    return LinearFunction.apply(input, weight, bias, mx_specs, prequantized_weights, name)
+
+
+class Linear(torch.nn.Linear):
+    def __init__(self, in_features, out_features, bias=True, mx_specs=None, name=None):
+        mx_assert_test(mx_specs)
+        self.mx_none = mx_specs is None
+        self.name = name
+        self.prequantized_weights = False
+        self.mx_specs = apply_mx_specs(mx_specs)
+        super().__init__(in_features, out_features, bias)
+
+    def apply_mx_specs(self, mx_specs):
+        mx_assert_test(mx_specs)
+        self.mx_none = mx_specs is None
+        self.mx_specs = apply_mx_specs(mx_specs)
+
+    def append_name(self, postfix):
+        self.name += postfix
+
+    def prequantize_weights(self):
+        """Store weight and bias as bfloat16 once, for inference (mx/linear.py:246-274)."""
+        if self.mx_none:
+            return
+        assert self.mx_specs["round"] == 'even', \
+            "Bfloat round should be 'even' for prequantizing weights."
+        assert torch.cuda.is_bf16_supported(), "Current device does not support bfloat16"
+        assert self.mx_specs['bfloat_subnorms'] == True, \
+            "Bfloat_subnorms should be set to True for prequantizing weights."
+        assert self.mx_specs["bfloat"] == 16, "Only Bfloat16 is supported for prequantizing weights."
+        with torch.no_grad():
+            self.weight.data = quantize_elemwise_op(
+                self.weight.data, mx_specs=self.mx_specs,
+                round=self.mx_specs["round_weight"]).to(torch.bfloat16)
+            if self.bias is not None:
+                self.bias.data = quantize_elemwise_op(
+                    self.bias.data, mx_specs=self.mx_specs,
+                    round=self.mx_specs["round_weight"]).to(torch.bfloat16)
+        self.prequantized_weights = True
+
+    def forward(self, inputs):
+        if self.mx_none:
+            return super().forward(inputs)
+        if self.prequantized_weights:
+            assert self.training == False, "Cannot use prequantized weights when training!"
+        return linear(input=inputs, weight=self.weight, bias=self.bias, mx_specs=self.mx_specs,
+                      prequantized_weights=self.prequantized_weights, name=self.name)

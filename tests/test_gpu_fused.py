@@ -1,0 +1,150 @@
+"""GPU tests of the packed MX form and the scaled-MFMA GEMM, and of the layers built on them."""
+import pytest
+import torch
+
+from helpers import assert_bits_equal
+from oracle import mx_oracle as O
+
+pytestmark = pytest.mark.gpu
+PACKABLE = ["fp8_e4m3", "fp8_e5m2", "fp6_e3m2", "fp6_e2m3", "fp4_e2m1"]
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available()
+    return torch.device("cuda:0")
+
+
+def rel_err(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return ((got - want).abs().max() / want.pow(2).mean().sqrt()).item()
+
+
+@pytest.mark.parametrize("fmt", PACKABLE)
+@pytest.mark.parametrize("rnd", ["nearest", "floor", "even"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pack_then_unpack_is_the_fake_quantized_tensor(dev, fmt, rnd, dtype):
+    """codes x 2^(scale-127) must be bit-identical to the oracle's _quantize_mx output, including
+    subnormal blocks, -0.0 and NaN blocks."""
+    from microxcaling_amd.fused import pack_mx, unpack_mx
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(96, 256, generator=g) * torch.exp(3 * torch.randn(96, 256, generator=g))
+    x[3, 40] = float("inf")
+    x[5, 70] = float("nan")
+    x[7, :64] *= 1e-38
+    x[9, :32] = 0.0
+    x[11, :32] = -1e-30 * torch.rand(32, generator=g)
+    x = x.to(dtype)
+    want = O.quantize_mx(x, 8, fmt, axes=[-1], block_size=32, round=rnd)
+    codes, scales, e5m2 = pack_mx(x.to(dev), fmt, 8, rnd)
+    assert codes.shape == x.shape and scales.shape == (96, 8) and e5m2 == (fmt == "fp8_e5m2")
+    got = unpack_mx(codes, scales, e5m2, dtype)
+    torch.cuda.synchronize()
+    assert_bits_equal(got, want, fmt)
+
+
+@pytest.mark.parametrize("M,N,K,batch", [(128, 128, 128, 1), (256, 384, 512, 1), (100, 72, 256, 1),
+                                         (130, 257, 128, 3), (16, 16, 128, 2), (1, 5, 384, 1)])
+@pytest.mark.parametrize("fa,fb", [("fp8_e4m3", "fp8_e4m3"), ("fp8_e5m2", "fp8_e4m3"),
+                                   ("fp6_e2m3", "fp8_e5m2"), ("fp4_e2m1", "fp6_e3m2")])
+def test_scaled_mfma_gemm_against_fp64(dev, M, N, K, batch, fa, fb):
+    """Per-block scale spread of 2^-3 .. 2^3 so that a wrong lane-to-scale mapping cannot hide.
+    Tolerance 1e-3 (max |diff| / RMS): one scaled MFMA keeps about 14 bits relative to the sum of
+    the magnitudes of the 128 products it adds, measured 7e-5 at worst."""
+    from microxcaling_amd.fused import pack_mx, unpack_mx, gemm_nt
+    g = torch.Generator().manual_seed(M * 7 + N * 3 + K + batch)
+    shape_a = (batch, M, K) if batch > 1 else (M, K)
+    shape_b = (batch, N, K) if batch > 1 else (N, K)
+    blk = lambda s: torch.exp2(torch.randint(-3, 4, s[:-1] + (s[-1] // 32, 1), generator=g).float())
+    a = (torch.randn(*shape_a, generator=g).view(*shape_a[:-1], K // 32, 32) * blk(shape_a)).view(shape_a)
+    b = (torch.randn(*shape_b, generator=g).view(*shape_b[:-1], K // 32, 32) * blk(shape_b)).view(shape_b)
+    pa = pack_mx(a.to(dev), fa)
+    pb = pack_mx(b.to(dev), fb)
+    got = gemm_nt(pa, pb, torch.float32)
+    qa = unpack_mx(*pa, torch.float32).double()
+    qb = unpack_mx(*pb, torch.float32).double()
+    want = qa @ qb.transpose(-1, -2)
+    torch.cuda.synchronize()
+    assert got.shape == want.shape
+    assert rel_err(got, want) < 1e-3
+    den = qa.abs() @ qb.abs().transpose(-1, -2)
+    assert ((got.double() - want).abs() <= 2e-4 * den + 1e-30).all()
+
+
+def test_gemm_propagates_nan_blocks(dev):
+    from microxcaling_amd.fused import pack_mx, gemm_nt
+    a = torch.randn(128, 128)
+    a[5, 40] = float("inf")
+    b = torch.randn(128, 128)
+    out = gemm_nt(pack_mx(a.to(dev), "fp8_e4m3"), pack_mx(b.to(dev), "fp8_e4m3")).cpu()
+    assert torch.isnan(out[5]).all() and torch.isfinite(out[torch.arange(128) != 5]).all()
+
+
+def _specs(**kw):
+    from microxcaling_amd.specs import finalize_mx_specs
+    return finalize_mx_specs(dict(kw))
+
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_forward_matches_reference_forward(dev, fused, dtype):
+    """mx.Linear forward (BASELINE config 4 at a reduced size): quantize-then-fp32-matmul oracle,
+    relative tolerance 1e-3 (max |diff| / RMS of the output)."""
+    from microxcaling_amd import gemm
+    from microxcaling_amd.linear import linear
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(512, 1024, generator=g).to(dtype)
+    w = (torch.randn(384, 1024, generator=g) * 0.02).to(dtype)
+    b = torch.randn(384, generator=g).to(dtype)
+    specs = _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32)
+    want = O.mx_linear_forward(x, w, b, "fp8_e4m3", "fp8_e4m3")      # same dtype as the GPU run
+    gemm.set_fused(fused)
+    try:
+        got = linear(x.to(dev), w.to(dev), b.to(dev), mx_specs=specs)
+    finally:
+        gemm.set_fused(True)
+    torch.cuda.synchronize()
+    assert got.dtype == dtype
+    if dtype == torch.float32:
+        assert rel_err(got, want) < 1e-3
+    else:
+        # bf16 tensors round the product and then the bias sum to bf16: allow one bf16 ulp of the
+        # larger of the two (|product| <= |result| + |bias|) on top of the accumulation tolerance
+        diff = (got.float().cpu() - want.float()).abs()
+        rms = want.float().pow(2).mean().sqrt()
+        mag = want.float().abs() + b.float().abs().view(1, -1)
+        assert (diff <= 2 ** -6 * mag + 2e-3 * rms).all()
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_bmm_and_softmax_forward(dev, fused):
+    """mx.bmm Q.K^T with MXFP6 e2m3 along head_dim, then the bfloat16 softmax chain (config 5 at a
+    reduced size).  Logits: relative 1e-3; softmax: absolute 2^-8 (one bf16 ulp at 1.0)."""
+    from microxcaling_amd import gemm
+    from microxcaling_amd.bmm import bmm
+    from microxcaling_amd.softmax import softmax
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(4, 256, 128, generator=g)
+    k = torch.randn(4, 256, 128, generator=g)
+    specs = _specs(a_elem_format="fp6_e2m3", block_size=32, bfloat=16)
+    want = O.mx_bmm_forward(q, k.transpose(-1, -2), "fp6_e2m3", bfloat=16)
+    gemm.set_fused(fused)
+    try:
+        got = bmm(q.to(dev), k.to(dev).transpose(-1, -2), mx_specs=specs)
+    finally:
+        gemm.set_fused(True)
+    torch.cuda.synchronize()
+    assert rel_err(got, want) < 1e-2                      # logits are re-rounded to bfloat16
+    sm = softmax(got, dim=-1, mx_specs=specs).cpu()
+    sm_want = O.softmax_forward(want, -1, bfloat=16)
+    assert (sm - sm_want).abs().max() <= 2 ** -8 * 4
+
+
+def test_linear_backward_runs(dev):
+    from microxcaling_amd.linear import Linear
+    specs = _specs(w_elem_format="fp6_e3m2", a_elem_format="fp6_e3m2", block_size=32, bfloat=16)
+    lin = Linear(256, 128, mx_specs=specs).to(dev)
+    x = torch.randn(64, 256, device=dev, requires_grad=True)
+    lin(x).sum().backward()
+    assert x.grad.shape == x.shape and lin.weight.grad.shape == lin.weight.shape
+    assert torch.isfinite(x.grad).all()
