@@ -97,6 +97,59 @@ def make_workload(name):
         return dict(x=x, gpu=fn, cpu=cpu, bytes=x.numel() * 4, dtype="f32", sample_axis=0 if dim == -1 else 1,
                     launches=1 if dim == -1 else 2,
                     desc="reduce %s over axis %d, fp32 [16384,8192]" % (op, dim))
+    if name in ("mx_linear", "mx_linear_unfused"):
+        # config 4: mx.Linear forward, MXFP8 e4m3 both operands, block 32 along K, bias
+        from microxcaling_amd import gemm
+        from microxcaling_amd.linear import linear
+        from microxcaling_amd.specs import finalize_mx_specs
+        g = torch.Generator().manual_seed(4)
+        M, N, K = 16384, 14336, 4096
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+        b = torch.randn(N, generator=g).to(torch.bfloat16)
+        specs = finalize_mx_specs({"w_elem_format": "fp8_e4m3", "a_elem_format": "fp8_e4m3", "block_size": 32})
+        dev_extra = {}
+        fused = name == "mx_linear"
+
+        def run(xd):
+            if "w" not in dev_extra:
+                dev_extra["w"], dev_extra["b"] = w.to(xd.device), b.to(xd.device)
+            gemm.set_fused(fused)
+            return linear(xd, dev_extra["w"], dev_extra["b"], mx_specs=specs)
+        return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, "fp8_e4m3", "fp8_e4m3"),
+                    flops=2.0 * M * N * K, bytes=0, dtype="fp8_e4m3 x fp8_e4m3 -> f32 acc", sample_axis=0,
+                    cpu_rows=1024, launches=5,
+                    desc="mx.Linear forward: x bf16 [16384,4096], W bf16 [14336,4096] ~N(0,0.02), bias; MXFP8 e4m3 "
+                         "block 32 along K, %s" % ("packed codes + scaled-MFMA GEMM" if fused else
+                                                   "fake-quantize kernels + torch (hipBLASLt) bf16 GEMM"))
+    if name in ("mx_bmm_softmax", "mx_bmm_softmax_unfused"):
+        # config 5: mx.bmm Q.K^T, MXFP6 e2m3 along head_dim, then the bfloat16 softmax chain
+        from microxcaling_amd import gemm
+        from microxcaling_amd.bmm import bmm
+        from microxcaling_amd.softmax import softmax
+        from microxcaling_amd.specs import finalize_mx_specs
+        g = torch.Generator().manual_seed(5)
+        B, S, D = 128, 2048, 128
+        q = torch.randn(B, S, D, generator=g).to(torch.bfloat16)
+        k = torch.randn(B, S, D, generator=g).to(torch.bfloat16)
+        specs = finalize_mx_specs({"a_elem_format": "fp6_e2m3", "block_size": 32, "bfloat": 16})
+        dev_extra = {}
+        fused = name == "mx_bmm_softmax"
+
+        def run(qd):
+            if "k" not in dev_extra:
+                dev_extra["k"] = k.to(qd.device)
+            gemm.set_fused(fused)
+            logits = bmm(qd, dev_extra["k"].transpose(-1, -2), mx_specs=specs)
+            return softmax(logits, dim=-1, mx_specs=specs)
+
+        def cpu(t):
+            n = t.shape[0]
+            return O.softmax_forward(O.mx_bmm_forward(t, k[:n].transpose(-1, -2), "fp6_e2m3", bfloat=16), -1)
+        return dict(x=q, gpu=run, cpu=cpu, flops=2.0 * B * S * S * D, bytes=0,
+                    dtype="fp6_e2m3 x fp6_e2m3 -> f32 acc", sample_axis=0, cpu_rows=8, launches=20,
+                    desc="mx.bmm Q.K^T bf16 [128,2048,128] MXFP6 e2m3 along head_dim + bfloat16 softmax, %s"
+                         % ("packed codes + scaled-MFMA GEMM" if fused else "fake-quantize + torch.bmm"))
     if name == "copy_fp32_8192":
         # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         x = torch.randn(8192, 8192, generator=torch.Generator().manual_seed(0))
@@ -133,6 +186,41 @@ def cpu_baseline(wl, budget_s=15.0):
                       "op-by-op oracle (oracle/mx_oracle.py), %d threads"
                       % ("x".join(str(n) for n in x.shape), len(times), time.perf_counter() - t_all, t,
                          torch.__version__, cores)}
+
+
+MFMA_PEAK_TFLOPS = {"fp8": 5000.0}          # MI355X dense fp8 (e4m3 / e5m2 codes), published
+
+
+def report_flops(args, wl, ms_per_step, step_gpu_ms):
+    """GEMM-shaped workloads: whole-step TFLOP/s (quantize + GEMM + epilogue ops all inside the
+    step) against the dense fp8 MFMA peak."""
+    value = wl["flops"] / (ms_per_step * 1e-3) / 1e12
+    achieved = wl["flops"] / (step_gpu_ms * 1e-3) / 1e12
+    out = {
+        "metric": "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"], "data": "synthetic",
+        "config": {"workload": args.workload, "detail": wl["desc"], "flop_per_step": wl["flops"]},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_PEAK_TFLOPS["fp8"],
+                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS["fp8"], 4),
+                     "traffic": None, "step_gpu_ms_avg": round(step_gpu_ms, 5),
+                     "note": "whole forward step (all launches) over the dense fp8 MFMA peak"},
+    }
+    if not args.no_cpu_baseline:
+        x = wl["x"]
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        rows = wl["cpu_rows"]
+        xs = x[:rows].contiguous()
+        t0 = time.perf_counter()
+        wl["cpu"](xs)
+        t = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(wl["flops"] * rows / x.shape[0] / t / 1e12, 5), "unit": "TFLOP/s",
+                               "cores": cores, "kind": "port",
+                               "sample": "first %d of %d rows/batches of the first operand, one pass, %.1f s; "
+                                         "torch op-by-op oracle" % (rows, x.shape[0], t)}
+    print(json.dumps(out, ensure_ascii=False), flush=True)
 
 
 def main():
@@ -176,6 +264,8 @@ def main():
 
     ms_per_step = wall * 1e3 / args.steps
     kern_avg_ms = ev0.elapsed_time(ev1) / args.steps
+    if "flops" in wl:
+        return report_flops(args, wl, ms_per_step, kern_avg_ms)
     value = wl["bytes"] / (ms_per_step * 1e-3) / 1e9
     achieved = wl["bytes"] / (kern_avg_ms * 1e-3) / 1e9
 

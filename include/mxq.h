@@ -111,6 +111,11 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, con
                    const void* b_scales, int b_is_e5m2, void* c, int c_dtype, int64_t batch,
                    int64_t M, int64_t N, int64_t K, void* hip_stream);
 
+/* Measurement aid (no counterpart in the reference): launches `workgroups` x 256 lanes, each wave
+ * issuing iters x 16 scaled 16x16x128 fp8 MFMAs on register-resident operands
+ * (workgroups * 4 * iters * 16 * 65536 flop in total).  `sink` is any 4 writable device bytes. */
+int mxq_probe_mfma_rate(int64_t workgroups, int iters, void* sink, void* hip_stream);
+
 /* ---- libmxq_host.so: the same arithmetic compiled for the host ----------------------------------
  * quantize_mx_func_cpp (mx/cpp/funcs.cpp:23-98) and quantize_elemwise_func_cpp
  * (mx/cpp/funcs.cpp:117-149) take CPU tensors; these are their stand-ins.  Pointers are host

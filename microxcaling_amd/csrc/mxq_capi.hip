@@ -140,11 +140,39 @@ struct LaunchPack {
     }
 };
 
+#ifndef MXQ_G2_WM
+#define MXQ_G2_WM 4
+#endif
+constexpr int G2_WM = MXQ_G2_WM;       // waves along M in the 256 x 256 kernel (4 -> 512 lanes)
+
+template <int CB, int BL, int ODT>
+int launch_gemm_dt(int64_t batch, const GemmArgs& g, hipStream_t s) {
+    // large problems: 256 x 256 tiles (148 KB of dynamic LDS); otherwise 128 x 128 tiles
+    if (g.M >= 512 && g.N >= 512) {
+        static bool configured = false;               // raising the dynamic-LDS limit is per kernel
+        if (!configured) {
+            hipError_t e = hipFuncSetAttribute(
+                reinterpret_cast<const void*>(&mx_gemm_nt_kernel_256<CB, BL, ODT, G2_WM>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, G2_LDS_BYTES);
+            if (e != hipSuccess)
+                return fail(MXQ_ERR_LAUNCH, "mxq_gemm_mx_nt: cannot reserve %d bytes of LDS: %s",
+                            G2_LDS_BYTES, hipGetErrorString(e));
+            configured = true;
+        }
+        dim3 grid((unsigned)(ceil_div(g.N, G2_BN) * ceil_div(g.M, G2_BM)), (unsigned)batch);
+        mx_gemm_nt_kernel_256<CB, BL, ODT, G2_WM><<<grid, G2_WM * 128, G2_LDS_BYTES, s>>>(g);
+    } else {
+        dim3 grid((unsigned)(ceil_div(g.N, GEMM_BN) * ceil_div(g.M, GEMM_BM)), (unsigned)batch);
+        mx_gemm_nt_kernel<CB, BL, ODT><<<grid, kThreads, 0, s>>>(g);
+    }
+    return MXQ_OK;
+}
+
 template <int CB, int BL>
-void launch_gemm(int c_dtype, dim3 grid, const GemmArgs& g, hipStream_t s) {
-    if (c_dtype == MXQ_DTYPE_F32) mx_gemm_nt_kernel<CB, BL, MXQ_F32><<<grid, kThreads, 0, s>>>(g);
-    else if (c_dtype == MXQ_DTYPE_BF16) mx_gemm_nt_kernel<CB, BL, MXQ_BF16><<<grid, kThreads, 0, s>>>(g);
-    else mx_gemm_nt_kernel<CB, BL, MXQ_F16><<<grid, kThreads, 0, s>>>(g);
+int launch_gemm(int c_dtype, int64_t batch, const GemmArgs& g, hipStream_t s) {
+    if (c_dtype == MXQ_DTYPE_F32) return launch_gemm_dt<CB, BL, MXQ_F32>(batch, g, s);
+    if (c_dtype == MXQ_DTYPE_BF16) return launch_gemm_dt<CB, BL, MXQ_BF16>(batch, g, s);
+    return launch_gemm_dt<CB, BL, MXQ_F16>(batch, g, s);
 }
 
 // splits of the outer axis for the two-pass outer reduction
@@ -346,12 +374,22 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, con
     g.batch_a = M * K; g.batch_sa = M * (K / 32);
     g.batch_b = N * K; g.batch_sb = N * (K / 32);
     g.batch_c = M * N;
-    dim3 grid((unsigned)ceil_div(N, GEMM_BN), (unsigned)ceil_div(M, GEMM_BM), (unsigned)batch);
     hipStream_t s = (hipStream_t)hip_stream;
-    if (!a_is_e5m2 && !b_is_e5m2) launch_gemm<0, 0>(c_dtype, grid, g, s);
-    else if (a_is_e5m2 && !b_is_e5m2) launch_gemm<1, 0>(c_dtype, grid, g, s);
-    else if (!a_is_e5m2 && b_is_e5m2) launch_gemm<0, 1>(c_dtype, grid, g, s);
-    else launch_gemm<1, 1>(c_dtype, grid, g, s);
+    int rc;
+    if (!a_is_e5m2 && !b_is_e5m2) rc = launch_gemm<0, 0>(c_dtype, batch, g, s);
+    else if (a_is_e5m2 && !b_is_e5m2) rc = launch_gemm<1, 0>(c_dtype, batch, g, s);
+    else if (!a_is_e5m2 && b_is_e5m2) rc = launch_gemm<0, 1>(c_dtype, batch, g, s);
+    else rc = launch_gemm<1, 1>(c_dtype, batch, g, s);
+    if (rc) return rc;
+    return check_launch(who);
+}
+
+int mxq_probe_mfma_rate(int64_t workgroups, int iters, void* sink, void* hip_stream) {
+    const char* who = "mxq_probe_mfma_rate";
+    if (workgroups <= 0 || workgroups > 0x7FFFFFFF || iters <= 0 || !sink)
+        return fail(MXQ_ERR_ARGUMENT, "%s: bad argument", who);
+    mfma_rate_probe_kernel<<<(unsigned)workgroups, kThreads, 0, (hipStream_t)hip_stream>>>(
+        iters, reinterpret_cast<float*>(sink));
     return check_launch(who);
 }
 

@@ -44,7 +44,8 @@ def test_pack_then_unpack_is_the_fake_quantized_tensor(dev, fmt, rnd, dtype):
 
 
 @pytest.mark.parametrize("M,N,K,batch", [(128, 128, 128, 1), (256, 384, 512, 1), (100, 72, 256, 1),
-                                         (130, 257, 128, 3), (16, 16, 128, 2), (1, 5, 384, 1)])
+                                         (130, 257, 128, 3), (16, 16, 128, 2), (1, 5, 384, 1),
+                                         (512, 768, 256, 1), (600, 520, 128, 2)])
 @pytest.mark.parametrize("fa,fb", [("fp8_e4m3", "fp8_e4m3"), ("fp8_e5m2", "fp8_e4m3"),
                                    ("fp6_e2m3", "fp8_e5m2"), ("fp4_e2m1", "fp6_e3m2")])
 def test_scaled_mfma_gemm_against_fp64(dev, M, N, K, batch, fa, fb):
