@@ -106,10 +106,12 @@ int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t ro
 int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, void* out, int dtype,
                   int64_t rows, int64_t K, void* hip_stream);
 /* C[b] (M, N) = A[b] (M, K) x B[b] (N, K)^T for b < batch, all tensors contiguous, fp32
- * accumulation on the scaled MFMA units; c_dtype is a MXQ_DTYPE_* code.  K % 128 == 0. */
+ * accumulation on the scaled MFMA units; c_dtype is a MXQ_DTYPE_* code.  K % 128 == 0.
+ * bias (optional, may be NULL): N values of dtype c_dtype; then C = round(round(A x B^T) + bias),
+ * both roundings to c_dtype, which is what "matmul, then add the bias" gives as tensor ops. */
 int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, const void* b_codes,
-                   const void* b_scales, int b_is_e5m2, void* c, int c_dtype, int64_t batch,
-                   int64_t M, int64_t N, int64_t K, void* hip_stream);
+                   const void* b_scales, int b_is_e5m2, const void* bias, void* c, int c_dtype,
+                   int64_t batch, int64_t M, int64_t N, int64_t K, void* hip_stream);
 
 /* Measurement aid (no counterpart in the reference): launches `workgroups` x 256 lanes, each wave
  * issuing iters x 16 scaled 16x16x128 fp8 MFMAs on register-resident operands

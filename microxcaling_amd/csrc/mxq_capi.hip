@@ -350,8 +350,8 @@ int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, voi
 }
 
 int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, const void* b_codes,
-                   const void* b_scales, int b_is_e5m2, void* c, int c_dtype, int64_t batch,
-                   int64_t M, int64_t N, int64_t K, void* hip_stream) {
+                   const void* b_scales, int b_is_e5m2, const void* bias, void* c, int c_dtype,
+                   int64_t batch, int64_t M, int64_t N, int64_t K, void* hip_stream) {
     const char* who = "mxq_gemm_mx_nt";
     if (c_dtype < 0 || c_dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, c_dtype);
     if (batch < 0 || M < 0 || N < 0 || K < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
@@ -370,6 +370,7 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, con
     g.b = reinterpret_cast<const unsigned char*>(b_codes);
     g.sb = reinterpret_cast<const unsigned char*>(b_scales);
     g.c = c;
+    g.bias = bias;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.batch_a = M * K; g.batch_sa = M * (K / 32);
     g.batch_b = N * K; g.batch_sb = N * (K / 32);

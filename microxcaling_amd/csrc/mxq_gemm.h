@@ -104,6 +104,7 @@ struct GemmArgs {
     const unsigned char* b;
     const unsigned char* sb;
     void* c;
+    const void* bias;     // optional (N), dtype of C: C = round(round(A x B^T) + bias)
     int M, N, K;
     int64_t batch_a, batch_sa, batch_b, batch_sb, batch_c;   // element strides between batches
 };
@@ -138,8 +139,19 @@ __device__ __forceinline__ v8i load_frag(const unsigned char* p) {
 // of C^T: a lane then holds four *consecutive columns* n = 4 * (lane / 16) + r of one row
 // m = lane % 16, which it can store with a single 8- or 16-byte access.
 template <int OUT_DT>
-__device__ __forceinline__ void store_c4(void* c, int64_t base, int m, int n, int M, int N,
-                                         bool tile_inside, const v4f& v) {
+__device__ __forceinline__ void store_c4(void* c, const void* bias, int64_t base, int m, int n,
+                                         int M, int N, bool tile_inside, v4f v) {
+    constexpr int ADT = Arith<OUT_DT>::DT_;
+    if (bias != nullptr) {
+        // what the layers do as separate tensor ops: the product is rounded to the tensor dtype,
+        // the bias is added, and the sum is rounded again (by the store below)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float b = (n + r < N) ? load_scalar<OUT_DT>(bias, n + r) : 0.0f;
+            const float p = (OUT_DT == MXQ_F16) ? (float)(_Float16)v[r] : mxq_round_dt<ADT>(v[r]);
+            v[r] = p + b;
+        }
+    }
     if (tile_inside) {                                       // uniform per workgroup
         const int64_t idx = base + (int64_t)m * N + n;
         if (OUT_DT == MXQ_F32) {
@@ -155,8 +167,7 @@ __device__ __forceinline__ void store_c4(void* c, int64_t base, int m, int n, in
 #pragma unroll
         for (int r = 0; r < 4; ++r)
             if (n + r < N)
-                store_scalar<OUT_DT>(c, base + (int64_t)m * N + n + r,
-                                     mxq_round_dt<Arith<OUT_DT>::DT_>(v[r]));
+                store_scalar<OUT_DT>(c, base + (int64_t)m * N + n + r, mxq_round_dt<ADT>(v[r]));
     }
 }
 
@@ -266,7 +277,7 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     for (int ti = 0; ti < 4; ++ti)
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj)
-            store_c4<OUT_DT>(g.c, cbase, m0 + wy * 64 + ti * 16 + frow, n0 + wx * 64 + tj * 16 + fg * 4,
+            store_c4<OUT_DT>(g.c, g.bias, cbase, m0 + wy * 64 + ti * 16 + frow, n0 + wx * 64 + tj * 16 + fg * 4,
                              g.M, g.N, inside, acc[ti][tj]);
 }
 
@@ -429,7 +440,7 @@ __global__ __launch_bounds__(WM * 128, 1) void mx_gemm_nt_kernel_256(GemmArgs g)
     for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
         for (int tj = 0; tj < 8; ++tj)
-            store_c4<OUT_DT>(g.c, cbase, m0 + wy * (TI * 16) + ti * 16 + frow,
+            store_c4<OUT_DT>(g.c, g.bias, cbase, m0 + wy * (TI * 16) + ti * 16 + frow,
                              n0 + wx * 128 + tj * 16 + fg * 4, g.M, g.N, inside, acc[ti][tj]);
 }
 

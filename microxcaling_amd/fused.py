@@ -65,9 +65,10 @@ def unpack_mx(codes, scales, codes_are_e5m2, dtype=torch.float32):
     return out
 
 
-def gemm_nt(a_packed, b_packed, out_dtype=torch.float32):
-    """C[b] = A[b] x B[b]^T.  a_packed / b_packed = (codes, scales, is_e5m2) with codes of shape
-    (batch, M, K) / (batch, N, K) or (M, K) / (N, K)."""
+def gemm_nt(a_packed, b_packed, out_dtype=torch.float32, bias=None):
+    """C[b] = A[b] x B[b]^T (+ bias).  a_packed / b_packed = (codes, scales, is_e5m2) with codes of
+    shape (batch, M, K) / (batch, N, K) or (M, K) / (N, K); bias: (N,) of out_dtype, added after the
+    product has been rounded to out_dtype, the sum being rounded again."""
     who = "gemm_nt"
     (ac, asc, ae), (bc, bsc, be) = a_packed, b_packed
     for t, n in ((ac, "a codes"), (asc, "a scales"), (bc, "b codes"), (bsc, "b scales")):
@@ -78,20 +79,25 @@ def gemm_nt(a_packed, b_packed, out_dtype=torch.float32):
                                                                           tuple(bc.shape)))
     batch = ac.shape[0] if ac.dim() == 3 else 1
     M, N, K = ac.shape[-2], bc.shape[-2], ac.shape[-1]
+    if bias is not None:
+        _check_gpu_input(bias, "bias", who)
+        if bias.dtype != out_dtype or bias.numel() != N:
+            raise RuntimeError("%s: bias must hold N values of the output dtype" % who)
     out = torch.empty(ac.shape[:-2] + (M, N), dtype=out_dtype, device=ac.device)
     lib = _lib.gpu()
     with torch.cuda.device(ac.device):
         rc = lib.mxq_gemm_mx_nt(ac.data_ptr(), asc.data_ptr(), int(ae), bc.data_ptr(),
-                                bsc.data_ptr(), int(be), out.data_ptr(), _DTYPE[out_dtype], batch, M,
-                                N, K, _stream(ac))
+                                bsc.data_ptr(), int(be), None if bias is None else bias.data_ptr(),
+                                out.data_ptr(), _DTYPE[out_dtype], batch, M, N, K, _stream(ac))
     _lib.check(rc, lib)
     return out
 
 
-def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round):
+def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None):
     """a (..., M, K) x b_kmajor (N, K) or (..., N, K), both MX-quantized along K: the fused
-    equivalent of quantize_mx_op(a, axes=[-1]) @ quantize_mx_op(b, axes=[-1]).T.
-    Returns None when the operands do not qualify (the caller then takes the unfused path)."""
+    equivalent of quantize_mx_op(a, axes=[-1]) @ quantize_mx_op(b, axes=[-1]).T (+ bias, see
+    gemm_nt).  Returns None when the operands do not qualify (the caller then takes the unfused
+    path)."""
     fa, fb = _as_format(a_fmt), _as_format(b_fmt)
     if fa not in _PACKABLE or fb not in _PACKABLE:
         return None
@@ -122,4 +128,6 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round):
     flush = mx_specs["mx_flush_fp32_subnorms"]
     pa = pack_mx(a2, fa, scale_bits, round, flush)
     pb = pack_mx(b2, fb, scale_bits, round, flush)
-    return gemm_nt(pa, pb, out_dtype=a.dtype).reshape(out_shape)
+    if bias is not None and (bias.dtype != a.dtype or bias.dim() != 1):
+        return None
+    return gemm_nt(pa, pb, out_dtype=a.dtype, bias=bias).reshape(out_shape)

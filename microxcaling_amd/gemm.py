@@ -25,26 +25,28 @@ def fused_enabled():
     return _use_fused
 
 
-def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round):
+def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None):
     """a: (..., M, K); b_kmajor: (..., N, K) -- both contiguous along K.  Returns None when the
     fused path does not apply."""
     if not _use_fused or not a.is_cuda:
         return None
     from . import fused
-    return fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round)
+    return fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=bias)
 
 
-def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round):
-    """x (..., K) times w (N, K) transposed: both operands share exponents along their last axis."""
-    out = _try_fused(x, w, a_fmt, w_fmt, mx_specs, round)
+def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, fuse_bias=None):
+    """x (..., K) times w (N, K) transposed: both operands share exponents along their last axis.
+    fuse_bias: a bias the caller would add right after the product with no quantization step in
+    between; returns (out, bias_was_added)."""
+    out = _try_fused(x, w, a_fmt, w_fmt, mx_specs, round, bias=fuse_bias)
     if out is not None:
-        return out
+        return out, fuse_bias is not None
     qx = quantize_mx_op(x, mx_specs, elem_format=a_fmt, axes=[-1], round=round)
     qw = quantize_mx_op(w, mx_specs, elem_format=w_fmt, axes=[-1], round=round)
     # prequantized bf16 weights meet inputs of another dtype (mx/linear.py:77-80)
     if qw.dtype == torch.bfloat16 and qx.dtype != torch.bfloat16:
         qw = qw.to(qx.dtype)
-    return torch.nn.functional.linear(qx, qw)
+    return torch.nn.functional.linear(qx, qw), False
 
 
 def mx_matmul_contract(a, b, a_fmt, b_fmt, mx_specs, round, batched=False):
