@@ -140,27 +140,32 @@ struct LaunchPack {
     }
 };
 
-#ifndef MXQ_G2_WM
-#define MXQ_G2_WM 4
-#endif
-constexpr int G2_WM = MXQ_G2_WM;       // waves along M in the 256 x 256 kernel (4 -> 512 lanes)
-
 template <int CB, int BL, int ODT>
 int launch_gemm_dt(int64_t batch, const GemmArgs& g, hipStream_t s) {
-    // large problems: 256 x 256 tiles (148 KB of dynamic LDS); otherwise 128 x 128 tiles
-    if (g.M >= 512 && g.N >= 512) {
+    // large problems: persistent 256 x 256 tile kernel (144 KB of dynamic LDS, one workgroup per CU);
+    // it fetches scales four K steps at a time, hence K % 512
+    const int64_t tiles_m = ceil_div(g.M, G2_BM), tiles_n = ceil_div(g.N, G2_BN);
+    const int64_t total = tiles_m * tiles_n * batch;
+    if (g.M >= 512 && g.N >= 512 && g.K % 512 == 0 && (int64_t)256 * g.K < ((int64_t)1 << 31) &&
+        total < ((int64_t)1 << 30)) {
         static bool configured = false;               // raising the dynamic-LDS limit is per kernel
+        static int cus = 0;
         if (!configured) {
             hipError_t e = hipFuncSetAttribute(
-                reinterpret_cast<const void*>(&mx_gemm_nt_kernel_256<CB, BL, ODT, G2_WM>),
-                hipFuncAttributeMaxDynamicSharedMemorySize, G2_LDS_BYTES);
-            if (e != hipSuccess)
-                return fail(MXQ_ERR_LAUNCH, "mxq_gemm_mx_nt: cannot reserve %d bytes of LDS: %s",
-                            G2_LDS_BYTES, hipGetErrorString(e));
+                reinterpret_cast<const void*>(&mx_gemm_nt_kernel_256p<CB, BL, ODT>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, G3_LDS_BYTES);
+            int dev = 0;
+            if (e == hipSuccess) e = hipGetDevice(&dev);
+            if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            if (e != hipSuccess || cus <= 0)
+                return fail(MXQ_ERR_LAUNCH, "mxq_gemm_mx_nt: cannot configure the tile kernel (%d bytes of LDS): %s",
+                            G3_LDS_BYTES, hipGetErrorString(e));
+            cus -= cus % 8;                           // a workgroup must stay on its XCD from tile to tile
+            if (cus < 8) cus = 8;
             configured = true;
         }
-        dim3 grid((unsigned)(ceil_div(g.N, G2_BN) * ceil_div(g.M, G2_BM)), (unsigned)batch);
-        mx_gemm_nt_kernel_256<CB, BL, ODT, G2_WM><<<grid, G2_WM * 128, G2_LDS_BYTES, s>>>(g);
+        const unsigned grid = (unsigned)(total < cus ? total : cus);
+        mx_gemm_nt_kernel_256p<CB, BL, ODT><<<grid, 512, G3_LDS_BYTES, s>>>(g, (int)tiles_m, (int)tiles_n, (int)total);
     } else {
         dim3 grid((unsigned)(ceil_div(g.N, GEMM_BN) * ceil_div(g.M, GEMM_BM)), (unsigned)batch);
         mx_gemm_nt_kernel<CB, BL, ODT><<<grid, kThreads, 0, s>>>(g);

@@ -171,6 +171,39 @@ __device__ __forceinline__ void store_c4(void* c, const void* bias, int64_t base
     }
 }
 
+// Eight consecutive columns of one row, 16-bit outputs: one 16-byte store (and bias load).
+template <int OUT_DT>
+__device__ __forceinline__ void store_c8(void* c, const void* bias, int64_t base, int m, int n,
+                                         int M, int N, bool tile_inside, v4f lo, v4f hi) {
+    constexpr int ADT = Arith<OUT_DT>::DT_;
+    float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    if (tile_inside) {                                       // uniform per workgroup
+        if (bias != nullptr) {
+            const u32x4 bw = *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned short*>(bias) + n);
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const float b = Pack<OUT_DT>::get(bw[r >> 1], r & 1);
+                const float p = (OUT_DT == MXQ_F16) ? (float)(_Float16)v[r] : mxq_round_dt<ADT>(v[r]);
+                v[r] = p + b;
+            }
+        }
+        *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned short*>(c) + base + (int64_t)m * N + n) =
+            u32x4{Pack<OUT_DT>::put(v[0], v[1]), Pack<OUT_DT>::put(v[2], v[3]),
+                  Pack<OUT_DT>::put(v[4], v[5]), Pack<OUT_DT>::put(v[6], v[7])};
+    } else if (m < M) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+            if (n + r < N) {
+                float x = v[r];
+                if (bias != nullptr) {
+                    const float p = (OUT_DT == MXQ_F16) ? (float)(_Float16)x : mxq_round_dt<ADT>(x);
+                    x = p + load_scalar<OUT_DT>(bias, n + r);
+                }
+                store_scalar<OUT_DT>(c, base + (int64_t)m * N + n + r, mxq_round_dt<ADT>(x));
+            }
+    }
+}
+
 template <int CBSZ, int BLGP, int OUT_DT>
 __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     __shared__ __attribute__((aligned(16))) unsigned char As[GEMM_BM * GEMM_PITCH];
@@ -281,167 +314,217 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
                              g.M, g.N, inside, acc[ti][tj]);
 }
 
-// ================================================================================================
-// Large-tile variant: workgroup tile 256 x 256 x 128, 2 x 2 waves, each wave 128 x 128 = 8 x 8 MFMA
-// tiles (256 accumulator registers).  Per K step a wave reads 8 A and 8 B fragments from LDS for 64
-// MFMAs, half the LDS traffic per flop of the 128 x 128 kernel.  LDS is double buffered
-// (2 x 2 x 256 rows x 144 bytes + scales = 148 KB): the global loads of step k+1 are issued before
-// the MFMAs of step k and land in the other buffer afterwards; one barrier per step.
-// ================================================================================================
 constexpr int G2_BM = 256, G2_BN = 256;
-constexpr int G2_TILE_BYTES = G2_BM * GEMM_PITCH;                   // one operand tile
-constexpr int G2_STAGE_BYTES = 2 * G2_TILE_BYTES + (G2_BM + G2_BN) * 4;
-constexpr int G2_LDS_BYTES = 2 * G2_STAGE_BYTES;
 
-// WM = waves along M (2 or 4); the workgroup has WM x 2 waves and each wave owns (256 / WM) x 128
-// outputs.  WM = 4 (512 lanes) halves the accumulators per wave so that two waves fit on every
-// SIMD: while one waits for LDS, memory or the barrier, the other keeps the MFMA pipe fed.
-template <int CBSZ, int BLGP, int OUT_DT, int WM>
-__global__ __launch_bounds__(WM * 128, 1) void mx_gemm_nt_kernel_256(GemmArgs g) {
-    constexpr int NT = WM * 128;                        // lanes in the workgroup
-    constexpr int TI = 16 / WM;                         // 16-row MFMA tiles per wave along M
-    constexpr int CH = 2048 / NT;                       // 16-byte chunks of A (and of B) per lane
-    constexpr int ROWS_PER_PASS = NT / 8;
+// ================================================================================================
+// Main GEMM kernel: persistent workgroups, tile 256 x 256 x 128, 512 lanes = 4 x 2 waves, wave tile
+// 64 x 128 = 4 x 8 MFMA tiles (128 accumulator registers, two waves per SIMD).
+//
+// Tile copy: global_load_lds_dwordx4 -- the memory pipe writes 16 bytes per lane straight into LDS
+// (lane L of a wave lands at base + 16 L), so there are no staging registers and no ds_write
+// instructions.  LDS holds two stages of codes (A 256 rows + B 256 rows, 128 bytes each, unpadded);
+// the 16-byte column c of row r is kept at position c ^ ((r >> 1) & 7), which makes the 16-byte
+// fragment reads of 16 consecutive rows hit 16 different bank groups, and the lanes pick their
+// global address so that the linear landing order produces exactly this image.  The loads of step
+// t + 1 are issued inside step t, spread over its MFMA groups.
+//
+// Scales: one byte per row and 32 K, i.e. 4 bytes per row and K step, each row in a different
+// cache line.  Fetching them per step would double the number of L2 requests of the kernel, so a
+// lane fetches 16 bytes = four K steps of one row at a time into a two-deep ring of scale groups.
+// This needs K % 512 == 0 and a K walk that starts at a multiple of four steps.
+//
+// A workgroup walks over tiles w, w + G, w + 2 G, ... (G = grid size, a multiple of 8 so that a
+// workgroup stays on its XCD) in one flat sequence of K steps: the last step of a tile already
+// fetches the first step of the next one, and the stores of a finished tile drain while the next
+// tile computes.
+// ================================================================================================
+constexpr int G3_TILE_BYTES = 256 * 128;
+constexpr int G3_STAGE_BYTES = 2 * G3_TILE_BYTES;            // codes of A and B for one K step
+constexpr int G3_SCALE_OFF = 2 * G3_STAGE_BYTES;
+constexpr int G3_SCALE_GROUP = 512 * 16;                     // 512 rows x 4 K steps x 4 bytes
+constexpr int G3_LDS_BYTES = G3_SCALE_OFF + 2 * G3_SCALE_GROUP;
+constexpr int G3_SPREAD = 6;        // the loads of the next step go out during the first 6 MFMA groups
+
+__device__ __forceinline__ void dma16(uint32_t lds_base, uint32_t voff, const unsigned char* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_base), "v"(voff), "s"(sbase) : "memory");
+}
+
+template <int CBSZ, int BLGP, int OUT_DT>
+__global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int tiles_m, int tiles_n,
+                                                                 int total) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wy = wave >> 1, wx = wave & 1;
-    int tile_m, tile_n;
-    tile_of_workgroup(blockIdx.x, gridDim.x, (g.M + G2_BM - 1) / G2_BM, (g.N + G2_BN - 1) / G2_BN,
-                      &tile_m, &tile_n);
-    const int m0 = tile_m * G2_BM, n0 = tile_n * G2_BN;
-    const int64_t bz = blockIdx.y;
-    const unsigned char* A = g.a + bz * g.batch_a;
-    const unsigned char* B = g.b + bz * g.batch_b;
-    const unsigned char* SA = g.sa + bz * g.batch_sa;
-    const unsigned char* SB = g.sb + bz * g.batch_sb;
     const int KB = g.K >> 5;
+    const int nk = g.K / GEMM_BK;
+    const int per_batch = tiles_m * tiles_n;
+    const int G = gridDim.x;
 
-    v4f acc[TI][8];
+    v4f acc[4][8];
 #pragma unroll
-    for (int i = 0; i < TI; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    // tile copy: 256 rows x 8 chunks of 16 bytes per operand, CH chunks of A and CH of B per lane
-    // (rows c_row + ROWS_PER_PASS * j).  Rows past the edge are clamped; they are never stored.
-    const int c_row = tid >> 3, c_col = (tid & 7) * 16;
-    int ra[CH], rb[CH];
-#pragma unroll
-    for (int j = 0; j < CH; ++j) {
-        ra[j] = min(m0 + c_row + ROWS_PER_PASS * j, g.M - 1);
-        rb[j] = min(n0 + c_row + ROWS_PER_PASS * j, g.N - 1);
-    }
-    // scales: lanes 0..255 carry a row of A, lanes 256.. (or the same lanes again) a row of B
-    const int s_row = tid & 255;
-    const bool two_scales = NT == 256;                  // every lane loads both
-    const bool s_is_b = tid >= 256;
-    const unsigned char* psa = SA + (int64_t)min(m0 + s_row, g.M - 1) * KB;
-    const unsigned char* psb = SB + (int64_t)min(n0 + s_row, g.N - 1) * KB;
-    const int st_off = c_row * GEMM_PITCH + c_col;
+    // Which rows of B make up MFMA fragment tj decides which columns of C a lane ends up with (it
+    // gets n_local = 4 (lane / 16) + 0..3 of every fragment).  For 16-bit outputs fragment tj, row i
+    // is B row (tj / 2) * 32 + (i / 4) * 8 + (tj % 2) * 4 + i % 4: a lane then owns 8 consecutive
+    // columns per fragment pair, and one store instruction writes 64 contiguous bytes per row
+    // (half as many write requests as 4 columns per lane).  fp32 outputs keep rows 16 tj + i
+    // (4 columns = 16 bytes per lane, 64 contiguous bytes per row as well).
+    constexpr bool PAIR = OUT_DT != MXQ_F32;
+    // position of 16-byte column c of row r inside its LDS row: c ^ key(r); the key must take 8
+    // different values over the even rows of a fragment (and again over the odd ones)
+    auto key_a = [](int r) { return (r >> 1) & 7; };
+    auto key_b = [](int r) { return PAIR ? ((r >> 1) & 1) | (((r >> 3) & 3) << 1) : (r >> 1) & 7; };
 
+    // ---- fetch side: which tile the tile copy is working on --------------------------------------
+    // Wave w brings in rows 32 w .. 32 w + 31 of A and of B, 8 rows per instruction; lane L lands at
+    // position L % 8 of row 8 i + L / 8 and therefore fetches column (L % 8) ^ ((row >> 1) & 7).
+    // Rows past the edge are clamped (their outputs are never stored).
+    const unsigned char *fA, *fB, *fS;
+    uint32_t offa[4], offb[4], offs;
+    int f_kstart;
+    const bool s_is_b = wave >= 4;
+    const int s_row = (wave & 3) * 64 + lane;
+    auto fetch_tile = [&](int logical) {
+        const int bz = logical / per_batch;
+        int tm, tn;
+        tile_of_workgroup(logical % per_batch, per_batch, tiles_m, tiles_n, &tm, &tn);
+        const int m0 = tm * G2_BM, n0 = tn * G2_BN;
+        fA = g.a + bz * g.batch_a + (int64_t)m0 * g.K;
+        fB = g.b + bz * g.batch_b + (int64_t)n0 * g.K;
+        fS = s_is_b ? g.sb + bz * g.batch_sb + (int64_t)n0 * KB : g.sa + bz * g.batch_sa + (int64_t)m0 * KB;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = wave * 32 + i * 8 + (lane >> 3);
+            offa[i] = (uint32_t)min(r, g.M - 1 - m0) * (uint32_t)g.K + ((lane & 7) ^ key_a(r)) * 16;
+            offb[i] = (uint32_t)min(r, g.N - 1 - n0) * (uint32_t)g.K + ((lane & 7) ^ key_b(r)) * 16;
+        }
+        offs = (uint32_t)min(s_row, (s_is_b ? g.N - n0 : g.M - m0) - 1) * (uint32_t)KB;
+        // Every tile walks K cyclically from its own starting step (a multiple of four), so that
+        // the K slices in flight at any moment are spread over the memory channels.
+        f_kstart = (int)(((unsigned)logical * 5u) % (unsigned)(nk >> 2)) << 2;
+    };
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds;     // LDS byte address of the array (normally 0)
+    // load i (0..7 codes, 8 scales) of flat step t, which is K step fs of the fetch-side tile
+    auto fetch_part = [&](int t, int fs, int i) {
+        int kidx = f_kstart + fs;
+        kidx = kidx >= nk ? kidx - nk : kidx;
+        const int k0 = kidx * GEMM_BK;
+        const uint32_t st = lds0 + (t & 1) * G3_STAGE_BYTES;
+        if (i < 4) {
+            dma16(st + (wave * 32 + i * 8) * 128, offa[i], fA + k0);
+        } else if (i < 8) {
+            dma16(st + G3_TILE_BYTES + (wave * 32 + (i - 4) * 8) * 128, offb[i - 4], fB + k0);
+        } else if ((t & 3) == 0) {                          // a new group of four K steps
+            dma16(lds0 + G3_SCALE_OFF + ((t >> 2) & 1) * G3_SCALE_GROUP + wave * 1024, offs, fS + (k0 >> 5));
+        }
+    };
+
+    // ---- compute side ---------------------------------------------------------------------------
     const int frow = lane & 15, fg = lane >> 4;
-    const int a_off = (wy * (TI * 16) + frow) * GEMM_PITCH + fg * 16;
-    const int b_off = G2_TILE_BYTES + (wx * 128 + frow) * GEMM_PITCH + fg * 16;
-    const int sa_off = 2 * G2_TILE_BYTES + (wy * (TI * 16) + frow) * 4 + fg;
-    const int sb_off = 2 * G2_TILE_BYTES + G2_BM * 4 + (wx * 128 + frow) * 4 + fg;
-
-    u32x4 va[CH], vb[CH];
-    uint32_t vsa = 0, vsb = 0;
-    auto fetch = [&](int k0) {
-#pragma unroll
-        for (int j = 0; j < CH; ++j) {
-            va[j] = *reinterpret_cast<const u32x4*>(A + (int64_t)ra[j] * g.K + (k0 + c_col));
-            vb[j] = *reinterpret_cast<const u32x4*>(B + (int64_t)rb[j] * g.K + (k0 + c_col));
-        }
-        if (two_scales) {
-            vsa = *reinterpret_cast<const uint32_t*>(psa + (k0 >> 5));
-            vsb = *reinterpret_cast<const uint32_t*>(psb + (k0 >> 5));
-        } else {
-            vsa = *reinterpret_cast<const uint32_t*>((s_is_b ? psb : psa) + (k0 >> 5));
-        }
+    const int a_lane = wy * 64 + frow;                                        // row of A fragment 0
+    const int b_lane = wx * 128 + (PAIR ? (frow >> 2) * 8 + (frow & 3) : frow);  // row of B fragment 0
+    auto b_step = [](int tj) { return PAIR ? (tj >> 1) * 32 + (tj & 1) * 4 : tj * 16; };
+    const int pa_lo = (fg ^ key_a(a_lane)) * 16, pb_lo = (fg ^ key_b(b_lane)) * 16;   // same for all fragments
+    const int a_row = a_lane * 128, b_row = G3_TILE_BYTES + b_lane * 128;
+    const int sa_off = G3_SCALE_OFF + a_lane * 16 + fg;
+    const int sb_off = G3_SCALE_OFF + 4096 + b_lane * 16 + fg;
+    auto frag = [&](const unsigned char* row, int p_lo) {
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(row + p_lo);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(row + (p_lo ^ 64));
+        return v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
     };
-    auto stash_rows = [&](unsigned char* stage, int j) {      // chunk j of A and of B
-        *reinterpret_cast<u32x4*>(stage + st_off + ROWS_PER_PASS * j * GEMM_PITCH) = va[j];
-        *reinterpret_cast<u32x4*>(stage + G2_TILE_BYTES + st_off + ROWS_PER_PASS * j * GEMM_PITCH) = vb[j];
-    };
-    auto stash_scales = [&](unsigned char* stage) {
-        if (two_scales) {
-            *reinterpret_cast<uint32_t*>(stage + 2 * G2_TILE_BYTES + s_row * 4) = vsa;
-            *reinterpret_cast<uint32_t*>(stage + 2 * G2_TILE_BYTES + G2_BM * 4 + s_row * 4) = vsb;
-        } else {
-            *reinterpret_cast<uint32_t*>(stage + 2 * G2_TILE_BYTES + (s_is_b ? G2_BM * 4 : 0) + s_row * 4) = vsa;
-        }
-    };
-
-    // Every workgroup walks K cyclically from its own starting step.  Rows are K bytes apart, so
-    // with K a power of two a given K slice of *every* row sits in the same L2 channel; staggering
-    // the start spreads the slices in flight at any moment over all channels.
-    const int nk = g.K / GEMM_BK;
-    const int kstart = (int)((blockIdx.x * 5u + blockIdx.y) % (unsigned)nk);
-    auto kof = [&](int step) { return ((kstart + step) % nk) * GEMM_BK; };
-
-    fetch(kof(0));
+    // flat step t: multiply the stage t & 1 while the tile copy fills the other one with K step
+    // fs of the fetch-side tile
+    auto step = [&](int t, int fs) {
+        const unsigned char* cur = lds + (t & 1) * G3_STAGE_BYTES;
+        const unsigned char* sc = lds + ((t >> 2) & 1) * G3_SCALE_GROUP + (t & 3) * 4;
+        v8i af[4];
+        int sa[4];
 #pragma unroll
-    for (int j = 0; j < CH; ++j) stash_rows(lds, j);
-    stash_scales(lds);
-    __syncthreads();
-
-    int buf = 0;
-    for (int step = 0; step < nk; ++step) {
-        const unsigned char* cur = lds + buf * G2_STAGE_BYTES;
-        unsigned char* nxt = lds + (buf ^ 1) * G2_STAGE_BYTES;   // nobody reads it during this step
-        // Fetch the next tile now; it is in flight during the MFMAs below.  The last step fetches
-        // one more (unused) tile and stores it into the idle buffer: keeping the loop body free of
-        // branches is what lets the instruction order below survive compilation.
-        fetch(kof(step + 1));
-
-        v8i af[TI];
-        int sa[TI];
-#pragma unroll
-        for (int ti = 0; ti < TI; ++ti) {
-            af[ti] = load_frag(cur + a_off + ti * 16 * GEMM_PITCH);
-            sa[ti] = cur[sa_off + ti * 64];
+        for (int ti = 0; ti < 4; ++ti) {
+            af[ti] = frag(cur + a_row + ti * 16 * 128, pa_lo);
+            sa[ti] = sc[sa_off + ti * 256];
         }
-        __builtin_amdgcn_sched_barrier(0);                   // keep the global loads up here
-        v8i bf = load_frag(cur + b_off);
-        int sb = cur[sb_off];
+        v8i bf = frag(cur + b_row, pb_lo);
+        int sb = sc[sb_off];
 #pragma unroll
         for (int tj = 0; tj < 8; ++tj) {
-            // the next B fragment is read in the shadow of this fragment's MFMAs
-            v8i bf_next = bf;
-            int sb_next = sb;
+            v8i bf_next = bf;                                // the next B fragment is read in the
+            int sb_next = sb;                                // shadow of this fragment's MFMAs
             if (tj + 1 < 8) {
-                bf_next = load_frag(cur + b_off + (tj + 1) * 16 * GEMM_PITCH);
-                sb_next = cur[sb_off + (tj + 1) * 64];
+                bf_next = frag(cur + b_row + b_step(tj + 1) * 128, pb_lo);
+                sb_next = sc[sb_off + b_step(tj + 1) * 16];
             }
 #pragma unroll
-            for (int ti = 0; ti < TI; ++ti)
+            for (int ti = 0; ti < 4; ++ti) {
                 acc[ti][tj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                     bf, af[ti], acc[ti][tj], BLGP, CBSZ, 0, sb, 0, sa[ti]);
-            // second half of the step: the tile fetched at its top has had time to arrive; its LDS
-            // writes go out in the shadow of the remaining MFMAs
-            if (tj >= 4) {
+                if (ti == 0) {
 #pragma unroll
-                for (int j = (tj - 4) * CH / 4; j < (tj - 3) * CH / 4; ++j) stash_rows(nxt, j);
+                    for (int i = 0; i < 9; ++i)
+                        if (i * G3_SPREAD / 9 == tj) fetch_part(t + 1, fs, i);
+                }
             }
-            if (tj == 7) stash_scales(nxt);
             __builtin_amdgcn_sched_barrier(0);
             bf = bf_next;
             sb = sb_next;
         }
-        __syncthreads();
-        buf ^= 1;
-    }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // this wave's share of the next stage is in
+        __syncthreads();                                     // ... everybody's is, and this stage is free
+    };
 
-    const int64_t cbase = bz * g.batch_c;
-    const bool inside = m0 + G2_BM <= g.M && n0 + G2_BN <= g.N && (g.N & 3) == 0;
+    int logical = blockIdx.x;                                // tile being multiplied
+    fetch_tile(logical);
 #pragma unroll
-    for (int ti = 0; ti < TI; ++ti)
+    for (int i = 0; i < 9; ++i) fetch_part(0, 0, i);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    int t = 0;
+    while (true) {
+        for (int cs = 0; cs + 1 < nk; ++cs, ++t) step(t, cs + 1);
+        // last K step of this tile: the tile copy moves on to the next tile (or, when there is none,
+        // fetches this tile's first step once more; nobody reads it)
+        const int next = logical + G;
+        if (next < total) fetch_tile(next);
+        step(t, 0);
+        ++t;
+
+        const int bz = logical / per_batch;
+        int tm, tn;
+        tile_of_workgroup(logical % per_batch, per_batch, tiles_m, tiles_n, &tm, &tn);
+        const int m0 = tm * G2_BM, n0 = tn * G2_BN;
+        const int64_t cbase = bz * g.batch_c;
+        const bool inside = m0 + G2_BM <= g.M && n0 + G2_BN <= g.N && (g.N & 3) == 0 &&
+                            ((uintptr_t)g.c & 15) == 0;
+        const bool inside8 = inside && (g.N & 7) == 0 && ((uintptr_t)g.bias & 15) == 0;
 #pragma unroll
-        for (int tj = 0; tj < 8; ++tj)
-            store_c4<OUT_DT>(g.c, g.bias, cbase, m0 + wy * (TI * 16) + ti * 16 + frow,
-                             n0 + wx * 128 + tj * 16 + fg * 4, g.M, g.N, inside, acc[ti][tj]);
+        for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < 8; ++tj) {
+                const int m = m0 + wy * 64 + ti * 16 + frow;
+                if constexpr (PAIR) {
+                    if (tj & 1)
+                        store_c8<OUT_DT>(g.c, g.bias, cbase, m, n0 + wx * 128 + (tj >> 1) * 32 + fg * 8, g.M,
+                                         g.N, inside8, acc[ti][tj - 1], acc[ti][tj]);
+                } else {
+                    store_c4<OUT_DT>(g.c, g.bias, cbase, m, n0 + wx * 128 + tj * 16 + fg * 4, g.M, g.N,
+                                     inside, acc[ti][tj]);
+                }
+            }
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < 8; ++tj) acc[ti][tj] = v4f{0.f, 0.f, 0.f, 0.f};
+        if (next >= total) break;
+        logical = next;
+    }
 }
 
 // Register-resident MFMA loop: every wave issues `iters` x 16 independent scaled MFMAs on operands

@@ -45,7 +45,11 @@ def test_pack_then_unpack_is_the_fake_quantized_tensor(dev, fmt, rnd, dtype):
 
 @pytest.mark.parametrize("M,N,K,batch", [(128, 128, 128, 1), (256, 384, 512, 1), (100, 72, 256, 1),
                                          (130, 257, 128, 3), (16, 16, 128, 2), (1, 5, 384, 1),
-                                         (512, 768, 256, 1), (600, 520, 128, 2)])
+                                         (512, 768, 256, 1), (600, 520, 128, 2),
+                                         # the persistent 256 x 256 kernel (K % 512 == 0): one tile
+                                         # per workgroup, ragged edges, several tiles per workgroup
+                                         (512, 768, 512, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
+                                         (2048, 2048, 512, 5), (2050, 1800, 1024, 5)])
 @pytest.mark.parametrize("fa,fb", [("fp8_e4m3", "fp8_e4m3"), ("fp8_e5m2", "fp8_e4m3"),
                                    ("fp6_e2m3", "fp8_e5m2"), ("fp4_e2m1", "fp6_e3m2")])
 def test_scaled_mfma_gemm_against_fp64(dev, M, N, K, batch, fa, fb):
@@ -70,6 +74,29 @@ def test_scaled_mfma_gemm_against_fp64(dev, M, N, K, batch, fa, fb):
     assert rel_err(got, want) < 1e-3
     den = qa.abs() @ qb.abs().transpose(-1, -2)
     assert ((got.double() - want).abs() <= 2e-4 * den + 1e-30).all()
+
+
+@pytest.mark.parametrize("M,N,K,batch", [(128, 136, 256, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
+                                         (2050, 1800, 512, 5), (520, 777, 512, 1)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_gemm_16bit_outputs_equal_rounded_fp32_output(dev, M, N, K, batch, dtype, with_bias):
+    """The accumulation does not depend on the output type, so a 16-bit output must be the fp32
+    output rounded once (and, with a bias, rounded, added to and rounded again), bit for bit --
+    whatever layout the kernel chooses for the output type."""
+    from microxcaling_amd.fused import pack_mx, gemm_nt
+    g = torch.Generator().manual_seed(M + N + K + batch)
+    sa = (batch, M, K) if batch > 1 else (M, K)
+    sb = (batch, N, K) if batch > 1 else (N, K)
+    pa = pack_mx(torch.randn(*sa, generator=g).to(dev), "fp8_e4m3")
+    pb = pack_mx(torch.randn(*sb, generator=g).to(dev), "fp8_e5m2")
+    bias = torch.randn(N, generator=g).to(dev).to(dtype) if with_bias else None
+    want = gemm_nt(pa, pb, torch.float32).to(dtype)
+    if with_bias:
+        want = want + bias
+    got = gemm_nt(pa, pb, dtype, bias=bias)
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
 def test_gemm_propagates_nan_blocks(dev):
