@@ -93,6 +93,21 @@ int mxq_reduce_sum_outer(const float* in, float* out, void* workspace, int64_t o
 int mxq_reduce_max_outer(const float* in, float* out, void* workspace, int64_t outer,
                          int64_t inner, void* hip_stream);
 
+/* SoftmaxFunction.forward (mx/softmax.py:20-54) over the last axis of a contiguous (rows, n) fp32
+ * or bf16 tensor, as one kernel: quantize, row maximum, subtract, exponential, row sum, divide, with
+ * the elementwise quantization of mx/vector_ops.py:38-130 (format bits / exp_bits / max_norm,
+ * overflow to Inf as in _quantize_bfloat / _quantize_fp) after every step.  bits == 0 means "no
+ * format": the steps are only rounded to the tensor dtype (what quantize_elemwise_op does without
+ * bfloat / fp, and for bfloat16 with round-half-even on a bf16 tensor).
+ * exp_mode 0: exp(x); 1: 2^x (mx_specs['softmax_exp2']); 2: 2^Q(x * 1.4453125) (['vec_use_exp2']).
+ * use_recip: e * Q(1 / sum) instead of e / sum (['vec_use_recip']).
+ * n must be a multiple of 16 bytes worth of elements and at most 4096.  The reference has no native
+ * counterpart (it runs ten tensor ops); results agree with that chain up to the last-bit
+ * differences of exp and of the summation order. */
+int mxq_softmax_lastdim(const void* in, void* out, int dtype, int64_t rows, int64_t n, int bits,
+                        int exp_bits, float max_norm, int rmode, int allow_denorm, int exp_mode,
+                        int use_recip, int flags, void* hip_stream);
+
 /* ---- packed MX tensors and the fused GEMM (no counterpart in the reference, which only ever
  * fake-quantizes and then calls a dense GEMM: mx/linear.py:62-86, mx/bmm.py:40-59) ---------------
  * Packed form of a (rows, K) tensor quantized along K in blocks of 32:
@@ -108,10 +123,14 @@ int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, voi
 /* C[b] (M, N) = A[b] (M, K) x B[b] (N, K)^T for b < batch, all tensors contiguous, fp32
  * accumulation on the scaled MFMA units; c_dtype is a MXQ_DTYPE_* code.  K % 128 == 0.
  * bias (optional, may be NULL): N values of dtype c_dtype; then C = round(round(A x B^T) + bias),
- * both roundings to c_dtype, which is what "matmul, then add the bias" gives as tensor ops. */
+ * both roundings to c_dtype, which is what "matmul, then add the bias" gives as tensor ops.
+ * epilogue_quant = 1 (bf16 C only): additionally apply the elementwise quantization of the layers
+ * with mx_specs['bfloat'] = 16 and round-half-away (quantize_elemwise_op, mx/linear.py:88-96,
+ * mx/bmm.py:55-57) to the rounded product and again to the rounded sum with the bias. */
 int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, const void* b_codes,
                    const void* b_scales, int b_is_e5m2, const void* bias, void* c, int c_dtype,
-                   int64_t batch, int64_t M, int64_t N, int64_t K, void* hip_stream);
+                   int64_t batch, int64_t M, int64_t N, int64_t K, int epilogue_quant,
+                   void* hip_stream);
 
 /* Measurement aid (no counterpart in the reference): launches `workgroups` x 256 lanes, each wave
  * issuing iters x 16 scaled 16x16x128 fp8 MFMAs on register-resident operands
@@ -125,6 +144,8 @@ int mxq_probe_mfma_rate(int64_t workgroups, int iters, void* sink, void* hip_str
  * CPU counterpart in the reference; it mirrors mxq_quantize_mx_by_tile so the kernel arithmetic
  * can be checked on a machine without a GPU. */
 #define MXQ_HOST_FLAG_ROUND_EVERY_OP 2 /* bf16: round to bf16 after every op, no shortcuts */
+#define MXQ_HOST_FLAG_CLOSED_FORM 4    /* elementwise, bf16 tensor -> bfloat16, nearest: the closed
+                                          form the fused softmax kernel uses (else: an error) */
 
 const char* mxq_host_last_error(void);
 int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_values, int dtype,

@@ -26,11 +26,13 @@ GPU_SYMBOLS = {
                                            _c_ptr]),
     "mxq_quantize_elemwise": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_f32,
                                        _c_int, _c_int, _c_int, _c_int, _c_ptr]),
+    "mxq_softmax_lastdim": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_int, _c_int, _c_f32,
+                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr]),
     "mxq_pack_mx": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_int, _c_int, _c_int,
                              _c_f32, _c_int, _c_int, _c_int, _c_ptr]),
     "mxq_unpack_mx": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_i64, _c_ptr]),
     "mxq_gemm_mx_nt": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int,
-                                _c_i64, _c_i64, _c_i64, _c_i64, _c_ptr]),
+                                _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr]),
     "mxq_probe_mfma_rate": (_c_int, [_c_i64, _c_int, _c_ptr, _c_ptr]),
     "mxq_reduce_sum_inner": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),
     "mxq_reduce_max_inner": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),

@@ -21,10 +21,12 @@ class BMMFunction(torch.autograd.Function):
             ctx.save_for_backward(bf_in1, bf_in2)
         else:
             ctx.save_for_backward(in1, in2)
-        out = mx_matmul_contract(bf_in1, bf_in2, mx_specs["a_elem_format"],
-                                 mx_specs["a_elem_format"], mx_specs, mx_specs["round_mx_output"],
-                                 batched=True)
-        out = quantize_elemwise_op(out, mx_specs=mx_specs, round=mx_specs["round_output"])
+        out, finished = mx_matmul_contract(bf_in1, bf_in2, mx_specs["a_elem_format"],
+                                           mx_specs["a_elem_format"], mx_specs,
+                                           mx_specs["round_mx_output"], batched=True,
+                                           out_round=mx_specs["round_output"])
+        if not finished:
+            out = quantize_elemwise_op(out, mx_specs=mx_specs, round=mx_specs["round_output"])
         ctx.mx_specs = get_backwards_mx_specs(mx_specs)
         return out
 

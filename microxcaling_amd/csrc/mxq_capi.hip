@@ -6,6 +6,7 @@
 #include "mxq.h"
 #include "mxq_kernels.h"
 #include "mxq_gemm.h"
+#include "mxq_softmax.h"
 
 namespace {
 
@@ -261,11 +262,11 @@ int mxq_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre, i
     if (post == 1 && ptr_ok && axis_size % tile == 0 && tile % vec_elems == 0) {
         const int64_t lpt = tile / vec_elems;
         if (lpt == 1 || lpt == 2 || lpt == 4 || lpt == 8 || lpt == 16) {
-            dispatch<LaunchLastAxis>(dtype, rmode, ze, lean_ok(dtype, p.fmt), in, out, total / vec_elems, (int)lpt, p, s);
+            dispatch<LaunchLastAxis>(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, total / vec_elems, (int)lpt, p, s);
             return check_launch(who);
         }
     }
-    dispatch<LaunchStrided>(dtype, rmode, ze, lean_ok(dtype, p.fmt), in, out, pre, axis_size, post, tile, ptr_ok, p, s);
+    dispatch<LaunchStrided>(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, pre, axis_size, post, tile, ptr_ok, p, s);
     return check_launch(who);
 }
 
@@ -284,7 +285,7 @@ int mxq_quantize_mx_given_max(const void* in, void* out, const void* max_values,
     if (mul_overflows(pre, axis_size, post, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
     if (total == 0) return MXQ_OK;
     if (!in || !out || !max_values) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
-    dispatch<LaunchGivenMax>(dtype, rmode, ze, lean_ok(dtype, p.fmt), in, out, max_values, total, axis_size, post, p,
+    dispatch<LaunchGivenMax>(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, max_values, total, axis_size, post, p,
                              (hipStream_t)hip_stream);
     return check_launch(who);
 }
@@ -302,7 +303,61 @@ int mxq_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int b
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     if (!aligned16(in) || !aligned16(out))
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
-    dispatch<LaunchElemwise>(dtype, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode), lean_ok(dtype, p.fmt), in, out, n, p, (hipStream_t)hip_stream);
+    dispatch<LaunchElemwise>(dtype, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode), lean_ok(dtype, p.fmt, rmode, true), in, out, n, p, (hipStream_t)hip_stream);
+    return check_launch(who);
+}
+
+int mxq_softmax_lastdim(const void* in, void* out, int dtype, int64_t rows, int64_t n, int bits,
+                        int exp_bits, float max_norm, int rmode, int allow_denorm, int exp_mode,
+                        int use_recip, int flags, void* hip_stream) {
+    const char* who = "mxq_softmax_lastdim";
+    SoftmaxParams p;
+    const bool ident = bits == 0;
+    if (dtype != MXQ_DTYPE_F32 && dtype != MXQ_DTYPE_BF16)
+        return fail(MXQ_ERR_ARGUMENT, "%s: dtype code %d (fp32 and bf16 tensors only)", who, dtype);
+    int rc = make_elem_params(dtype, ident ? 9 : bits, ident ? 8 : exp_bits, ident ? 1.0f : max_norm,
+                              ident ? MXQ_ROUND_NEAREST : rmode, 0, allow_denorm, flags, &p.q, who);
+    if (rc) return rc;
+    if (!ident && !lean_ok(dtype, p.q.fmt, rmode, true))
+        return fail(MXQ_ERR_ARGUMENT, "%s: round-half-even to %d fraction bits on a bf16 tensor is "
+                    "only available through the separate elementwise steps", who, p.q.fmt.t);
+    if (exp_mode < 0 || exp_mode > 2) return fail(MXQ_ERR_ARGUMENT, "%s: exp_mode %d outside [0, 2]", who, exp_mode);
+    p.exp_mode = exp_mode;
+    p.use_recip = use_recip ? 1 : 0;
+    const int epv = dtype == MXQ_DTYPE_F32 ? 4 : 8;
+    if (rows < 0 || n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (n > 4096 || n % epv != 0)
+        return fail(MXQ_ERR_ARGUMENT, "%s: row length %lld must be a multiple of %d and at most 4096",
+                    who, (long long)n, epv);
+    if (rows == 0 || n == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(in) || !aligned16(out))
+        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int grid = grid_for(ceil_div(rows, kThreads / 64));
+    const int64_t nvec = n / epv;                       // 16-byte vectors per row, 64 lanes
+    const bool closed = !ident && dtype == MXQ_DTYPE_BF16 && bits == 9 && exp_bits == 8 &&
+                        rmode == MXQ_ROUND_NEAREST && allow_denorm && p.q.fmt.max_bits == 0x7F7F0000u;
+#define MXQ_SM(DT, RM, QM)                                                                         \
+    do {                                                                                           \
+        constexpr int V = (DT == MXQ_F32) ? 2 : 1;                                                 \
+        if (nvec <= 128 * V) softmax_row_kernel<DT, RM, QM, 2 * V><<<grid, kThreads, 0, s>>>(in, out, rows, (int)n, p);      \
+        else if (nvec <= 256 * V) softmax_row_kernel<DT, RM, QM, 4 * V><<<grid, kThreads, 0, s>>>(in, out, rows, (int)n, p); \
+        else softmax_row_kernel<DT, RM, QM, 8 * V><<<grid, kThreads, 0, s>>>(in, out, rows, (int)n, p);                     \
+    } while (0)
+    if (dtype == MXQ_DTYPE_F32) {
+        if (ident) MXQ_SM(MXQ_F32, MXQ_NEAREST, SMQ_IDENT);
+        else if (rmode == MXQ_ROUND_FLOOR) MXQ_SM(MXQ_F32, MXQ_FLOOR, SMQ_GENERIC);
+        else if (rmode == MXQ_ROUND_NEAREST) MXQ_SM(MXQ_F32, MXQ_NEAREST, SMQ_GENERIC);
+        else MXQ_SM(MXQ_F32, MXQ_EVEN, SMQ_GENERIC);
+    } else {
+        if (ident) MXQ_SM(MXQ_BF16, MXQ_NEAREST, SMQ_IDENT);
+        else if (closed) MXQ_SM(MXQ_BF16, MXQ_NEAREST, SMQ_BF16);
+        else if (rmode == MXQ_ROUND_FLOOR) MXQ_SM(MXQ_BF16, MXQ_FLOOR, SMQ_GENERIC);
+        else if (rmode == MXQ_ROUND_NEAREST) MXQ_SM(MXQ_BF16, MXQ_NEAREST, SMQ_GENERIC);
+        else MXQ_SM(MXQ_BF16, MXQ_EVEN, SMQ_GENERIC);
+    }
+#undef MXQ_SM
     return check_launch(who);
 }
 
@@ -356,9 +411,12 @@ int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, voi
 
 int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, const void* b_codes,
                    const void* b_scales, int b_is_e5m2, const void* bias, void* c, int c_dtype,
-                   int64_t batch, int64_t M, int64_t N, int64_t K, void* hip_stream) {
+                   int64_t batch, int64_t M, int64_t N, int64_t K, int epilogue_quant,
+                   void* hip_stream) {
     const char* who = "mxq_gemm_mx_nt";
     if (c_dtype < 0 || c_dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, c_dtype);
+    if (epilogue_quant != 0 && (epilogue_quant != 1 || c_dtype != MXQ_DTYPE_BF16))
+        return fail(MXQ_ERR_ARGUMENT, "%s: epilogue_quant must be 0, or 1 with a bf16 output", who);
     if (batch < 0 || M < 0 || N < 0 || K < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
     if (K % GEMM_BK != 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be a multiple of %d", who, GEMM_BK);
     if (batch == 0 || M == 0 || N == 0) return MXQ_OK;
@@ -376,6 +434,13 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, con
     g.sb = reinterpret_cast<const unsigned char*>(b_scales);
     g.c = c;
     g.bias = bias;
+    g.q_nan_from = 0u;
+    if (epilogue_quant) {                               // bfloat16, nearest: only the NaN threshold is needed
+        ElemParams q;
+        int rc = make_elem_params(MXQ_DTYPE_BF16, 9, 8, 3.3895313892515355e38f, MXQ_ROUND_NEAREST, 0, 1, 0, &q, who);
+        if (rc) return rc;
+        g.q_nan_from = q.fmt.nan_from;
+    }
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.batch_a = M * K; g.batch_sa = M * (K / 32);
     g.batch_b = N * K; g.batch_sb = N * (K / 32);

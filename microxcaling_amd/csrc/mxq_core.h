@@ -62,6 +62,7 @@ struct MxqFmt {
     float half;         // what "+ 0.5" must add so that floor() sees the dtype-rounded sum
     float tie_fix;      // the one input of the scaled domain whose "+ 0.5" rounds up to 1.0
     uint32_t nan_from;  // elementwise only: |x| bit pattern from which floor(log2|x|) is 128
+    float bump_lo;      // bf16 tensors, t >= 7: 128 (see mxq_round_lean<.., BUMP>); else +inf
 };
 
 // ---- floor(log2(x)) in the tensor dtype --------------------------------------------------------
@@ -110,7 +111,11 @@ MXQ_HD MxqScale mxq_block_scale(uint32_t um, int emax, int scale_emax, bool flus
 // and torch's even-mode emulation equals round-half-even except for that same input.
 // Inf/NaN inputs give unspecified results here; callers overwrite them.
 // sign_src: a value with the sign the result must carry (+0.0 when the result must be +0).
-template <int RMODE, bool ZONE>
+// BUMP (bf16 tensors, nearest and floor modes, any t): with 7 or more fraction bits the scaled
+// value s can be an integer in [128, 256), where bf16 has no halves: "s + 0.5" then ties to the
+// even neighbour, so an odd s comes out as s + 1.  Everything else is exact: s has 8 significant
+// bits, larger s are integers that "+ 0.5" leaves alone, smaller ones have room for the half.
+template <int RMODE, bool ZONE, bool BUMP = false>
 MXQ_HD float mxq_round_lean(float a, float sign_src, const MxqFmt& f, bool saturate,
                             const unsigned char* zone, int zshift) {
     const uint32_t ua = mxq_bits(a) & 0x7FFFFFFFu;
@@ -129,6 +134,10 @@ MXQ_HD float mxq_round_lean(float a, float sign_src, const MxqFmt& f, bool satur
         r = floorf(s);
     } else if (RMODE == MXQ_NEAREST) {
         r = floorf(s + f.half);
+        if (BUMP) {
+            const float odd = r - 2.0f * floorf(r * 0.5f);
+            r += (s >= f.bump_lo && s < 2.0f * f.bump_lo) ? odd : 0.0f;
+        }
     } else {
         r = __builtin_rintf(s);                 // ties to even (default rounding mode)
         r = (s == f.tie_fix) ? 1.0f : r;
@@ -253,13 +262,27 @@ MXQ_HD uint32_t mxq_encode_e8m0(float scale) {
     return (u >> 23) ? (u >> 23) : 0u;            // 2^-127 is the fp32 subnormal 0x00400000 -> 0
 }
 
+// The elementwise quantizer for the commonest case, closed form: a bf16 tensor rounded to bfloat16
+// (8 exponent bits, bits = 9), round-half-away, subnormals allowed, overflow to Inf.  The format
+// holds every bf16 value, yet the op-by-op arithmetic is not the identity: the scaled significand
+// is an integer in [128, 256) (or, in the round-up zone of the exponent, a half-integer in
+// [64, 128)), and "+ 0.5" then moves an odd significand to the next even one.  Subnormals scale
+// below 128 and stay.  x: already a bf16 value.
+MXQ_HD float mxq_quant_bf16_to_bfloat16_nearest(float x, uint32_t nan_from) {
+    const uint32_t u = mxq_bits(x), ua = u & 0x7FFFFFFFu;
+    uint32_t r = u + (u & 0x10000u);                      // odd significand -> + 1 (may carry to Inf)
+    r = (ua >> 23) == 0u ? (ua == 0u ? 0u : u) : r;       // subnormals stay, +-0 -> +0
+    if (ua >= nan_from) r = (ua == MXQ_INF_BITS) ? u : MXQ_QNAN_BITS;
+    return mxq_float(r);
+}
+
 // One element of the elementwise quantizer (mx/elemwise_ops.py:127-163).
 template <int RMODE, int DT, bool ZONE, bool LEAN>
 MXQ_HD float mxq_quant_elemwise(float x, const MxqFmt& f, bool saturate, bool allow_denorm,
                                 const unsigned char* zone, int zshift) {
     const uint32_t ux = mxq_bits(x) & 0x7FFFFFFFu;
     float y;
-    if (LEAN) y = mxq_round_lean<RMODE, ZONE>(x, x + 0.0f, f, saturate || f.ebits == 0, zone, zshift);
+    if (LEAN) y = mxq_round_lean<RMODE, ZONE, DT == MXQ_BF16>(x, x + 0.0f, f, saturate || f.ebits == 0, zone, zshift);
     else y = mxq_round_every_op<RMODE, DT>(ux < MXQ_INF_BITS ? x : 0.0f, f, saturate, zone, zshift);
     // (|A| >= min_norm) * A is +-0, and sign(+-0) is 0
     if (!allow_denorm && f.ebits > 0 && (ux >> 23) < f.min_eb) y = 0.0f;

@@ -105,6 +105,9 @@ struct GemmArgs {
     const unsigned char* sb;
     void* c;
     const void* bias;     // optional (N), dtype of C: C = round(round(A x B^T) + bias)
+    uint32_t q_nan_from;  // 0: no output quantization.  Else C is bf16 and is quantized to bfloat16,
+                          // round-half-away, after the product and again after the bias add (the
+                          // closed form mxq_quant_bf16_to_bfloat16_nearest with this threshold)
     int M, N, K;
     int64_t batch_a, batch_sa, batch_b, batch_sb, batch_c;   // element strides between batches
 };
@@ -138,18 +141,32 @@ __device__ __forceinline__ v8i load_frag(const unsigned char* p) {
 // The MFMAs are issued with the B fragment as the first operand, i.e. they compute 16 x 16 blocks
 // of C^T: a lane then holds four *consecutive columns* n = 4 * (lane / 16) + r of one row
 // m = lane % 16, which it can store with a single 8- or 16-byte access.
+// What the layers do as separate tensor ops after the product: round it to the tensor dtype,
+// (quantize,) add the bias, round again (, quantize again).  The last rounding to the dtype is left
+// to the store when nothing follows it.
 template <int OUT_DT>
-__device__ __forceinline__ void store_c4(void* c, const void* bias, int64_t base, int m, int n,
-                                         int M, int N, bool tile_inside, v4f v) {
+__device__ __forceinline__ float epilogue_value(float acc, bool has_bias, float b, uint32_t q_nan_from) {
     constexpr int ADT = Arith<OUT_DT>::DT_;
-    if (bias != nullptr) {
-        // what the layers do as separate tensor ops: the product is rounded to the tensor dtype,
-        // the bias is added, and the sum is rounded again (by the store below)
+    if (!has_bias && q_nan_from == 0u) return acc;
+    float p = (OUT_DT == MXQ_F16) ? (float)(_Float16)acc : mxq_round_dt<ADT>(acc);
+    if (OUT_DT == MXQ_BF16 && q_nan_from != 0u) p = mxq_quant_bf16_to_bfloat16_nearest(p, q_nan_from);
+    if (has_bias) {
+        p += b;
+        if (OUT_DT == MXQ_BF16 && q_nan_from != 0u)
+            p = mxq_quant_bf16_to_bfloat16_nearest(mxq_round_dt<ADT>(p), q_nan_from);
+    }
+    return p;
+}
+
+template <int OUT_DT>
+__device__ __forceinline__ void store_c4(void* c, const void* bias, uint32_t q_nan_from, int64_t base,
+                                         int m, int n, int M, int N, bool tile_inside, v4f v) {
+    constexpr int ADT = Arith<OUT_DT>::DT_;
+    if (bias != nullptr || q_nan_from != 0u) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float b = (n + r < N) ? load_scalar<OUT_DT>(bias, n + r) : 0.0f;
-            const float p = (OUT_DT == MXQ_F16) ? (float)(_Float16)v[r] : mxq_round_dt<ADT>(v[r]);
-            v[r] = p + b;
+            const float b = (bias != nullptr && n + r < N) ? load_scalar<OUT_DT>(bias, n + r) : 0.0f;
+            v[r] = epilogue_value<OUT_DT>(v[r], bias != nullptr, b, q_nan_from);
         }
     }
     if (tile_inside) {                                       // uniform per workgroup
@@ -173,19 +190,19 @@ __device__ __forceinline__ void store_c4(void* c, const void* bias, int64_t base
 
 // Eight consecutive columns of one row, 16-bit outputs: one 16-byte store (and bias load).
 template <int OUT_DT>
-__device__ __forceinline__ void store_c8(void* c, const void* bias, int64_t base, int m, int n,
-                                         int M, int N, bool tile_inside, v4f lo, v4f hi) {
+__device__ __forceinline__ void store_c8(void* c, const void* bias, uint32_t q_nan_from, int64_t base,
+                                         int m, int n, int M, int N, bool tile_inside, v4f lo, v4f hi) {
     constexpr int ADT = Arith<OUT_DT>::DT_;
     float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     if (tile_inside) {                                       // uniform per workgroup
         if (bias != nullptr) {
             const u32x4 bw = *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned short*>(bias) + n);
 #pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                const float b = Pack<OUT_DT>::get(bw[r >> 1], r & 1);
-                const float p = (OUT_DT == MXQ_F16) ? (float)(_Float16)v[r] : mxq_round_dt<ADT>(v[r]);
-                v[r] = p + b;
-            }
+            for (int r = 0; r < 8; ++r)
+                v[r] = epilogue_value<OUT_DT>(v[r], true, Pack<OUT_DT>::get(bw[r >> 1], r & 1), q_nan_from);
+        } else if (q_nan_from != 0u) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) v[r] = epilogue_value<OUT_DT>(v[r], false, 0.0f, q_nan_from);
         }
         *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned short*>(c) + base + (int64_t)m * N + n) =
             u32x4{Pack<OUT_DT>::put(v[0], v[1]), Pack<OUT_DT>::put(v[2], v[3]),
@@ -194,11 +211,8 @@ __device__ __forceinline__ void store_c8(void* c, const void* bias, int64_t base
 #pragma unroll
         for (int r = 0; r < 8; ++r)
             if (n + r < N) {
-                float x = v[r];
-                if (bias != nullptr) {
-                    const float p = (OUT_DT == MXQ_F16) ? (float)(_Float16)x : mxq_round_dt<ADT>(x);
-                    x = p + load_scalar<OUT_DT>(bias, n + r);
-                }
+                const float b = bias != nullptr ? load_scalar<OUT_DT>(bias, n + r) : 0.0f;
+                const float x = epilogue_value<OUT_DT>(v[r], bias != nullptr, b, q_nan_from);
                 store_scalar<OUT_DT>(c, base + (int64_t)m * N + n + r, mxq_round_dt<ADT>(x));
             }
     }
@@ -310,7 +324,7 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     for (int ti = 0; ti < 4; ++ti)
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj)
-            store_c4<OUT_DT>(g.c, g.bias, cbase, m0 + wy * 64 + ti * 16 + frow, n0 + wx * 64 + tj * 16 + fg * 4,
+            store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m0 + wy * 64 + ti * 16 + frow, n0 + wx * 64 + tj * 16 + fg * 4,
                              g.M, g.N, inside, acc[ti][tj]);
 }
 
@@ -511,10 +525,10 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
                 const int m = m0 + wy * 64 + ti * 16 + frow;
                 if constexpr (PAIR) {
                     if (tj & 1)
-                        store_c8<OUT_DT>(g.c, g.bias, cbase, m, n0 + wx * 128 + (tj >> 1) * 32 + fg * 8, g.M,
+                        store_c8<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, n0 + wx * 128 + (tj >> 1) * 32 + fg * 8, g.M,
                                          g.N, inside8, acc[ti][tj - 1], acc[ti][tj]);
                 } else {
-                    store_c4<OUT_DT>(g.c, g.bias, cbase, m, n0 + wx * 128 + tj * 16 + fg * 4, g.M, g.N,
+                    store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, n0 + wx * 128 + tj * 16 + fg * 4, g.M, g.N,
                                      inside, acc[ti][tj]);
                 }
             }

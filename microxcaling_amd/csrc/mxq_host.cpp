@@ -85,7 +85,7 @@ int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t p
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const int64_t tile = (tile_size <= 0 || tile_size > axis_size) ? axis_size : tile_size;
     const unsigned char* zone = kZone[p.zone_row];
-    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
+    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < pre; ++i)
         for (int64_t k0 = 0; k0 < axis_size; k0 += tile)
             for (int64_t j = 0; j < post; ++j) {
@@ -118,7 +118,7 @@ int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_va
     if (total == 0) return MXQ_OK;
     if (!in || !out || !max_values) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const unsigned char* zone = kZone[p.zone_row];
-    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
+    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < pre; ++i)
         for (int64_t j = 0; j < post; ++j) {
             const uint32_t um = mxq_bits(load_as_float(max_values, dtype, i * post + j)) & 0x7FFFFFFFu;
@@ -142,9 +142,18 @@ int mxq_host_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, 
     if (n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
     if (n == 0) return MXQ_OK;
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (flags & MXQ_HOST_FLAG_CLOSED_FORM) {
+        if (!(dtype == MXQ_DTYPE_BF16 && bits == 9 && exp_bits == 8 && rmode == MXQ_ROUND_NEAREST &&
+              allow_denorm && !saturate_normals && p.fmt.max_bits == 0x7F7F0000u))
+            return fail(MXQ_ERR_ARGUMENT, "%s: no closed form for this case", who);
+        for (int64_t i = 0; i < n; ++i)
+            store_from_float(out, dtype, i,
+                             mxq_quant_bf16_to_bfloat16_nearest(load_as_float(in, dtype, i), p.fmt.nan_from));
+        return MXQ_OK;
+    }
     const unsigned char* zone = kZone[p.zone_row];
     ElemFn fn = pick_elem(dtype, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode),
-                           lean_ok(dtype, p.fmt) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
+                           lean_ok(dtype, p.fmt, rmode, true) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < n; ++i)
         store_from_float(out, dtype, i,
                          fn(load_as_float(in, dtype, i), p.fmt, p.saturate != 0, p.allow_denorm != 0, zone, p.zshift));

@@ -78,6 +78,7 @@ inline int make_fmt(int dtype, int ebits, int mbits, float max_norm, MxqFmt* fmt
     fmt->half = dtype == MXQ_DTYPE_BF16 ? 0.5f + 0.001953125f : 0.5f;
     fmt->tie_fix = dtype == MXQ_DTYPE_BF16 ? 0.5f - 0.001953125f : 0.5f - 2.98023223876953125e-8f;
     fmt->nan_from = MXQ_INF_BITS;
+    fmt->bump_lo = (dtype == MXQ_DTYPE_BF16 && fmt->t >= 7) ? 128.0f : __builtin_inff();
     return MXQ_OK;
 }
 
@@ -94,8 +95,12 @@ inline void zone_for(int dtype, int flags, int* row, int* zshift) {
 }
 
 // May the lean element rounding be used (see mxq_round_lean)?  bf16 tensors with 7 or more
-// fraction bits need the op-by-op form: there "s + 0.5" itself ties in bf16.
-inline bool lean_ok(int dtype, const MxqFmt& f) { return dtype != MXQ_DTYPE_BF16 || f.t <= 6; }
+// fraction bits: the elementwise quantizer handles the one extra case of nearest mode (BUMP), floor
+// mode has none, torch's emulation of even mode has too many (op-by-op form).  MX element formats
+// never have more than 6 fraction bits.
+inline bool lean_ok(int dtype, const MxqFmt& f, int rmode, bool elementwise) {
+    return dtype != MXQ_DTYPE_BF16 || f.t <= 6 || (elementwise && rmode != MXQ_ROUND_EVEN);
+}
 
 // Does the round-up zone of the *element* exponent change results?  In nearest / even modes a
 // value in the zone rounds to the next power of two whichever exponent is used, as long as the

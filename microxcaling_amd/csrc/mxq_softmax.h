@@ -1,0 +1,114 @@
+// Softmax over the last axis with an elementwise quantization after every step
+// (mx/softmax.py:20-54 over mx/vector_ops.py:38-130): one kernel instead of ten tensor passes.
+#pragma once
+#include "mxq_kernels.h"
+
+struct SoftmaxParams {
+    ElemParams q;      // the elementwise format applied after every step
+    int exp_mode;      // 0: exp(x)   1: 2^x (softmax_exp2)   2: 2^Q(x * log2(e) at bfloat16 precision)
+    int use_recip;     // divide as e * Q(1 / sum) instead of e / sum (vec_use_recip)
+};
+
+namespace {
+
+// One wave per row; a lane keeps VPL 16-byte vectors of the row in registers from the load to the
+// store (vector j of lane l is vector 64 j + l of the row), so the row is read once and written
+// once.  QMODE: SMQ_GENERIC = the elementwise quantizer with the format in p.q; SMQ_IDENT = the
+// identity on values of the tensor dtype (no format configured, or bfloat16 with round-half-even on
+// a bf16 tensor); SMQ_BF16 = closed form for bf16 tensor -> bfloat16, round-half-away.
+// Every step rounds to the tensor dtype first, like the tensor op it stands for, then quantizes.
+enum { SMQ_GENERIC = 0, SMQ_IDENT = 1, SMQ_BF16 = 2 };
+
+template <int DT, int RMODE, int QMODE, int VPL>
+__global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict__ in_,
+                                                          void* __restrict__ out_, int64_t rows,
+                                                          int n, SoftmaxParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int EPV = 4 * PD;
+    constexpr int EPL = VPL * EPV;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.q.zone_row]);
+
+    auto Q = [&](float v) {
+        v = mxq_round_dt<ADT>(v);
+        if (QMODE == SMQ_IDENT) return v;
+        if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, p.q.fmt.nan_from);
+        return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
+                                                          p.q.allow_denorm != 0, zone, ZS);
+    };
+
+    const int lane = threadIdx.x & 63;
+    const int nvec = n / EPV;
+    const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
+    for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows; row += waves) {
+        const u32x4* in = reinterpret_cast<const u32x4*>(in_) + row * nvec;
+        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec;
+        u32x4 raw[VPL];
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const int v = j * 64 + lane;
+            if (v < nvec) raw[j] = in[v];
+        }
+        // positions past the end of the row behave like -inf: they drop out of the maximum and
+        // contribute exp(-inf) = 0 to the sum
+        float x[EPL];
+        float m = -__builtin_inff();
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const bool valid = j * 64 + lane < nvec;
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const int e = (j * 4 + d) * PD + h;
+                    x[e] = valid ? Q(Pack<DT>::get(raw[j][d], h)) : -__builtin_inff();
+                    m = MaxOp::apply(m, x[e]);                 // NaN sticks, like torch.max
+                }
+        }
+        m = wave_reduce<MaxOp>(m);
+
+        float sum = 0.0f;
+        if (p.exp_mode == 0) {                               // one loop per mode: no branch per element
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                x[e] = Q(expf(Q(x[e] - m)));
+                sum += x[e];
+            }
+        } else if (p.exp_mode == 1) {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                x[e] = Q(exp2f(Q(x[e] - m)));
+                sum += x[e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                x[e] = Q(exp2f(Q(1.4453125f * Q(x[e] - m))));
+                sum += x[e];
+            }
+        }
+        sum = Q(wave_reduce<SumOp>(sum));
+        const bool recip = p.use_recip != 0;
+        const float r = recip ? Q(1.0f / sum) : 0.0f;
+
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            u32x4 o;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                float q[2];
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const float e = x[(j * 4 + d) * PD + h];
+                    q[h] = Q(recip ? e * r : e / sum);
+                }
+                o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+            }
+            if (j * 64 + lane < nvec) __builtin_nontemporal_store(o, &out[j * 64 + lane]);
+        }
+    }
+}
+
+}  // namespace

@@ -37,6 +37,12 @@ def _quantize_elemwise_core(A, bits, exp_bits, max_norm, round='nearest',
                                        device=sp.device, requires_grad=sp.requires_grad)
 
     from . import custom_extensions
+    if not A.is_contiguous() and A.dim() >= 2 and A.transpose(-1, -2).is_contiguous():
+        # elementwise work does not care about the order of the axes: keep a transposed view
+        # transposed (a K-major operand of the fused GEMM stays K-major) instead of copying it
+        return _quantize_elemwise_core(A.transpose(-1, -2), bits, exp_bits, max_norm, round=round,
+                                       saturate_normals=saturate_normals, allow_denorm=allow_denorm,
+                                       custom_cuda=custom_cuda).transpose(-1, -2)
     A = A.contiguous()
     if A.device.type == "cuda":
         return custom_extensions.funcs.quantize_elemwise_func_cuda(
@@ -75,6 +81,34 @@ def _quantize_fp(A, exp_bits=None, mantissa_bits=None, round='nearest', custom_c
     return _quantize_elemwise_core(A, bits=mantissa_bits + 2, exp_bits=exp_bits,
                                    max_norm=_get_max_norm(exp_bits, mantissa_bits + 2),
                                    round=round, allow_denorm=allow_denorm, custom_cuda=custom_cuda)
+
+
+def elemwise_plan(mx_specs, round=None):
+    """What quantize_elemwise_op(., mx_specs, round) amounts to, without a tensor:
+    ("identity",), ("to_bf16",) or ("quantize", bits, exp_bits, max_norm, allow_denorm).  Raises the
+    same ValueErrors.  Used by fused kernels that apply the quantizer between their own steps."""
+    if mx_specs is None:
+        return ("identity",)
+    if round is None:
+        round = mx_specs['round']
+    if mx_specs['bfloat'] == 16 and round == 'even' and torch.cuda.is_bf16_supported() \
+            and mx_specs['bfloat_subnorms'] == True:
+        return ("to_bf16",)
+    if mx_specs['bfloat'] > 0 and mx_specs['fp'] > 0:
+        raise ValueError("Cannot set both [bfloat] and [fp] in mx_specs.")
+    if mx_specs['bfloat'] > 9:
+        b = mx_specs['bfloat']
+        if b == 32:
+            return ("identity",)
+        return ("quantize", b - 7, 8, _get_max_norm(8, b - 7), bool(mx_specs['bfloat_subnorms']))
+    if mx_specs['bfloat'] > 0:
+        raise ValueError("Cannot set [bfloat] <= 9 in mx_specs.")
+    if mx_specs['fp'] > 6:
+        m = mx_specs['fp'] - 6
+        return ("quantize", m + 2, 5, _get_max_norm(5, m + 2), bool(mx_specs['bfloat_subnorms']))
+    if mx_specs['fp'] > 0:
+        raise ValueError("Cannot set [fp] <= 6 in mx_specs.")
+    return ("identity",)
 
 
 def quantize_elemwise_op(A, mx_specs, round=None):

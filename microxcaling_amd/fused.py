@@ -65,10 +65,12 @@ def unpack_mx(codes, scales, codes_are_e5m2, dtype=torch.float32):
     return out
 
 
-def gemm_nt(a_packed, b_packed, out_dtype=torch.float32, bias=None):
+def gemm_nt(a_packed, b_packed, out_dtype=torch.float32, bias=None, epilogue_quant=False):
     """C[b] = A[b] x B[b]^T (+ bias).  a_packed / b_packed = (codes, scales, is_e5m2) with codes of
     shape (batch, M, K) / (batch, N, K) or (M, K) / (N, K); bias: (N,) of out_dtype, added after the
-    product has been rounded to out_dtype, the sum being rounded again."""
+    product has been rounded to out_dtype, the sum being rounded again.  epilogue_quant (bf16
+    output only): also apply the bfloat16 / round-half-away elementwise quantization after the
+    product and after the bias add."""
     who = "gemm_nt"
     (ac, asc, ae), (bc, bsc, be) = a_packed, b_packed
     for t, n in ((ac, "a codes"), (asc, "a scales"), (bc, "b codes"), (bsc, "b scales")):
@@ -88,12 +90,13 @@ def gemm_nt(a_packed, b_packed, out_dtype=torch.float32, bias=None):
     with torch.cuda.device(ac.device):
         rc = lib.mxq_gemm_mx_nt(ac.data_ptr(), asc.data_ptr(), int(ae), bc.data_ptr(),
                                 bsc.data_ptr(), int(be), None if bias is None else bias.data_ptr(),
-                                out.data_ptr(), _DTYPE[out_dtype], batch, M, N, K, _stream(ac))
+                                out.data_ptr(), _DTYPE[out_dtype], batch, M, N, K,
+                                int(bool(epilogue_quant)), _stream(ac))
     _lib.check(rc, lib)
     return out
 
 
-def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None):
+def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_quant=False):
     """a (..., M, K) x b_kmajor (N, K) or (..., N, K), both MX-quantized along K: the fused
     equivalent of quantize_mx_op(a, axes=[-1]) @ quantize_mx_op(b, axes=[-1]).T (+ bias, see
     gemm_nt).  Returns None when the operands do not qualify (the caller then takes the unfused
@@ -126,8 +129,10 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None):
         return None                                      # broadcast batch axes
     scale_bits = mx_specs["scale_bits"] if mx_specs["scale_bits"] != 0 else 8
     flush = mx_specs["mx_flush_fp32_subnorms"]
-    pa = pack_mx(a2, fa, scale_bits, round, flush)
-    pb = pack_mx(b2, fb, scale_bits, round, flush)
     if bias is not None and (bias.dtype != a.dtype or bias.dim() != 1):
         return None
-    return gemm_nt(pa, pb, out_dtype=a.dtype, bias=bias).reshape(out_shape)
+    if epilogue_quant and a.dtype != torch.bfloat16:
+        return None
+    pa = pack_mx(a2, fa, scale_bits, round, flush)
+    pb = pack_mx(b2, fb, scale_bits, round, flush)
+    return gemm_nt(pa, pb, out_dtype=a.dtype, bias=bias, epilogue_quant=epilogue_quant).reshape(out_shape)

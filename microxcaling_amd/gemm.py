@@ -25,22 +25,46 @@ def fused_enabled():
     return _use_fused
 
 
-def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None):
-    """a: (..., M, K); b_kmajor: (..., N, K) -- both contiguous along K.  Returns None when the
-    fused path does not apply."""
+def _epilogue_mode(mx_specs, round, dtype):
+    """How the layers' "elementwise-quantize the product (, add the bias, quantize again)" can ride
+    in the fused GEMM's epilogue: 0 = the quantizer is the identity (plain rounding to the tensor
+    dtype), 1 = bfloat16 with round-half-away on a bf16 tensor (closed form in the kernel),
+    None = neither, the caller runs the separate steps."""
+    from .elemwise_ops import elemwise_plan
+    from .formats import _get_max_norm
+    plan = elemwise_plan(mx_specs, round)
+    if plan[0] == "identity":
+        return 0
+    if plan == ("quantize", 9, 8, _get_max_norm(8, 9), True) and round == "nearest" \
+            and dtype == torch.bfloat16:
+        return 1
+    return None
+
+
+def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, out_round=None, bias=None):
+    """a: (..., M, K); b_kmajor: (..., N, K) -- both contiguous along K.  Returns (out, finished):
+    out is None when the fused path does not apply; finished says whether the output quantization
+    with rounding `out_round` and the bias add have been done in the epilogue."""
     if not _use_fused or not a.is_cuda:
-        return None
+        return None, False
     from . import fused
-    return fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=bias)
+    mode = _epilogue_mode(mx_specs, out_round, a.dtype) if out_round is not None else None
+    if mode is not None and (bias is None or bias.dtype == a.dtype):
+        out = fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=bias,
+                               epilogue_quant=mode == 1)
+        if out is not None:
+            return out, True
+    return fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round), False
 
 
-def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, fuse_bias=None):
+def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, out_round=None, bias=None):
     """x (..., K) times w (N, K) transposed: both operands share exponents along their last axis.
-    fuse_bias: a bias the caller would add right after the product with no quantization step in
-    between; returns (out, bias_was_added)."""
-    out = _try_fused(x, w, a_fmt, w_fmt, mx_specs, round, bias=fuse_bias)
+    out_round / bias: what the caller does next -- elementwise-quantize the product with that
+    rounding, add the (already quantized) bias, quantize again.  Returns (out, finished); when
+    finished, those steps have been done in the GEMM's epilogue."""
+    out, finished = _try_fused(x, w, a_fmt, w_fmt, mx_specs, round, out_round, bias)
     if out is not None:
-        return out, fuse_bias is not None
+        return out, finished
     qx = quantize_mx_op(x, mx_specs, elem_format=a_fmt, axes=[-1], round=round)
     qw = quantize_mx_op(w, mx_specs, elem_format=w_fmt, axes=[-1], round=round)
     # prequantized bf16 weights meet inputs of another dtype (mx/linear.py:77-80)
@@ -49,15 +73,16 @@ def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, fuse_bias=None):
     return torch.nn.functional.linear(qx, qw), False
 
 
-def mx_matmul_contract(a, b, a_fmt, b_fmt, mx_specs, round, batched=False):
-    """a (..., M, K) times b (..., K, N): a shares exponents along -1, b along -2."""
+def mx_matmul_contract(a, b, a_fmt, b_fmt, mx_specs, round, batched=False, out_round=None, bias=None):
+    """a (..., M, K) times b (..., K, N): a shares exponents along -1, b along -2.  out_round / bias
+    and the return value: as for mx_linear_contract."""
     if b.dim() >= 2 and a.dim() >= 2:
         # the fused kernel wants both operands K-major; a transposed view of b often already is
         bt = b.transpose(-1, -2)
         if bt.is_contiguous() and a.is_contiguous():
-            out = _try_fused(a, bt, a_fmt, b_fmt, mx_specs, round)
+            out, finished = _try_fused(a, bt, a_fmt, b_fmt, mx_specs, round, out_round, bias)
             if out is not None:
-                return out
+                return out, finished
     qa = quantize_mx_op(a, mx_specs, elem_format=a_fmt, axes=[-1], round=round)
     qb = quantize_mx_op(b, mx_specs, elem_format=b_fmt, axes=[-2], round=round)
-    return torch.bmm(qa, qb) if batched else torch.matmul(qa, qb)
+    return (torch.bmm(qa, qb) if batched else torch.matmul(qa, qb)), False

@@ -35,18 +35,17 @@ class LinearFunction(torch.autograd.Function):
         else:
             ctx.save_for_backward(input, weight)
 
-        # with no bfloat / fp quantization configured, "quantize, add bias, quantize" is a plain
-        # add in the tensor dtype, which the fused GEMM does in its epilogue
-        plain_add = bias is not None and mx_specs["bfloat"] == 0 and mx_specs["fp"] == 0 \
-            and bf_bias.dtype == bf_in.dtype
-        output, bias_added = mx_linear_contract(bf_in, bf_weight, mx_specs["a_elem_format"],
-                                                mx_specs["w_elem_format"], mx_specs,
-                                                mx_specs["round_mx_output"],
-                                                fuse_bias=bf_bias if plain_add else None)
-        output = quantize_elemwise_op(output, mx_specs=mx_specs, round=mx_specs["round_output"])
-        if bias is not None and not bias_added:
-            output = quantize_elemwise_op(output + bf_bias, mx_specs=mx_specs,
-                                          round=mx_specs["round_output"])
+        # the steps after the product -- quantize, add the bias, quantize -- ride in the fused
+        # GEMM's epilogue when the quantizer allows it (finished)
+        output, finished = mx_linear_contract(bf_in, bf_weight, mx_specs["a_elem_format"],
+                                              mx_specs["w_elem_format"], mx_specs,
+                                              mx_specs["round_mx_output"],
+                                              out_round=mx_specs["round_output"], bias=bf_bias)
+        if not finished:
+            output = quantize_elemwise_op(output, mx_specs=mx_specs, round=mx_specs["round_output"])
+            if bias is not None:
+                output = quantize_elemwise_op(output + bf_bias, mx_specs=mx_specs,
+                                              round=mx_specs["round_output"])
         ctx.mx_specs = get_backwards_mx_specs(mx_specs)
         ctx.prequantized_weights = prequantized_weights
         ctx.name = name

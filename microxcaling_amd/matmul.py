@@ -35,13 +35,15 @@ class MatMulFunction(torch.autograd.Function):
         else:
             ctx.save_for_backward(in1, in2)
 
-        out = mx_matmul_contract(bf_in1, bf_in2, _fmt(mx_specs, mode_config[0]),
-                                 _fmt(mx_specs, mode_config[1]), mx_specs,
-                                 mx_specs["round_mx_output"])
-        out = quantize_elemwise_op(out, mx_specs=mx_specs, round=mx_specs["round_output"])
-        if bias is not None:
-            out = quantize_elemwise_op(out + bf_bias, mx_specs=mx_specs,
-                                       round=mx_specs["round_output"])
+        out, finished = mx_matmul_contract(bf_in1, bf_in2, _fmt(mx_specs, mode_config[0]),
+                                           _fmt(mx_specs, mode_config[1]), mx_specs,
+                                           mx_specs["round_mx_output"],
+                                           out_round=mx_specs["round_output"], bias=bf_bias)
+        if not finished:
+            out = quantize_elemwise_op(out, mx_specs=mx_specs, round=mx_specs["round_output"])
+            if bias is not None:
+                out = quantize_elemwise_op(out + bf_bias, mx_specs=mx_specs,
+                                           round=mx_specs["round_output"])
         ctx.mx_specs = get_backwards_mx_specs(mx_specs)
         return out
 

@@ -10,6 +10,51 @@ from .vector_ops import (vec_div, vec_exp, vec_exp2, vec_mul, vec_quantize, vec_
 f_softmax = F.softmax
 LN_2_BF16 = 0.69140625           # ln(2) at bfloat16 precision
 
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
+MAX_FUSED_ROW = 4096
+
+
+def _fused_forward(input, dim, mx_specs):
+    """The whole forward chain as one kernel launch (mxq_softmax_lastdim), or None when the kernel
+    does not cover the case: CPU tensors, another axis than the last, rows longer than 4096 or not
+    a multiple of 16 bytes, fp16 tensors, round-half-even to a wide format on a bf16 tensor."""
+    from . import _lib, gemm
+    from .elemwise_ops import _native_round, elemwise_plan
+    if not (gemm.fused_enabled() and input.is_cuda and dim == input.dim() - 1):
+        return None
+    rnd = mx_specs['round']
+    plan = elemwise_plan(mx_specs, rnd)
+    if plan[0] == "to_bf16":
+        input = input.to(torch.bfloat16)       # the first quantization of the chain does this
+        plan = ("identity",)
+    if input.dtype not in _DTYPE_CODE:
+        return None
+    n = input.shape[-1]
+    if n == 0 or n > MAX_FUSED_ROW or n % (16 // input.element_size()) != 0:
+        return None
+    if plan[0] == "identity":
+        bits, exp_bits, max_norm, denorm, rmode = 0, 0, 1.0, True, 0
+    else:
+        _, bits, exp_bits, max_norm, denorm = plan
+        rmode = _native_round(rnd)
+        if input.dtype == torch.bfloat16 and bits >= 9 and rnd == 'even':
+            return None
+    if mx_specs.get('softmax_exp2', False):
+        exp_mode = 1
+    else:
+        exp_mode = 2 if mx_specs['vec_use_exp2'] else 0
+    x = input.contiguous()
+    out = torch.empty_like(x)
+    lib = _lib.gpu()
+    from .custom_extensions import _flags_value
+    with torch.cuda.device(x.device):
+        rc = lib.mxq_softmax_lastdim(x.data_ptr(), out.data_ptr(), _DTYPE_CODE[x.dtype],
+                                     x.numel() // n, n, bits, exp_bits, max_norm, rmode, int(denorm),
+                                     exp_mode, int(bool(mx_specs['vec_use_recip'])), _flags_value(),
+                                     torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, lib)
+    return out
+
 
 class SoftmaxFunction(torch.autograd.Function):
     """quantize -> max -> subtract -> exp (or 2^x) -> sum -> divide, re-quantizing after every
@@ -20,6 +65,11 @@ class SoftmaxFunction(torch.autograd.Function):
         dim = dim + len(input.shape) if dim < 0 else dim
         ctx.dim = dim
         rnd = mx_specs['round']
+        fused = _fused_forward(input, dim, mx_specs)
+        if fused is not None:
+            ctx.save_for_backward(fused)
+            ctx.mx_specs = get_backwards_mx_specs(mx_specs)
+            return fused
         input = vec_quantize(input, mx_specs=mx_specs)
         max_data, _ = input.max(dim, keepdim=True)
         input = vec_sub(input, max_data, mx_specs=mx_specs, round=rnd)

@@ -290,16 +290,23 @@ def mx_bmm_forward(a, b, fmt, block_size=32, scale_bits=8, bfloat=0, round="near
     return q(torch.bmm(qa, qb))
 
 
-def softmax_forward(x, dim, bfloat=16, round="nearest", use_exp2=False):
+def softmax_forward(x, dim, bfloat=16, round="nearest", use_exp2=False, vec_use_exp2=False,
+                    vec_use_recip=False, fp=0):
     """Forward of the bfloat softmax chain.  mx/softmax.py:20-54 over mx/vector_ops.py:38-130:
-    every step is a torch op followed by an elementwise quantization."""
-    q = lambda t: quantize_elemwise_op(t, bfloat=bfloat, round=round)
+    every step is a torch op followed by an elementwise quantization.  use_exp2 =
+    mx_specs['softmax_exp2'] (softmax.py:35-37); vec_use_exp2 / vec_use_recip: vector_ops.py:73-77,
+    59-62."""
+    q = lambda t: quantize_elemwise_op(t, bfloat=bfloat, fp=fp, round=round)
     x = q(x)
     mx = torch.max(x, dim, keepdim=True).values
     x = q(x - mx)
     if use_exp2:
         e = q(torch.exp2(x))
+    elif vec_use_exp2:
+        e = q(torch.exp2(q(1.4453125 * x)))
     else:
         e = q(torch.exp(x))
     s = q(e.sum(dim, keepdim=True))
+    if vec_use_recip:
+        return q(e * q(1.0 / s))
     return q(e / s)

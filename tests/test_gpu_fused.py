@@ -99,6 +99,31 @@ def test_gemm_16bit_outputs_equal_rounded_fp32_output(dev, M, N, K, batch, dtype
     assert got.dtype == dtype and torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
+@pytest.mark.parametrize("M,N,K,batch", [(128, 136, 256, 1), (600, 520, 1024, 2), (2050, 1800, 512, 3)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_gemm_epilogue_quantization_equals_separate_steps(dev, M, N, K, batch, with_bias):
+    """epilogue_quant: the bfloat16 / round-half-away quantization after the product and after the
+    bias add, done inside the GEMM, against the same steps done with the elementwise kernel
+    (itself bit-identical to the oracle) on the fp32 product -- bit for bit."""
+    from microxcaling_amd.fused import pack_mx, gemm_nt
+    from microxcaling_amd.elemwise_ops import _quantize_bfloat
+    g = torch.Generator().manual_seed(M + N + K + batch + 1)
+    sa = (batch, M, K) if batch > 1 else (M, K)
+    sb = (batch, N, K) if batch > 1 else (N, K)
+    pa = pack_mx((torch.randn(*sa, generator=g) * 7).to(dev), "fp8_e4m3")
+    pb = pack_mx(torch.randn(*sb, generator=g).to(dev), "fp6_e2m3")
+    bias = torch.randn(N, generator=g).to(dev).to(torch.bfloat16) if with_bias else None
+    want = _quantize_bfloat(gemm_nt(pa, pb, torch.float32).to(torch.bfloat16), 16, round="nearest")
+    if with_bias:
+        want = _quantize_bfloat(want + bias, 16, round="nearest")
+    got = gemm_nt(pa, pb, torch.bfloat16, bias=bias, epilogue_quant=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # the quantizer is not the identity on bf16: about half of the values must have moved
+    plain = gemm_nt(pa, pb, torch.bfloat16, bias=bias)
+    assert (plain != got).float().mean().item() > 0.2
+
+
 def test_gemm_propagates_nan_blocks(dev):
     from microxcaling_amd.fused import pack_mx, gemm_nt
     a = torch.randn(128, 128)
@@ -176,3 +201,79 @@ def test_linear_backward_runs(dev):
     lin(x).sum().backward()
     assert x.grad.shape == x.shape and lin.weight.grad.shape == lin.weight.shape
     assert torch.isfinite(x.grad).all()
+
+
+# ---- fused softmax kernel against the oracle's chain of tensor ops --------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(3, 5, 2048), (64, 1000), (7, 8), (2, 4096), (33, 264)])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, softmax_exp2=True),
+                                  dict(bfloat=16, vec_use_exp2=True, vec_use_recip=True),
+                                  dict(bfloat=16, round="floor"), dict(bfloat=16, round="even"),
+                                  dict(fp=16), dict(bfloat=12), dict(fp=10, round="even"),
+                                  dict(fp=16, round="even"), dict()])
+def test_fused_softmax_against_chain(dev, dtype, shape, spec):
+    """One-kernel softmax vs the reference's chain (max, sub, exp, sum, div, each followed by the
+    elementwise quantizer) on the CPU.  exp and the order of the row sum differ in the last bit
+    between the two, which the quantizer can turn into one step of the element format: tolerance
+    2^-8 absolute (one bf16 step at 1.0) and 1 % of the elements allowed to differ at all
+    (floor rounding: 3 %)."""
+    from microxcaling_amd.softmax import softmax, _fused_forward
+    from microxcaling_amd.specs import apply_mx_specs
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g) * 3).to(dtype)
+    x[0, ..., 3] = 9.5                                   # a clear maximum somewhere
+    specs = _specs(**spec)
+    if specs is not None:                                # the kernel is the path under test
+        bits = spec["bfloat"] - 7 if "bfloat" in spec else spec.get("fp", 11) - 4
+        unfusable = dtype == torch.bfloat16 and spec.get("round") == "even" and bits >= 9 \
+            and spec.get("bfloat") != 16
+        assert (_fused_forward(x.to(dev), x.dim() - 1, apply_mx_specs(specs)) is None) == unfusable
+    got = softmax(x.to(dev), dim=-1, mx_specs=specs).cpu()
+    want = O.softmax_forward(x, -1, bfloat=spec.get("bfloat", 0), fp=spec.get("fp", 0),
+                             round=spec.get("round", "nearest"), use_exp2=spec.get("softmax_exp2", False),
+                             vec_use_exp2=spec.get("vec_use_exp2", False),
+                             vec_use_recip=spec.get("vec_use_recip", False))
+    assert got.dtype == want.dtype and got.shape == want.shape
+    diff = (got.float() - want.float()).abs()
+    assert diff.max().item() <= 2.0 ** -8
+    if specs is None:                                    # the reference then calls torch's softmax
+        plain = torch.softmax(x, -1).float()
+        assert torch.allclose(got.float(), plain, rtol=2.0 ** -7 if dtype == torch.bfloat16 else 1e-5, atol=1e-9)
+        return
+    frac = (diff > 0).float().mean().item()
+    assert frac <= (0.03 if spec.get("round") == "floor" else 0.01), frac
+
+
+def test_fused_softmax_special_rows(dev):
+    """Rows holding -inf, +inf and NaN: -inf entries get weight 0; a row with +inf or NaN is NaN
+    throughout (inf - inf), exactly like the chain of tensor ops."""
+    from microxcaling_amd.softmax import softmax
+    x = torch.randn(6, 64)
+    x[1, 5] = float("-inf")
+    x[2, 7] = float("inf")
+    x[3, 9] = float("nan")
+    x[4, :] = float("-inf")
+    specs = _specs(bfloat=16)
+    got = softmax(x.to(dev), dim=-1, mx_specs=specs).cpu()
+    want = O.softmax_forward(x, -1, bfloat=16)
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    assert got[1, 5] == 0 and torch.isnan(got[2]).all() and torch.isnan(got[3]).all() and torch.isnan(got[4]).all()
+    ok = ~torch.isnan(want)
+    assert (got[ok] - want[ok]).abs().max() <= 2.0 ** -8
+
+
+def test_softmax_unfused_path_still_matches(dev):
+    from microxcaling_amd import gemm
+    from microxcaling_amd.softmax import softmax
+    x = torch.randn(16, 2048).to(torch.bfloat16)
+    specs = _specs(bfloat=16)
+    gemm.set_fused(False)
+    try:
+        a = softmax(x.to(dev), dim=-1, mx_specs=specs).cpu()
+    finally:
+        gemm.set_fused(True)
+    b = softmax(x.to(dev), dim=-1, mx_specs=specs).cpu()
+    assert (a.float() - b.float()).abs().max() <= 2.0 ** -8
+    # another axis than the last one is served by the separate steps
+    c = softmax(x.to(dev), dim=0, mx_specs=specs).cpu()
+    assert (c.float() - O.softmax_forward(x, 0, bfloat=16).float()).abs().max() <= 2.0 ** -8

@@ -123,7 +123,10 @@ def all_bf16():
 
 @pytest.mark.parametrize("bits,ebits,max_norm", [(9, 8, 2 ** 127 * 255 / 128), (12, 5, 65504.0),
                                                  (5, 4, 448.0), (4, 5, 57344.0), (3, 2, 6.0),
-                                                 (8, 0, 127 / 64), (5, 8, 2 ** 127 * 15 / 8)])
+                                                 (8, 0, 127 / 64), (5, 8, 2 ** 127 * 15 / 8),
+                                                 # more fraction bits than a bf16 tensor has
+                                                 (10, 8, 2 ** 127 * 255 / 128), (16, 8, 3.0e38),
+                                                 (9, 5, 65408.0), (10, 4, 480.0), (9, 0, 255 / 128)])
 @pytest.mark.parametrize("rnd", ROUNDS)
 def test_elementwise_every_bf16_code(bits, ebits, max_norm, rnd):
     x = all_bf16()
@@ -134,6 +137,25 @@ def test_elementwise_every_bf16_code(bits, ebits, max_norm, rnd):
             got = _quantize_elemwise_core(x.clone(), bits, ebits, max_norm, round=rnd,
                                           saturate_normals=sat, allow_denorm=den)
             assert_bits_equal(got, want, "sat=%s den=%s" % (sat, den))
+
+
+def test_closed_form_bf16_to_bfloat16_nearest_every_code():
+    """The closed form the fused softmax kernel uses for its commonest case (bf16 tensor, bfloat16,
+    round-half-away) against the op-by-op oracle on all 65536 bf16 codes."""
+    import ctypes
+    from microxcaling_amd import _lib
+    x = all_bf16().contiguous()
+    out = torch.empty_like(x)
+    lib = _lib.host()
+    max_norm = 2 ** 127 * 255 / 128
+    rc = lib.mxq_host_quantize_elemwise(x.data_ptr(), out.data_ptr(), 2, x.numel(), 9, 8, max_norm, 0, 0, 1, 4)
+    assert rc == 0, lib.mxq_host_last_error()
+    want = O.quantize_elemwise_core(x.clone(), 9, 8, max_norm, round="nearest",
+                                    saturate_normals=False, allow_denorm=True)
+    assert_bits_equal(out, want, "closed form")
+    # and it refuses what it does not cover
+    assert lib.mxq_host_quantize_elemwise(x.data_ptr(), out.data_ptr(), 2, x.numel(), 9, 8, max_norm, 2, 0, 1, 4) != 0
+    assert lib.mxq_host_quantize_elemwise(x.data_ptr(), out.data_ptr(), 2, x.numel(), 9, 8, 1000.0, 0, 0, 1, 4) != 0
 
 
 def fp32_probe_values():
