@@ -146,6 +146,8 @@ int mxq_probe_mfma_rate(int64_t workgroups, int iters, void* sink, void* hip_str
 #define MXQ_HOST_FLAG_ROUND_EVERY_OP 2 /* bf16: round to bf16 after every op, no shortcuts */
 #define MXQ_HOST_FLAG_CLOSED_FORM 4    /* elementwise, bf16 tensor -> bfloat16, nearest: the closed
                                           form the fused softmax kernel uses (else: an error) */
+#define MXQ_HOST_FLAG_CLOSED_FORM_NONNEG 8 /* with CLOSED_FORM: its variant for +0 <= x < 2^127,
+                                              +Inf and NaN (other inputs: unspecified) */
 
 const char* mxq_host_last_error(void);
 int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_values, int dtype,

@@ -276,6 +276,13 @@ MXQ_HD float mxq_quant_bf16_to_bfloat16_nearest(float x, uint32_t nan_from) {
     return mxq_float(r);
 }
 
+// The same closed form for values known to be >= +0, below 2^127, or NaN / +Inf (exponentials, their
+// sums and quotients): no sign of zero to fix and no top-binade zone to reach.
+MXQ_HD float mxq_quant_bf16_to_bfloat16_nearest_nonneg(float x) {
+    const uint32_t u = mxq_bits(x);
+    return mxq_float(u + ((u - 0x00800000u) < 0x7F000000u ? (u & 0x10000u) : 0u));   // finite normals only
+}
+
 // One element of the elementwise quantizer (mx/elemwise_ops.py:127-163).
 template <int RMODE, int DT, bool ZONE, bool LEAN>
 MXQ_HD float mxq_quant_elemwise(float x, const MxqFmt& f, bool saturate, bool allow_denorm,

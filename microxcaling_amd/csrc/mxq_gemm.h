@@ -220,6 +220,7 @@ __device__ __forceinline__ void store_c8(void* c, const void* bias, uint32_t q_n
 
 template <int CBSZ, int BLGP, int OUT_DT>
 __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
+    constexpr bool PAIR = OUT_DT != MXQ_F32;
     __shared__ __attribute__((aligned(16))) unsigned char As[GEMM_BM * GEMM_PITCH];
     __shared__ __attribute__((aligned(16))) unsigned char Bs[GEMM_BN * GEMM_PITCH];
     __shared__ __attribute__((aligned(16))) unsigned char sAs[GEMM_BM * 4];
@@ -298,7 +299,10 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
         int sb[4];
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) {
-            const int n = wx * 64 + tj * 16 + frow;
+            // 16-bit outputs: fragment rows permuted so that a lane owns 8 consecutive columns per
+            // fragment pair (see the 256 x 256 kernel)
+            const int n = wx * 64 + (PAIR ? (tj >> 1) * 32 + (frow >> 2) * 8 + (tj & 1) * 4 + (frow & 3)
+                                          : tj * 16 + frow);
             bf[tj] = load_frag(Bs + n * GEMM_PITCH + fg * 16);
             sb[tj] = sBs[n * 4 + fg];
         }
@@ -319,13 +323,23 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     }
 
     const int64_t cbase = bz * g.batch_c;
-    const bool inside = m0 + GEMM_BM <= g.M && n0 + GEMM_BN <= g.N && (g.N & 3) == 0;
+    const bool inside = m0 + GEMM_BM <= g.M && n0 + GEMM_BN <= g.N && (g.N & 3) == 0 &&
+                        ((uintptr_t)g.c & 15) == 0;
+    const bool inside8 = inside && (g.N & 7) == 0 && ((uintptr_t)g.bias & 15) == 0;
 #pragma unroll
     for (int ti = 0; ti < 4; ++ti)
 #pragma unroll
-        for (int tj = 0; tj < 4; ++tj)
-            store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m0 + wy * 64 + ti * 16 + frow, n0 + wx * 64 + tj * 16 + fg * 4,
-                             g.M, g.N, inside, acc[ti][tj]);
+        for (int tj = 0; tj < 4; ++tj) {
+            const int m = m0 + wy * 64 + ti * 16 + frow;
+            if constexpr (PAIR) {
+                if (tj & 1)
+                    store_c8<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, n0 + wx * 64 + (tj >> 1) * 32 + fg * 8,
+                                     g.M, g.N, inside8, acc[ti][tj - 1], acc[ti][tj]);
+            } else {
+                store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, n0 + wx * 64 + tj * 16 + fg * 4, g.M, g.N,
+                                 inside, acc[ti][tj]);
+            }
+        }
 }
 
 constexpr int G2_BM = 256, G2_BN = 256;

@@ -146,9 +146,12 @@ int mxq_host_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, 
         if (!(dtype == MXQ_DTYPE_BF16 && bits == 9 && exp_bits == 8 && rmode == MXQ_ROUND_NEAREST &&
               allow_denorm && !saturate_normals && p.fmt.max_bits == 0x7F7F0000u))
             return fail(MXQ_ERR_ARGUMENT, "%s: no closed form for this case", who);
-        for (int64_t i = 0; i < n; ++i)
-            store_from_float(out, dtype, i,
-                             mxq_quant_bf16_to_bfloat16_nearest(load_as_float(in, dtype, i), p.fmt.nan_from));
+        const bool nonneg = (flags & MXQ_HOST_FLAG_CLOSED_FORM_NONNEG) != 0;
+        for (int64_t i = 0; i < n; ++i) {
+            const float x = load_as_float(in, dtype, i);
+            store_from_float(out, dtype, i, nonneg ? mxq_quant_bf16_to_bfloat16_nearest_nonneg(x)
+                                                   : mxq_quant_bf16_to_bfloat16_nearest(x, p.fmt.nan_from));
+        }
         return MXQ_OK;
     }
     const unsigned char* zone = kZone[p.zone_row];

@@ -39,6 +39,13 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
                                                           p.q.allow_denorm != 0, zone, ZS);
     };
 
+    // the quantizer for exponentials, their row sum and the quotients: all >= +0 and <= 4096 (or
+    // NaN / +Inf), where the closed form needs no special cases
+    auto Qp = [&](float v) {
+        if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest_nonneg(mxq_round_dt<ADT>(v));
+        return Q(v);
+    };
+
     const int lane = threadIdx.x & 63;
     const int nvec = n / EPV;
     const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
@@ -73,25 +80,25 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
         if (p.exp_mode == 0) {                               // one loop per mode: no branch per element
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
-                x[e] = Q(expf(Q(x[e] - m)));
+                x[e] = Qp(expf(Q(x[e] - m)));
                 sum += x[e];
             }
         } else if (p.exp_mode == 1) {
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
-                x[e] = Q(exp2f(Q(x[e] - m)));
+                x[e] = Qp(exp2f(Q(x[e] - m)));
                 sum += x[e];
             }
         } else {
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
-                x[e] = Q(exp2f(Q(1.4453125f * Q(x[e] - m))));
+                x[e] = Qp(exp2f(Q(1.4453125f * Q(x[e] - m))));
                 sum += x[e];
             }
         }
-        sum = Q(wave_reduce<SumOp>(sum));
+        sum = Qp(wave_reduce<SumOp>(sum));
         const bool recip = p.use_recip != 0;
-        const float r = recip ? Q(1.0f / sum) : 0.0f;
+        const float r = recip ? Qp(1.0f / sum) : 0.0f;
 
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
@@ -102,7 +109,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
 #pragma unroll
                 for (int h = 0; h < PD; ++h) {
                     const float e = x[(j * 4 + d) * PD + h];
-                    q[h] = Q(recip ? e * r : e / sum);
+                    q[h] = Qp(recip ? e * r : e / sum);
                 }
                 o[d] = Pack<DT>::put(q[0], q[PD - 1]);
             }

@@ -153,6 +153,14 @@ def test_closed_form_bf16_to_bfloat16_nearest_every_code():
     want = O.quantize_elemwise_core(x.clone(), 9, 8, max_norm, round="nearest",
                                     saturate_normals=False, allow_denorm=True)
     assert_bits_equal(out, want, "closed form")
+    # the variant for exponentials, sums and quotients: +0 <= x < 2^127, +Inf, NaN
+    codes = torch.cat([torch.arange(0, 0x7F00), torch.arange(0x7F80, 0x8000)]).to(torch.int16)
+    xp = codes.view(torch.bfloat16).contiguous()
+    outp = torch.empty_like(xp)
+    rc = lib.mxq_host_quantize_elemwise(xp.data_ptr(), outp.data_ptr(), 2, xp.numel(), 9, 8, max_norm, 0, 0, 1, 4 | 8)
+    assert rc == 0, lib.mxq_host_last_error()
+    assert_bits_equal(outp, O.quantize_elemwise_core(xp.clone(), 9, 8, max_norm, round="nearest",
+                                                     saturate_normals=False, allow_denorm=True), "nonneg")
     # and it refuses what it does not cover
     assert lib.mxq_host_quantize_elemwise(x.data_ptr(), out.data_ptr(), 2, x.numel(), 9, 8, max_norm, 2, 0, 1, 4) != 0
     assert lib.mxq_host_quantize_elemwise(x.data_ptr(), out.data_ptr(), 2, x.numel(), 9, 8, 1000.0, 0, 0, 1, 4) != 0
