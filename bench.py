@@ -191,6 +191,16 @@ def cpu_baseline(wl, budget_s=15.0):
 MFMA_PEAK_TFLOPS = {"fp8": 5000.0}          # MI355X dense fp8 (e4m3 / e5m2 codes), published
 
 
+def measured_traffic(workload):
+    """HBM bytes per launch of the workload's dominant kernel, measured separately with
+    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (the summaries are in profiles/)."""
+    tfile = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
+    if not os.path.exists(tfile):
+        return None
+    with open(tfile) as f:
+        return json.load(f).get(workload)
+
+
 def report_flops(args, wl, ms_per_step, step_gpu_ms):
     """GEMM-shaped workloads: whole-step TFLOP/s (quantize + GEMM + epilogue ops all inside the
     step) against the dense fp8 MFMA peak."""
@@ -204,7 +214,7 @@ def report_flops(args, wl, ms_per_step, step_gpu_ms):
         "config": {"workload": args.workload, "detail": wl["desc"], "flop_per_step": wl["flops"]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_PEAK_TFLOPS["fp8"],
                      "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS["fp8"], 4),
-                     "traffic": None, "step_gpu_ms_avg": round(step_gpu_ms, 5),
+                     "traffic": measured_traffic(args.workload), "step_gpu_ms_avg": round(step_gpu_ms, 5),
                      "note": "whole forward step (all launches) over the dense fp8 MFMA peak"},
     }
     if not args.no_cpu_baseline:
@@ -269,11 +279,7 @@ def main():
     value = wl["bytes"] / (ms_per_step * 1e-3) / 1e9
     achieved = wl["bytes"] / (kern_avg_ms * 1e-3) / 1e9
 
-    traffic = None
-    tfile = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
-    if os.path.exists(tfile):
-        with open(tfile) as f:
-            traffic = json.load(f).get(args.workload)       # measured separately with rocprofv3 --pmc
+    traffic = measured_traffic(args.workload)
 
     out = {
         "metric": "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s",
