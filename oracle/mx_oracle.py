@@ -30,6 +30,13 @@ Parity status of every function here ("pinned" = checked against something other
                             62-67,84-112; exact-rational brute force; golden fixtures for bf16.
   * reduce_*_inner_dim      are torch.sum / torch.max themselves (the reference's own oracle,
                             mx/tests/test_reduce.py:17-20).
+  * mx_linear_forward / _backward, mx_bmm_forward / _backward, softmax_forward / _backward
+                            pinned (fp32 and bf16 tensors, bfloat 0 / 16, e^x and 2^x softmax):
+                            forward outputs and gradients written by the reference's own layers on
+                            the CPU (tests/golden/reference_layer_vectors.npz), reproduced bit for
+                            bit (tests/test_layer_golden.py).  The vec_use_exp2 / vec_use_recip
+                            variants of softmax_forward and the fp= formats are not in the
+                            fixtures: parity unpinned for those two switches.
 """
 import torch
 
@@ -310,3 +317,47 @@ def softmax_forward(x, dim, bfloat=16, round="nearest", use_exp2=False, vec_use_
     if vec_use_recip:
         return q(e * q(1.0 / s))
     return q(e / s)
+
+
+# ---- backward passes (mx_specs['quantize_backprop'] = True, one format / rounding throughout) ----
+def mx_linear_backward(x, w, grad_out, has_bias, fmt, block_size=32, scale_bits=8, bfloat=0,
+                       round="nearest"):
+    """Backward of the MX linear layer.  mx/linear.py:103-198: the saved tensors are the
+    elementwise-quantized input and weight (62-66); grad_weight contracts over the example axis
+    (both operands MX-quantized along axis -2, 124-150), grad_input over the output features
+    (weight along axis 0, grad_output along -1, 160-182), grad_bias is a plain sum (187-196).
+    Returns (grad_input, grad_weight, grad_bias)."""
+    q = lambda t: quantize_elemwise_op(t, bfloat=bfloat, round=round)
+    mxq = lambda t, ax: quantize_mx(t, scale_bits, fmt, axes=[ax], block_size=block_size, round=round)
+    bx, bw = q(x), q(w)
+    out_dim, in_dim = w.shape
+    go = q(grad_out)
+    qex_in = mxq(bx, -2).reshape(-1, in_dim)
+    qex_go = mxq(go, -2).reshape(-1, out_dim)
+    grad_w = q(torch.matmul(qex_go.transpose(0, 1), qex_in))
+    grad_in = q(torch.matmul(mxq(go, -1), mxq(bw, 0)))
+    grad_b = q(go.reshape(-1, out_dim).sum(0)) if has_bias else None
+    return grad_in, grad_w, grad_b
+
+
+def mx_bmm_backward(a, b, grad_out, fmt, block_size=32, scale_bits=8, bfloat=0, round="nearest"):
+    """Backward of MX bmm.  mx/bmm.py:69-127: in1 along -2 and in2 along -1 (the axes that are
+    contracted now), grad_out once along -1 and once along -2.  Returns (grad_in1, grad_in2)."""
+    q = lambda t: quantize_elemwise_op(t, bfloat=bfloat, round=round)
+    mxq = lambda t, ax: quantize_mx(t, scale_bits, fmt, axes=[ax], block_size=block_size, round=round)
+    ba, bb, go = q(a), q(b), q(grad_out)
+    g1 = q(torch.bmm(mxq(go, -1), mxq(bb, -1).transpose(-1, -2)))
+    g2 = q(torch.bmm(mxq(ba, -2).transpose(-1, -2), mxq(go, -2)))
+    return g1, g2
+
+
+def softmax_backward(out, grad_out, dim, bfloat=16, round="nearest", use_exp2=False):
+    """Backward of the bfloat softmax.  mx/softmax.py:56-88: out * (g - sum(g * out)), every op
+    followed by the elementwise quantizer; * ln2 at bfloat16 precision for the 2^x variant."""
+    q = lambda t: quantize_elemwise_op(t, bfloat=bfloat, round=round)
+    g = q(grad_out)
+    dot = q(q(g * out).sum(dim, keepdim=True))
+    gi = q(out * q(g - dot))
+    if use_exp2:
+        gi = q(gi * 0.69140625)
+    return gi

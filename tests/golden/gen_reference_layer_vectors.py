@@ -1,0 +1,85 @@
+"""Writes reference_layer_vectors.npz: forward outputs and gradients of the reference's MX layers
+(linear, bmm, softmax) on the CPU (``custom_cuda=False``), on small seeded inputs.  Run once, in a
+container where the reference checkout exists:
+``python tests/golden/gen_reference_layer_vectors.py /root/reference``.
+Only inputs and the reference's outputs are stored; none of the reference's code is.  The fixtures
+pin the order of the quantization steps inside the layers (oracle/mx_oracle.py: mx_linear_forward /
+_backward, mx_bmm_forward / _backward, softmax_forward / _backward), which no literal vector of the
+reference's own tests does."""
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def store(d, name, t):
+    t = t.detach()
+    if t.dtype == torch.bfloat16:
+        d[name + ":bf16"] = t.contiguous().view(torch.int16).numpy().copy()
+    else:
+        d[name + ":f32"] = t.contiguous().view(torch.int32).numpy().copy()
+
+
+def main(ref_root):
+    sys.path.insert(0, ref_root)
+    from mx.specs import finalize_mx_specs
+    from mx.linear import linear
+    from mx.bmm import bmm
+    from mx.softmax import softmax
+
+    torch.set_num_threads(1)                      # fixed summation order inside torch's CPU GEMM
+    d = {}
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(2, 32, 64, generator=g)
+    w = torch.randn(48, 64, generator=g) * 0.2
+    b = torch.randn(48, generator=g)
+    go = torch.randn(2, 32, 48, generator=g)
+    a2 = torch.randn(2, 64, 48, generator=g)
+    go2 = torch.randn(2, 32, 48, generator=g)
+    sx = torch.randn(4, 128, generator=g) * 2
+    sgo = torch.randn(4, 128, generator=g)
+    for name, t in (("x", x), ("w", w), ("b", b), ("go", go), ("a2", a2), ("go2", go2), ("sx", sx), ("sgo", sgo)):
+        store(d, "in/" + name, t)
+
+    for dt_name, dt in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+        for bfloat in (0, 16):
+            specs = finalize_mx_specs(dict(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32,
+                                           bfloat=bfloat, quantize_backprop=True, custom_cuda=False))
+            xi, wi, bi = (t.to(dt).clone().requires_grad_(True) for t in (x, w, b))
+            out = linear(xi, wi, bi, mx_specs=specs)
+            out.backward(go.to(dt))
+            key = "linear/%s/bfloat%d/" % (dt_name, bfloat)
+            store(d, key + "out", out)
+            store(d, key + "gx", xi.grad)
+            store(d, key + "gw", wi.grad)
+            store(d, key + "gb", bi.grad)
+
+        specs = finalize_mx_specs(dict(a_elem_format="fp6_e2m3", block_size=32, quantize_backprop=True,
+                                       custom_cuda=False))
+        ai, bi2 = x.to(dt).clone().requires_grad_(True), a2.to(dt).clone().requires_grad_(True)
+        out = bmm(ai, bi2, mx_specs=specs)
+        out.backward(go2.to(dt))
+        key = "bmm/%s/" % dt_name
+        store(d, key + "out", out)
+        store(d, key + "g1", ai.grad)
+        store(d, key + "g2", bi2.grad)
+
+        for exp2 in (False, True):
+            specs = finalize_mx_specs(dict(bfloat=16, softmax_exp2=exp2, quantize_backprop=True,
+                                           custom_cuda=False))
+            si = sx.to(dt).clone().requires_grad_(True)
+            out = softmax(si, dim=-1, mx_specs=specs)
+            out.backward(sgo.to(dt))
+            key = "softmax/%s/exp2_%d/" % (dt_name, int(exp2))
+            store(d, key + "out", out)
+            store(d, key + "gx", si.grad)
+
+    np.savez_compressed(os.path.join(HERE, "reference_layer_vectors.npz"), **d)
+    print("wrote %d arrays, torch %s" % (len(d), torch.__version__))
+
+
+if __name__ == "__main__":
+    main(sys.argv[1] if len(sys.argv) > 1 else "/root/reference")

@@ -277,3 +277,69 @@ def test_softmax_unfused_path_still_matches(dev):
     # another axis than the last one is served by the separate steps
     c = softmax(x.to(dev), dim=0, mx_specs=specs).cpu()
     assert (c.float() - O.softmax_forward(x, 0, bfloat=16).float()).abs().max() <= 2.0 ** -8
+
+
+# ---- backward passes against the oracle's restatement --------------------------------------------
+def _close(got, want, rel):
+    got, want = got.float().cpu(), want.float()
+    assert got.shape == want.shape
+    rms = want.pow(2).mean().sqrt().item() + 1e-30
+    assert (got - want).abs().max().item() <= rel * rms, ((got - want).abs().max().item(), rms)
+
+
+@pytest.mark.parametrize("dtype,rel", [(torch.float32, 1e-3), (torch.bfloat16, 4e-2)])
+@pytest.mark.parametrize("bfloat", [0, 16])
+def test_linear_backward_against_oracle(dev, dtype, rel, bfloat):
+    """grad_input / grad_weight / grad_bias of mx.Linear (MXFP8 e4m3 forward and backward) vs the
+    oracle's restatement of mx/linear.py:103-198 on the CPU.  The operands of every contraction are
+    bit-identical on both sides; fp32: only the summation order differs (1e-3 of the RMS);
+    bf16: the GEMM output is rounded to bf16, so one bf16 step of the largest entries (4e-2 RMS)."""
+    from microxcaling_amd.linear import linear
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(3, 64, 128, generator=g).to(dtype)
+    w = (torch.randn(96, 128, generator=g) * 0.1).to(dtype)
+    b = torch.randn(96, generator=g).to(dtype)
+    go = torch.randn(3, 64, 96, generator=g).to(dtype)
+    specs = _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32, bfloat=bfloat,
+                   quantize_backprop=True)
+    xd, wd, bd = (t.to(dev).requires_grad_(True) for t in (x, w, b))
+    out = linear(xd, wd, bd, mx_specs=specs)
+    out.backward(go.to(dev))
+    gi, gw, gb = O.mx_linear_backward(x, w, go, True, "fp8_e4m3", bfloat=bfloat)
+    _close(xd.grad, gi, rel)
+    _close(wd.grad, gw, rel)
+    _close(bd.grad, gb, rel)
+
+
+@pytest.mark.parametrize("dtype,rel", [(torch.float32, 1e-3), (torch.bfloat16, 4e-2)])
+def test_bmm_backward_against_oracle(dev, dtype, rel):
+    from microxcaling_amd.bmm import bmm
+    g = torch.Generator().manual_seed(22)
+    a = torch.randn(4, 64, 128, generator=g).to(dtype)
+    b = torch.randn(4, 128, 96, generator=g).to(dtype)
+    go = torch.randn(4, 64, 96, generator=g).to(dtype)
+    specs = _specs(a_elem_format="fp6_e2m3", block_size=32, quantize_backprop=True)
+    ad, bd = a.to(dev).requires_grad_(True), b.to(dev).requires_grad_(True)
+    bmm(ad, bd, mx_specs=specs).backward(go.to(dev))
+    g1, g2 = O.mx_bmm_backward(a, b, go, "fp6_e2m3")
+    _close(ad.grad, g1, rel)
+    _close(bd.grad, g2, rel)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("exp2", [False, True])
+def test_softmax_backward_against_oracle(dev, dtype, exp2):
+    """Backward of the bfloat16 softmax from the same saved output on both sides: only the order of
+    the row sum differs."""
+    from microxcaling_amd.softmax import softmax
+    g = torch.Generator().manual_seed(23)
+    x = (torch.randn(8, 256, generator=g) * 2).to(dtype)
+    go = torch.randn(8, 256, generator=g).to(dtype)
+    specs = _specs(bfloat=16, softmax_exp2=exp2, quantize_backprop=True)
+    xd = x.to(dev).requires_grad_(True)
+    out = softmax(xd, dim=-1, mx_specs=specs)
+    out.backward(go.to(dev))
+    want = O.softmax_backward(out.detach().cpu(), go, -1, bfloat=16, use_exp2=exp2)
+    diff = (xd.grad.float().cpu() - want.float()).abs()
+    assert diff.max().item() <= 2.0 ** -7 * want.float().abs().max().item()
+    assert (diff > 0).float().mean().item() < 0.02

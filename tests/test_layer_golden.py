@@ -1,0 +1,98 @@
+"""Forward outputs and gradients of the MX layers against fixtures written by the reference's own
+CPU path (tests/golden/gen_reference_layer_vectors.py): the oracle's restatements, and the
+package's layers on CPU tensors (host library quantizers + torch's GEMM).  Bit for bit -- same
+torch, same op order, single-threaded GEMM."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import ROOT_DIR, assert_bits_equal
+from oracle import mx_oracle as O
+
+FIX = np.load(os.path.join(ROOT_DIR, "tests", "golden", "reference_layer_vectors.npz"))
+
+
+def fx(name):
+    if name + ":bf16" in FIX:
+        return torch.from_numpy(FIX[name + ":bf16"].copy()).view(torch.bfloat16)
+    return torch.from_numpy(FIX[name + ":f32"].copy()).view(torch.float32)
+
+
+@pytest.fixture(autouse=True)
+def one_thread():
+    n = torch.get_num_threads()
+    torch.set_num_threads(1)
+    yield
+    torch.set_num_threads(n)
+
+
+DT = {"f32": torch.float32, "bf16": torch.bfloat16}
+
+
+def _specs(**kw):
+    from microxcaling_amd.specs import finalize_mx_specs
+    return finalize_mx_specs(dict(kw))
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("bfloat", [0, 16])
+def test_linear_oracle_and_cpu_layer(dt, bfloat):
+    x, w, b, go = (fx("in/" + n).to(DT[dt]) for n in ("x", "w", "b", "go"))
+    key = "linear/%s/bfloat%d/" % (dt, bfloat)
+    out = O.mx_linear_forward(x, w, b, "fp8_e4m3", "fp8_e4m3", bfloat=bfloat)
+    assert_bits_equal(out, fx(key + "out"), "oracle forward")
+    gi, gw, gb = O.mx_linear_backward(x, w, go, True, "fp8_e4m3", bfloat=bfloat)
+    assert_bits_equal(gi, fx(key + "gx"), "oracle grad_input")
+    assert_bits_equal(gw, fx(key + "gw"), "oracle grad_weight")
+    assert_bits_equal(gb, fx(key + "gb"), "oracle grad_bias")
+
+    from microxcaling_amd.linear import linear
+    specs = _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32, bfloat=bfloat,
+                   quantize_backprop=True)
+    xi, wi, bi = (t.clone().requires_grad_(True) for t in (x, w, b))
+    o = linear(xi, wi, bi, mx_specs=specs)
+    o.backward(go)
+    assert_bits_equal(o.detach(), fx(key + "out"), "layer forward")
+    assert_bits_equal(xi.grad, fx(key + "gx"), "layer grad_input")
+    assert_bits_equal(wi.grad, fx(key + "gw"), "layer grad_weight")
+    assert_bits_equal(bi.grad, fx(key + "gb"), "layer grad_bias")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_bmm_oracle_and_cpu_layer(dt):
+    a, b, go = (fx("in/" + n).to(DT[dt]) for n in ("x", "a2", "go2"))
+    key = "bmm/%s/" % dt
+    assert_bits_equal(O.mx_bmm_forward(a, b, "fp6_e2m3"), fx(key + "out"), "oracle forward")
+    g1, g2 = O.mx_bmm_backward(a, b, go, "fp6_e2m3")
+    assert_bits_equal(g1, fx(key + "g1"), "oracle grad_in1")
+    assert_bits_equal(g2, fx(key + "g2"), "oracle grad_in2")
+
+    from microxcaling_amd.bmm import bmm
+    specs = _specs(a_elem_format="fp6_e2m3", block_size=32, quantize_backprop=True)
+    ai, bi = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    o = bmm(ai, bi, mx_specs=specs)
+    o.backward(go)
+    assert_bits_equal(o.detach(), fx(key + "out"), "layer forward")
+    assert_bits_equal(ai.grad, fx(key + "g1"), "layer grad_in1")
+    assert_bits_equal(bi.grad, fx(key + "g2"), "layer grad_in2")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("exp2", [False, True])
+def test_softmax_oracle_and_cpu_layer(dt, exp2):
+    x, go = fx("in/sx").to(DT[dt]), fx("in/sgo").to(DT[dt])
+    key = "softmax/%s/exp2_%d/" % (dt, int(exp2))
+    out = O.softmax_forward(x, -1, bfloat=16, use_exp2=exp2)
+    assert_bits_equal(out, fx(key + "out"), "oracle forward")
+    assert_bits_equal(O.softmax_backward(out, go, -1, bfloat=16, use_exp2=exp2), fx(key + "gx"),
+                      "oracle backward")
+
+    from microxcaling_amd.softmax import softmax
+    specs = _specs(bfloat=16, softmax_exp2=exp2, quantize_backprop=True)
+    xi = x.clone().requires_grad_(True)
+    o = softmax(xi, dim=-1, mx_specs=specs)
+    o.backward(go)
+    assert_bits_equal(o.detach(), fx(key + "out"), "layer forward")
+    assert_bits_equal(xi.grad, fx(key + "gx"), "layer backward")
