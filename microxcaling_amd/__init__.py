@@ -9,3 +9,11 @@ from .specs import (MxSpecs, get_default_mx_specs, get_backwards_mx_specs, apply
 from .formats import ElemFormat, RoundingMode
 from .mx_ops import quantize_mx_op
 from .elemwise_ops import quantize_elemwise_op
+from .quantize import quantize_bfloat
+from .linear import Linear, linear
+from .matmul import matmul
+from .bmm import bmm
+from .softmax import Softmax, softmax
+from .layernorm import LayerNorm, RMSNorm, layer_norm
+from .activations import (sigmoid, tanh, relu, relu6, leaky_relu, silu, gelu,
+                          Sigmoid, Tanh, ReLU, ReLU6, LeakyReLU, SiLU, GELU)

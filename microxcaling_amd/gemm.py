@@ -12,6 +12,12 @@ import torch
 
 from .mx_ops import quantize_mx_op
 
+# the stock torch functions, taken now: inject_pyt_ops later rebinds the names in the torch
+# namespace to the MX versions, which end up here
+f_linear = torch.nn.functional.linear
+torch_matmul = torch.matmul
+torch_bmm = torch.bmm
+
 _use_fused = True
 
 
@@ -70,7 +76,7 @@ def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, out_round=None, bias
     # prequantized bf16 weights meet inputs of another dtype (mx/linear.py:77-80)
     if qw.dtype == torch.bfloat16 and qx.dtype != torch.bfloat16:
         qw = qw.to(qx.dtype)
-    return torch.nn.functional.linear(qx, qw), False
+    return f_linear(qx, qw), False
 
 
 def mx_matmul_contract(a, b, a_fmt, b_fmt, mx_specs, round, batched=False, out_round=None, bias=None):
@@ -85,4 +91,4 @@ def mx_matmul_contract(a, b, a_fmt, b_fmt, mx_specs, round, batched=False, out_r
                 return out, finished
     qa = quantize_mx_op(a, mx_specs, elem_format=a_fmt, axes=[-1], round=round)
     qb = quantize_mx_op(b, mx_specs, elem_format=b_fmt, axes=[-2], round=round)
-    return (torch.bmm(qa, qb) if batched else torch.matmul(qa, qb)), False
+    return (torch_bmm(qa, qb) if batched else torch_matmul(qa, qb)), False

@@ -1,0 +1,120 @@
+"""LayerNorm and RMSNorm over the last axis: same interface as the reference's mx/layernorm.py."""
+import torch
+import torch.nn.functional as F
+
+from .norm_utils import _norm_backward_LN, _norm_forward
+from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
+from .vector_ops import (vec_add, vec_mul, vec_quantize, vec_recip, vec_reduce_mean, vec_reduce_sum,
+                         vec_sqrt, vec_sub)
+
+torch_layer_norm = F.layer_norm
+
+
+def _leading_axes(t):
+    return list(range(t.ndim - 1))
+
+
+def _param_grads(grad_output, x_norm, specs):
+    """grad_bias = sum(g), grad_weight = sum(g * x_norm) over every axis but the last."""
+    axes = _leading_axes(grad_output)
+    grad_bias = vec_reduce_sum(grad_output, axes, mx_specs=specs)
+    grad_weight = vec_reduce_sum(vec_mul(grad_output, x_norm, mx_specs=specs), axes, mx_specs=specs)
+    return grad_weight, grad_bias
+
+
+class LayerNormFunction(torch.autograd.Function):
+    """mx/layernorm.py:17-69."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps, mx_specs=None, name=None):
+        ctx.eps = eps
+        x = vec_quantize(x, mx_specs=mx_specs)
+        bf_weight = vec_quantize(weight, mx_specs=mx_specs)
+        bf_bias = vec_quantize(bias, mx_specs=mx_specs)
+        output, _, x_norm, _, _, x_vare = _norm_forward(x, -1, bf_weight, bf_bias, eps, mx_specs)
+        ctx.save_for_backward(x_norm, x_vare, bf_weight if mx_specs['quantize_backprop'] else weight)
+        ctx.mx_specs = get_backwards_mx_specs(mx_specs)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x_norm, x_vare, weight = ctx.saved_tensors
+        s = ctx.mx_specs
+        grad_output = vec_quantize(grad_output, mx_specs=s)
+        grad_weight, grad_bias = _param_grads(grad_output, x_norm, s)
+        grad_input = _norm_backward_LN(grad_output, -1, weight, x_norm, x_vare, s)
+        return (grad_input, grad_weight, grad_bias, None, None, None)
+
+
+class RMSNormFunction(torch.autograd.Function):
+    """x / sqrt(mean(x^2) + eps) * weight + bias (mx/layernorm.py:100-168)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps, mx_specs=None, name=None):
+        ctx.eps = eps
+        s = mx_specs
+        x = vec_quantize(x, mx_specs=s)
+        ms = vec_reduce_mean(vec_mul(x, x, mx_specs=s), -1, keepdim=True, mx_specs=s)
+        rms_inv = vec_recip(vec_sqrt(vec_add(ms, eps, mx_specs=s), mx_specs=s), mx_specs=s)
+        x_norm = vec_mul(x, rms_inv, mx_specs=s)
+        bf_weight = vec_quantize(weight, mx_specs=s)
+        bf_bias = vec_quantize(bias, mx_specs=s)
+        output = vec_add(vec_mul(bf_weight, x_norm, mx_specs=s), bf_bias, mx_specs=s)
+        ctx.save_for_backward(x_norm, rms_inv, bf_weight if s['quantize_backprop'] else weight)
+        ctx.mx_specs = get_backwards_mx_specs(s)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x_norm, rms_inv, weight = ctx.saved_tensors
+        s = ctx.mx_specs
+        grad_output = vec_quantize(grad_output, mx_specs=s)
+        grad_weight, grad_bias = _param_grads(grad_output, x_norm, s)
+        dx1 = vec_mul(vec_mul(grad_output, weight, mx_specs=s), rms_inv, mx_specs=s)
+        proj = vec_reduce_mean(vec_mul(dx1, x_norm, mx_specs=s), -1, keepdim=True, mx_specs=s)
+        # the last subtraction carries no mx_specs in the reference (mx/layernorm.py:166): unquantized
+        grad_input = vec_sub(dx1, vec_mul(x_norm, proj, mx_specs=s))
+        return (grad_input, grad_weight, grad_bias, None, None, None)
+
+
+class _NormModule(torch.nn.LayerNorm):
+    """TF-style layer norm module (epsilon inside the square root)."""
+    _function = None
+    _plain_without_specs = True
+
+    def __init__(self, hidden_size, eps=1e-12, mx_specs=None, name=None):
+        mx_assert_test(mx_specs)
+        self.mx_none = mx_specs is None
+        self.name = name
+        self.mx_specs = apply_mx_specs(mx_specs)
+        super().__init__(normalized_shape=hidden_size, eps=eps)
+
+    def apply_mx_specs(self, mx_specs):
+        self.mx_none = mx_specs is None
+        self.mx_specs = apply_mx_specs(mx_specs)
+
+    def append_name(self, postfix):
+        self.name += postfix
+
+    def forward(self, x):
+        if self.mx_none and self._plain_without_specs:
+            return super().forward(x)
+        return self._function.apply(x, self.weight, self.bias, self.eps, self.mx_specs, self.name)
+
+
+class LayerNorm(_NormModule):
+    _function = LayerNormFunction
+
+
+class RMSNorm(_NormModule):
+    """torch has no RMSNorm to fall back to: always the vector-op chain (mx/layernorm.py:171-196)."""
+    _function = RMSNormFunction
+    _plain_without_specs = False
+
+
+def layer_norm(input, normalized_shape, weight, bias, eps=1e-12, mx_specs=None, name=None):
+    mx_assert_test(mx_specs)
+    if mx_specs is None:
+        return torch_layer_norm(input, normalized_shape, weight, bias, eps)
+    assert normalized_shape == weight.shape
+    return LayerNormFunction.apply(input, weight, bias, eps, apply_mx_specs(mx_specs), name)

@@ -8,6 +8,7 @@ from .mx_ops import quantize_mx_op
 from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
 
 f_linear = F.linear
+torch_matmul = torch.matmul      # the stock function: inject_pyt_ops rebinds torch.matmul later
 
 
 class LinearFunction(torch.autograd.Function):
@@ -65,7 +66,7 @@ class LinearFunction(torch.autograd.Function):
                               round=specs["round_mx_input_grad_weight"])
         q_go = quantize_mx_op(grad_output, specs, elem_format=specs["a_elem_format_bp_ex"],
                               axes=[-2], round=specs["round_mx_grad_output_grad_weight"])
-        grad_weight = torch.matmul(q_go.reshape(-1, out_dim).transpose(0, 1),
+        grad_weight = torch_matmul(q_go.reshape(-1, out_dim).transpose(0, 1),
                                    q_in.reshape(-1, in_dim))
         grad_weight = quantize_elemwise_op(grad_weight, mx_specs=specs,
                                            round=specs["round_grad_weight"])
@@ -75,7 +76,7 @@ class LinearFunction(torch.autograd.Function):
                              round=specs["round_mx_weight_grad_input"])
         q_go = quantize_mx_op(grad_output, specs, elem_format=specs["a_elem_format_bp_os"],
                               axes=[-1], round=specs["round_mx_grad_output_grad_input"])
-        grad_input = quantize_elemwise_op(torch.matmul(q_go, q_w), mx_specs=specs,
+        grad_input = quantize_elemwise_op(torch_matmul(q_go, q_w), mx_specs=specs,
                                           round=specs["round_grad_input"])
 
         grad_bias = None

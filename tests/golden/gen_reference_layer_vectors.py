@@ -1,5 +1,5 @@
 """Writes reference_layer_vectors.npz: forward outputs and gradients of the reference's MX layers
-(linear, bmm, softmax) on the CPU (``custom_cuda=False``), on small seeded inputs.  Run once, in a
+(linear, bmm, softmax, LayerNorm, RMSNorm, the activations) on the CPU (``custom_cuda=False``), on small seeded inputs.  Run once, in a
 container where the reference checkout exists:
 ``python tests/golden/gen_reference_layer_vectors.py /root/reference``.
 Only inputs and the reference's outputs are stored; none of the reference's code is.  The fixtures
@@ -76,6 +76,42 @@ def main(ref_root):
             key = "softmax/%s/exp2_%d/" % (dt_name, int(exp2))
             store(d, key + "out", out)
             store(d, key + "gx", si.grad)
+
+    # normalization layers and activations (bfloat16 vector-op chains)
+    from mx.layernorm import LayerNorm, RMSNorm
+    from mx import activations as act
+    nx = torch.randn(2, 16, 64, generator=g) * 2 + 0.5
+    nw = torch.randn(64, generator=g)
+    nb = torch.randn(64, generator=g)
+    ngo = torch.randn(2, 16, 64, generator=g)
+    for name, t in (("nx", nx), ("nw", nw), ("nb", nb), ("ngo", ngo)):
+        store(d, "in/" + name, t)
+    specs = finalize_mx_specs(dict(bfloat=16, quantize_backprop=True, custom_cuda=False))
+    for dt_name, dt in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+        for lname, cls in (("layernorm", LayerNorm), ("rmsnorm", RMSNorm)):
+            m = cls(64, eps=1e-5, mx_specs=specs).to(dt)
+            with torch.no_grad():
+                m.weight.copy_(nw.to(dt))
+                m.bias.copy_(nb.to(dt))
+            xi = nx.to(dt).clone().requires_grad_(True)
+            out = m(xi)
+            out.backward(ngo.to(dt))
+            key = "%s/%s/" % (lname, dt_name)
+            store(d, key + "out", out)
+            store(d, key + "gx", xi.grad)
+            store(d, key + "gw", m.weight.grad)
+            store(d, key + "gb", m.bias.grad)
+        acts = {"sigmoid": lambda t: act.sigmoid(t, mx_specs=specs), "tanh": lambda t: act.tanh(t, mx_specs=specs),
+                "relu": lambda t: act.relu(t, mx_specs=specs), "relu6": lambda t: act.relu6(t, mx_specs=specs),
+                "leaky_relu": lambda t: act.leaky_relu(t, 0.1, mx_specs=specs),
+                "silu": lambda t: act.silu(t, mx_specs=specs), "gelu": lambda t: act.gelu(t, mx_specs=specs),
+                "gelu1": lambda t: act.gelu(t, mx_specs=specs, first_order_gelu=True)}
+        for aname, fn in acts.items():
+            xi = (nx * 2).to(dt).clone().requires_grad_(True)
+            out = fn(xi)
+            out.backward(ngo.to(dt))
+            store(d, "act/%s/%s/out" % (aname, dt_name), out)
+            store(d, "act/%s/%s/gx" % (aname, dt_name), xi.grad)
 
     np.savez_compressed(os.path.join(HERE, "reference_layer_vectors.npz"), **d)
     print("wrote %d arrays, torch %s" % (len(d), torch.__version__))

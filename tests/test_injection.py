@@ -1,0 +1,72 @@
+"""inject_pyt_ops on a stock torch model: the residual MLP of the reference's
+examples/ffn_mx_auto.py (LayerNorm -> Linear -> GELU -> Linear, + residual), written with plain
+torch.nn / torch.nn.functional names.  Injection rewrites the global torch namespace, so each case
+runs in its own interpreter."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+from helpers import ROOT_DIR
+
+SCRIPT = r'''
+import sys
+sys.path.insert(0, %(root)r)
+import torch
+import torch.nn.functional as F
+from microxcaling_amd import finalize_mx_specs, mx_mapping, LayerNorm, Linear, gelu
+
+device = %(device)r
+specs = finalize_mx_specs({'w_elem_format': 'fp6_e3m2', 'a_elem_format': 'fp6_e3m2', 'block_size': 32,
+                           'bfloat': 16, 'custom_cuda': device == 'cuda', 'quantize_backprop': False})
+torch.manual_seed(3)
+H = 128
+x = torch.randn(16, H)
+
+# the same network written explicitly with the MX modules, before anything is injected
+ln, d1, d2 = LayerNorm(H, eps=1e-5, mx_specs=specs), Linear(H, 4 * H, mx_specs=specs), Linear(4 * H, H, mx_specs=specs)
+state = [p.detach().clone() for m in (ln, d1, d2) for p in m.parameters()]
+
+mx_mapping.inject_pyt_ops(specs)
+
+class ResidualMLP(torch.nn.Module):
+    def __init__(self, hidden):
+        super().__init__()
+        self.layernorm = torch.nn.LayerNorm(hidden, eps=1e-5)
+        self.dense_4h = torch.nn.Linear(hidden, 4 * hidden)
+        self.dense_h = torch.nn.Linear(4 * hidden, hidden)
+    def forward(self, inputs):
+        h = F.gelu(self.dense_4h(self.layernorm(inputs)))
+        return inputs + self.dense_h(h)
+
+mlp = ResidualMLP(H)
+assert type(mlp.layernorm).__name__ == 'LayerNorm_inj' and type(mlp.dense_h).__name__ == 'Linear_inj'
+with torch.no_grad():
+    for p, v in zip(mlp.parameters(), state):
+        p.copy_(v)
+mlp.to(device); ln.to(device); d1.to(device); d2.to(device)
+xd = x.to(device).requires_grad_(True)
+y = mlp(xd)
+y.sum().backward()
+want = x.to(device) + d2(gelu(d1(ln(x.to(device))), mx_specs=specs))
+assert y.shape == (16, H) and torch.isfinite(y).all() and xd.grad is not None
+assert torch.equal(y.detach(), want.detach()), (y - want).abs().max()
+print("OK", float(y.abs().mean()))
+'''
+
+
+def _run(device):
+    code = SCRIPT % {"root": ROOT_DIR, "device": device}
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0, res.stdout + res.stderr
+    assert "OK" in res.stdout
+
+
+def test_injected_ffn_on_cpu():
+    _run("cpu")
+
+
+@pytest.mark.gpu
+def test_injected_ffn_on_gpu():
+    _run("cuda")

@@ -96,3 +96,39 @@ def test_softmax_oracle_and_cpu_layer(dt, exp2):
     o.backward(go)
     assert_bits_equal(o.detach(), fx(key + "out"), "layer forward")
     assert_bits_equal(xi.grad, fx(key + "gx"), "layer backward")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("layer", ["layernorm", "rmsnorm"])
+def test_norm_layers_on_cpu(dt, layer):
+    from microxcaling_amd.layernorm import LayerNorm, RMSNorm
+    specs = _specs(bfloat=16, quantize_backprop=True)
+    m = {"layernorm": LayerNorm, "rmsnorm": RMSNorm}[layer](64, eps=1e-5, mx_specs=specs).to(DT[dt])
+    with torch.no_grad():
+        m.weight.copy_(fx("in/nw").to(DT[dt]))
+        m.bias.copy_(fx("in/nb").to(DT[dt]))
+    x = fx("in/nx").to(DT[dt]).clone().requires_grad_(True)
+    out = m(x)
+    out.backward(fx("in/ngo").to(DT[dt]))
+    key = "%s/%s/" % (layer, dt)
+    assert_bits_equal(out.detach(), fx(key + "out"), "forward")
+    assert_bits_equal(x.grad, fx(key + "gx"), "grad_input")
+    assert_bits_equal(m.weight.grad, fx(key + "gw"), "grad_weight")
+    assert_bits_equal(m.bias.grad, fx(key + "gb"), "grad_bias")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("name", ["sigmoid", "tanh", "relu", "relu6", "leaky_relu", "silu", "gelu", "gelu1"])
+def test_activations_on_cpu(dt, name):
+    from microxcaling_amd import activations as act
+    specs = _specs(bfloat=16, quantize_backprop=True)
+    fn = {"sigmoid": lambda t: act.sigmoid(t, mx_specs=specs), "tanh": lambda t: act.tanh(t, mx_specs=specs),
+          "relu": lambda t: act.relu(t, mx_specs=specs), "relu6": lambda t: act.relu6(t, mx_specs=specs),
+          "leaky_relu": lambda t: act.leaky_relu(t, 0.1, mx_specs=specs),
+          "silu": lambda t: act.silu(t, mx_specs=specs), "gelu": lambda t: act.gelu(t, mx_specs=specs),
+          "gelu1": lambda t: act.gelu(t, mx_specs=specs, first_order_gelu=True)}[name]
+    x = (fx("in/nx") * 2).to(DT[dt]).clone().requires_grad_(True)
+    out = fn(x)
+    out.backward(fx("in/ngo").to(DT[dt]))
+    assert_bits_equal(out.detach(), fx("act/%s/%s/out" % (name, dt)), "forward")
+    assert_bits_equal(x.grad, fx("act/%s/%s/gx" % (name, dt)), "backward")
