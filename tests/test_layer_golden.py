@@ -132,3 +132,124 @@ def test_activations_on_cpu(dt, name):
     out.backward(fx("in/ngo").to(DT[dt]))
     assert_bits_equal(out.detach(), fx("act/%s/%s/out" % (name, dt)), "forward")
     assert_bits_equal(x.grad, fx("act/%s/%s/gx" % (name, dt)), "backward")
+
+
+# ---- convolutions, batch / group norm, pooling, simd ops, LSTM (fp32, bfloat16 + MXFP8 specs) ----
+def _cspecs():
+    return _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32, bfloat=16,
+                  quantize_backprop=True)
+
+
+def _load_params(m, key):
+    with torch.no_grad():
+        for n, p in m.named_parameters():
+            p.copy_(fx(key + "p_" + n))
+
+
+def _check_module(key, m, x, go, params=True):
+    if params:
+        _load_params(m, key)
+    xi = x.clone().requires_grad_(True)
+    out = m(xi)
+    out.backward(go)
+    assert_bits_equal(out.detach(), fx(key + "out"), key + "out")
+    assert_bits_equal(xi.grad, fx(key + "gx"), key + "gx")
+    if params:
+        for n, p in m.named_parameters():
+            assert_bits_equal(p.grad, fx(key + "g_" + n), key + "g_" + n)
+
+
+def test_convolutions_on_cpu():
+    from microxcaling_amd.convolution import Conv1d, Conv2d
+    from microxcaling_amd.transpose_convolution import ConvTranspose2d
+    s = _cspecs()
+    cx = fx("in/cx")
+    _check_module("conv2d/", Conv2d(64, 48, 3, stride=2, padding=1, mx_specs=s), cx, fx("in/cgo"))
+    _check_module("conv2d_groups/", Conv2d(64, 64, 3, padding=1, groups=2, bias=False, mx_specs=s), cx,
+                  fx("in/cgo2"))
+    _check_module("conv1d/", Conv1d(32, 40, 5, padding=2, mx_specs=s), fx("in/c1"), fx("in/c1go"))
+    _check_module("convT2d/", ConvTranspose2d(64, 32, 3, stride=2, padding=1, output_padding=1, mx_specs=s),
+                  cx, fx("in/tgo"))
+
+
+def test_batch_and_group_norm_on_cpu():
+    from microxcaling_amd.batchnorm import BatchNorm2d
+    from microxcaling_amd.groupnorm import GroupNorm
+    s = _specs(bfloat=16, quantize_backprop=True)
+    cx, go = fx("in/cx"), fx("in/bgo")
+    bn = BatchNorm2d(64, mx_specs=s)
+    _check_module("bn_train/", bn, cx, go)
+    assert_bits_equal(bn.running_mean, fx("bn_train/running_mean"), "running_mean")
+    assert_bits_equal(bn.running_var, fx("bn_train/running_var"), "running_var")
+    bn.eval()
+    _check_module("bn_eval/", bn, cx, go, params=False)
+    _check_module("gn/", GroupNorm(4, 64, mx_specs=s), cx, go)
+
+
+def test_adaptive_avg_pool_on_cpu():
+    from microxcaling_amd.adaptive_avg_pooling import adaptive_avg_pool2d
+    s = _specs(bfloat=16, quantize_backprop=True)
+    x = fx("in/cx").clone().requires_grad_(True)
+    out = adaptive_avg_pool2d(x, (2, 3), mx_specs=s)
+    out.backward(fx("in/pgo"))
+    assert_bits_equal(out.detach(), fx("pool/out"), "out")
+    assert_bits_equal(x.grad, fx("pool/gx"), "gx")
+
+
+def test_simd_ops_on_cpu():
+    from microxcaling_amd import simd_ops as so
+    s = _specs(bfloat=16, quantize_backprop=True)
+    sa, sb, go = fx("in/sa"), fx("in/sb"), fx("in/ssgo")
+    for name, fn in {"add": so.simd_add, "sub": so.simd_sub, "mul": so.simd_mul, "div": so.simd_div}.items():
+        a, b = sa.clone().requires_grad_(True), sb.clone().requires_grad_(True)
+        out = fn(a, b, mx_specs=s)
+        out.backward(go)
+        assert_bits_equal(out.detach(), fx("simd/%s/out" % name), name)
+        assert_bits_equal(a.grad, fx("simd/%s/g1" % name), name + " g1")
+        assert_bits_equal(b.grad, fx("simd/%s/g2" % name), name + " g2")
+        a = sa.clone().requires_grad_(True)
+        out = fn(a, 1.7, mx_specs=s)
+        out.backward(go)
+        assert_bits_equal(out.detach(), fx("simd/%s_const/out" % name), name + " const")
+        assert_bits_equal(a.grad, fx("simd/%s_const/g1" % name), name + " const g1")
+    for name, fn in {"square": so.simd_square, "sqrt": so.simd_sqrt, "exp": so.simd_exp, "log": so.simd_log}.items():
+        a = (sa.abs() + 0.1).clone().requires_grad_(True)
+        out = fn(a, mx_specs=s)
+        out.backward(go)
+        assert_bits_equal(out.detach(), fx("simd/%s/out" % name), name)
+        assert_bits_equal(a.grad, fx("simd/%s/g1" % name), name + " g1")
+    a = sa.clone().requires_grad_(True)
+    out = so.simd_reduce_sum(a, [0, 2], mx_specs=s)
+    out.backward(torch.ones_like(out) * 0.37)
+    assert_bits_equal(out.detach(), fx("simd/reduce_sum/out"), "reduce_sum")
+    assert_bits_equal(a.grad, fx("simd/reduce_sum/g1"), "reduce_sum g1")
+    a = sa.clone().requires_grad_(True)
+    out = so.simd_reduce_mean(a, -1, keepdim=True, mx_specs=s)
+    out.backward(torch.ones_like(out) * 0.37)
+    assert_bits_equal(out.detach(), fx("simd/reduce_mean/out"), "reduce_mean")
+    assert_bits_equal(a.grad, fx("simd/reduce_mean/g1"), "reduce_mean g1")
+    a = sa.clone().requires_grad_(True)
+    out = so.simd_norm(a, mx_specs=s)
+    out.backward()
+    assert_bits_equal(out.detach(), fx("simd/norm/out"), "norm")
+    assert_bits_equal(a.grad, fx("simd/norm/g1"), "norm g1")
+
+
+def test_lstm_on_cpu():
+    from torch.nn.utils.rnn import pack_padded_sequence
+    from microxcaling_amd.rnn import LSTM
+    m = LSTM(32, 64, num_layers=2, bidirectional=True, mx_specs=_cspecs())
+    _load_params(m, "lstm/")
+    x = fx("in/lx").clone().requires_grad_(True)
+    out, (hn, cn) = m(x)
+    (out * fx("in/lgo")).sum().backward()
+    assert_bits_equal(out.detach(), fx("lstm/out"), "out")
+    assert_bits_equal(hn.detach(), fx("lstm/hn"), "hn")
+    assert_bits_equal(cn.detach(), fx("lstm/cn"), "cn")
+    assert_bits_equal(x.grad, fx("lstm/gx"), "gx")
+    for n, p in m.named_parameters():
+        assert_bits_equal(p.grad, fx("lstm/g_" + n), "g_" + n)
+    outp, (hn, cn) = m(pack_padded_sequence(fx("in/lx"), [5, 3, 2]))
+    assert_bits_equal(outp.data.detach(), fx("lstm_packed/out"), "packed out")
+    assert_bits_equal(hn.detach(), fx("lstm_packed/hn"), "packed hn")
+    assert_bits_equal(cn.detach(), fx("lstm_packed/cn"), "packed cn")
