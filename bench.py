@@ -150,6 +150,41 @@ def make_workload(name):
                     dtype="fp6_e2m3 x fp6_e2m3 -> f32 acc", sample_axis=0, cpu_rows=8, launches=20,
                     desc="mx.bmm Q.K^T bf16 [128,2048,128] MXFP6 e2m3 along head_dim + bfloat16 softmax, %s"
                          % ("packed codes + scaled-MFMA GEMM" if fused else "fake-quantize + torch.bmm"))
+    if name in ("softmax_bf16", "softmax_bf16_unfused", "layernorm_bf16", "layernorm_bf16_unfused"):
+        # the fused row kernels on their own: bfloat16 softmax over [128*2048, 2048] (the logits of
+        # config 5) and bfloat16 LayerNorm over [32768, 4096]
+        from microxcaling_amd import gemm
+        from microxcaling_amd.layernorm import LayerNorm
+        from microxcaling_amd.softmax import softmax
+        from microxcaling_amd.specs import finalize_mx_specs
+        specs = finalize_mx_specs({"bfloat": 16})
+        fused = not name.endswith("unfused")
+        g = torch.Generator().manual_seed(6)
+        if name.startswith("softmax"):
+            x = (torch.randn(16384, 2048, generator=g) * 3).to(torch.bfloat16).repeat(16, 1)
+            per_elem, what = 4, "softmax over the last axis, bf16 [262144,2048]"
+
+            def run(xd):
+                gemm.set_fused(fused)
+                return softmax(xd, dim=-1, mx_specs=specs)
+            cpu = lambda t: O.softmax_forward(t, -1, bfloat=16)
+        else:
+            x = (torch.randn(32768, 4096, generator=g) * 2 + 0.5).to(torch.bfloat16)
+            per_elem, what = 6, "LayerNorm (output + saved normalized input), bf16 [32768,4096]"
+            ln = {}
+
+            def run(xd):
+                if "m" not in ln:
+                    ln["m"] = LayerNorm(4096, eps=1e-5, mx_specs=specs).to(torch.bfloat16).to(xd.device)
+                gemm.set_fused(fused)
+                with torch.no_grad():
+                    return ln["m"](xd)
+            cpu_ln = LayerNorm(4096, eps=1e-5, mx_specs=specs).to(torch.bfloat16)
+            cpu = lambda t: cpu_ln(t)
+        return dict(x=x, gpu=run, cpu=cpu, bytes=x.numel() * per_elem, dtype="bf16", sample_axis=0,
+                    launches=1 if fused else 12,
+                    desc="%s, bfloat16 quantization after every step, %s" % (what, "one kernel" if fused else
+                                                                             "separate tensor passes"))
     if name == "copy_fp32_8192":
         # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         x = torch.randn(8192, 8192, generator=torch.Generator().manual_seed(0))

@@ -108,6 +108,19 @@ int mxq_softmax_lastdim(const void* in, void* out, int dtype, int64_t rows, int6
                         int exp_bits, float max_norm, int rmode, int allow_denorm, int exp_mode,
                         int use_recip, int flags, void* hip_stream);
 
+/* LayerNormFunction.forward / RMSNormFunction.forward (mx/layernorm.py:17-45, 100-131, over
+ * mx/norm_utils.py:25-114) for the last axis of a contiguous (rows, n) fp32 or bf16 tensor, as one
+ * kernel, with the elementwise quantizer (bits / exp_bits / max_norm as in mxq_softmax_lastdim,
+ * bits == 0: none) after every step.  weight, bias: n values of the tensor dtype, already quantized.
+ * out: (rows, n).  x_norm (may be NULL): (rows, n), the normalized input the layer saves for its
+ * backward pass.  row_stat: rows values, var + eps (LayerNorm) or 1 / rms (RMSNorm), also saved.
+ * n: multiple of 16 bytes worth of elements, at most 4096.  Agrees with the reference's chain of
+ * tensor ops up to the order of the two row sums. */
+int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void* out, void* x_norm,
+                     void* row_stat, int dtype, int64_t rows, int64_t n, float eps, int rms_norm,
+                     int bits, int exp_bits, float max_norm, int rmode, int allow_denorm, int flags,
+                     void* hip_stream);
+
 /* ---- packed MX tensors and the fused GEMM (no counterpart in the reference, which only ever
  * fake-quantizes and then calls a dense GEMM: mx/linear.py:62-86, mx/bmm.py:40-59) ---------------
  * Packed form of a (rows, K) tensor quantized along K in blocks of 32:

@@ -361,6 +361,60 @@ int mxq_softmax_lastdim(const void* in, void* out, int dtype, int64_t rows, int6
     return check_launch(who);
 }
 
+int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void* out, void* x_norm,
+                     void* row_stat, int dtype, int64_t rows, int64_t n, float eps, int rms_norm,
+                     int bits, int exp_bits, float max_norm, int rmode, int allow_denorm, int flags,
+                     void* hip_stream) {
+    const char* who = "mxq_norm_lastdim";
+    NormParams p;
+    const bool ident = bits == 0;
+    if (dtype != MXQ_DTYPE_F32 && dtype != MXQ_DTYPE_BF16)
+        return fail(MXQ_ERR_ARGUMENT, "%s: dtype code %d (fp32 and bf16 tensors only)", who, dtype);
+    int rc = make_elem_params(dtype, ident ? 9 : bits, ident ? 8 : exp_bits, ident ? 1.0f : max_norm,
+                              ident ? MXQ_ROUND_NEAREST : rmode, 0, allow_denorm, flags, &p.q, who);
+    if (rc) return rc;
+    if (!ident && !lean_ok(dtype, p.q.fmt, rmode, true))
+        return fail(MXQ_ERR_ARGUMENT, "%s: round-half-even to %d fraction bits on a bf16 tensor is "
+                    "only available through the separate elementwise steps", who, p.q.fmt.t);
+    p.eps = eps;
+    p.rms = rms_norm ? 1 : 0;
+    const int epv = dtype == MXQ_DTYPE_F32 ? 4 : 8;
+    if (rows < 0 || n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (n > 4096 || n % epv != 0)
+        return fail(MXQ_ERR_ARGUMENT, "%s: row length %lld must be a multiple of %d and at most 4096",
+                    who, (long long)n, epv);
+    if (rows == 0 || n == 0) return MXQ_OK;
+    if (!in || !out || !weight || !bias || !row_stat) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(in) || !aligned16(out) || !aligned16(weight) || !aligned16(bias) || !aligned16(x_norm))
+        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int grid = grid_for(ceil_div(rows, kThreads / 64));
+    const int64_t nvec = n / epv;
+    const bool closed = !ident && dtype == MXQ_DTYPE_BF16 && bits == 9 && exp_bits == 8 &&
+                        rmode == MXQ_ROUND_NEAREST && allow_denorm && p.q.fmt.max_bits == 0x7F7F0000u;
+#define MXQ_NM(DT, RM, QM)                                                                         \
+    do {                                                                                           \
+        constexpr int V = (DT == MXQ_F32) ? 2 : 1;                                                 \
+        if (nvec <= 128 * V) norm_row_kernel<DT, RM, QM, 2 * V><<<grid, kThreads, 0, s>>>(in, weight, bias, out, x_norm, row_stat, rows, (int)n, p);      \
+        else if (nvec <= 256 * V) norm_row_kernel<DT, RM, QM, 4 * V><<<grid, kThreads, 0, s>>>(in, weight, bias, out, x_norm, row_stat, rows, (int)n, p); \
+        else norm_row_kernel<DT, RM, QM, 8 * V><<<grid, kThreads, 0, s>>>(in, weight, bias, out, x_norm, row_stat, rows, (int)n, p);                     \
+    } while (0)
+    if (dtype == MXQ_DTYPE_F32) {
+        if (ident) MXQ_NM(MXQ_F32, MXQ_NEAREST, SMQ_IDENT);
+        else if (rmode == MXQ_ROUND_FLOOR) MXQ_NM(MXQ_F32, MXQ_FLOOR, SMQ_GENERIC);
+        else if (rmode == MXQ_ROUND_NEAREST) MXQ_NM(MXQ_F32, MXQ_NEAREST, SMQ_GENERIC);
+        else MXQ_NM(MXQ_F32, MXQ_EVEN, SMQ_GENERIC);
+    } else {
+        if (ident) MXQ_NM(MXQ_BF16, MXQ_NEAREST, SMQ_IDENT);
+        else if (closed) MXQ_NM(MXQ_BF16, MXQ_NEAREST, SMQ_BF16);
+        else if (rmode == MXQ_ROUND_FLOOR) MXQ_NM(MXQ_BF16, MXQ_FLOOR, SMQ_GENERIC);
+        else if (rmode == MXQ_ROUND_NEAREST) MXQ_NM(MXQ_BF16, MXQ_NEAREST, SMQ_GENERIC);
+        else MXQ_NM(MXQ_BF16, MXQ_EVEN, SMQ_GENERIC);
+    }
+#undef MXQ_NM
+    return check_launch(who);
+}
+
 int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t rows, int64_t K,
                 int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
                 int flush_fp32_subnorms, int rmode, int flags, void* hip_stream) {

@@ -119,3 +119,113 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
 }
 
 }  // namespace
+
+// ================================================================================================
+// LayerNorm / RMSNorm over the last axis with the elementwise quantizer after every step
+// (mx/norm_utils.py:25-114 with axes = -1, mx/layernorm.py:100-131): one kernel instead of about
+// fifteen tensor passes.  Same work mapping as the softmax kernel.  Besides the output it writes
+// what the backward pass of the layer keeps: the normalized input (optional) and one statistic per
+// row (LayerNorm: var + eps; RMSNorm: 1 / rms).
+//   LayerNorm: mean = Q(Q(sum x) / n); d = Q(x - mean); var = Q(Q(sum Q(d d)) / n);
+//              v = Q(var + eps); r = Q(1 / Q(sqrt v)); z = Q(d r); out = Q(Q(w z) + b)
+//   RMSNorm:   ms = Q(Q(sum Q(x x)) / n); v = Q(ms + eps); r = Q(1 / Q(sqrt v)); z = Q(x r); same out
+// weight and bias are already quantized.
+// ================================================================================================
+struct NormParams {
+    ElemParams q;
+    float eps;
+    int rms;           // 1: RMSNorm
+};
+
+namespace {
+
+template <int DT, int RMODE, int QMODE, int VPL>
+__global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ in_,
+                                                       const void* __restrict__ weight_,
+                                                       const void* __restrict__ bias_,
+                                                       void* __restrict__ out_, void* __restrict__ znorm_,
+                                                       void* __restrict__ stat_, int64_t rows, int n,
+                                                       NormParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int EPV = 4 * PD;
+    constexpr int EPL = VPL * EPV;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.q.zone_row]);
+
+    auto Q = [&](float v) {
+        v = mxq_round_dt<ADT>(v);
+        if (QMODE == SMQ_IDENT) return v;
+        if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, p.q.fmt.nan_from);
+        return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
+                                                          p.q.allow_denorm != 0, zone, ZS);
+    };
+
+    const int lane = threadIdx.x & 63;
+    const int nvec = n / EPV;
+    const float count = (float)n;
+    const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
+    for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows; row += waves) {
+        const u32x4* in = reinterpret_cast<const u32x4*>(in_) + row * nvec;
+        float x[EPL];
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const bool valid = j * 64 + lane < nvec;
+            u32x4 raw = {0, 0, 0, 0};
+            if (valid) raw = in[j * 64 + lane];
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const int e = (j * 4 + d) * PD + h;
+                    x[e] = valid ? Q(Pack<DT>::get(raw[d], h)) : 0.0f;    // zeros add nothing to the sums
+                    sum += p.rms ? 0.0f : x[e];
+                }
+        }
+        if (!p.rms) {
+            const float mean = Q(Q(wave_reduce<SumOp>(sum)) / count);
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) {
+                const bool valid = j * 64 + lane < nvec;
+#pragma unroll
+                for (int k = 0; k < EPV; ++k) x[j * EPV + k] = valid ? Q(x[j * EPV + k] - mean) : 0.0f;
+            }
+        }
+        float sq = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) sq += Q(x[e] * x[e]);
+        const float var = Q(Q(wave_reduce<SumOp>(sq)) / count);
+        const float vare = Q(var + p.eps);
+        const float rinv = Q(1.0f / Q(sqrtf(vare)));
+        if (lane == 0) store_scalar<DT>(stat_, row, p.rms ? rinv : vare);
+
+        const u32x4* wv = reinterpret_cast<const u32x4*>(weight_);
+        const u32x4* bv = reinterpret_cast<const u32x4*>(bias_);
+        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec;
+        u32x4* zn = znorm_ ? reinterpret_cast<u32x4*>(znorm_) + row * nvec : nullptr;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const int v = j * 64 + lane;
+            if (v >= nvec) continue;
+            const u32x4 w4 = wv[v], b4 = bv[v];
+            u32x4 o, z4;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                float q[2], z[2];
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    z[h] = Q(x[(j * 4 + d) * PD + h] * rinv);
+                    q[h] = Q(Q(Pack<DT>::get(w4[d], h) * z[h]) + Pack<DT>::get(b4[d], h));
+                }
+                o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+                z4[d] = Pack<DT>::put(z[0], z[PD - 1]);
+            }
+            __builtin_nontemporal_store(o, &out[v]);
+            if (zn) __builtin_nontemporal_store(z4, &zn[v]);
+        }
+    }
+}
+
+}  // namespace

@@ -10,6 +10,51 @@ from .vector_ops import (vec_add, vec_mul, vec_quantize, vec_recip, vec_reduce_m
 torch_layer_norm = F.layer_norm
 
 
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
+MAX_FUSED_ROW = 4096
+
+
+def _fused_forward(x, bf_weight, bf_bias, eps, mx_specs, rms):
+    """The forward chain as one kernel launch (mxq_norm_lastdim): returns (output, x_norm, row
+    statistic) or None when the kernel does not cover the case (CPU tensors, rows longer than 4096
+    or not a multiple of 16 bytes, fp16, mixed dtypes, vec_use_recip, round-half-even to a wide
+    format on bf16 tensors)."""
+    from . import _lib, gemm
+    from .custom_extensions import _flags_value
+    from .elemwise_ops import _native_round, elemwise_plan
+    if not (gemm.fused_enabled() and x.is_cuda) or mx_specs['vec_use_recip']:
+        return None
+    rnd = mx_specs['round']
+    plan = elemwise_plan(mx_specs, rnd)
+    if plan[0] == "to_bf16":                   # the inputs were already cast by vec_quantize
+        plan = ("identity",)
+    if x.dtype not in _DTYPE_CODE or bf_weight.dtype != x.dtype or bf_bias.dtype != x.dtype:
+        return None
+    n = x.shape[-1]
+    if n == 0 or n > MAX_FUSED_ROW or n % (16 // x.element_size()) != 0 or bf_weight.numel() != n:
+        return None
+    if plan[0] == "identity":
+        bits, exp_bits, max_norm, denorm, rmode = 0, 0, 1.0, True, 0
+    else:
+        _, bits, exp_bits, max_norm, denorm = plan
+        rmode = _native_round(rnd)
+        if x.dtype == torch.bfloat16 and bits >= 9 and rnd == 'even':
+            return None
+    x = x.contiguous()
+    w, b = bf_weight.contiguous(), bf_bias.contiguous()
+    out, x_norm = torch.empty_like(x), torch.empty_like(x)
+    stat = torch.empty(x.shape[:-1] + (1,), dtype=x.dtype, device=x.device)
+    lib = _lib.gpu()
+    with torch.cuda.device(x.device):
+        rc = lib.mxq_norm_lastdim(x.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(),
+                                  x_norm.data_ptr(), stat.data_ptr(), _DTYPE_CODE[x.dtype],
+                                  x.numel() // n, n, float(eps), int(rms), bits, exp_bits, max_norm,
+                                  rmode, int(denorm), _flags_value(),
+                                  torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, lib)
+    return out, x_norm, stat
+
+
 def _leading_axes(t):
     return list(range(t.ndim - 1))
 
@@ -31,7 +76,11 @@ class LayerNormFunction(torch.autograd.Function):
         x = vec_quantize(x, mx_specs=mx_specs)
         bf_weight = vec_quantize(weight, mx_specs=mx_specs)
         bf_bias = vec_quantize(bias, mx_specs=mx_specs)
-        output, _, x_norm, _, _, x_vare = _norm_forward(x, -1, bf_weight, bf_bias, eps, mx_specs)
+        fused = _fused_forward(x, bf_weight, bf_bias, eps, mx_specs, rms=False)
+        if fused is not None:
+            output, x_norm, x_vare = fused
+        else:
+            output, _, x_norm, _, _, x_vare = _norm_forward(x, -1, bf_weight, bf_bias, eps, mx_specs)
         ctx.save_for_backward(x_norm, x_vare, bf_weight if mx_specs['quantize_backprop'] else weight)
         ctx.mx_specs = get_backwards_mx_specs(mx_specs)
         return output
@@ -54,12 +103,16 @@ class RMSNormFunction(torch.autograd.Function):
         ctx.eps = eps
         s = mx_specs
         x = vec_quantize(x, mx_specs=s)
-        ms = vec_reduce_mean(vec_mul(x, x, mx_specs=s), -1, keepdim=True, mx_specs=s)
-        rms_inv = vec_recip(vec_sqrt(vec_add(ms, eps, mx_specs=s), mx_specs=s), mx_specs=s)
-        x_norm = vec_mul(x, rms_inv, mx_specs=s)
         bf_weight = vec_quantize(weight, mx_specs=s)
         bf_bias = vec_quantize(bias, mx_specs=s)
-        output = vec_add(vec_mul(bf_weight, x_norm, mx_specs=s), bf_bias, mx_specs=s)
+        fused = _fused_forward(x, bf_weight, bf_bias, eps, s, rms=True)
+        if fused is not None:
+            output, x_norm, rms_inv = fused
+        else:
+            ms = vec_reduce_mean(vec_mul(x, x, mx_specs=s), -1, keepdim=True, mx_specs=s)
+            rms_inv = vec_recip(vec_sqrt(vec_add(ms, eps, mx_specs=s), mx_specs=s), mx_specs=s)
+            x_norm = vec_mul(x, rms_inv, mx_specs=s)
+            output = vec_add(vec_mul(bf_weight, x_norm, mx_specs=s), bf_bias, mx_specs=s)
         ctx.save_for_backward(x_norm, rms_inv, bf_weight if s['quantize_backprop'] else weight)
         ctx.mx_specs = get_backwards_mx_specs(s)
         return output

@@ -180,3 +180,39 @@ def test_lstm(dev):
     for got, want in ((og, oc), (hg, hc), (cg, cc)):
         diff = (got.detach().cpu() - want.detach()).abs()
         assert diff.max().item() <= 0.05 and diff.mean().item() <= 2e-3, (diff.max().item(), diff.mean().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("layer", ["layernorm", "rmsnorm"])
+@pytest.mark.parametrize("shape", [(64, 4096), (5, 7, 1000), (33, 264), (9, 8)])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, round="floor"), dict(fp=16),
+                                  dict(bfloat=16, round="even")])
+def test_fused_norm_kernel_against_the_separate_steps(dev, dtype, layer, shape, spec):
+    """mxq_norm_lastdim vs the chain of vector ops it replaces, both on the GPU (set_fused switches
+    between them): output, saved normalized input, row statistic and gradients.  Only the order of
+    the two row sums differs."""
+    from microxcaling_amd import gemm
+    from microxcaling_amd.layernorm import LayerNorm, RMSNorm, _fused_forward
+    cls = {"layernorm": LayerNorm, "rmsnorm": RMSNorm}[layer]
+    specs = _specs(quantize_backprop=True, **spec)
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g) * 2 + 0.3).to(dtype)
+    go = torch.randn(*shape, generator=g).to(dtype)
+    m = cls(shape[-1], eps=1e-5, mx_specs=specs).to(dtype)
+    with torch.no_grad():
+        m.weight.copy_(torch.randn(shape[-1], generator=g))
+        m.bias.copy_(torch.randn(shape[-1], generator=g))
+    m.to(dev)
+    res = []
+    for fused in (True, False):
+        gemm.set_fused(fused)
+        try:
+            xi = x.to(dev).requires_grad_(True)
+            m.zero_grad()
+            out = m(xi)
+            out.backward(go.to(dev))
+            res.append((out.detach().cpu(), xi.grad.cpu(), m.weight.grad.cpu().clone(), m.bias.grad.cpu().clone()))
+        finally:
+            gemm.set_fused(True)
+    for got, want, what in zip(res[0], res[1], ("forward", "grad_input", "grad_weight", "grad_bias")):
+        _near(got, want, what)
