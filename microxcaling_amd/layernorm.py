@@ -15,7 +15,8 @@ MAX_FUSED_ROW = 4096
 
 
 def _fused_forward(x, bf_weight, bf_bias, eps, mx_specs, rms):
-    """The forward chain as one kernel launch (mxq_norm_lastdim): returns (output, x_norm, row
+    """The forward chain, including the quantization of the input x, as one kernel launch
+    (mxq_norm_lastdim); weight and bias are already quantized.  Returns (output, x_norm, row
     statistic) or None when the kernel does not cover the case (CPU tensors, rows longer than 4096
     or not a multiple of 16 bytes, fp16, mixed dtypes, vec_use_recip, round-half-even to a wide
     format on bf16 tensors)."""
@@ -26,7 +27,8 @@ def _fused_forward(x, bf_weight, bf_bias, eps, mx_specs, rms):
         return None
     rnd = mx_specs['round']
     plan = elemwise_plan(mx_specs, rnd)
-    if plan[0] == "to_bf16":                   # the inputs were already cast by vec_quantize
+    if plan[0] == "to_bf16":                   # what the first quantization of the chain does
+        x = x.to(torch.bfloat16)
         plan = ("identity",)
     if x.dtype not in _DTYPE_CODE or bf_weight.dtype != x.dtype or bf_bias.dtype != x.dtype:
         return None
@@ -73,13 +75,13 @@ class LayerNormFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias, eps, mx_specs=None, name=None):
         ctx.eps = eps
-        x = vec_quantize(x, mx_specs=mx_specs)
         bf_weight = vec_quantize(weight, mx_specs=mx_specs)
         bf_bias = vec_quantize(bias, mx_specs=mx_specs)
         fused = _fused_forward(x, bf_weight, bf_bias, eps, mx_specs, rms=False)
         if fused is not None:
             output, x_norm, x_vare = fused
         else:
+            x = vec_quantize(x, mx_specs=mx_specs)
             output, _, x_norm, _, _, x_vare = _norm_forward(x, -1, bf_weight, bf_bias, eps, mx_specs)
         ctx.save_for_backward(x_norm, x_vare, bf_weight if mx_specs['quantize_backprop'] else weight)
         ctx.mx_specs = get_backwards_mx_specs(mx_specs)
@@ -102,13 +104,13 @@ class RMSNormFunction(torch.autograd.Function):
     def forward(ctx, x, weight, bias, eps, mx_specs=None, name=None):
         ctx.eps = eps
         s = mx_specs
-        x = vec_quantize(x, mx_specs=s)
         bf_weight = vec_quantize(weight, mx_specs=s)
         bf_bias = vec_quantize(bias, mx_specs=s)
         fused = _fused_forward(x, bf_weight, bf_bias, eps, s, rms=True)
         if fused is not None:
             output, x_norm, rms_inv = fused
         else:
+            x = vec_quantize(x, mx_specs=s)
             ms = vec_reduce_mean(vec_mul(x, x, mx_specs=s), -1, keepdim=True, mx_specs=s)
             rms_inv = vec_recip(vec_sqrt(vec_add(ms, eps, mx_specs=s), mx_specs=s), mx_specs=s)
             x_norm = vec_mul(x, rms_inv, mx_specs=s)
