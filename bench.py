@@ -271,8 +271,8 @@ def report_flops(args, wl, ms_per_step, step_gpu_ms):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)     # the clocks need a few ms to ramp up
     ap.add_argument("--workload", default="mxfp8_fp32_8192")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()

@@ -34,9 +34,8 @@ Parity status of every function here ("pinned" = checked against something other
                             pinned (fp32 and bf16 tensors, bfloat 0 / 16, e^x and 2^x softmax):
                             forward outputs and gradients written by the reference's own layers on
                             the CPU (tests/golden/reference_layer_vectors.npz), reproduced bit for
-                            bit (tests/test_layer_golden.py).  The vec_use_exp2 / vec_use_recip
-                            variants of softmax_forward and the fp= formats are not in the
-                            fixtures: parity unpinned for those two switches.
+                            bit (tests/test_layer_golden.py), including the vec_use_exp2 and
+                            vec_use_recip switches and an fp= format of softmax_forward.
 """
 import torch
 

@@ -77,6 +77,11 @@ def main(ref_root):
             key = "softmax/%s/exp2_%d/" % (dt_name, int(exp2))
             store(d, key + "out", out)
             store(d, key + "gx", si.grad)
+        for sw in ("vec_use_exp2", "vec_use_recip"):
+            specs = finalize_mx_specs({"bfloat": 16, sw: True, "quantize_backprop": True, "custom_cuda": False})
+            store(d, "softmax/%s/%s/out" % (dt_name, sw), softmax(sx.to(dt), dim=-1, mx_specs=specs))
+        specs = finalize_mx_specs(dict(fp=16, quantize_backprop=True, custom_cuda=False))
+        store(d, "softmax/%s/fp16/out" % dt_name, softmax(sx.to(dt), dim=-1, mx_specs=specs))
 
     # normalization layers and activations (bfloat16 vector-op chains)
     from mx.layernorm import LayerNorm, RMSNorm

@@ -99,6 +99,20 @@ def test_softmax_oracle_and_cpu_layer(dt, exp2):
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_softmax_switches(dt):
+    """vec_use_exp2 (2^Q(x log2 e)), vec_use_recip (e * Q(1 / sum)) and an fp format."""
+    from microxcaling_amd.softmax import softmax
+    x = fx("in/sx").to(DT[dt])
+    for sw in ("vec_use_exp2", "vec_use_recip"):
+        want = fx("softmax/%s/%s/out" % (dt, sw))
+        assert_bits_equal(O.softmax_forward(x, -1, bfloat=16, **{sw: True}), want, "oracle " + sw)
+        assert_bits_equal(softmax(x, dim=-1, mx_specs=_specs(bfloat=16, **{sw: True})), want, "layer " + sw)
+    want = fx("softmax/%s/fp16/out" % dt)
+    assert_bits_equal(O.softmax_forward(x, -1, bfloat=0, fp=16), want, "oracle fp16")
+    assert_bits_equal(softmax(x, dim=-1, mx_specs=_specs(fp=16)), want, "layer fp16")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("layer", ["layernorm", "rmsnorm"])
 def test_norm_layers_on_cpu(dt, layer):
     from microxcaling_amd.layernorm import LayerNorm, RMSNorm
