@@ -122,6 +122,40 @@ def make_workload(name):
                     desc="mx.Linear forward: x bf16 [16384,4096], W bf16 [14336,4096] ~N(0,0.02), bias; MXFP8 e4m3 "
                          "block 32 along K, %s" % ("packed codes + scaled-MFMA GEMM" if fused else
                                                    "fake-quantize kernels + torch (hipBLASLt) bf16 GEMM"))
+    if name in ("mx_linear_train", "mx_linear_train_unfused"):
+        # forward + backward of the same layer (three GEMMs: output, grad_input, grad_weight), every
+        # operand MX-quantized along its contraction axis (mx/linear.py:20-198)
+        from microxcaling_amd import gemm
+        from microxcaling_amd.linear import linear
+        from microxcaling_amd.specs import finalize_mx_specs
+        g = torch.Generator().manual_seed(4)
+        M, N, K = 16384, 14336, 4096
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+        b = torch.randn(N, generator=g).to(torch.bfloat16)
+        specs = finalize_mx_specs({"w_elem_format": "fp8_e4m3", "a_elem_format": "fp8_e4m3", "block_size": 32,
+                                   "quantize_backprop": True})
+        st = {}
+        fused = name == "mx_linear_train"
+
+        def run(xd):
+            if "w" not in st:
+                st["w"] = w.to(xd.device).requires_grad_(True)
+                st["b"] = b.to(xd.device).requires_grad_(True)
+                st["x"] = xd.clone().requires_grad_(True)
+                st["go"] = torch.randn(M, N, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(xd.device)
+            gemm.set_fused(fused)
+            for t in (st["w"], st["b"], st["x"]):
+                t.grad = None
+            out = linear(st["x"], st["w"], st["b"], mx_specs=specs)
+            out.backward(st["go"])
+            return out
+        return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, "fp8_e4m3", "fp8_e4m3"),
+                    flops=6.0 * M * N * K, bytes=0, dtype="fp8_e4m3 x fp8_e4m3 -> f32 acc", sample_axis=0,
+                    cpu_rows=1024, launches=20,
+                    desc="mx.Linear forward + backward: x bf16 [16384,4096], W bf16 [14336,4096], bias; MXFP8 "
+                         "e4m3 block 32 along every contraction axis, %s" %
+                         ("packed codes + scaled-MFMA GEMMs" if fused else "fake-quantize kernels + torch GEMMs"))
     if name in ("mx_bmm_softmax", "mx_bmm_softmax_unfused"):
         # config 5: mx.bmm Q.K^T, MXFP6 e2m3 along head_dim, then the bfloat16 softmax chain
         from microxcaling_amd import gemm

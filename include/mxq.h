@@ -133,6 +133,14 @@ int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t ro
                 int flush_fp32_subnorms, int rmode, int flags, void* hip_stream);
 int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, void* out, int dtype,
                   int64_t rows, int64_t K, void* hip_stream);
+/* Quantize along the second-to-last axis and transpose while packing: in (batch, R, C) contiguous,
+ * blocks of 32 along R; codes (batch, C, R), scales (batch, C, R / 32) -- the K-major operand of
+ * mxq_gemm_mx_nt when the contraction runs over R, as in the gradient GEMMs of the layers
+ * (mx/linear.py:124-173: input and grad_output along axis -2, the weight along axis 0).
+ * unpack(codes, scales) is the transpose of mxq_quantize_mx_by_tile(in, axis = R). */
+int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t batch, int64_t R,
+                  int64_t C, int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                  int flush_fp32_subnorms, int rmode, int flags, void* hip_stream);
 /* C[b] (M, N) = A[b] (M, K) x B[b] (N, K)^T for b < batch, all tensors contiguous, fp32
  * accumulation on the scaled MFMA units; c_dtype is a MXQ_DTYPE_* code.  K % 128 == 0.
  * bias (optional, may be NULL): N values of dtype c_dtype; then C = round(round(A x B^T) + bias),

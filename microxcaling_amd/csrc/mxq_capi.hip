@@ -141,6 +141,19 @@ struct LaunchPack {
     }
 };
 
+template <int DT, int RMODE, bool ZE, bool LEAN>
+struct LaunchPackT {
+    static void run(const void* in, void* codes, void* scales, int64_t items, int64_t n_tiles,
+                    int64_t pv, bool bf8, MxParams p, hipStream_t s) {
+        const unsigned grid = (unsigned)ceil_div(items, kThreads);
+        const u32x2* i2 = reinterpret_cast<const u32x2*>(in);
+        unsigned char* c = reinterpret_cast<unsigned char*>(codes);
+        unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
+        if (bf8) mx_pack_t_kernel<DT, RMODE, ZE, true><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+        else mx_pack_t_kernel<DT, RMODE, ZE, false><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+    }
+};
+
 template <int CB, int BL, int ODT>
 int launch_gemm_dt(int64_t batch, const GemmArgs& g, hipStream_t s) {
     // large problems: persistent 256 x 256 tile kernel (144 KB of dynamic LDS, one workgroup per CU);
@@ -438,6 +451,36 @@ int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t ro
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
     dispatch<LaunchPack>(dtype, rmode, ze, true, in, codes, scales, total / (16 / elem_size(dtype)), bf8,
                          p, (hipStream_t)hip_stream);
+    return check_launch(who);
+}
+
+int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t batch, int64_t R,
+                  int64_t C, int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                  int flush_fp32_subnorms, int rmode, int flags, void* hip_stream) {
+    const char* who = "mxq_pack_mx_t";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    const bool bf8 = elem_ebits == 5 && elem_mbits <= 4;
+    if (!bf8 && !(elem_ebits >= 2 && elem_ebits <= 4 && elem_mbits <= 5))
+        return fail(MXQ_ERR_ARGUMENT, "%s: element format e%dm%d has no 8-bit float code "
+                    "(supported: up to e4m3, and e5m2)", who, elem_ebits, elem_mbits - 2);
+    if (batch < 0 || R < 0 || C < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    const int vw = 8 / elem_size(dtype);                 // columns in the 8 bytes a lane owns
+    if (R % 32 != 0 || C % vw != 0)
+        return fail(MXQ_ERR_ARGUMENT, "%s: R must be a multiple of 32 and C of %d", who, vw);
+    int64_t total;
+    if (mul_overflows(batch, R, C, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !codes || !scales) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if ((reinterpret_cast<uintptr_t>(in) & 7) || !aligned16(codes))
+        return fail(MXQ_ERR_ARGUMENT, "%s: input must be 8-byte and codes 16-byte aligned", who);
+    const int64_t n_tiles = R / 32, pv = C / vw, items = batch * n_tiles * pv;
+    if (ceil_div(items, kThreads) > 0x7FFFFFFF) return fail(MXQ_ERR_ARGUMENT, "%s: tensor too large", who);
+    dispatch<LaunchPackT>(dtype, rmode, ze, true, in, codes, scales, items, n_tiles, pv, bf8, p,
+                          (hipStream_t)hip_stream);
     return check_launch(who);
 }
 

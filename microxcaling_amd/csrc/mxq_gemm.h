@@ -72,6 +72,71 @@ __global__ __launch_bounds__(TPB) void mx_pack_kernel(const u32x4* __restrict__ 
     }
 }
 
+// ================================================================================================
+// quantize + pack + transpose: input (pre, R, C) with the shared axis = R (blocks of 32 rows, the
+// second-to-last axis), output codes (pre, C, R) and scales (pre, C, R / 32) -- the K-major operand
+// the GEMM wants when the contraction runs over R (gradients: x^T, grad_output^T, W^T).
+// A lane keeps a 32-row x 8-byte column strip in registers (like mx_strided_tile_kernel) and writes,
+// per column, the 32 codes of the block as 32 contiguous bytes.
+// ================================================================================================
+template <int DT, int RMODE, bool ZONE_ELEM, bool BF8>
+__global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict__ in,
+                                                        unsigned char* __restrict__ codes,
+                                                        unsigned char* __restrict__ scales,
+                                                        int64_t items, int64_t n_tiles, int64_t pv,
+                                                        MxParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int VW = Col8<DT>::VW;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int ROWS = 32;
+    __shared__ unsigned char zone[ZONE_PAD];
+
+    const int64_t w = (int64_t)blockIdx.x * TPB + threadIdx.x;     // (pre_i, tile_i, column group)
+    const bool live = w < items;
+    const int64_t c = live ? w % pv : 0;
+    const int64_t pt = live ? w / pv : 0;                           // pre_i * n_tiles + tile_i
+    const int64_t off0 = pt * ROWS * pv + c;                        // in units of 8 bytes
+
+    u32x2 raw[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) raw[r] = live ? in[off0 + (int64_t)r * pv] : u32x2{0, 0};
+    load_zone(zone, g_zone_tables[p.zone_row]);
+
+    uint32_t um[VW];
+#pragma unroll
+    for (int k = 0; k < VW; ++k) um[k] = 0;
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+        for (int d = 0; d < 2; ++d)
+#pragma unroll
+            for (int h = 0; h < PD; ++h)
+                um[d * PD + h] = max(um[d * PD + h], abs_bits(Pack<DT>::get(raw[r][d], h)));
+
+    const int64_t pre_i = pt / n_tiles, tile_i = pt % n_tiles;
+    const int64_t C = pv * VW, R = n_tiles * ROWS;
+#pragma unroll
+    for (int k = 0; k < VW; ++k) {
+        const MxqScale sc = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+        uint32_t out[8] = {};
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const float y = mxq_quant_mx_elem_unscaled<RMODE, ADT, ZONE_ELEM>(
+                Pack<DT>::get(raw[r][k / PD], k % PD), sc, p.fmt, zone, ZS);
+            const uint32_t code = BF8 ? mxq_encode_e5m2(y) : mxq_encode_e4m3(y);
+            out[r / 4] |= code << (8 * (r % 4));
+        }
+        if (live) {
+            const int64_t col = c * VW + k;
+            u32x4* dst = reinterpret_cast<u32x4*>(codes + (pre_i * C + col) * R + tile_i * ROWS);
+            dst[0] = u32x4{out[0], out[1], out[2], out[3]};
+            dst[1] = u32x4{out[4], out[5], out[6], out[7]};
+            scales[(pre_i * C + col) * n_tiles + tile_i] = (unsigned char)mxq_encode_e8m0(sc.scale);
+        }
+    }
+}
+
 // unpack: codes * 2^(scale-127) -> fp32 / bf16 / fp16 (for tests and for callers that want the
 // fake-quantized view of a packed tensor)
 template <int DT, bool BF8>

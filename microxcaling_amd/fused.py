@@ -49,6 +49,37 @@ def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=F
     return codes, scales, fmt == ElemFormat.fp8_e5m2
 
 
+def pack_mx_t(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=False):
+    """MX-quantize A (..., R, C) along its second-to-last axis (block 32) and transpose while
+    packing: codes uint8 (..., C, R), scales uint8 (..., C, R / 32) -- K-major for a contraction
+    over R.  Returns (codes, scales, codes_are_e5m2)."""
+    who = "pack_mx_t"
+    fmt = _as_format(elem_format)
+    if fmt not in _PACKABLE:
+        raise RuntimeError("%s: element format %s has no packed form" % (who, fmt))
+    _check_gpu_input(A, "A", who)
+    if A.dtype not in _DTYPE:
+        raise RuntimeError("%s: Tensor dtype not supported (%s)" % (who, A.dtype))
+    if A.dim() < 2:
+        raise RuntimeError("%s: needs at least two axes" % who)
+    R, C = A.shape[-2], A.shape[-1]
+    if R % 32 != 0 or C % (8 // A.element_size()) != 0:
+        raise RuntimeError("%s: shape %s: the second-to-last axis must be a multiple of 32 and the "
+                           "last one of 8 bytes" % (who, tuple(A.shape)))
+    ebits, mbits, _, max_norm, _ = _get_format_params(fmt)
+    batch = A.numel() // (R * C) if R * C else 0
+    codes = torch.empty(A.shape[:-2] + (C, R), dtype=torch.uint8, device=A.device)
+    scales = torch.empty(A.shape[:-2] + (C, R // 32), dtype=torch.uint8, device=A.device)
+    lib = _lib.gpu()
+    with torch.cuda.device(A.device):
+        rc = lib.mxq_pack_mx_t(A.data_ptr(), codes.data_ptr(), scales.data_ptr(), _DTYPE[A.dtype],
+                               batch, R, C, scale_bits, ebits, mbits, max_norm,
+                               int(bool(flush_fp32_subnorms)), int(RoundingMode[round]),
+                               _flags_value(), _stream(A))
+    _lib.check(rc, lib)
+    return codes, scales, fmt == ElemFormat.fp8_e5m2
+
+
 def unpack_mx(codes, scales, codes_are_e5m2, dtype=torch.float32):
     """codes * 2^(scales - 127) as a tensor of `dtype` (255 in scales -> NaN block)."""
     who = "unpack_mx"
@@ -136,3 +167,46 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
     pa = pack_mx(a2, fa, scale_bits, round, flush)
     pb = pack_mx(b2, fb, scale_bits, round, flush)
     return gemm_nt(pa, pb, out_dtype=a.dtype, bias=bias, epilogue_quant=epilogue_quant).reshape(out_shape)
+
+
+def mx_gemm_operands(operands, mx_specs, out_dtype):
+    """General form of mx_gemm_nt for the gradient GEMMs: `operands` = two (tensor, format, round,
+    transposed) entries.  transposed=False: the tensor is (..., rows, K), quantized along its last
+    axis; True: it is (..., K, rows), quantized along its second-to-last axis and transposed while
+    packing.  Returns rows_a x rows_b (leading axes must match, or the second operand has none),
+    or None when the operands do not qualify."""
+    if mx_specs["block_size"] != 32 or mx_specs["shared_exp_method"] != "max":
+        return None
+    packed, shapes = [], []
+    for t, fmt, rnd, transposed in operands:
+        f = _as_format(fmt)
+        if f not in _PACKABLE or rnd not in RoundingMode.string_enums():
+            return None
+        if not t.is_cuda or t.dtype not in _DTYPE or t.dim() < 2 or t.numel() == 0:
+            return None
+        K = t.shape[-2] if transposed else t.shape[-1]
+        if K % GEMM_K_MULTIPLE != 0 or (transposed and t.shape[-1] % (8 // t.element_size()) != 0):
+            return None
+        shapes.append((t.shape[:-2], t.shape[-1] if transposed else t.shape[-2], K, transposed, f, rnd))
+    (lead_a, rows_a, Ka, _, _, _), (lead_b, rows_b, Kb, _, _, _) = shapes
+    if Ka != Kb or (len(lead_b) and lead_b != lead_a):
+        return None
+    if len(lead_a) and not len(lead_b) and operands[0][3]:
+        return None                                   # a transposed batched A cannot be folded into rows
+    scale_bits = mx_specs["scale_bits"] if mx_specs["scale_bits"] != 0 else 8
+    flush = mx_specs["mx_flush_fp32_subnorms"]
+    for (t, _, _, _), (lead, rows, K, transposed, f, rnd) in zip(operands, shapes):
+        t = t.contiguous()
+        p = (pack_mx_t if transposed else pack_mx)(t, f, scale_bits, rnd, flush)
+        packed.append(p)
+    (ac, asc, ae), (bc, bsc, be) = packed
+    if len(lead_b):                                   # batched x batched
+        batch = ac.numel() // (rows_a * Ka)
+        if batch > 65535:
+            return None
+        ac, asc = ac.reshape(batch, rows_a, Ka), asc.reshape(batch, rows_a, Ka // 32)
+        bc, bsc = bc.reshape(batch, rows_b, Ka), bsc.reshape(batch, rows_b, Ka // 32)
+    else:                                             # every leading axis of A folds into its rows
+        ac, asc = ac.reshape(-1, Ka), asc.reshape(-1, Ka // 32)
+    out = gemm_nt((ac, asc, ae), (bc, bsc, be), out_dtype=out_dtype)
+    return out.reshape(tuple(lead_a) + (rows_a, rows_b))

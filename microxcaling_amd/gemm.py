@@ -92,3 +92,25 @@ def mx_matmul_contract(a, b, a_fmt, b_fmt, mx_specs, round, batched=False, out_r
     qa = quantize_mx_op(a, mx_specs, elem_format=a_fmt, axes=[-1], round=round)
     qb = quantize_mx_op(b, mx_specs, elem_format=b_fmt, axes=[-2], round=round)
     return (torch_bmm(qa, qb) if batched else torch_matmul(qa, qb)), False
+
+
+def mx_grad_contract(a, a_fmt, a_round, a_transposed, b, b_fmt, b_round, b_transposed, mx_specs,
+                     batched=False):
+    """The contractions of the backward passes: rows(a) x rows(b)^T over a shared K axis, each
+    operand either (..., rows, K) quantized along -1, or -- transposed -- (..., K, rows) quantized
+    along -2 (mx/linear.py:124-173, mx/matmul.py:131-172, mx/bmm.py:82-121).  Fused path: packed
+    codes (transposed while packing where needed) + the scaled-MFMA GEMM; otherwise the
+    fake-quantize kernels + torch's GEMM."""
+    if _use_fused and a.is_cuda:
+        from . import fused
+        out = fused.mx_gemm_operands(((a, a_fmt, a_round, a_transposed), (b, b_fmt, b_round, b_transposed)),
+                                     mx_specs, a.dtype)
+        if out is not None:
+            return out
+    qa = quantize_mx_op(a, mx_specs, elem_format=a_fmt, axes=[-2 if a_transposed else -1], round=a_round)
+    qb = quantize_mx_op(b, mx_specs, elem_format=b_fmt, axes=[-2 if b_transposed else -1], round=b_round)
+    if a_transposed:
+        qa = qa.transpose(-1, -2)
+    if not b_transposed:
+        qb = qb.transpose(-1, -2)
+    return torch_bmm(qa, qb) if batched else torch_matmul(qa, qb)

@@ -3,7 +3,7 @@ import torch
 import torch.nn.functional as F
 
 from .elemwise_ops import quantize_elemwise_op
-from .gemm import mx_linear_contract, mx_matmul_contract
+from .gemm import mx_grad_contract, mx_linear_contract
 from .mx_ops import quantize_mx_op
 from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
 
@@ -61,23 +61,30 @@ class LinearFunction(torch.autograd.Function):
         grad_output = quantize_elemwise_op(grad_output, mx_specs=specs,
                                            round=specs["round_grad_input"])
 
-        # grad_weight = grad_output^T x input, contracted over the example axis
-        q_in = quantize_mx_op(input, specs, elem_format=specs["a_elem_format_bp"], axes=[-2],
-                              round=specs["round_mx_input_grad_weight"])
-        q_go = quantize_mx_op(grad_output, specs, elem_format=specs["a_elem_format_bp_ex"],
-                              axes=[-2], round=specs["round_mx_grad_output_grad_weight"])
-        grad_weight = torch_matmul(q_go.reshape(-1, out_dim).transpose(0, 1),
-                                   q_in.reshape(-1, in_dim))
+        # grad_weight = grad_output^T x input, contracted over the example axis; both operands share
+        # exponents along axis -2.  When that axis is a multiple of 32 the blocks do not straddle
+        # batch entries and the tensors can be flattened to 2-D first (one GEMM over all examples)
+        if input.dim() == 2 or input.shape[-2] % 32 == 0:
+            grad_weight = mx_grad_contract(
+                grad_output.reshape(-1, out_dim), specs["a_elem_format_bp_ex"],
+                specs["round_mx_grad_output_grad_weight"], True,
+                input.reshape(-1, in_dim), specs["a_elem_format_bp"],
+                specs["round_mx_input_grad_weight"], True, specs)
+        else:
+            q_in = quantize_mx_op(input, specs, elem_format=specs["a_elem_format_bp"], axes=[-2],
+                                  round=specs["round_mx_input_grad_weight"])
+            q_go = quantize_mx_op(grad_output, specs, elem_format=specs["a_elem_format_bp_ex"],
+                                  axes=[-2], round=specs["round_mx_grad_output_grad_weight"])
+            grad_weight = torch_matmul(q_go.reshape(-1, out_dim).transpose(0, 1),
+                                       q_in.reshape(-1, in_dim))
         grad_weight = quantize_elemwise_op(grad_weight, mx_specs=specs,
                                            round=specs["round_grad_weight"])
 
         # grad_input = grad_output x weight, contracted over the output-feature axis
-        q_w = quantize_mx_op(weight, specs, elem_format=specs["w_elem_format_bp"], axes=[0],
-                             round=specs["round_mx_weight_grad_input"])
-        q_go = quantize_mx_op(grad_output, specs, elem_format=specs["a_elem_format_bp_os"],
-                              axes=[-1], round=specs["round_mx_grad_output_grad_input"])
-        grad_input = quantize_elemwise_op(torch_matmul(q_go, q_w), mx_specs=specs,
-                                          round=specs["round_grad_input"])
+        grad_input = mx_grad_contract(
+            grad_output, specs["a_elem_format_bp_os"], specs["round_mx_grad_output_grad_input"], False,
+            weight, specs["w_elem_format_bp"], specs["round_mx_weight_grad_input"], True, specs)
+        grad_input = quantize_elemwise_op(grad_input, mx_specs=specs, round=specs["round_grad_input"])
 
         grad_bias = None
         if ctx.has_bias:

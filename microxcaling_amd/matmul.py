@@ -3,7 +3,7 @@ import numpy as np
 import torch
 
 from .elemwise_ops import quantize_elemwise_op
-from .gemm import mx_matmul_contract
+from .gemm import mx_grad_contract, mx_matmul_contract
 from .mx_ops import quantize_mx_op
 from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
 
@@ -56,16 +56,22 @@ class MatMulFunction(torch.autograd.Function):
         in1, in2 = ctx.saved_tensors
         grad_out = quantize_elemwise_op(grad_out, mx_specs=specs, round=specs["round_grad_input"])
 
-        q1 = quantize_mx_op(in1, specs, elem_format=fmt1, axes=[-2],
-                            round=specs["round_mx_input_grad_input"])
-        q2 = quantize_mx_op(in2, specs, elem_format=fmt2, axes=[-1],
-                            round=specs["round_mx_input_grad_input"])
-        g_cols = quantize_mx_op(grad_out, specs, elem_format=fmt_g, axes=[-1],
-                                round=specs["round_mx_grad_output_grad_input"])
-        g_rows = quantize_mx_op(grad_out, specs, elem_format=fmt_g, axes=[-2],
-                                round=specs["round_mx_grad_output_grad_input"])
-        grad_in1 = torch_matmul(g_cols, q2.transpose(-1, -2))
-        grad_in2 = torch_matmul(q1.transpose(-1, -2), g_rows)
+        r_in, r_g = specs["round_mx_input_grad_input"], specs["round_mx_grad_output_grad_input"]
+        if in1.dim() == in2.dim() and in1.shape[:-2] == in2.shape[:-2]:
+            # grad_in1 = grad_out x in2^T over N (both along -1); grad_in2 = in1^T x grad_out over M
+            # (both along -2)
+            batched = in1.dim() == 3
+            grad_in1 = mx_grad_contract(grad_out, fmt_g, r_g, False, in2, fmt2, r_in, False, specs,
+                                        batched=batched)
+            grad_in2 = mx_grad_contract(in1, fmt1, r_in, True, grad_out, fmt_g, r_g, True, specs,
+                                        batched=batched)
+        else:                                    # broadcast leading axes: torch.matmul sorts them out
+            q1 = quantize_mx_op(in1, specs, elem_format=fmt1, axes=[-2], round=r_in)
+            q2 = quantize_mx_op(in2, specs, elem_format=fmt2, axes=[-1], round=r_in)
+            g_cols = quantize_mx_op(grad_out, specs, elem_format=fmt_g, axes=[-1], round=r_g)
+            g_rows = quantize_mx_op(grad_out, specs, elem_format=fmt_g, axes=[-2], round=r_g)
+            grad_in1 = torch_matmul(g_cols, q2.transpose(-1, -2))
+            grad_in2 = torch_matmul(q1.transpose(-1, -2), g_rows)
         grad_in1 = quantize_elemwise_op(grad_in1, mx_specs=specs, round=specs["round_grad_input"])
         grad_in2 = quantize_elemwise_op(grad_in2, mx_specs=specs, round=specs["round_grad_input"])
 
