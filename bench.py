@@ -97,8 +97,8 @@ def make_workload(name):
         return dict(x=x, gpu=fn, cpu=cpu, bytes=x.numel() * 4, dtype="f32", sample_axis=0 if dim == -1 else 1,
                     launches=1 if dim == -1 else 2,
                     desc="reduce %s over axis %d, fp32 [16384,8192]" % (op, dim))
-    if name in ("mx_linear", "mx_linear_unfused"):
-        # config 4: mx.Linear forward, MXFP8 e4m3 both operands, block 32 along K, bias
+    if name in ("mx_linear", "mx_linear_unfused", "mx_linear_fp4", "mx_linear_fp4_unfused"):
+        # config 4: mx.Linear forward, MXFP8 e4m3 (or MXFP4 e2m1) both operands, block 32 along K, bias
         from microxcaling_amd import gemm
         from microxcaling_amd.linear import linear
         from microxcaling_amd.specs import finalize_mx_specs
@@ -107,21 +107,23 @@ def make_workload(name):
         x = torch.randn(M, K, generator=g).to(torch.bfloat16)
         w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
         b = torch.randn(N, generator=g).to(torch.bfloat16)
-        specs = finalize_mx_specs({"w_elem_format": "fp8_e4m3", "a_elem_format": "fp8_e4m3", "block_size": 32})
+        ef = "fp4_e2m1" if "fp4" in name else "fp8_e4m3"
+        specs = finalize_mx_specs({"w_elem_format": ef, "a_elem_format": ef, "block_size": 32})
         dev_extra = {}
-        fused = name == "mx_linear"
+        fused = not name.endswith("_unfused")
 
         def run(xd):
             if "w" not in dev_extra:
                 dev_extra["w"], dev_extra["b"] = w.to(xd.device), b.to(xd.device)
             gemm.set_fused(fused)
             return linear(xd, dev_extra["w"], dev_extra["b"], mx_specs=specs)
-        return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, "fp8_e4m3", "fp8_e4m3"),
-                    flops=2.0 * M * N * K, bytes=0, dtype="fp8_e4m3 x fp8_e4m3 -> f32 acc", sample_axis=0,
-                    cpu_rows=1024, launches=5,
-                    desc="mx.Linear forward: x bf16 [16384,4096], W bf16 [14336,4096] ~N(0,0.02), bias; MXFP8 e4m3 "
-                         "block 32 along K, %s" % ("packed codes + scaled-MFMA GEMM" if fused else
-                                                   "fake-quantize kernels + torch (hipBLASLt) bf16 GEMM"))
+        return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, ef, ef),
+                    flops=2.0 * M * N * K, bytes=0, dtype="%s x %s -> f32 acc" % (ef, ef), sample_axis=0,
+                    cpu_rows=1024, launches=5, peak="fp4" if ef == "fp4_e2m1" else "fp8",
+                    desc="mx.Linear forward: x bf16 [16384,4096], W bf16 [14336,4096] ~N(0,0.02), bias; %s "
+                         "block 32 along K, %s" % ("MXFP4 e2m1" if ef == "fp4_e2m1" else "MXFP8 e4m3",
+                                                   ("packed codes + scaled-MFMA GEMM" if fused else
+                                                    "fake-quantize kernels + torch (hipBLASLt) bf16 GEMM")))
     if name in ("mx_linear_train", "mx_linear_train_unfused"):
         # forward + backward of the same layer (three GEMMs: output, grad_input, grad_weight), every
         # operand MX-quantized along its contraction axis (mx/linear.py:20-198)
@@ -257,7 +259,8 @@ def cpu_baseline(wl, budget_s=15.0):
                          torch.__version__, cores)}
 
 
-MFMA_PEAK_TFLOPS = {"fp8": 5000.0}          # MI355X dense fp8 (e4m3 / e5m2 codes), published
+# MI355X dense MFMA peaks, published: fp8 (e4m3 / e5m2 byte codes) and fp4 (e2m1 nibble codes)
+MFMA_PEAK_TFLOPS = {"fp8": 5000.0, "fp4": 10100.0}
 
 
 def measured_traffic(workload):
@@ -275,16 +278,17 @@ def report_flops(args, wl, ms_per_step, step_gpu_ms):
     step) against the dense fp8 MFMA peak."""
     value = wl["flops"] / (ms_per_step * 1e-3) / 1e12
     achieved = wl["flops"] / (step_gpu_ms * 1e-3) / 1e12
+    peak = MFMA_PEAK_TFLOPS[wl.get("peak", "fp8")]
     out = {
         "metric": "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"], "data": "synthetic",
         "config": {"workload": args.workload, "detail": wl["desc"], "flop_per_step": wl["flops"]},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_PEAK_TFLOPS["fp8"],
-                     "unit": "TFLOP/s", "frac": round(achieved / MFMA_PEAK_TFLOPS["fp8"], 4),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak,
+                     "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
                      "traffic": measured_traffic(args.workload), "step_gpu_ms_avg": round(step_gpu_ms, 5),
-                     "note": "whole forward step (all launches) over the dense fp8 MFMA peak"},
+                     "note": "whole forward step (all launches) over the dense %s MFMA peak" % wl.get("peak", "fp8")},
     }
     if not args.no_cpu_baseline:
         x = wl["x"]

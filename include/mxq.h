@@ -41,6 +41,12 @@ extern "C" {
 
 /* flags */
 #define MXQ_FLAG_EXACT_EXPONENT 1 /* bit-field exponents instead of torch's floor(log2(x)) */
+#define MXQ_FLAG_PACK_NIBBLES 4   /* mxq_pack_mx / _t, fp4 (e2m1) only: 4-bit codes, two per byte */
+
+/* kinds of packed element codes */
+#define MXQ_CODES_E4M3 0 /* one OCP e4m3 byte per element */
+#define MXQ_CODES_E5M2 1 /* one OCP e5m2 byte per element */
+#define MXQ_CODES_E2M1 4 /* one OCP e2m1 nibble per element, the lower K index in the low nibble */
 
 /* status codes */
 #define MXQ_OK 0
@@ -125,13 +131,14 @@ int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void*
  * fake-quantizes and then calls a dense GEMM: mx/linear.py:62-86, mx/bmm.py:40-59) ---------------
  * Packed form of a (rows, K) tensor quantized along K in blocks of 32:
  *   codes  uint8 (rows, K)     OCP e4m3 for fp8_e4m3 / fp6_e3m2 / fp6_e2m3 / fp4_e2m1 elements (e4m3
- *                              holds all their values exactly), OCP e5m2 for fp8_e5m2 elements
+ *                              holds all their values exactly), OCP e5m2 for fp8_e5m2 elements;
+ *          or uint8 (rows, K/2) OCP e2m1 nibbles for fp4_e2m1 with MXQ_FLAG_PACK_NIBBLES
  *   scales uint8 (rows, K/32)  E8M0 (shared exponent + 127; 255 = the block is NaN)
  * value = code * 2^(scale - 127), identical to what mxq_quantize_mx_by_tile returns. */
 int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t rows, int64_t K,
                 int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
                 int flush_fp32_subnorms, int rmode, int flags, void* hip_stream);
-int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, void* out, int dtype,
+int mxq_unpack_mx(const void* codes, const void* scales, int code_kind, void* out, int dtype,
                   int64_t rows, int64_t K, void* hip_stream);
 /* Quantize along the second-to-last axis and transpose while packing: in (batch, R, C) contiguous,
  * blocks of 32 along R; codes (batch, C, R), scales (batch, C, R / 32) -- the K-major operand of
@@ -142,21 +149,24 @@ int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t 
                   int64_t C, int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
                   int flush_fp32_subnorms, int rmode, int flags, void* hip_stream);
 /* C[b] (M, N) = A[b] (M, K) x B[b] (N, K)^T for b < batch, all tensors contiguous, fp32
- * accumulation on the scaled MFMA units; c_dtype is a MXQ_DTYPE_* code.  K % 128 == 0.
+ * accumulation on the scaled MFMA units; c_dtype is a MXQ_DTYPE_* code.  a_kind, b_kind:
+ * MXQ_CODES_* of the operands; e4m3 and e5m2 bytes mix freely (K % 128 == 0), e2m1 nibbles need both
+ * operands in that form (K % 256 == 0) and run at the 4-bit MFMA rate.
  * bias (optional, may be NULL): N values of dtype c_dtype; then C = round(round(A x B^T) + bias),
  * both roundings to c_dtype, which is what "matmul, then add the bias" gives as tensor ops.
  * epilogue_quant = 1 (bf16 C only): additionally apply the elementwise quantization of the layers
  * with mx_specs['bfloat'] = 16 and round-half-away (quantize_elemwise_op, mx/linear.py:88-96,
  * mx/bmm.py:55-57) to the rounded product and again to the rounded sum with the bias. */
-int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, const void* b_codes,
-                   const void* b_scales, int b_is_e5m2, const void* bias, void* c, int c_dtype,
+int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const void* b_codes,
+                   const void* b_scales, int b_kind, const void* bias, void* c, int c_dtype,
                    int64_t batch, int64_t M, int64_t N, int64_t K, int epilogue_quant,
                    void* hip_stream);
 
 /* Measurement aid (no counterpart in the reference): launches `workgroups` x 256 lanes, each wave
- * issuing iters x 16 scaled 16x16x128 fp8 MFMAs on register-resident operands
- * (workgroups * 4 * iters * 16 * 65536 flop in total).  `sink` is any 4 writable device bytes. */
-int mxq_probe_mfma_rate(int64_t workgroups, int iters, void* sink, void* hip_stream);
+ * issuing iters x 16 scaled 16x16x128 MFMAs on register-resident operands of kind MXQ_CODES_E4M3 or
+ * MXQ_CODES_E2M1 (workgroups * 4 * iters * 16 * 65536 flop in total).  `sink` is any 4 writable
+ * device bytes. */
+int mxq_probe_mfma_rate(int64_t workgroups, int iters, int code_kind, void* sink, void* hip_stream);
 
 /* ---- libmxq_host.so: the same arithmetic compiled for the host ----------------------------------
  * quantize_mx_func_cpp (mx/cpp/funcs.cpp:23-98) and quantize_elemwise_func_cpp

@@ -131,36 +131,38 @@ struct LaunchElemwise {
 
 template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchPack {
-    static void run(const void* in, void* codes, void* scales, int64_t n_vec, bool bf8, MxParams p,
+    static void run(const void* in, void* codes, void* scales, int64_t n_vec, int kind, MxParams p,
                     hipStream_t s) {
         const int grid = grid_for(ceil_div(n_vec, (int64_t)kThreads * 4));
         const u32x4* i4 = reinterpret_cast<const u32x4*>(in);
         unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
-        if (bf8) mx_pack_kernel<DT, RMODE, ZE, true, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
-        else mx_pack_kernel<DT, RMODE, ZE, false, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+        if (kind == 1) mx_pack_kernel<DT, RMODE, ZE, 1, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+        else if (kind == 4) mx_pack_kernel<DT, RMODE, ZE, 4, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+        else mx_pack_kernel<DT, RMODE, ZE, 0, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
     }
 };
 
 template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchPackT {
     static void run(const void* in, void* codes, void* scales, int64_t items, int64_t n_tiles,
-                    int64_t pv, bool bf8, MxParams p, hipStream_t s) {
+                    int64_t pv, int kind, MxParams p, hipStream_t s) {
         const unsigned grid = (unsigned)ceil_div(items, kThreads);
         const u32x2* i2 = reinterpret_cast<const u32x2*>(in);
         unsigned char* c = reinterpret_cast<unsigned char*>(codes);
         unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
-        if (bf8) mx_pack_t_kernel<DT, RMODE, ZE, true><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
-        else mx_pack_t_kernel<DT, RMODE, ZE, false><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+        if (kind == 1) mx_pack_t_kernel<DT, RMODE, ZE, 1><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+        else if (kind == 4) mx_pack_t_kernel<DT, RMODE, ZE, 4><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+        else mx_pack_t_kernel<DT, RMODE, ZE, 0><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
     }
 };
 
 template <int CB, int BL, int ODT>
 int launch_gemm_dt(int64_t batch, const GemmArgs& g, hipStream_t s) {
     // large problems: persistent 256 x 256 tile kernel (144 KB of dynamic LDS, one workgroup per CU);
-    // it fetches scales four K steps at a time, hence K % 512
+    // it fetches 16 scale bytes per row at a time, hence K % 512
     const int64_t tiles_m = ceil_div(g.M, G2_BM), tiles_n = ceil_div(g.N, G2_BN);
     const int64_t total = tiles_m * tiles_n * batch;
-    if (g.M >= 512 && g.N >= 512 && g.K % 512 == 0 && (int64_t)256 * g.K < ((int64_t)1 << 31) &&
+    if (g.M >= 512 && g.N >= 512 && g.K % 512 == 0 && (int64_t)256 * g.kbytes < ((int64_t)1 << 31) &&
         total < ((int64_t)1 << 30)) {
         static bool configured = false;               // raising the dynamic-LDS limit is per kernel
         static int cus = 0;
@@ -241,6 +243,24 @@ int reduce_outer(const float* in, float* out, void* workspace, int64_t outer, in
     if (rc || splits == 1) return rc;
     reduce_outer_final_kernel<OP><<<(unsigned)ceil_div(inner, 64), kThreads, 0, s>>>(partial, out, splits, inner);
     return check_launch(who);
+}
+
+// Which code the element format packs to: MXQ_CODES_E4M3 / _E5M2 bytes, or _E2M1 nibbles when the
+// caller asks for them (MXQ_FLAG_PACK_NIBBLES, fp4 only); -1 = no packed form.
+int code_kind(int ebits, int mbits, int flags, const char* who) {
+    const bool fp4 = ebits == 2 && mbits == 3;
+    if (flags & MXQ_FLAG_PACK_NIBBLES) {
+        if (!fp4) {
+            fail(MXQ_ERR_ARGUMENT, "%s: 4-bit codes exist for the e2m1 format only", who);
+            return -1;
+        }
+        return MXQ_CODES_E2M1;
+    }
+    if (ebits == 5 && mbits <= 4) return MXQ_CODES_E5M2;
+    if (ebits >= 2 && ebits <= 4 && mbits <= 5) return MXQ_CODES_E4M3;
+    fail(MXQ_ERR_ARGUMENT, "%s: element format e%dm%d has no 8-bit float code (supported: up to "
+         "e4m3, and e5m2)", who, ebits, mbits - 2);
+    return -1;
 }
 
 }  // namespace
@@ -437,10 +457,8 @@ int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t ro
     int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
                             flush_fp32_subnorms, rmode, flags, &p, &ze, who);
     if (rc) return rc;
-    const bool bf8 = elem_ebits == 5 && elem_mbits <= 4;
-    if (!bf8 && !(elem_ebits >= 2 && elem_ebits <= 4 && elem_mbits <= 5))
-        return fail(MXQ_ERR_ARGUMENT, "%s: element format e%dm%d has no 8-bit float code "
-                    "(supported: up to e4m3, and e5m2)", who, elem_ebits, elem_mbits - 2);
+    const int kind = code_kind(elem_ebits, elem_mbits, flags, who);
+    if (kind < 0) return MXQ_ERR_ARGUMENT;
     if (rows < 0 || K < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
     if (K % 32 != 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be a multiple of the block size 32", who);
     int64_t total;
@@ -449,7 +467,7 @@ int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t ro
     if (!in || !codes || !scales) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     if (!aligned16(in) || !aligned16(codes))
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
-    dispatch<LaunchPack>(dtype, rmode, ze, true, in, codes, scales, total / (16 / elem_size(dtype)), bf8,
+    dispatch<LaunchPack>(dtype, rmode, ze, true, in, codes, scales, total / (16 / elem_size(dtype)), kind,
                          p, (hipStream_t)hip_stream);
     return check_launch(who);
 }
@@ -463,10 +481,8 @@ int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t 
     int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
                             flush_fp32_subnorms, rmode, flags, &p, &ze, who);
     if (rc) return rc;
-    const bool bf8 = elem_ebits == 5 && elem_mbits <= 4;
-    if (!bf8 && !(elem_ebits >= 2 && elem_ebits <= 4 && elem_mbits <= 5))
-        return fail(MXQ_ERR_ARGUMENT, "%s: element format e%dm%d has no 8-bit float code "
-                    "(supported: up to e4m3, and e5m2)", who, elem_ebits, elem_mbits - 2);
+    const int kind = code_kind(elem_ebits, elem_mbits, flags, who);
+    if (kind < 0) return MXQ_ERR_ARGUMENT;
     if (batch < 0 || R < 0 || C < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
     const int vw = 8 / elem_size(dtype);                 // columns in the 8 bytes a lane owns
     if (R % 32 != 0 || C % vw != 0)
@@ -479,15 +495,17 @@ int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t 
         return fail(MXQ_ERR_ARGUMENT, "%s: input must be 8-byte and codes 16-byte aligned", who);
     const int64_t n_tiles = R / 32, pv = C / vw, items = batch * n_tiles * pv;
     if (ceil_div(items, kThreads) > 0x7FFFFFFF) return fail(MXQ_ERR_ARGUMENT, "%s: tensor too large", who);
-    dispatch<LaunchPackT>(dtype, rmode, ze, true, in, codes, scales, items, n_tiles, pv, bf8, p,
+    dispatch<LaunchPackT>(dtype, rmode, ze, true, in, codes, scales, items, n_tiles, pv, kind, p,
                           (hipStream_t)hip_stream);
     return check_launch(who);
 }
 
-int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, void* out, int dtype,
+int mxq_unpack_mx(const void* codes, const void* scales, int code_kind, void* out, int dtype,
                   int64_t rows, int64_t K, void* hip_stream) {
     const char* who = "mxq_unpack_mx";
     if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
+    if (code_kind != MXQ_CODES_E4M3 && code_kind != MXQ_CODES_E5M2 && code_kind != MXQ_CODES_E2M1)
+        return fail(MXQ_ERR_ARGUMENT, "%s: unknown code kind %d", who, code_kind);
     if (rows < 0 || K < 0 || K % 32 != 0) return fail(MXQ_ERR_ARGUMENT, "%s: bad size", who);
     const int64_t n = rows * K;
     if (n == 0) return MXQ_OK;
@@ -497,8 +515,9 @@ int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, voi
     hipStream_t s = (hipStream_t)hip_stream;
     const int grid = grid_for(ceil_div(n, kThreads * 4));
 #define MXQ_UNPACK(DT)                                                                       \
-    if (codes_are_e5m2) mx_unpack_kernel<DT, true><<<grid, kThreads, 0, s>>>(cd, sc, out, n); \
-    else mx_unpack_kernel<DT, false><<<grid, kThreads, 0, s>>>(cd, sc, out, n);
+    if (code_kind == 1) mx_unpack_kernel<DT, 1><<<grid, kThreads, 0, s>>>(cd, sc, out, n);      \
+    else if (code_kind == 4) mx_unpack_kernel<DT, 4><<<grid, kThreads, 0, s>>>(cd, sc, out, n); \
+    else mx_unpack_kernel<DT, 0><<<grid, kThreads, 0, s>>>(cd, sc, out, n);
     if (dtype == MXQ_DTYPE_F32) { MXQ_UNPACK(MXQ_F32) }
     else if (dtype == MXQ_DTYPE_BF16) { MXQ_UNPACK(MXQ_BF16) }
     else { MXQ_UNPACK(MXQ_F16) }
@@ -506,8 +525,8 @@ int mxq_unpack_mx(const void* codes, const void* scales, int codes_are_e5m2, voi
     return check_launch(who);
 }
 
-int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, const void* b_codes,
-                   const void* b_scales, int b_is_e5m2, const void* bias, void* c, int c_dtype,
+int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const void* b_codes,
+                   const void* b_scales, int b_kind, const void* bias, void* c, int c_dtype,
                    int64_t batch, int64_t M, int64_t N, int64_t K, int epilogue_quant,
                    void* hip_stream) {
     const char* who = "mxq_gemm_mx_nt";
@@ -515,7 +534,14 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, con
     if (epilogue_quant != 0 && (epilogue_quant != 1 || c_dtype != MXQ_DTYPE_BF16))
         return fail(MXQ_ERR_ARGUMENT, "%s: epilogue_quant must be 0, or 1 with a bf16 output", who);
     if (batch < 0 || M < 0 || N < 0 || K < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
-    if (K % GEMM_BK != 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be a multiple of %d", who, GEMM_BK);
+    const bool nib = a_kind == MXQ_CODES_E2M1;
+    if ((a_kind != MXQ_CODES_E4M3 && a_kind != MXQ_CODES_E5M2 && a_kind != MXQ_CODES_E2M1) ||
+        (b_kind != MXQ_CODES_E4M3 && b_kind != MXQ_CODES_E5M2 && b_kind != MXQ_CODES_E2M1))
+        return fail(MXQ_ERR_ARGUMENT, "%s: unknown code kind %d / %d", who, a_kind, b_kind);
+    if (nib != (b_kind == MXQ_CODES_E2M1))
+        return fail(MXQ_ERR_ARGUMENT, "%s: e2m1 nibble codes need both operands in that form", who);
+    const int kstep = nib ? 2 * GEMM_BK : GEMM_BK;      // elements in a 128-byte K step
+    if (K % kstep != 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be a multiple of %d", who, kstep);
     if (batch == 0 || M == 0 || N == 0) return MXQ_OK;
     if (K == 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be positive", who);
     if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF || batch > 65535)
@@ -539,25 +565,32 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_is_e5m2, con
         g.q_nan_from = q.fmt.nan_from;
     }
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
-    g.batch_a = M * K; g.batch_sa = M * (K / 32);
-    g.batch_b = N * K; g.batch_sb = N * (K / 32);
+    g.kbytes = (int)(nib ? K / 2 : K);
+    g.batch_a = M * g.kbytes; g.batch_sa = M * (K / 32);
+    g.batch_b = N * g.kbytes; g.batch_sb = N * (K / 32);
     g.batch_c = M * N;
     hipStream_t s = (hipStream_t)hip_stream;
     int rc;
-    if (!a_is_e5m2 && !b_is_e5m2) rc = launch_gemm<0, 0>(c_dtype, batch, g, s);
-    else if (a_is_e5m2 && !b_is_e5m2) rc = launch_gemm<1, 0>(c_dtype, batch, g, s);
-    else if (!a_is_e5m2 && b_is_e5m2) rc = launch_gemm<0, 1>(c_dtype, batch, g, s);
+    if (nib) rc = launch_gemm<4, 4>(c_dtype, batch, g, s);
+    else if (!a_kind && !b_kind) rc = launch_gemm<0, 0>(c_dtype, batch, g, s);
+    else if (a_kind && !b_kind) rc = launch_gemm<1, 0>(c_dtype, batch, g, s);
+    else if (!a_kind && b_kind) rc = launch_gemm<0, 1>(c_dtype, batch, g, s);
     else rc = launch_gemm<1, 1>(c_dtype, batch, g, s);
     if (rc) return rc;
     return check_launch(who);
 }
 
-int mxq_probe_mfma_rate(int64_t workgroups, int iters, void* sink, void* hip_stream) {
+int mxq_probe_mfma_rate(int64_t workgroups, int iters, int code_kind, void* sink, void* hip_stream) {
     const char* who = "mxq_probe_mfma_rate";
-    if (workgroups <= 0 || workgroups > 0x7FFFFFFF || iters <= 0 || !sink)
+    if (workgroups <= 0 || workgroups > 0x7FFFFFFF || iters <= 0 || !sink ||
+        (code_kind != MXQ_CODES_E4M3 && code_kind != MXQ_CODES_E2M1))
         return fail(MXQ_ERR_ARGUMENT, "%s: bad argument", who);
-    mfma_rate_probe_kernel<<<(unsigned)workgroups, kThreads, 0, (hipStream_t)hip_stream>>>(
-        iters, reinterpret_cast<float*>(sink));
+    if (code_kind == MXQ_CODES_E2M1)
+        mfma_rate_probe_kernel<4><<<(unsigned)workgroups, kThreads, 0, (hipStream_t)hip_stream>>>(
+            iters, reinterpret_cast<float*>(sink));
+    else
+        mfma_rate_probe_kernel<0><<<(unsigned)workgroups, kThreads, 0, (hipStream_t)hip_stream>>>(
+            iters, reinterpret_cast<float*>(sink));
     return check_launch(who);
 }
 

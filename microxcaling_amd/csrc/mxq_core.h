@@ -255,6 +255,19 @@ MXQ_HD float mxq_decode_e5m2(uint32_t c) {
     return (c & 0x80u) ? -v : v;
 }
 
+// OCP e2m1 (fp4) code of a value that the format represents exactly: 0, 0.5, 1, 1.5, 2, 3, 4, 6
+MXQ_HD uint32_t mxq_encode_e2m1(float y) {
+    const uint32_t u = mxq_bits(y), ua = u & 0x7FFFFFFFu;
+    const uint32_t normal = (ua >> 22) - 252u;                      // ((e + 1) << 1) | mantissa bit
+    const uint32_t subnormal = (uint32_t)(mxq_float(ua) * 2.0f);    // 0 or 0.5
+    return ((u >> 28) & 0x8u) | (ua >= 0x3F800000u ? normal : subnormal);
+}
+MXQ_HD float mxq_decode_e2m1(uint32_t c) {
+    const uint32_t e = (c >> 1) & 3u, m = c & 1u;
+    const float v = e ? ldexpf((float)(2u + m), (int)e - 2) : 0.5f * (float)m;
+    return (c & 0x8u) ? -v : v;
+}
+
 // E8M0 byte of a block scale: exponent + 127, 255 for a NaN block (MxqScale.scale is NaN)
 MXQ_HD uint32_t mxq_encode_e8m0(float scale) {
     const uint32_t u = mxq_bits(scale);

@@ -24,7 +24,16 @@ namespace {
 // ================================================================================================
 // quantize + pack, shared axis innermost, block size 32
 // ================================================================================================
-template <int DT, int RMODE, bool ZONE_ELEM, bool BF8, int UNROLL>
+// KIND of the codes: 0 = OCP e4m3 bytes, 1 = OCP e5m2 bytes, 4 = OCP e2m1 nibbles (two per byte, the
+// element with the lower K index in the low nibble)
+template <int KIND>
+__device__ __forceinline__ uint32_t mx_encode(float y) {
+    if (KIND == 1) return mxq_encode_e5m2(y);
+    if (KIND == 4) return mxq_encode_e2m1(y);
+    return mxq_encode_e4m3(y);
+}
+
+template <int DT, int RMODE, bool ZONE_ELEM, int KIND, int UNROLL>
 __global__ __launch_bounds__(TPB) void mx_pack_kernel(const u32x4* __restrict__ in,
                                                       void* __restrict__ codes_,
                                                       unsigned char* __restrict__ scales,
@@ -58,12 +67,16 @@ __global__ __launch_bounds__(TPB) void mx_pack_kernel(const u32x4* __restrict__ 
                 for (int h = 0; h < PD; ++h) {
                     const float y = mxq_quant_mx_elem_unscaled<RMODE, ADT, ZONE_ELEM>(
                         Pack<DT>::get(v[j][d], h), sc, p.fmt, zone, ZS);
-                    const uint32_t c = BF8 ? mxq_encode_e5m2(y) : mxq_encode_e4m3(y);
+                    const uint32_t c = mx_encode<KIND>(y);
                     const int e = d * PD + h;              // element index inside the vector
-                    out[e / 4] |= c << (8 * (e % 4));
+                    if (KIND == 4) out[0] |= c << (4 * e);
+                    else out[e / 4] |= c << (8 * (e % 4));
                 }
             if (i < n_vec) {
-                if (PD == 1) reinterpret_cast<uint32_t*>(codes_)[i] = out[0];
+                if (KIND == 4) {
+                    if (PD == 1) reinterpret_cast<unsigned short*>(codes_)[i] = (unsigned short)out[0];
+                    else reinterpret_cast<uint32_t*>(codes_)[i] = out[0];
+                } else if (PD == 1) reinterpret_cast<uint32_t*>(codes_)[i] = out[0];
                 else reinterpret_cast<u32x2*>(codes_)[i] = u32x2{out[0], out[PD - 1]};
                 if ((threadIdx.x & (LPT - 1)) == 0)
                     scales[i / LPT] = (unsigned char)mxq_encode_e8m0(sc.scale);
@@ -79,7 +92,7 @@ __global__ __launch_bounds__(TPB) void mx_pack_kernel(const u32x4* __restrict__ 
 // A lane keeps a 32-row x 8-byte column strip in registers (like mx_strided_tile_kernel) and writes,
 // per column, the 32 codes of the block as 32 contiguous bytes.
 // ================================================================================================
-template <int DT, int RMODE, bool ZONE_ELEM, bool BF8>
+template <int DT, int RMODE, bool ZONE_ELEM, int KIND>
 __global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict__ in,
                                                         unsigned char* __restrict__ codes,
                                                         unsigned char* __restrict__ scales,
@@ -124,14 +137,20 @@ __global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict_
         for (int r = 0; r < ROWS; ++r) {
             const float y = mxq_quant_mx_elem_unscaled<RMODE, ADT, ZONE_ELEM>(
                 Pack<DT>::get(raw[r][k / PD], k % PD), sc, p.fmt, zone, ZS);
-            const uint32_t code = BF8 ? mxq_encode_e5m2(y) : mxq_encode_e4m3(y);
-            out[r / 4] |= code << (8 * (r % 4));
+            const uint32_t code = mx_encode<KIND>(y);
+            if (KIND == 4) out[r / 8] |= code << (4 * (r % 8));
+            else out[r / 4] |= code << (8 * (r % 4));
         }
         if (live) {
             const int64_t col = c * VW + k;
-            u32x4* dst = reinterpret_cast<u32x4*>(codes + (pre_i * C + col) * R + tile_i * ROWS);
-            dst[0] = u32x4{out[0], out[1], out[2], out[3]};
-            dst[1] = u32x4{out[4], out[5], out[6], out[7]};
+            if (KIND == 4) {
+                *reinterpret_cast<u32x4*>(codes + ((pre_i * C + col) * R + tile_i * ROWS) / 2) =
+                    u32x4{out[0], out[1], out[2], out[3]};
+            } else {
+                u32x4* dst = reinterpret_cast<u32x4*>(codes + (pre_i * C + col) * R + tile_i * ROWS);
+                dst[0] = u32x4{out[0], out[1], out[2], out[3]};
+                dst[1] = u32x4{out[4], out[5], out[6], out[7]};
+            }
             scales[(pre_i * C + col) * n_tiles + tile_i] = (unsigned char)mxq_encode_e8m0(sc.scale);
         }
     }
@@ -139,13 +158,15 @@ __global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict_
 
 // unpack: codes * 2^(scale-127) -> fp32 / bf16 / fp16 (for tests and for callers that want the
 // fake-quantized view of a packed tensor)
-template <int DT, bool BF8>
+template <int DT, int KIND>
 __global__ __launch_bounds__(TPB) void mx_unpack_kernel(const unsigned char* __restrict__ codes,
                                                         const unsigned char* __restrict__ scales,
                                                         void* __restrict__ out, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (int64_t)gridDim.x * TPB) {
         const uint32_t s = scales[i >> 5];
-        const float y = BF8 ? mxq_decode_e5m2(codes[i]) : mxq_decode_e4m3(codes[i]);
+        float y;
+        if (KIND == 4) y = mxq_decode_e2m1((codes[i >> 1] >> (4 * (i & 1))) & 15u);
+        else y = (KIND == 1) ? mxq_decode_e5m2(codes[i]) : mxq_decode_e4m3(codes[i]);
         float v = y * ldexpf(1.0f, (int)s - 127);
         if (s == 255u) v = mxq_float(MXQ_QNAN_BITS);
         store_scalar<DT>(out, i, mxq_round_dt<Arith<DT>::DT_>(v));
@@ -160,6 +181,7 @@ __global__ __launch_bounds__(TPB) void mx_unpack_kernel(const unsigned char* __r
 // ================================================================================================
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int GEMM_BM = 128, GEMM_BN = 128, GEMM_BK = 128, GEMM_PITCH = GEMM_BK + 16;
 
@@ -174,7 +196,8 @@ struct GemmArgs {
                           // round-half-away, after the product and again after the bias add (the
                           // closed form mxq_quant_bf16_to_bfloat16_nearest with this threshold)
     int M, N, K;
-    int64_t batch_a, batch_sa, batch_b, batch_sb, batch_c;   // element strides between batches
+    int kbytes;           // bytes of codes per row: K (8-bit codes) or K / 2 (e2m1 nibbles)
+    int64_t batch_a, batch_sa, batch_b, batch_sb, batch_c;   // strides between batches (bytes / elements of C)
 };
 
 // Which output tile a workgroup computes.  Workgroups are dealt round-robin to the 8 XCDs, each
@@ -201,6 +224,47 @@ __device__ __forceinline__ v8i load_frag(const unsigned char* p) {
     const u32x4 lo = *reinterpret_cast<const u32x4*>(p);
     const u32x4 hi = *reinterpret_cast<const u32x4*>(p + 64);
     return v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+}
+
+// One K = 128 MFMA.  e2m1 operands (CBSZ = BLGP = 4) are 16 bytes per lane: the fragment a lane reads
+// for a 128-byte K step (16 bytes at p, 16 at p + 64) then holds the operands of *two* MFMAs, K
+// 0..127 in registers 0-3 (HALF = 0) and K 128..255 in registers 4-7 (HALF = 1).
+template <int CBSZ, int BLGP, int HALF>
+__device__ __forceinline__ v4f mx_mfma(const v8i& b, const v8i& a, v4f c, int sb, int sa) {
+    if constexpr (CBSZ == 4) {
+        const v8i b4 = {b[4 * HALF], b[4 * HALF + 1], b[4 * HALF + 2], b[4 * HALF + 3], 0, 0, 0, 0};
+        const v8i a4 = {a[4 * HALF], a[4 * HALF + 1], a[4 * HALF + 2], a[4 * HALF + 3], 0, 0, 0, 0};
+        return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b4, a4, c, 4, 4, 0, sb, 0, sa);
+    } else {
+        return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b, a, c, BLGP, CBSZ, 0, sb, 0, sa);
+    }
+}
+
+// One 32 x 32 x 64 MFMA of the large-tile kernel: operand registers and scale byte of MFMA h of a
+// K step out of the four 16-byte reads r[0..3] of a lane (see the kernel).  `sb`, `sa` hold the
+// row's scale bytes shifted so that this lane's block comes first; op_sel picks byte 0 or 2.
+template <int CBSZ, int BLGP, class Frag, class Scales>
+__device__ __forceinline__ v16f mx_mfma32(const Frag& b, const Frag& a, v16f c, const Scales& sb,
+                                          const Scales& sa, int h) {
+    if constexpr (CBSZ == 4) {
+#define MXQ_MMA4(H)                                                                                       \
+    __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                                                      \
+        v8i{(int)b.r[H][0], (int)b.r[H][1], (int)b.r[H][2], (int)b.r[H][3], 0, 0, 0, 0},                  \
+        v8i{(int)a.r[H][0], (int)a.r[H][1], (int)a.r[H][2], (int)a.r[H][3], 0, 0, 0, 0}, c, 4, 4,          \
+        ((H) & 1) * 2, sb.w[(H) >> 1], ((H) & 1) * 2, sa.w[(H) >> 1])
+        return h == 0 ? MXQ_MMA4(0) : h == 1 ? MXQ_MMA4(1) : h == 2 ? MXQ_MMA4(2) : MXQ_MMA4(3);
+#undef MXQ_MMA4
+    } else {
+#define MXQ_MMA8(H)                                                                                       \
+    __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                                                      \
+        v8i{(int)b.r[2 * H][0], (int)b.r[2 * H][1], (int)b.r[2 * H][2], (int)b.r[2 * H][3],               \
+            (int)b.r[2 * H + 1][0], (int)b.r[2 * H + 1][1], (int)b.r[2 * H + 1][2], (int)b.r[2 * H + 1][3]}, \
+        v8i{(int)a.r[2 * H][0], (int)a.r[2 * H][1], (int)a.r[2 * H][2], (int)a.r[2 * H][3],               \
+            (int)a.r[2 * H + 1][0], (int)a.r[2 * H + 1][1], (int)a.r[2 * H + 1][2], (int)a.r[2 * H + 1][3]}, \
+        c, BLGP, CBSZ, (H) * 2, sb.w[0], (H) * 2, sa.w[0])
+        return h == 0 ? MXQ_MMA8(0) : MXQ_MMA8(1);
+#undef MXQ_MMA8
+    }
 }
 
 // The MFMAs are issued with the B fragment as the first operand, i.e. they compute 16 x 16 blocks
@@ -286,10 +350,12 @@ __device__ __forceinline__ void store_c8(void* c, const void* bias, uint32_t q_n
 template <int CBSZ, int BLGP, int OUT_DT>
 __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     constexpr bool PAIR = OUT_DT != MXQ_F32;
+    constexpr int EPB = (CBSZ == 4) ? 2 : 1;                 // elements per byte of codes
+    constexpr int SBY = 4 * EPB;                             // scale bytes per row and 128-byte K step
     __shared__ __attribute__((aligned(16))) unsigned char As[GEMM_BM * GEMM_PITCH];
     __shared__ __attribute__((aligned(16))) unsigned char Bs[GEMM_BN * GEMM_PITCH];
-    __shared__ __attribute__((aligned(16))) unsigned char sAs[GEMM_BM * 4];
-    __shared__ __attribute__((aligned(16))) unsigned char sBs[GEMM_BN * 4];
+    __shared__ __attribute__((aligned(16))) unsigned char sAs[GEMM_BM * SBY];
+    __shared__ __attribute__((aligned(16))) unsigned char sBs[GEMM_BN * SBY];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wy = wave >> 1, wx = wave & 1;
@@ -320,8 +386,8 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
         ld_col[j] = (c & 7) * 16;
         const int gm = min(m0 + ld_row[j], g.M - 1);         // rows past the edge are never stored
         const int gn = min(n0 + ld_row[j], g.N - 1);
-        ga[j] = (int64_t)gm * g.K + ld_col[j];
-        gb[j] = (int64_t)gn * g.K + ld_col[j];
+        ga[j] = (int64_t)gm * g.kbytes + ld_col[j];
+        gb[j] = (int64_t)gn * g.kbytes + ld_col[j];
     }
     const int srow = tid & 127;
     const bool s_is_a = tid < 128;
@@ -330,14 +396,16 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
 
     const int frow = lane & 15, fg = lane >> 4;
     u32x4 va[4], vb[4];
-    uint32_t sv;
-    auto fetch = [&](int k0) {
+    uint32_t sv[EPB];
+    auto fetch = [&](int k0) {                               // k0: byte offset of the K step in a row
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             va[j] = *reinterpret_cast<const u32x4*>(A + ga[j] + k0);
             vb[j] = *reinterpret_cast<const u32x4*>(B + gb[j] + k0);
         }
-        sv = *reinterpret_cast<const uint32_t*>((s_is_a ? SA : SB) + gs + (k0 >> 5));
+#pragma unroll
+        for (int e = 0; e < EPB; ++e)
+            sv[e] = *reinterpret_cast<const uint32_t*>((s_is_a ? SA : SB) + gs + ((k0 * EPB) >> 5) + 4 * e);
     };
     auto stash = [&]() {
 #pragma unroll
@@ -345,10 +413,12 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
             *reinterpret_cast<u32x4*>(As + ld_row[j] * GEMM_PITCH + ld_col[j]) = va[j];
             *reinterpret_cast<u32x4*>(Bs + ld_row[j] * GEMM_PITCH + ld_col[j]) = vb[j];
         }
-        *reinterpret_cast<uint32_t*>((s_is_a ? sAs : sBs) + srow * 4) = sv;
+#pragma unroll
+        for (int e = 0; e < EPB; ++e)
+            *reinterpret_cast<uint32_t*>((s_is_a ? sAs : sBs) + srow * SBY + 4 * e) = sv[e];
     };
     // K is walked cyclically from a per-workgroup starting step (see the 256 x 256 kernel)
-    const int nk = g.K / GEMM_BK;
+    const int nk = g.kbytes / GEMM_BK;
     const int kstart = (int)((blockIdx.x * 5u + blockIdx.y) % (unsigned)nk);
     auto kof = [&](int step) { return ((kstart + step) % nk) * GEMM_BK; };
     fetch(kof(0));
@@ -361,7 +431,7 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
         __builtin_amdgcn_sched_barrier(0);
 
         v8i bf[4];
-        int sb[4];
+        int sb[4][EPB];
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) {
             // 16-bit outputs: fragment rows permuted so that a lane owns 8 consecutive columns per
@@ -369,17 +439,24 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
             const int n = wx * 64 + (PAIR ? (tj >> 1) * 32 + (frow >> 2) * 8 + (tj & 1) * 4 + (frow & 3)
                                           : tj * 16 + frow);
             bf[tj] = load_frag(Bs + n * GEMM_PITCH + fg * 16);
-            sb[tj] = sBs[n * 4 + fg];
+#pragma unroll
+            for (int e = 0; e < EPB; ++e) sb[tj][e] = sBs[n * SBY + 4 * e + fg];
         }
 #pragma unroll
         for (int ti = 0; ti < 4; ++ti) {
             const int m = wy * 64 + ti * 16 + frow;
             const v8i af = load_frag(As + m * GEMM_PITCH + fg * 16);
-            const int sa = sAs[m * 4 + fg];
+            int sa[EPB];
+#pragma unroll
+            for (int e = 0; e < EPB; ++e) sa[e] = sAs[m * SBY + 4 * e + fg];
 #pragma unroll
             for (int tj = 0; tj < 4; ++tj)
-                acc[ti][tj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    bf[tj], af, acc[ti][tj], BLGP, CBSZ, 0, sb[tj], 0, sa);
+                acc[ti][tj] = mx_mfma<CBSZ, BLGP, 0>(bf[tj], af, acc[ti][tj], sb[tj][0], sa[0]);
+            if constexpr (EPB == 2) {
+#pragma unroll
+                for (int tj = 0; tj < 4; ++tj)
+                    acc[ti][tj] = mx_mfma<CBSZ, BLGP, 1>(bf[tj], af, acc[ti][tj], sb[tj][1], sa[1]);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();                                     // every wave is done with this tile
@@ -410,8 +487,10 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
 constexpr int G2_BM = 256, G2_BN = 256;
 
 // ================================================================================================
-// Main GEMM kernel: persistent workgroups, tile 256 x 256 x 128, 512 lanes = 4 x 2 waves, wave tile
-// 64 x 128 = 4 x 8 MFMA tiles (128 accumulator registers, two waves per SIMD).
+// Main GEMM kernel: persistent workgroups, tile 256 x 256 x 128 bytes of K, 512 lanes = 4 x 2 waves,
+// wave tile 64 x 128 = 2 x 4 MFMA tiles of 32 x 32 (128 accumulator registers, two waves per SIMD).
+// 32 x 32 x 64 MFMAs because the matrix pipes cannot be kept busy with 16 x 16 x 128 ones on 4-bit
+// operands (a register-resident loop of those reaches 5-7 PFLOP/s, of 32 x 32 x 64 ones 9.2-9.5).
 //
 // Tile copy: global_load_lds_dwordx4 -- the memory pipe writes 16 bytes per lane straight into LDS
 // (lane L of a wave lands at base + 16 L), so there are no staging registers and no ds_write
@@ -419,7 +498,7 @@ constexpr int G2_BM = 256, G2_BN = 256;
 // the 16-byte column c of row r is kept at position c ^ ((r >> 1) & 7), which makes the 16-byte
 // fragment reads of 16 consecutive rows hit 16 different bank groups, and the lanes pick their
 // global address so that the linear landing order produces exactly this image.  The loads of step
-// t + 1 are issued inside step t, spread over its MFMA groups.
+// t + 1 are issued inside step t, behind its first three MFMA groups.
 //
 // Scales: one byte per row and 32 K, i.e. 4 bytes per row and K step, each row in a different
 // cache line.  Fetching them per step would double the number of L2 requests of the kernel, so a
@@ -436,7 +515,6 @@ constexpr int G3_STAGE_BYTES = 2 * G3_TILE_BYTES;            // codes of A and B
 constexpr int G3_SCALE_OFF = 2 * G3_STAGE_BYTES;
 constexpr int G3_SCALE_GROUP = 512 * 16;                     // 512 rows x 4 K steps x 4 bytes
 constexpr int G3_LDS_BYTES = G3_SCALE_OFF + 2 * G3_SCALE_GROUP;
-constexpr int G3_SPREAD = 6;        // the loads of the next step go out during the first 6 MFMA groups
 
 __device__ __forceinline__ void dma16(uint32_t lds_base, uint32_t voff, const unsigned char* sbase) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -451,28 +529,34 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wy = wave >> 1, wx = wave & 1;
+    constexpr int EPB = (CBSZ == 4) ? 2 : 1;                 // elements per byte of codes
+    constexpr int SBY = 4 * EPB;                             // scale bytes per row and K step
+    constexpr int GS = 16 / SBY;                             // K steps covered by a 16-byte scale group
     const int KB = g.K >> 5;
-    const int nk = g.K / GEMM_BK;
+    const int nk = g.kbytes / GEMM_BK;
     const int per_batch = tiles_m * tiles_n;
     const int G = gridDim.x;
 
-    v4f acc[4][8];
+    v16f acc[2][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    // Which rows of B make up MFMA fragment tj decides which columns of C a lane ends up with (it
-    // gets n_local = 4 (lane / 16) + 0..3 of every fragment).  For 16-bit outputs fragment tj, row i
-    // is B row (tj / 2) * 32 + (i / 4) * 8 + (tj % 2) * 4 + i % 4: a lane then owns 8 consecutive
-    // columns per fragment pair, and one store instruction writes 64 contiguous bytes per row
-    // (half as many write requests as 4 columns per lane).  fp32 outputs keep rows 16 tj + i
-    // (4 columns = 16 bytes per lane, 64 contiguous bytes per row as well).
+    // The MFMAs are 32 x 32 x 64 with the B fragment as the first operand: lane L, accumulator
+    // register v then holds C[m = L % 32][n = fragment row 8 (v / 4) + 4 (L / 32) + v % 4].  Which
+    // rows of B make up the fragment decides which columns a lane ends up with.  fp32 outputs keep
+    // fragment row i = B row i: 4 consecutive columns (16 bytes) per register quad.  For 16-bit
+    // outputs fragment row i = 8 q + 4 h + r is B row 16 (q / 2) + 8 h + 4 (q % 2) + r, so that two
+    // register quads of a lane are 8 consecutive columns: one 16-byte store.
     constexpr bool PAIR = OUT_DT != MXQ_F32;
-    // position of 16-byte column c of row r inside its LDS row: c ^ key(r); the key must take 8
-    // different values over the even rows of a fragment (and again over the odd ones)
+    // position of 16-byte column c of row r inside its LDS row: c ^ key(r); the key takes 8
+    // different values over the even rows of any 16 consecutive rows (and again over the odd ones),
+    // which is what a 16-byte read by 16 lanes needs to touch every bank once
     auto key_a = [](int r) { return (r >> 1) & 7; };
-    auto key_b = [](int r) { return PAIR ? ((r >> 1) & 1) | (((r >> 3) & 3) << 1) : (r >> 1) & 7; };
+    auto key_b = key_a;
 
     // ---- fetch side: which tile the tile copy is working on --------------------------------------
     // Wave w brings in rows 32 w .. 32 w + 31 of A and of B, 8 rows per instruction; lane L lands at
@@ -488,19 +572,19 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
         int tm, tn;
         tile_of_workgroup(logical % per_batch, per_batch, tiles_m, tiles_n, &tm, &tn);
         const int m0 = tm * G2_BM, n0 = tn * G2_BN;
-        fA = g.a + bz * g.batch_a + (int64_t)m0 * g.K;
-        fB = g.b + bz * g.batch_b + (int64_t)n0 * g.K;
+        fA = g.a + bz * g.batch_a + (int64_t)m0 * g.kbytes;
+        fB = g.b + bz * g.batch_b + (int64_t)n0 * g.kbytes;
         fS = s_is_b ? g.sb + bz * g.batch_sb + (int64_t)n0 * KB : g.sa + bz * g.batch_sa + (int64_t)m0 * KB;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = wave * 32 + i * 8 + (lane >> 3);
-            offa[i] = (uint32_t)min(r, g.M - 1 - m0) * (uint32_t)g.K + ((lane & 7) ^ key_a(r)) * 16;
-            offb[i] = (uint32_t)min(r, g.N - 1 - n0) * (uint32_t)g.K + ((lane & 7) ^ key_b(r)) * 16;
+            offa[i] = (uint32_t)min(r, g.M - 1 - m0) * (uint32_t)g.kbytes + ((lane & 7) ^ key_a(r)) * 16;
+            offb[i] = (uint32_t)min(r, g.N - 1 - n0) * (uint32_t)g.kbytes + ((lane & 7) ^ key_b(r)) * 16;
         }
         offs = (uint32_t)min(s_row, (s_is_b ? g.N - n0 : g.M - m0) - 1) * (uint32_t)KB;
         // Every tile walks K cyclically from its own starting step (a multiple of four), so that
         // the K slices in flight at any moment are spread over the memory channels.
-        f_kstart = (int)(((unsigned)logical * 5u) % (unsigned)(nk >> 2)) << 2;
+        f_kstart = (int)(((unsigned)logical * 5u) % (unsigned)(nk / GS)) * GS;
     };
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;     // LDS byte address of the array (normally 0)
     // load i (0..7 codes, 8 scales) of flat step t, which is K step fs of the fetch-side tile
@@ -513,58 +597,80 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
             dma16(st + (wave * 32 + i * 8) * 128, offa[i], fA + k0);
         } else if (i < 8) {
             dma16(st + G3_TILE_BYTES + (wave * 32 + (i - 4) * 8) * 128, offb[i - 4], fB + k0);
-        } else if ((t & 3) == 0) {                          // a new group of four K steps
-            dma16(lds0 + G3_SCALE_OFF + ((t >> 2) & 1) * G3_SCALE_GROUP + wave * 1024, offs, fS + (k0 >> 5));
+        } else if (t % GS == 0) {                           // a new group of GS K steps
+            dma16(lds0 + G3_SCALE_OFF + ((t / GS) & 1) * G3_SCALE_GROUP + wave * 1024, offs,
+                  fS + ((k0 * EPB) >> 5));
         }
     };
 
     // ---- compute side ---------------------------------------------------------------------------
-    const int frow = lane & 15, fg = lane >> 4;
-    const int a_lane = wy * 64 + frow;                                        // row of A fragment 0
-    const int b_lane = wx * 128 + (PAIR ? (frow >> 2) * 8 + (frow & 3) : frow);  // row of B fragment 0
-    auto b_step = [](int tj) { return PAIR ? (tj >> 1) * 32 + (tj & 1) * 4 : tj * 16; };
-    const int pa_lo = (fg ^ key_a(a_lane)) * 16, pb_lo = (fg ^ key_b(b_lane)) * 16;   // same for all fragments
-    const int a_row = a_lane * 128, b_row = G3_TILE_BYTES + b_lane * 128;
-    const int sa_off = G3_SCALE_OFF + a_lane * 16 + fg;
-    const int sb_off = G3_SCALE_OFF + 4096 + b_lane * 16 + fg;
-    auto frag = [&](const unsigned char* row, int p_lo) {
-        const u32x4 lo = *reinterpret_cast<const u32x4*>(row + p_lo);
-        const u32x4 hi = *reinterpret_cast<const u32x4*>(row + (p_lo ^ 64));
-        return v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    // A K step is 128 bytes per row: two (8-bit codes) or four (nibbles) K = 64 MFMAs per pair of
+    // fragments.  Lane (i = L % 32, g = L / 32) reads the 16-byte columns 2 q + g, q = 0..3, of its
+    // row: 8-bit MFMA h takes columns 4 h + g and 4 h + 2 + g (K 16 g.. and 32 + 16 g.. of its 64),
+    // nibble MFMA h takes column 2 h + g (K 32 g.. of its 64).  The lane's scale is the one of block
+    // g of the MFMA's two blocks, i.e. byte 2 h + g of the row's scale bytes for this step.
+    constexpr int NH = 2 * EPB;                              // MFMAs per fragment pair and K step
+    const int fi = lane & 31, fg = lane >> 5;
+    const int a_lane = wy * 64 + fi;                                          // row of A fragment 0
+    const int b_lane = wx * 128 + (PAIR ? (fi & 16) + ((fi & 4) << 1) + ((fi & 8) >> 1) + (fi & 3) : fi);
+    int a_addr[4], b_addr[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        a_addr[q] = a_lane * 128 + ((fg ^ key_a(a_lane) ^ (2 * q)) * 16);
+        b_addr[q] = G3_TILE_BYTES + b_lane * 128 + ((fg ^ key_b(b_lane) ^ (2 * q)) * 16);
+    }
+    const int sa_off = G3_SCALE_OFF + a_lane * 16;
+    const int sb_off = G3_SCALE_OFF + 4096 + b_lane * 16;
+    const int sshift = fg * 8;
+    struct Frag { u32x4 r[4]; };
+    auto frag = [&](const unsigned char* stage, const int* addr, int tile) {
+        Frag f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) f.r[q] = *reinterpret_cast<const u32x4*>(stage + addr[q] + tile * 32 * 128);
+        return f;
+    };
+    struct Scales { int w[EPB]; };
+    auto scales = [&](const unsigned char* p) {              // the row's scale bytes, this lane's block first
+        Scales sc;
+#pragma unroll
+        for (int e = 0; e < EPB; ++e) sc.w[e] = (int)(reinterpret_cast<const uint32_t*>(p)[e] >> sshift);
+        return sc;
     };
     // flat step t: multiply the stage t & 1 while the tile copy fills the other one with K step
     // fs of the fetch-side tile
     auto step = [&](int t, int fs) {
         const unsigned char* cur = lds + (t & 1) * G3_STAGE_BYTES;
-        const unsigned char* sc = lds + ((t >> 2) & 1) * G3_SCALE_GROUP + (t & 3) * 4;
-        v8i af[4];
-        int sa[4];
+        const unsigned char* sc = lds + ((t / GS) & 1) * G3_SCALE_GROUP + (t % GS) * SBY;
+        Frag af[2];
+        Scales sa[2];
 #pragma unroll
-        for (int ti = 0; ti < 4; ++ti) {
-            af[ti] = frag(cur + a_row + ti * 16 * 128, pa_lo);
-            sa[ti] = sc[sa_off + ti * 256];
+        for (int ti = 0; ti < 2; ++ti) {
+            af[ti] = frag(cur, a_addr, ti);
+            sa[ti] = scales(sc + sa_off + ti * 512);
         }
-        v8i bf = frag(cur + b_row, pb_lo);
-        int sb = sc[sb_off];
+        Frag bf = frag(cur, b_addr, 0);
+        Scales sb = scales(sc + sb_off);
 #pragma unroll
-        for (int tj = 0; tj < 8; ++tj) {
-            v8i bf_next = bf;                                // the next B fragment is read in the
-            int sb_next = sb;                                // shadow of this fragment's MFMAs
-            if (tj + 1 < 8) {
-                bf_next = frag(cur + b_row + b_step(tj + 1) * 128, pb_lo);
-                sb_next = sc[sb_off + b_step(tj + 1) * 16];
+        for (int tj = 0; tj < 4; ++tj) {
+            Frag bf_next = bf;                               // the next B fragment is read in the
+            Scales sb_next = sb;                             // shadow of this fragment's MFMAs
+            if (tj + 1 < 4) {
+                bf_next = frag(cur, b_addr, tj + 1);
+                sb_next = scales(sc + sb_off + (tj + 1) * 512);
             }
 #pragma unroll
-            for (int ti = 0; ti < 4; ++ti) {
-                acc[ti][tj] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    bf, af[ti], acc[ti][tj], BLGP, CBSZ, 0, sb, 0, sa[ti]);
-                if (ti == 0) {
+            for (int h = 0; h < NH; ++h)
 #pragma unroll
-                    for (int i = 0; i < 9; ++i)
-                        if (i * G3_SPREAD / 9 == tj) fetch_part(t + 1, fs, i);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
+                for (int ti = 0; ti < 2; ++ti)
+                    acc[ti][tj] = mx_mfma32<CBSZ, BLGP>(bf, af[ti], acc[ti][tj], sb, sa[ti], h);
+            // The tile copy of the next step goes out behind this group's MFMAs, three loads per
+            // group.  The empty asm pins the MFMAs above it: the compiler would otherwise issue
+            // all loads first, and every wave of the workgroup would sit in the memory pipe's
+            // queue at the same time with the matrix pipes idle.
+            asm volatile("" : "+v"(acc[0][tj]), "+v"(acc[1][tj]));
+#pragma unroll
+            for (int i = 0; i < 9; ++i)
+                if (i / 3 == tj) fetch_part(t + 1, fs, i);
             bf = bf_next;
             sb = sb_next;
         }
@@ -598,23 +704,31 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
                             ((uintptr_t)g.c & 15) == 0;
         const bool inside8 = inside && (g.N & 7) == 0 && ((uintptr_t)g.bias & 15) == 0;
 #pragma unroll
-        for (int ti = 0; ti < 4; ++ti)
+        for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
-            for (int tj = 0; tj < 8; ++tj) {
-                const int m = m0 + wy * 64 + ti * 16 + frow;
+            for (int tj = 0; tj < 4; ++tj) {
+                const int m = m0 + wy * 64 + ti * 32 + fi;
+                const int nt = n0 + wx * 128 + tj * 32;
+                const v16f& c = acc[ti][tj];
                 if constexpr (PAIR) {
-                    if (tj & 1)
-                        store_c8<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, n0 + wx * 128 + (tj >> 1) * 32 + fg * 8, g.M,
-                                         g.N, inside8, acc[ti][tj - 1], acc[ti][tj]);
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        store_c8<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, nt + 16 * h + 8 * fg, g.M, g.N, inside8,
+                                         v4f{c[8 * h], c[8 * h + 1], c[8 * h + 2], c[8 * h + 3]},
+                                         v4f{c[8 * h + 4], c[8 * h + 5], c[8 * h + 6], c[8 * h + 7]});
                 } else {
-                    store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, n0 + wx * 128 + tj * 16 + fg * 4, g.M, g.N,
-                                     inside, acc[ti][tj]);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, nt + 8 * q + 4 * fg, g.M, g.N, inside,
+                                         v4f{c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]});
                 }
             }
 #pragma unroll
-        for (int ti = 0; ti < 4; ++ti)
+        for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
-            for (int tj = 0; tj < 8; ++tj) acc[ti][tj] = v4f{0.f, 0.f, 0.f, 0.f};
+            for (int tj = 0; tj < 4; ++tj)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[ti][tj][v] = 0.f;
         if (next >= total) break;
         logical = next;
     }
@@ -622,7 +736,9 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
 
 // Register-resident MFMA loop: every wave issues `iters` x 16 independent scaled MFMAs on operands
 // it never reloads.  Its rate is the practical ceiling of the matrix pipes under this instruction
-// (datasheet: 5 PFLOP/s dense fp8).  `sink` only keeps the compiler from deleting the loop.
+// (datasheet: 5 PFLOP/s dense fp8, 10.1 PFLOP/s fp4).  FMT: 0 e4m3 bytes, 4 e2m1 nibbles.
+// `sink` only keeps the compiler from deleting the loop.
+template <int FMT>
 __global__ __launch_bounds__(TPB) void mfma_rate_probe_kernel(int iters, float* sink) {
     v8i a = {(int)threadIdx.x, 1, 2, 3, 4, 5, 6, 7}, b = {7, 6, 5, 4, 3, 2, 1, (int)blockIdx.x};
     v4f acc[16];
@@ -631,7 +747,7 @@ __global__ __launch_bounds__(TPB) void mfma_rate_probe_kernel(int iters, float* 
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
         for (int i = 0; i < 16; ++i)
-            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[i], 0, 0, 0, 127, 0, 127);
+            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[i], FMT, FMT, 0, 127, 0, 127);
     }
     float t = 0.f;
 #pragma unroll

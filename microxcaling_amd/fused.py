@@ -14,6 +14,9 @@ from .formats import ElemFormat, RoundingMode, _get_format_params
 _PACKABLE = (ElemFormat.fp8_e4m3, ElemFormat.fp8_e5m2, ElemFormat.fp6_e3m2, ElemFormat.fp6_e2m3,
              ElemFormat.fp4)
 GEMM_K_MULTIPLE = 128
+# kinds of element codes (include/mxq.h MXQ_CODES_*): e4m3 bytes, e5m2 bytes, e2m1 nibbles
+CODES_E4M3, CODES_E5M2, CODES_E2M1 = 0, 1, 4
+_FLAG_PACK_NIBBLES = 4
 
 
 def _as_format(fmt):
@@ -22,13 +25,24 @@ def _as_format(fmt):
     return ElemFormat.from_str(fmt) if type(fmt) is str else fmt
 
 
-def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=False):
-    """MX-quantize A along its last axis (block 32) into (codes, scales, codes_are_e5m2):
-    codes uint8 of A's shape, scales uint8 with the last axis divided by 32."""
+def _code_kind(fmt, nibbles, who):
+    if nibbles:
+        if fmt != ElemFormat.fp4:
+            raise RuntimeError("%s: only fp4 elements pack into nibbles (got %s)" % (who, fmt))
+        return CODES_E2M1
+    return CODES_E5M2 if fmt == ElemFormat.fp8_e5m2 else CODES_E4M3
+
+
+def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=False, nibbles=False):
+    """MX-quantize A along its last axis (block 32) into (codes, scales, code_kind): codes uint8 of
+    A's shape (one e4m3 / e5m2 byte per element) or, with nibbles=True (fp4 only), of half the last
+    axis (two e2m1 codes per byte, the lower index in the low nibble); scales uint8 with the last
+    axis divided by 32."""
     who = "pack_mx"
     fmt = _as_format(elem_format)
     if fmt not in _PACKABLE:
         raise RuntimeError("%s: element format %s has no packed form" % (who, fmt))
+    kind = _code_kind(fmt, nibbles, who)
     _check_gpu_input(A, "A", who)
     if A.dtype not in _DTYPE:
         raise RuntimeError("%s: Tensor dtype not supported (%s)" % (who, A.dtype))
@@ -37,26 +51,27 @@ def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=F
         raise RuntimeError("%s: the last axis must be a multiple of 32" % who)
     ebits, mbits, _, max_norm, _ = _get_format_params(fmt)
     rows = A.numel() // K if K else 0
-    codes = torch.empty(A.shape, dtype=torch.uint8, device=A.device)
+    codes = torch.empty(A.shape[:-1] + (K // 2 if nibbles else K,), dtype=torch.uint8, device=A.device)
     scales = torch.empty(A.shape[:-1] + (K // 32,), dtype=torch.uint8, device=A.device)
     lib = _lib.gpu()
     with torch.cuda.device(A.device):
         rc = lib.mxq_pack_mx(A.data_ptr(), codes.data_ptr(), scales.data_ptr(), _DTYPE[A.dtype],
                              rows, K, scale_bits, ebits, mbits, max_norm,
                              int(bool(flush_fp32_subnorms)), int(RoundingMode[round]),
-                             _flags_value(), _stream(A))
+                             _flags_value() | (_FLAG_PACK_NIBBLES if nibbles else 0), _stream(A))
     _lib.check(rc, lib)
-    return codes, scales, fmt == ElemFormat.fp8_e5m2
+    return codes, scales, kind
 
 
-def pack_mx_t(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=False):
+def pack_mx_t(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=False, nibbles=False):
     """MX-quantize A (..., R, C) along its second-to-last axis (block 32) and transpose while
-    packing: codes uint8 (..., C, R), scales uint8 (..., C, R / 32) -- K-major for a contraction
-    over R.  Returns (codes, scales, codes_are_e5m2)."""
+    packing: codes uint8 (..., C, R) (or (..., C, R / 2) e2m1 nibbles), scales uint8
+    (..., C, R / 32) -- K-major for a contraction over R.  Returns (codes, scales, code_kind)."""
     who = "pack_mx_t"
     fmt = _as_format(elem_format)
     if fmt not in _PACKABLE:
         raise RuntimeError("%s: element format %s has no packed form" % (who, fmt))
+    kind = _code_kind(fmt, nibbles, who)
     _check_gpu_input(A, "A", who)
     if A.dtype not in _DTYPE:
         raise RuntimeError("%s: Tensor dtype not supported (%s)" % (who, A.dtype))
@@ -68,37 +83,47 @@ def pack_mx_t(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms
                            "last one of 8 bytes" % (who, tuple(A.shape)))
     ebits, mbits, _, max_norm, _ = _get_format_params(fmt)
     batch = A.numel() // (R * C) if R * C else 0
-    codes = torch.empty(A.shape[:-2] + (C, R), dtype=torch.uint8, device=A.device)
+    codes = torch.empty(A.shape[:-2] + (C, R // 2 if nibbles else R), dtype=torch.uint8, device=A.device)
     scales = torch.empty(A.shape[:-2] + (C, R // 32), dtype=torch.uint8, device=A.device)
     lib = _lib.gpu()
     with torch.cuda.device(A.device):
         rc = lib.mxq_pack_mx_t(A.data_ptr(), codes.data_ptr(), scales.data_ptr(), _DTYPE[A.dtype],
                                batch, R, C, scale_bits, ebits, mbits, max_norm,
                                int(bool(flush_fp32_subnorms)), int(RoundingMode[round]),
-                               _flags_value(), _stream(A))
+                               _flags_value() | (_FLAG_PACK_NIBBLES if nibbles else 0), _stream(A))
     _lib.check(rc, lib)
-    return codes, scales, fmt == ElemFormat.fp8_e5m2
+    return codes, scales, kind
 
 
-def unpack_mx(codes, scales, codes_are_e5m2, dtype=torch.float32):
+def _packed_k(codes, scales, kind, who):
+    """Length of the quantized axis of a packed tensor, after checking that codes and scales fit."""
+    K = scales.shape[-1] * 32
+    if codes.shape[:-1] != scales.shape[:-1] or codes.shape[-1] != (K // 2 if int(kind) == CODES_E2M1 else K):
+        raise RuntimeError("%s: codes %s and scales %s do not belong together (code kind %d)"
+                           % (who, tuple(codes.shape), tuple(scales.shape), int(kind)))
+    return K
+
+
+def unpack_mx(codes, scales, code_kind, dtype=torch.float32):
     """codes * 2^(scales - 127) as a tensor of `dtype` (255 in scales -> NaN block)."""
     who = "unpack_mx"
     _check_gpu_input(codes, "codes", who)
     _check_gpu_input(scales, "scales", who)
-    K = codes.shape[-1]
-    out = torch.empty(codes.shape, dtype=dtype, device=codes.device)
+    K = _packed_k(codes, scales, code_kind, who)
+    out = torch.empty(codes.shape[:-1] + (K,), dtype=dtype, device=codes.device)
     lib = _lib.gpu()
     with torch.cuda.device(codes.device):
-        rc = lib.mxq_unpack_mx(codes.data_ptr(), scales.data_ptr(), int(codes_are_e5m2),
-                               out.data_ptr(), _DTYPE[dtype], codes.numel() // K if K else 0, K,
+        rc = lib.mxq_unpack_mx(codes.data_ptr(), scales.data_ptr(), int(code_kind),
+                               out.data_ptr(), _DTYPE[dtype], out.numel() // K if K else 0, K,
                                _stream(codes))
     _lib.check(rc, lib)
     return out
 
 
 def gemm_nt(a_packed, b_packed, out_dtype=torch.float32, bias=None, epilogue_quant=False):
-    """C[b] = A[b] x B[b]^T (+ bias).  a_packed / b_packed = (codes, scales, is_e5m2) with codes of
-    shape (batch, M, K) / (batch, N, K) or (M, K) / (N, K); bias: (N,) of out_dtype, added after the
+    """C[b] = A[b] x B[b]^T (+ bias).  a_packed / b_packed = (codes, scales, code_kind) as returned
+    by pack_mx, of a (batch, M, K) / (batch, N, K) or (M, K) / (N, K) tensor; e2m1 nibble codes need
+    both operands in that form; bias: (N,) of out_dtype, added after the
     product has been rounded to out_dtype, the sum being rounded again.  epilogue_quant (bf16
     output only): also apply the bfloat16 / round-half-away elementwise quantization after the
     product and after the bias add."""
@@ -106,12 +131,13 @@ def gemm_nt(a_packed, b_packed, out_dtype=torch.float32, bias=None, epilogue_qua
     (ac, asc, ae), (bc, bsc, be) = a_packed, b_packed
     for t, n in ((ac, "a codes"), (asc, "a scales"), (bc, "b codes"), (bsc, "b scales")):
         _check_gpu_input(t, n, who)
-    if ac.dim() != bc.dim() or ac.dim() not in (2, 3) or ac.shape[-1] != bc.shape[-1] \
+    K = _packed_k(ac, asc, ae, who)
+    if ac.dim() != bc.dim() or ac.dim() not in (2, 3) or _packed_k(bc, bsc, be, who) != K \
             or ac.shape[:-2] != bc.shape[:-2]:
         raise RuntimeError("%s: operand shapes %s and %s do not match" % (who, tuple(ac.shape),
                                                                           tuple(bc.shape)))
     batch = ac.shape[0] if ac.dim() == 3 else 1
-    M, N, K = ac.shape[-2], bc.shape[-2], ac.shape[-1]
+    M, N = ac.shape[-2], bc.shape[-2]
     if bias is not None:
         _check_gpu_input(bias, "bias", who)
         if bias.dtype != out_dtype or bias.numel() != N:
@@ -125,6 +151,11 @@ def gemm_nt(a_packed, b_packed, out_dtype=torch.float32, bias=None, epilogue_qua
                                 int(bool(epilogue_quant)), _stream(ac))
     _lib.check(rc, lib)
     return out
+
+
+def _use_nibbles(fa, fb, K):
+    """Two fp4 operands go to the MFMA units as e2m1 nibbles (half the bytes, twice the rate)."""
+    return fa == ElemFormat.fp4 and fb == ElemFormat.fp4 and K % (2 * GEMM_K_MULTIPLE) == 0
 
 
 def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_quant=False):
@@ -164,8 +195,9 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
         return None
     if epilogue_quant and a.dtype != torch.bfloat16:
         return None
-    pa = pack_mx(a2, fa, scale_bits, round, flush)
-    pb = pack_mx(b2, fb, scale_bits, round, flush)
+    nibbles = _use_nibbles(fa, fb, K)
+    pa = pack_mx(a2, fa, scale_bits, round, flush, nibbles)
+    pb = pack_mx(b2, fb, scale_bits, round, flush, nibbles)
     return gemm_nt(pa, pb, out_dtype=a.dtype, bias=bias, epilogue_quant=epilogue_quant).reshape(out_shape)
 
 
@@ -195,18 +227,20 @@ def mx_gemm_operands(operands, mx_specs, out_dtype):
         return None                                   # a transposed batched A cannot be folded into rows
     scale_bits = mx_specs["scale_bits"] if mx_specs["scale_bits"] != 0 else 8
     flush = mx_specs["mx_flush_fp32_subnorms"]
+    nibbles = _use_nibbles(shapes[0][4], shapes[1][4], Ka)
     for (t, _, _, _), (lead, rows, K, transposed, f, rnd) in zip(operands, shapes):
         t = t.contiguous()
-        p = (pack_mx_t if transposed else pack_mx)(t, f, scale_bits, rnd, flush)
+        p = (pack_mx_t if transposed else pack_mx)(t, f, scale_bits, rnd, flush, nibbles)
         packed.append(p)
     (ac, asc, ae), (bc, bsc, be) = packed
+    kb = Ka // 2 if nibbles else Ka                   # bytes of codes per row
     if len(lead_b):                                   # batched x batched
-        batch = ac.numel() // (rows_a * Ka)
+        batch = asc.numel() // (rows_a * (Ka // 32))
         if batch > 65535:
             return None
-        ac, asc = ac.reshape(batch, rows_a, Ka), asc.reshape(batch, rows_a, Ka // 32)
-        bc, bsc = bc.reshape(batch, rows_b, Ka), bsc.reshape(batch, rows_b, Ka // 32)
+        ac, asc = ac.reshape(batch, rows_a, kb), asc.reshape(batch, rows_a, Ka // 32)
+        bc, bsc = bc.reshape(batch, rows_b, kb), bsc.reshape(batch, rows_b, Ka // 32)
     else:                                             # every leading axis of A folds into its rows
-        ac, asc = ac.reshape(-1, Ka), asc.reshape(-1, Ka // 32)
+        ac, asc = ac.reshape(-1, kb), asc.reshape(-1, Ka // 32)
     out = gemm_nt((ac, asc, ae), (bc, bsc, be), out_dtype=out_dtype)
     return out.reshape(tuple(lead_a) + (rows_a, rows_b))

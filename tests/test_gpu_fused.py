@@ -146,6 +146,81 @@ def test_transposing_pack_equals_axis_minus2_quantization(dev, fmt, rnd, dtype, 
     assert_bits_equal(got.contiguous().cpu(), want.cpu(), "pack_mx_t")
 
 
+@pytest.mark.parametrize("rnd", ["nearest", "floor", "even"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_nibble_pack_is_the_fake_quantized_tensor(dev, rnd, dtype):
+    """fp4 elements as e2m1 nibbles (two per byte): unpacking gives the oracle's _quantize_mx output
+    bit for bit, for the row-wise and for the transposing pack; the low nibble is the lower index."""
+    from microxcaling_amd.fused import pack_mx, pack_mx_t, unpack_mx, CODES_E2M1
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(96, 256, generator=g) * torch.exp(3 * torch.randn(96, 256, generator=g))
+    x[3, 40] = float("inf")
+    x[5, 70] = float("nan")
+    x[7, :64] *= 1e-38
+    x[9, :32] = 0.0
+    x[11, :32] = -1e-30 * torch.rand(32, generator=g)
+    x = x.to(dtype)
+    want = O.quantize_mx(x, 8, "fp4_e2m1", axes=[-1], block_size=32, round=rnd)
+    codes, scales, kind = pack_mx(x.to(dev), "fp4_e2m1", 8, rnd, nibbles=True)
+    assert codes.shape == (96, 128) and scales.shape == (96, 8) and kind == CODES_E2M1
+    assert_bits_equal(unpack_mx(codes, scales, kind, dtype), want, "nibbles")
+    # same values as the byte codes, element 2i in the low nibble of byte i
+    bytes_, scales8, kind8 = pack_mx(x.to(dev), "fp4_e2m1", 8, rnd)
+    assert torch.equal(scales8, scales)
+    lut = torch.tensor([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6], device=dev)
+    ones = torch.full_like(scales8, 127)
+    lo, hi = lut[(codes & 15).long()], lut[(codes >> 4).long()]
+    elems = unpack_mx(bytes_, ones, kind8, torch.float32)
+    finite = (scales8 != 255).repeat_interleave(32, dim=-1)
+    assert torch.equal(torch.stack([lo, hi], -1).reshape(96, 256)[finite], elems[finite])
+    # transposing pack
+    want_t = O.quantize_mx(x, 8, "fp4_e2m1", axes=[-2], block_size=32, round=rnd)
+    codes, scales, kind = pack_mx_t(x.to(dev), "fp4_e2m1", 8, rnd, nibbles=True)
+    assert codes.shape == (256, 48) and scales.shape == (256, 3) and kind == CODES_E2M1
+    got = unpack_mx(codes, scales, kind, dtype).transpose(-1, -2).contiguous()
+    assert_bits_equal(got, want_t, "nibbles, transposed")
+    with pytest.raises(RuntimeError, match="nibbles"):
+        pack_mx(x.to(dev), "fp6_e2m3", nibbles=True)
+
+
+@pytest.mark.parametrize("M,N,K,batch", [(128, 128, 256, 1), (100, 72, 256, 1), (130, 257, 768, 3),
+                                         (1, 5, 512, 1), (600, 520, 256, 2),
+                                         # persistent kernel (K % 512 == 0)
+                                         (512, 768, 512, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
+                                         (2050, 1800, 1536, 3)])
+def test_fp4_gemm_on_nibbles_against_fp64(dev, M, N, K, batch):
+    """Both operands as e2m1 nibbles at the 4-bit MFMA rate: against fp64 on the unpacked operands,
+    with a 2^-3 .. 2^3 spread of block scales, and against the same GEMM on byte codes (same
+    products; only the grouping of the additions differs)."""
+    from microxcaling_amd.fused import pack_mx, unpack_mx, gemm_nt
+    g = torch.Generator().manual_seed(M * 7 + N * 3 + K + batch)
+    shape_a = (batch, M, K) if batch > 1 else (M, K)
+    shape_b = (batch, N, K) if batch > 1 else (N, K)
+    blk = lambda s: torch.exp2(torch.randint(-3, 4, s[:-1] + (s[-1] // 32, 1), generator=g).float())
+    a = (torch.randn(*shape_a, generator=g).view(*shape_a[:-1], K // 32, 32) * blk(shape_a)).view(shape_a)
+    b = (torch.randn(*shape_b, generator=g).view(*shape_b[:-1], K // 32, 32) * blk(shape_b)).view(shape_b)
+    pa = pack_mx(a.to(dev), "fp4_e2m1", nibbles=True)
+    pb = pack_mx(b.to(dev), "fp4_e2m1", nibbles=True)
+    got = gemm_nt(pa, pb, torch.float32)
+    qa = unpack_mx(*pa, torch.float32).double()
+    qb = unpack_mx(*pb, torch.float32).double()
+    want = qa @ qb.transpose(-1, -2)
+    assert got.shape == want.shape
+    assert rel_err(got, want) < 1e-3
+    den = qa.abs() @ qb.abs().transpose(-1, -2)
+    assert ((got.double() - want).abs() <= 2e-4 * den + 1e-30).all()
+    on_bytes = gemm_nt(pack_mx(a.to(dev), "fp4_e2m1"), pack_mx(b.to(dev), "fp4_e2m1"), torch.float32)
+    assert rel_err(got, on_bytes) < 1e-3
+    # 16-bit output with bias and epilogue quantization: the fp32 result pushed through the same steps
+    from microxcaling_amd.elemwise_ops import _quantize_bfloat
+    bias = torch.randn(N, generator=g).to(dev).to(torch.bfloat16)
+    want16 = _quantize_bfloat(_quantize_bfloat(got.to(torch.bfloat16), 16, round="nearest") + bias, 16, round="nearest")
+    got16 = gemm_nt(pa, pb, torch.bfloat16, bias=bias, epilogue_quant=True)
+    assert torch.equal(got16.view(torch.int16), want16.view(torch.int16))
+    with pytest.raises(RuntimeError, match="both operands"):
+        gemm_nt(pa, pack_mx(b.to(dev), "fp4_e2m1"), torch.float32)
+
+
 def test_gemm_propagates_nan_blocks(dev):
     from microxcaling_amd.fused import pack_mx, gemm_nt
     a = torch.randn(128, 128)
