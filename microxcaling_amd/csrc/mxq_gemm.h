@@ -347,6 +347,37 @@ __device__ __forceinline__ void store_c8(void* c, const void* bias, uint32_t q_n
     }
 }
 
+// Epilogue of eight consecutive columns n .. n + 7 of one row, packed to a 16-bit output type
+// (inside tiles only: n + 7 < N, bias 16-byte aligned at n).
+template <int OUT_DT>
+__device__ __forceinline__ u32x4 epilogue_pack8(const void* bias, uint32_t q_nan_from, int n, v4f lo, v4f hi) {
+    float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    if (bias != nullptr) {
+        const u32x4 bw = *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned short*>(bias) + n);
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+            v[r] = epilogue_value<OUT_DT>(v[r], true, Pack<OUT_DT>::get(bw[r >> 1], r & 1), q_nan_from);
+    } else if (q_nan_from != 0u) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) v[r] = epilogue_value<OUT_DT>(v[r], false, 0.0f, q_nan_from);
+    }
+    return u32x4{Pack<OUT_DT>::put(v[0], v[1]), Pack<OUT_DT>::put(v[2], v[3]),
+                 Pack<OUT_DT>::put(v[4], v[5]), Pack<OUT_DT>::put(v[6], v[7])};
+}
+
+// Swaps `b` of the lanes 0-15 / 32-47 of a wave with `a` of the lanes 16-31 / 48-63 (lane L with
+// lane L + 16).  The large-tile kernel uses it so that the four lanes L, L + 16, L + 32, L + 48 hold
+// four consecutive 16-byte pieces of one output row: a store instruction then writes 64 contiguous
+// bytes per row instead of 32, half as many write requests.
+__device__ __forceinline__ void swap_with_lane16(u32x4& a, u32x4& b) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const auto r = __builtin_amdgcn_permlane16_swap(a[k], b[k], false, false);
+        a[k] = r[0];
+        b[k] = r[1];
+    }
+}
+
 template <int CBSZ, int BLGP, int OUT_DT>
 __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     constexpr bool PAIR = OUT_DT != MXQ_F32;
@@ -703,24 +734,58 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
         const bool inside = m0 + G2_BM <= g.M && n0 + G2_BN <= g.N && (g.N & 3) == 0 &&
                             ((uintptr_t)g.c & 15) == 0;
         const bool inside8 = inside && (g.N & 7) == 0 && ((uintptr_t)g.bias & 15) == 0;
+        // Inside tiles: a lane holds the 16-byte pieces fg, 2 + fg (, 4 + fg, 6 + fg) of its row of
+        // a fragment; after the exchange with lane L +- 16 it holds piece 2 * (L / 16 % 2) + fg of
+        // row L % 16 and the same piece of row 16 + L % 16 (see swap_with_lane16).
+        const int half = (lane >> 4) & 1, m16 = lane & 15;
 #pragma unroll
         for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
             for (int tj = 0; tj < 4; ++tj) {
-                const int m = m0 + wy * 64 + ti * 32 + fi;
+                const int mt = m0 + wy * 64 + ti * 32;
                 const int nt = n0 + wx * 128 + tj * 32;
                 const v16f& c = acc[ti][tj];
                 if constexpr (PAIR) {
+                    if (inside8) {
+                        u32x4 p[2];
 #pragma unroll
-                    for (int h = 0; h < 2; ++h)
-                        store_c8<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, nt + 16 * h + 8 * fg, g.M, g.N, inside8,
-                                         v4f{c[8 * h], c[8 * h + 1], c[8 * h + 2], c[8 * h + 3]},
-                                         v4f{c[8 * h + 4], c[8 * h + 5], c[8 * h + 6], c[8 * h + 7]});
+                        for (int h = 0; h < 2; ++h)
+                            p[h] = epilogue_pack8<OUT_DT>(g.bias, g.q_nan_from, nt + 16 * h + 8 * fg,
+                                                          v4f{c[8 * h], c[8 * h + 1], c[8 * h + 2], c[8 * h + 3]},
+                                                          v4f{c[8 * h + 4], c[8 * h + 5], c[8 * h + 6], c[8 * h + 7]});
+                        swap_with_lane16(p[0], p[1]);
+                        unsigned short* out = reinterpret_cast<unsigned short*>(g.c) + cbase +
+                                              (int64_t)(mt + m16) * g.N + nt + 8 * (2 * half + fg);
+                        *reinterpret_cast<u32x4*>(out) = p[0];
+                        *reinterpret_cast<u32x4*>(out + (int64_t)16 * g.N) = p[1];
+                    } else {
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+                            store_c8<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, mt + fi, nt + 16 * h + 8 * fg, g.M, g.N,
+                                             false, v4f{c[8 * h], c[8 * h + 1], c[8 * h + 2], c[8 * h + 3]},
+                                             v4f{c[8 * h + 4], c[8 * h + 5], c[8 * h + 6], c[8 * h + 7]});
+                    }
                 } else {
+                    if (inside && g.bias == nullptr) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, nt + 8 * q + 4 * fg, g.M, g.N, inside,
-                                         v4f{c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]});
+                        for (int q = 0; q < 4; q += 2) {
+                            u32x4 p[2];
+#pragma unroll
+                            for (int e = 0; e < 2; ++e)
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) p[e][r] = __float_as_uint(c[4 * (q + e) + r]);
+                            swap_with_lane16(p[0], p[1]);
+                            float* out = reinterpret_cast<float*>(g.c) + cbase + (int64_t)(mt + m16) * g.N + nt +
+                                         8 * q + 4 * (2 * half + fg);
+                            *reinterpret_cast<u32x4*>(out) = p[0];
+                            *reinterpret_cast<u32x4*>(out + (int64_t)16 * g.N) = p[1];
+                        }
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, mt + fi, nt + 8 * q + 4 * fg, g.M, g.N,
+                                             inside, v4f{c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]});
+                    }
                 }
             }
 #pragma unroll
