@@ -31,13 +31,13 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
     __shared__ unsigned char zone[ZONE_PAD];
     load_zone(zone, g_zone_tables[p.q.zone_row]);
 
-    auto Q = [&](float v) {
-        v = mxq_round_dt<ADT>(v);
+    auto Qd = [&](float v) {                                 // v already is a value of the tensor dtype
         if (QMODE == SMQ_IDENT) return v;
         if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, p.q.fmt.nan_from);
         return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
                                                           p.q.allow_denorm != 0, zone, ZS);
     };
+    auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
 
     // the quantizer for exponentials, their row sum and the quotients: all >= +0 and <= 4096 (or
     // NaN / +Inf), where the closed form needs no special cases
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
 #pragma unroll
                 for (int h = 0; h < PD; ++h) {
                     const int e = (j * 4 + d) * PD + h;
-                    x[e] = valid ? Q(Pack<DT>::get(raw[j][d], h)) : -__builtin_inff();
+                    x[e] = valid ? Qd(Pack<DT>::get(raw[j][d], h)) : -__builtin_inff();
                     m = MaxOp::apply(m, x[e]);                 // NaN sticks, like torch.max
                 }
         }
@@ -99,6 +99,17 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
         sum = Qp(wave_reduce<SumOp>(sum));
         const bool recip = p.use_recip != 0;
         const float r = recip ? Qp(1.0f / sum) : 0.0f;
+        // e / sum without a division per element: one refined reciprocal per row, then a product
+        // and a residual correction.  For operands with 8-bit significands (the dtype-rounded
+        // exponentials and sum of a bf16 tensor) this is the correctly rounded fp32 quotient,
+        // checked over every pair of significands; fp32 tensors keep the division.
+        const float r0 = __builtin_amdgcn_rcpf(sum);
+        const float r1 = fmaf(fmaf(-sum, r0, 1.0f), r0, r0);
+        auto quotient = [&](float e) {
+            if (ADT != MXQ_BF16) return e / sum;
+            const float q0 = e * r1;
+            return fmaf(fmaf(-q0, sum, e), r1, q0);
+        };
 
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
@@ -109,7 +120,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
 #pragma unroll
                 for (int h = 0; h < PD; ++h) {
                     const float e = x[(j * 4 + d) * PD + h];
-                    q[h] = Qp(recip ? e * r : e / sum);
+                    q[h] = Qp(recip ? e * r : quotient(e));
                 }
                 o[d] = Pack<DT>::put(q[0], q[PD - 1]);
             }
@@ -154,13 +165,13 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
     __shared__ unsigned char zone[ZONE_PAD];
     load_zone(zone, g_zone_tables[p.q.zone_row]);
 
-    auto Q = [&](float v) {
-        v = mxq_round_dt<ADT>(v);
+    auto Qd = [&](float v) {                                 // v already is a value of the tensor dtype
         if (QMODE == SMQ_IDENT) return v;
         if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, p.q.fmt.nan_from);
         return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
                                                           p.q.allow_denorm != 0, zone, ZS);
     };
+    auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
 
     const int lane = threadIdx.x & 63;
     const int nvec = n / EPV;
@@ -180,7 +191,7 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
 #pragma unroll
                 for (int h = 0; h < PD; ++h) {
                     const int e = (j * 4 + d) * PD + h;
-                    x[e] = valid ? Q(Pack<DT>::get(raw[d], h)) : 0.0f;    // zeros add nothing to the sums
+                    x[e] = valid ? Qd(Pack<DT>::get(raw[d], h)) : 0.0f;   // zeros add nothing to the sums
                     sum += p.rms ? 0.0f : x[e];
                 }
         }
