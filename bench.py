@@ -221,6 +221,25 @@ def make_workload(name):
                     launches=1 if fused else 12,
                     desc="%s, bfloat16 quantization after every step, %s" % (what, "one kernel" if fused else
                                                                              "separate tensor passes"))
+    if name in ("gelu_bf16", "gelu_bf16_unfused", "silu_bf16", "silu_bf16_unfused"):
+        # fused activation kernels: GELU (writes the result, phi and the quantized input: what the
+        # layer saves for its backward pass) and SiLU (result and sigmoid) over bf16 [16384, 8192]
+        from microxcaling_amd import activations, gemm
+        from microxcaling_amd.specs import finalize_mx_specs
+        specs = finalize_mx_specs({"bfloat": 16})
+        fused = not name.endswith("unfused")
+        is_gelu = name.startswith("gelu")
+        x = (torch.randn(4096, 8192, generator=torch.Generator().manual_seed(7)) * 2).to(torch.bfloat16).repeat(4, 1)
+
+        def run(xd):
+            gemm.set_fused(fused)
+            xi = xd.requires_grad_(True)                # the layers only save tensors when a gradient is wanted
+            return activations.gelu(xi, mx_specs=specs) if is_gelu else activations.silu(xi, mx_specs=specs)
+        cpu = (lambda t: activations.gelu(t, mx_specs=specs)) if is_gelu else (lambda t: activations.silu(t, mx_specs=specs))
+        return dict(x=x, gpu=run, cpu=cpu, bytes=x.numel() * (8 if is_gelu else 6), dtype="bf16", sample_axis=0,
+                    launches=1 if fused else (22 if is_gelu else 12),
+                    desc="%s forward, bf16 [16384,8192], bfloat16 quantization after every step, %s"
+                         % ("GELU (cubic)" if is_gelu else "SiLU", "one kernel" if fused else "separate tensor passes"))
     if name == "copy_fp32_8192":
         # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         x = torch.randn(8192, 8192, generator=torch.Generator().manual_seed(0))

@@ -127,6 +127,23 @@ int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void*
                      int bits, int exp_bits, float max_norm, int rmode, int allow_denorm, int flags,
                      void* hip_stream);
 
+/* The forward passes of SigmoidFunction, TanhFunction, SiLUFunction and GELUFunction
+ * (mx/activations.py:237-297, 418-557) on a contiguous fp32 or bf16 tensor of n elements, as one
+ * kernel, with the elementwise quantizer (bits / exp_bits / max_norm as in mxq_softmax_lastdim,
+ * bits == 0: none) after every step of the reference's chain of vec_* ops.
+ * act: MXQ_ACT_*.  exp_mode 0: exp(x); 2: 2^Q(x * 1.4453125) (mx_specs['vec_use_exp2']).
+ * out: the result.  aux (may be NULL): the logistic factor that silu (sigmoid(x)) and gelu (phi) save
+ * for their backward passes.  q_in (may be NULL): the quantized input, which gelu saves.
+ * Agrees with the reference's chain up to the last-bit differences of exp and tanh. */
+#define MXQ_ACT_SIGMOID 0
+#define MXQ_ACT_TANH 1
+#define MXQ_ACT_SILU 2
+#define MXQ_ACT_GELU_FIRST_ORDER 3 /* x * sigmoid(1.702 x) */
+#define MXQ_ACT_GELU 4             /* x * sigmoid(1.5958 (x + 0.044715 x^3)) */
+int mxq_activation_forward(const void* in, void* out, void* aux, void* q_in, int dtype, int64_t n,
+                           int act, int bits, int exp_bits, float max_norm, int rmode,
+                           int allow_denorm, int exp_mode, int flags, void* hip_stream);
+
 /* ---- packed MX tensors and the fused GEMM (no counterpart in the reference, which only ever
  * fake-quantizes and then calls a dense GEMM: mx/linear.py:62-86, mx/bmm.py:40-59) ---------------
  * Packed form of a (rows, K) tensor quantized along K in blocks of 32:

@@ -24,6 +24,50 @@ GELU_SCALE = 1.59375              # ~1.5958
 GELU_SCALE_DERIV = 0.21386719     # ~3 * 0.044715 * 1.5958
 
 
+ACT_SIGMOID, ACT_TANH, ACT_SILU, ACT_GELU_FIRST_ORDER, ACT_GELU = range(5)
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
+
+
+def _fused_forward(input, act, mx_specs, want_aux=False, want_q=False):
+    """The whole forward chain of one activation as a single kernel launch
+    (mxq_activation_forward): (output, logistic factor or None, quantized input or None), or None
+    when the kernel does not cover the case: CPU tensors, fp16 tensors, round-half-even to a wide
+    format on a bf16 tensor."""
+    from . import _lib, gemm
+    from .custom_extensions import _flags_value
+    from .elemwise_ops import _native_round, elemwise_plan
+    if not (gemm.fused_enabled() and input.is_cuda):
+        return None
+    rnd = mx_specs['round']
+    plan = elemwise_plan(mx_specs, rnd)
+    if plan[0] == "to_bf16":
+        input = input.to(torch.bfloat16)       # the first quantization of the chain does this
+        plan = ("identity",)
+    if input.dtype not in _DTYPE_CODE or input.numel() == 0:
+        return None
+    if plan[0] == "identity":
+        bits, exp_bits, max_norm, denorm, rmode = 0, 0, 1.0, True, 0
+    else:
+        _, bits, exp_bits, max_norm, denorm = plan
+        rmode = _native_round(rnd)
+        if input.dtype == torch.bfloat16 and bits >= 9 and rnd == 'even':
+            return None
+    x = input.contiguous()
+    out = torch.empty_like(x)
+    aux = torch.empty_like(x) if want_aux else None
+    q = torch.empty_like(x) if want_q else None
+    lib = _lib.gpu()
+    with torch.cuda.device(x.device):
+        rc = lib.mxq_activation_forward(x.data_ptr(), out.data_ptr(),
+                                        None if aux is None else aux.data_ptr(),
+                                        None if q is None else q.data_ptr(), _DTYPE_CODE[x.dtype],
+                                        x.numel(), act, bits, exp_bits, max_norm, rmode, int(denorm),
+                                        2 if mx_specs['vec_use_exp2'] else 0, _flags_value(),
+                                        torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, lib)
+    return out, aux, q
+
+
 def _logistic(x, specs):
     """1 / (1 + exp(-x)) as three quantized steps (mx/activations.py:245-249)."""
     return vec_recip(vec_add(vec_exp(-x, mx_specs=specs), 1., mx_specs=specs), mx_specs=specs)
@@ -47,7 +91,8 @@ class SigmoidFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, mx_specs=None, name=None):
-        out = _logistic(vec_quantize(input, mx_specs=mx_specs), mx_specs)
+        fused = _fused_forward(input, ACT_SIGMOID, mx_specs)
+        out = fused[0] if fused else _logistic(vec_quantize(input, mx_specs=mx_specs), mx_specs)
         ctx.save_for_backward(out)
         ctx.mx_specs = get_backwards_mx_specs(mx_specs)
         return out
@@ -66,7 +111,8 @@ class TanhFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, mx_specs=None, name=None):
-        out = vec_tanh(vec_quantize(input, mx_specs=mx_specs), mx_specs=mx_specs)
+        fused = _fused_forward(input, ACT_TANH, mx_specs)
+        out = fused[0] if fused else vec_tanh(vec_quantize(input, mx_specs=mx_specs), mx_specs=mx_specs)
         ctx.save_for_backward(out)
         ctx.mx_specs = get_backwards_mx_specs(mx_specs)
         return out
@@ -151,9 +197,14 @@ class SiLUFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, inplace=False, mx_specs=None, name=None):
-        q = vec_quantize(input, mx_specs=mx_specs)
-        sig = _logistic(q, mx_specs)
-        out = _finish_inplace(ctx, input, vec_mul(q, sig, mx_specs=mx_specs), inplace)
+        fused = _fused_forward(input, ACT_SILU, mx_specs, want_aux=True)
+        if fused:
+            out, sig, _ = fused
+        else:
+            q = vec_quantize(input, mx_specs=mx_specs)
+            sig = _logistic(q, mx_specs)
+            out = vec_mul(q, sig, mx_specs=mx_specs)
+        out = _finish_inplace(ctx, input, out, inplace)
         ctx.save_for_backward(out, sig)
         ctx.mx_specs = get_backwards_mx_specs(mx_specs)
         return out
@@ -175,6 +226,13 @@ class GELUFunction(torch.autograd.Function):
     def forward(ctx, input, mx_specs=None, first_order_gelu=False, name=None):
         ctx.first_order_gelu = first_order_gelu
         s = mx_specs
+        fused = _fused_forward(input, ACT_GELU_FIRST_ORDER if first_order_gelu else ACT_GELU, s,
+                               want_aux=True, want_q=bool(s['quantize_backprop']))
+        if fused:
+            out, phi, q = fused
+            ctx.save_for_backward(q if s['quantize_backprop'] else input, phi)
+            ctx.mx_specs = get_backwards_mx_specs(s)
+            return out
         q = vec_quantize(input, mx_specs=s)
         if first_order_gelu:
             y = vec_mul(GELU_FIRST_ORDER, q, mx_specs=s)

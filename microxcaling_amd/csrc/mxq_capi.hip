@@ -394,6 +394,51 @@ int mxq_softmax_lastdim(const void* in, void* out, int dtype, int64_t rows, int6
     return check_launch(who);
 }
 
+int mxq_activation_forward(const void* in, void* out, void* aux, void* q_in, int dtype, int64_t n,
+                           int act, int bits, int exp_bits, float max_norm, int rmode,
+                           int allow_denorm, int exp_mode, int flags, void* hip_stream) {
+    const char* who = "mxq_activation_forward";
+    ActParams p;
+    const bool ident = bits == 0;
+    if (dtype != MXQ_DTYPE_F32 && dtype != MXQ_DTYPE_BF16)
+        return fail(MXQ_ERR_ARGUMENT, "%s: dtype code %d (fp32 and bf16 tensors only)", who, dtype);
+    int rc = make_elem_params(dtype, ident ? 9 : bits, ident ? 8 : exp_bits, ident ? 1.0f : max_norm,
+                              ident ? MXQ_ROUND_NEAREST : rmode, 0, allow_denorm, flags, &p.q, who);
+    if (rc) return rc;
+    if (!ident && !lean_ok(dtype, p.q.fmt, rmode, true))
+        return fail(MXQ_ERR_ARGUMENT, "%s: round-half-even to %d fraction bits on a bf16 tensor is "
+                    "only available through the separate elementwise steps", who, p.q.fmt.t);
+    if (act < ACT_SIGMOID || act > ACT_GELU) return fail(MXQ_ERR_ARGUMENT, "%s: unknown activation %d", who, act);
+    if (exp_mode != 0 && exp_mode != 2) return fail(MXQ_ERR_ARGUMENT, "%s: exp_mode %d (0 or 2)", who, exp_mode);
+    p.act = act;
+    p.exp_mode = exp_mode;
+    if (n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (n == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(in) || !aligned16(out) || !aligned16(aux) || !aligned16(q_in))
+        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int epv = dtype == MXQ_DTYPE_F32 ? 4 : 8;
+    const int grid = grid_for(ceil_div(ceil_div(n, epv), (int64_t)kThreads));
+    const bool closed = !ident && dtype == MXQ_DTYPE_BF16 && bits == 9 && exp_bits == 8 &&
+                        rmode == MXQ_ROUND_NEAREST && allow_denorm && p.q.fmt.max_bits == 0x7F7F0000u;
+#define MXQ_ACT(DT, RM, QM) activation_kernel<DT, RM, QM><<<grid, kThreads, 0, s>>>(in, out, aux, q_in, n, p)
+    if (dtype == MXQ_DTYPE_F32) {
+        if (ident) MXQ_ACT(MXQ_F32, MXQ_NEAREST, SMQ_IDENT);
+        else if (rmode == MXQ_ROUND_FLOOR) MXQ_ACT(MXQ_F32, MXQ_FLOOR, SMQ_GENERIC);
+        else if (rmode == MXQ_ROUND_NEAREST) MXQ_ACT(MXQ_F32, MXQ_NEAREST, SMQ_GENERIC);
+        else MXQ_ACT(MXQ_F32, MXQ_EVEN, SMQ_GENERIC);
+    } else {
+        if (ident) MXQ_ACT(MXQ_BF16, MXQ_NEAREST, SMQ_IDENT);
+        else if (closed) MXQ_ACT(MXQ_BF16, MXQ_NEAREST, SMQ_BF16);
+        else if (rmode == MXQ_ROUND_FLOOR) MXQ_ACT(MXQ_BF16, MXQ_FLOOR, SMQ_GENERIC);
+        else if (rmode == MXQ_ROUND_NEAREST) MXQ_ACT(MXQ_BF16, MXQ_NEAREST, SMQ_GENERIC);
+        else MXQ_ACT(MXQ_BF16, MXQ_EVEN, SMQ_GENERIC);
+    }
+#undef MXQ_ACT
+    return check_launch(who);
+}
+
 int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void* out, void* x_norm,
                      void* row_stat, int dtype, int64_t rows, int64_t n, float eps, int rms_norm,
                      int bits, int exp_bits, float max_norm, int rmode, int allow_denorm, int flags,

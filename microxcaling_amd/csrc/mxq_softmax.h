@@ -240,3 +240,102 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
 }
 
 }  // namespace
+
+// ================================================================================================
+// Activations with the elementwise quantizer after every step (mx/activations.py:237-557): one
+// kernel instead of 3 to 22 tensor passes.  Elementwise, 16 bytes per lane, grid-stride.
+//   logistic(y) = Q(1 / Q(Q(exp(-y)) + 1)); with vec_use_exp2: exp(t) = Q(2^Q(1.4453125 t))
+//   sigmoid: logistic(q)        tanh: Q(tanh q)        silu: Q(q s), s = logistic(q)
+//   gelu:    Q(q phi), phi = logistic(y), y = Q(1.703125 q)                           (first order)
+//            or y = Q(1.59375 Q(Q(0.044677734375 Q(Q(q q) q)) + q))                   (cubic)
+// with q = Q(input).  Besides the result it writes what the backward passes keep: the logistic
+// factor (silu, gelu) and the quantized input (gelu), when the pointers are given.
+// ================================================================================================
+enum { ACT_SIGMOID = 0, ACT_TANH = 1, ACT_SILU = 2, ACT_GELU_FIRST_ORDER = 3, ACT_GELU = 4 };
+
+struct ActParams {
+    ElemParams q;
+    int act;
+    int exp_mode;      // 0: exp(x)   2: 2^Q(x * log2(e) at bfloat16 precision)  (vec_use_exp2)
+};
+
+namespace {
+
+template <int DT, int RMODE, int QMODE>
+__global__ __launch_bounds__(TPB) void activation_kernel(const void* __restrict__ in_, void* __restrict__ out_,
+                                                         void* __restrict__ aux_, void* __restrict__ qin_,
+                                                         int64_t n, ActParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int EPV = 4 * PD;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.q.zone_row]);
+
+    auto Qd = [&](float v) {                                 // v already is a value of the tensor dtype
+        if (QMODE == SMQ_IDENT) return v;
+        if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, p.q.fmt.nan_from);
+        return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
+                                                          p.q.allow_denorm != 0, zone, ZS);
+    };
+    auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
+    const bool via_exp2 = p.exp_mode == 2;
+    auto logistic = [&](float y) {
+        const float t = -y;
+        const float e = via_exp2 ? Q(exp2f(Q(1.4453125f * t))) : Q(expf(t));
+        return Q(1.0f / Q(e + 1.0f));
+    };
+    // one element: result, logistic factor (silu, gelu), quantized input
+    auto eval = [&](float x, float& aux, float& q) {
+        q = Qd(x);
+        aux = 0.0f;
+        switch (p.act) {
+            case ACT_SIGMOID: return logistic(q);
+            case ACT_TANH: return Q(tanhf(q));
+            case ACT_SILU: aux = logistic(q); return Q(q * aux);
+            case ACT_GELU_FIRST_ORDER: aux = logistic(Q(1.703125f * q)); return Q(q * aux);
+            default: {
+                const float cube = Q(Q(q * q) * q);
+                const float y = Q(1.59375f * Q(Q(0.044677734375f * cube) + q));
+                aux = logistic(y);
+                return Q(q * aux);
+            }
+        }
+    };
+
+    const u32x4* in = reinterpret_cast<const u32x4*>(in_);
+    u32x4* out = reinterpret_cast<u32x4*>(out_);
+    u32x4* auxv = reinterpret_cast<u32x4*>(aux_);
+    u32x4* qinv = reinterpret_cast<u32x4*>(qin_);
+    const int64_t n_vec = n / EPV;
+    const int64_t stride = (int64_t)gridDim.x * TPB;
+    for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n_vec; i += stride) {
+        const u32x4 v = in[i];
+        u32x4 o, a, qv;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            float r[2], ax[2], qq[2];
+#pragma unroll
+            for (int h = 0; h < PD; ++h) r[h] = eval(Pack<DT>::get(v[d], h), ax[h], qq[h]);
+            o[d] = Pack<DT>::put(r[0], r[PD - 1]);
+            a[d] = Pack<DT>::put(ax[0], ax[PD - 1]);
+            qv[d] = Pack<DT>::put(qq[0], qq[PD - 1]);
+        }
+        __builtin_nontemporal_store(o, &out[i]);
+        if (auxv) __builtin_nontemporal_store(a, &auxv[i]);
+        if (qinv) __builtin_nontemporal_store(qv, &qinv[i]);
+    }
+    // tail
+    const int64_t t0 = n_vec * EPV;
+    const int64_t gi = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (gi < n - t0) {
+        float ax, qq;
+        const float r = eval(load_scalar<DT>(in_, t0 + gi), ax, qq);
+        store_scalar<DT>(out_, t0 + gi, mxq_round_dt<ADT>(r));
+        if (aux_) store_scalar<DT>(aux_, t0 + gi, mxq_round_dt<ADT>(ax));
+        if (qin_) store_scalar<DT>(qin_, t0 + gi, qq);
+    }
+}
+
+}  // namespace
+

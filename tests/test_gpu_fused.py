@@ -448,3 +448,74 @@ def test_softmax_backward_against_oracle(dev, dtype, exp2):
     diff = (xd.grad.float().cpu() - want.float()).abs()
     assert diff.max().item() <= 2.0 ** -7 * want.float().abs().max().item()
     assert (diff > 0).float().mean().item() < 0.02
+
+
+_ACTS = {
+    "sigmoid": lambda A, x, s: A.sigmoid(x, mx_specs=s),
+    "tanh": lambda A, x, s: A.tanh(x, mx_specs=s),
+    "silu": lambda A, x, s: A.silu(x, mx_specs=s),
+    "gelu": lambda A, x, s: A.gelu(x, mx_specs=s),
+    "gelu_first_order": lambda A, x, s: A.gelu(x, mx_specs=s, first_order_gelu=True),
+}
+
+
+def _one_step_apart(got, want, frac_allowed):
+    """exp / tanh differ in the last bit between the GPU and the CPU library; a quantizer turns that
+    into one step of the format now and then.  At most two steps of the coarsest grid in play
+    (2^-6 relative), on at most `frac_allowed` of the elements; NaNs in the same places."""
+    got, want = got.float().cpu(), want.float().cpu()
+    assert got.shape == want.shape
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    ok = ~torch.isnan(want)
+    g, w = got[ok], want[ok]
+    inf = torch.isinf(w)
+    assert torch.equal(g[inf], w[inf])
+    d = (g[~inf] - w[~inf]).abs()
+    assert (d <= 2.0 ** -5 * w[~inf].abs() + 1e-37).all(), d.max().item()
+    assert (d > 0).float().mean().item() <= frac_allowed
+
+
+@pytest.mark.parametrize("act", sorted(_ACTS))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, vec_use_exp2=True), dict(bfloat=12),
+                                  dict(bfloat=16, round="floor")],
+                         ids=["bfloat16", "bfloat16-exp2", "bfloat12", "bfloat16-floor"])
+def test_fused_activation_against_chain(dev, act, dtype, spec):
+    """One-kernel activation forward (and the backward pass fed by what it saved) against the chain
+    of vec_* ops on the CPU, which is bit-identical to the reference's layers."""
+    from microxcaling_amd import activations as A, gemm
+    from microxcaling_amd.specs import apply_mx_specs
+    specs = _specs(**spec)
+    g = torch.Generator().manual_seed(len(act) + spec.get("bfloat", 0))
+    x = (torch.randn(257, 130, generator=g) * 3).to(dtype)            # 33410 elements: a ragged tail
+    w = torch.randn(257, 130, generator=g).to(dtype)
+    outs = {}
+    for where in ("cpu", "gpu"):
+        xi = (x.to(dev) if where == "gpu" else x.clone()).requires_grad_(True)
+        y = _ACTS[act](A, xi, specs)
+        (y * (w.to(dev) if where == "gpu" else w)).sum().backward()
+        outs[where] = (y.detach(), xi.grad.detach())
+    assert A._fused_forward(x.to(dev), A.ACT_TANH, apply_mx_specs(specs)) is not None      # the path under test
+    assert outs["gpu"][0].dtype == outs["cpu"][0].dtype
+    loose = 0.06 if spec.get("round") == "floor" else 0.03
+    _one_step_apart(outs["gpu"][0], outs["cpu"][0], loose)
+    _one_step_apart(outs["gpu"][1], outs["cpu"][1], 2 * loose)
+    # the separate steps on the GPU give the same as the kernel, to the same tolerance
+    gemm.set_fused(False)
+    try:
+        y_chain = _ACTS[act](A, x.to(dev), specs)
+    finally:
+        gemm.set_fused(True)
+    _one_step_apart(outs["gpu"][0], y_chain, loose)
+
+
+@pytest.mark.parametrize("act", sorted(_ACTS))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_activation_special_values(dev, act, dtype):
+    from microxcaling_amd import activations as A
+    specs = _specs(bfloat=16)
+    x = torch.tensor([0.0, -0.0, float("inf"), float("-inf"), float("nan"), 1e-30, -1e-30, 88.0, -88.0,
+                      100.0, -100.0, 3e38, -3e38, 1e-40, 20.0, -20.0], dtype=torch.float32).to(dtype)
+    got = _ACTS[act](A, x.to(dev), specs)
+    want = _ACTS[act](A, x, specs)
+    _one_step_apart(got, want, 0.2)
