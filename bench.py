@@ -221,6 +221,39 @@ def make_workload(name):
                     launches=1 if fused else 12,
                     desc="%s, bfloat16 quantization after every step, %s" % (what, "one kernel" if fused else
                                                                              "separate tensor passes"))
+    if name in ("gelu_bf16_train", "gelu_bf16_train_unfused", "softmax_bf16_train", "softmax_bf16_train_unfused"):
+        # forward + backward of one bfloat16 layer: the fused forward kernel writes what the fused
+        # backward kernel reads
+        from microxcaling_amd import activations, gemm
+        from microxcaling_amd.softmax import softmax
+        from microxcaling_amd.specs import finalize_mx_specs
+        specs = finalize_mx_specs({"bfloat": 16})
+        fused = not name.endswith("unfused")
+        is_gelu = name.startswith("gelu")
+        gen = torch.Generator().manual_seed(8)
+        if is_gelu:
+            x = (torch.randn(4096, 8192, generator=gen) * 2).to(torch.bfloat16).repeat(4, 1)
+            per_elem = 8 + 8                              # fwd: 1 read, 3 writes; bwd: 3 reads, 1 write
+        else:
+            x = (torch.randn(16384, 2048, generator=gen) * 3).to(torch.bfloat16).repeat(8, 1)
+            per_elem = 4 + 6                              # fwd: read, write; bwd: 2 reads, 1 write
+        extra = {}
+
+        def run(xd):
+            if "g" not in extra:
+                extra["g"] = torch.randn(xd.shape, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(xd.device)
+            gemm.set_fused(fused)
+            xi = xd.requires_grad_(True)
+            xi.grad = None
+            y = activations.gelu(xi, mx_specs=specs) if is_gelu else softmax(xi, dim=-1, mx_specs=specs)
+            y.backward(extra["g"])
+            return xi.grad
+        cpu = (lambda t: activations.gelu(t, mx_specs=specs)) if is_gelu else (lambda t: O.softmax_forward(t, -1, bfloat=16))
+        return dict(x=x, gpu=run, cpu=cpu, bytes=x.numel() * per_elem, dtype="bf16", sample_axis=0,
+                    launches=2 if fused else 40,
+                    desc="%s forward + backward, bf16 %s, bfloat16 quantization after every step, %s"
+                         % ("GELU (cubic)" if is_gelu else "softmax over the last axis", list(x.shape),
+                            "two kernels" if fused else "separate tensor passes"))
     if name in ("gelu_bf16", "gelu_bf16_unfused", "silu_bf16", "silu_bf16_unfused"):
         # fused activation kernels: GELU (writes the result, phi and the quantized input: what the
         # layer saves for its backward pass) and SiLU (result and sigmoid) over bf16 [16384, 8192]

@@ -144,6 +144,22 @@ int mxq_activation_forward(const void* in, void* out, void* aux, void* q_in, int
                            int act, int bits, int exp_bits, float max_norm, int rmode,
                            int allow_denorm, int exp_mode, int flags, void* hip_stream);
 
+/* The backward passes of the same four layers (mx/activations.py:251-267, 284-297, 437-455,
+ * 500-557) from what their forward passes saved: `saved` = the output (sigmoid, tanh, silu) or the
+ * (quantized) input (gelu); `aux` = sigmoid(x) (silu) or phi (gelu), NULL otherwise.  Exact
+ * arithmetic and the quantizer only: bit-identical to the reference's chain of vec_* ops. */
+int mxq_activation_backward(const void* grad_out, const void* saved, const void* aux, void* grad_in,
+                            int dtype, int64_t n, int act, int bits, int exp_bits, float max_norm,
+                            int rmode, int allow_denorm, int flags, void* hip_stream);
+
+/* SoftmaxFunction.backward (mx/softmax.py:56-88) over the last axis of contiguous (rows, n) tensors:
+ * y is the saved output.  scale_ln2: the extra multiplication by ln 2 of mx_specs['softmax_exp2'].
+ * Same limits as mxq_softmax_lastdim; agrees with the reference's chain up to the order of the
+ * row sum. */
+int mxq_softmax_backward_lastdim(const void* grad_out, const void* y, void* grad_in, int dtype,
+                                 int64_t rows, int64_t n, int bits, int exp_bits, float max_norm,
+                                 int rmode, int allow_denorm, int scale_ln2, int flags, void* hip_stream);
+
 /* ---- packed MX tensors and the fused GEMM (no counterpart in the reference, which only ever
  * fake-quantizes and then calls a dense GEMM: mx/linear.py:62-86, mx/bmm.py:40-59) ---------------
  * Packed form of a (rows, K) tensor quantized along K in blocks of 32:

@@ -25,34 +25,20 @@ GELU_SCALE_DERIV = 0.21386719     # ~3 * 0.044715 * 1.5958
 
 
 ACT_SIGMOID, ACT_TANH, ACT_SILU, ACT_GELU_FIRST_ORDER, ACT_GELU = range(5)
-_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
 
 
 def _fused_forward(input, act, mx_specs, want_aux=False, want_q=False):
     """The whole forward chain of one activation as a single kernel launch
     (mxq_activation_forward): (output, logistic factor or None, quantized input or None), or None
-    when the kernel does not cover the case: CPU tensors, fp16 tensors, round-half-even to a wide
-    format on a bf16 tensor."""
-    from . import _lib, gemm
+    when the kernel does not cover the case (see fused_chain_args)."""
+    from . import _lib
     from .custom_extensions import _flags_value
-    from .elemwise_ops import _native_round, elemwise_plan
-    if not (gemm.fused_enabled() and input.is_cuda):
+    from .elemwise_ops import fused_chain_args
+    args = fused_chain_args(input, mx_specs)
+    if args is None or input.numel() == 0:
         return None
-    rnd = mx_specs['round']
-    plan = elemwise_plan(mx_specs, rnd)
-    if plan[0] == "to_bf16":
-        input = input.to(torch.bfloat16)       # the first quantization of the chain does this
-        plan = ("identity",)
-    if input.dtype not in _DTYPE_CODE or input.numel() == 0:
-        return None
-    if plan[0] == "identity":
-        bits, exp_bits, max_norm, denorm, rmode = 0, 0, 1.0, True, 0
-    else:
-        _, bits, exp_bits, max_norm, denorm = plan
-        rmode = _native_round(rnd)
-        if input.dtype == torch.bfloat16 and bits >= 9 and rnd == 'even':
-            return None
-    x = input.contiguous()
+    x, code, (bits, exp_bits, max_norm, rmode, denorm) = args
+    x = x.contiguous()
     out = torch.empty_like(x)
     aux = torch.empty_like(x) if want_aux else None
     q = torch.empty_like(x) if want_q else None
@@ -60,12 +46,38 @@ def _fused_forward(input, act, mx_specs, want_aux=False, want_q=False):
     with torch.cuda.device(x.device):
         rc = lib.mxq_activation_forward(x.data_ptr(), out.data_ptr(),
                                         None if aux is None else aux.data_ptr(),
-                                        None if q is None else q.data_ptr(), _DTYPE_CODE[x.dtype],
-                                        x.numel(), act, bits, exp_bits, max_norm, rmode, int(denorm),
+                                        None if q is None else q.data_ptr(), code, x.numel(), act,
+                                        bits, exp_bits, max_norm, rmode, denorm,
                                         2 if mx_specs['vec_use_exp2'] else 0, _flags_value(),
                                         torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, lib)
     return out, aux, q
+
+
+def _fused_backward(grad_output, act, saved, aux, mx_specs):
+    """The backward chain of one activation as a single kernel launch (mxq_activation_backward)
+    from the tensors the forward pass saved, or None when the kernel does not cover the case."""
+    from . import _lib
+    from .custom_extensions import _flags_value
+    from .elemwise_ops import fused_chain_args
+    args = fused_chain_args(grad_output, mx_specs)
+    if args is None or grad_output.numel() == 0:
+        return None
+    g, code, (bits, exp_bits, max_norm, rmode, denorm) = args
+    others = [saved] + ([aux] if aux is not None else [])
+    if any(t.dtype != g.dtype or t.shape != g.shape or t.device != g.device for t in others):
+        return None
+    g, saved = g.contiguous(), saved.contiguous()
+    aux = None if aux is None else aux.contiguous()
+    out = torch.empty_like(g)
+    lib = _lib.gpu()
+    with torch.cuda.device(g.device):
+        rc = lib.mxq_activation_backward(g.data_ptr(), saved.data_ptr(),
+                                         None if aux is None else aux.data_ptr(), out.data_ptr(),
+                                         code, g.numel(), act, bits, exp_bits, max_norm, rmode, denorm,
+                                         _flags_value(), torch.cuda.current_stream(g.device).cuda_stream)
+    _lib.check(rc, lib)
+    return out
 
 
 def _logistic(x, specs):
@@ -101,6 +113,9 @@ class SigmoidFunction(torch.autograd.Function):
     def backward(ctx, grad_output):
         out, = ctx.saved_tensors
         s = ctx.mx_specs
+        fused = _fused_backward(grad_output, ACT_SIGMOID, out, None, s)
+        if fused is not None:
+            return (fused, None, None)
         g = vec_quantize(grad_output, mx_specs=s)
         d = vec_mul(out, vec_sub(1, out, mx_specs=s), mx_specs=s)
         return (vec_mul(d, g, mx_specs=s), None, None)
@@ -121,6 +136,9 @@ class TanhFunction(torch.autograd.Function):
     def backward(ctx, grad_output):
         out, = ctx.saved_tensors
         s = ctx.mx_specs
+        fused = _fused_backward(grad_output, ACT_TANH, out, None, s)
+        if fused is not None:
+            return (fused, None, None)
         g = vec_quantize(grad_output, mx_specs=s)
         d = vec_sub(1, vec_mul(out, out, mx_specs=s), mx_specs=s)
         return (vec_mul(d, g, mx_specs=s), None, None)
@@ -213,6 +231,9 @@ class SiLUFunction(torch.autograd.Function):
     def backward(ctx, grad_output):
         y, sig = ctx.saved_tensors
         s = ctx.mx_specs
+        fused = _fused_backward(grad_output, ACT_SILU, y, sig, s)
+        if fused is not None:
+            return (fused, None, None, None)
         g = vec_quantize(grad_output, mx_specs=s)
         d = vec_add(sig, vec_mul(y, vec_sub(1., sig, mx_specs=s), mx_specs=s), mx_specs=s)
         return (vec_mul(d, g, mx_specs=s), None, None, None)
@@ -249,6 +270,10 @@ class GELUFunction(torch.autograd.Function):
     def backward(ctx, grad_output):
         x, phi = ctx.saved_tensors
         s = ctx.mx_specs
+        fused = _fused_backward(grad_output, ACT_GELU_FIRST_ORDER if ctx.first_order_gelu else ACT_GELU,
+                                x, phi, s)
+        if fused is not None:
+            return (fused, None, None, None)
         g = vec_quantize(grad_output, mx_specs=s)
         dphi = vec_mul(phi, vec_sub(1, phi, mx_specs=s), mx_specs=s)       # sigmoid'(y)
         if ctx.first_order_gelu:

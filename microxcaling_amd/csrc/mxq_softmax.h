@@ -337,5 +337,152 @@ __global__ __launch_bounds__(TPB) void activation_kernel(const void* __restrict_
     }
 }
 
-}  // namespace
+// The backward passes of the same activations (mx/activations.py:251-267, 284-297, 437-455,
+// 500-557) from the tensors their forward passes saved; only exact arithmetic and the quantizer,
+// so the results are those of the chain of vec_* ops bit for bit.
+//   g = Q(grad_output)
+//   sigmoid: d = Q(s Q(1 - s))                       s = saved output
+//   tanh:    d = Q(1 - Q(t t))                       t = saved output
+//   silu:    d = Q(s + Q(y Q(1 - s)))                y = saved output, s = saved sigmoid
+//   gelu:    p = Q(phi Q(1 - phi)); first order: p = Q(1.703125 p);
+//            cubic: p = Q(Q(1.59375 + Q(0.2138671875 Q(x x))) p);  d = Q(phi + Q(x p))
+//   grad_input = Q(d g)
+template <int DT, int RMODE, int QMODE>
+__global__ __launch_bounds__(TPB) void activation_backward_kernel(const void* __restrict__ grad_,
+                                                                  const void* __restrict__ saved_,
+                                                                  const void* __restrict__ aux_,
+                                                                  void* __restrict__ out_, int64_t n,
+                                                                  ActParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int EPV = 4 * PD;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.q.zone_row]);
 
+    auto Qd = [&](float v) {
+        if (QMODE == SMQ_IDENT) return v;
+        if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, p.q.fmt.nan_from);
+        return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
+                                                          p.q.allow_denorm != 0, zone, ZS);
+    };
+    auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
+    auto eval = [&](float grad, float sv, float ax) {
+        const float g = Qd(grad);
+        float d;
+        switch (p.act) {
+            case ACT_SIGMOID: d = Q(sv * Q(1.0f - sv)); break;
+            case ACT_TANH: d = Q(1.0f - Q(sv * sv)); break;
+            case ACT_SILU: d = Q(ax + Q(sv * Q(1.0f - ax))); break;
+            default: {
+                float dphi = Q(ax * Q(1.0f - ax));
+                if (p.act == ACT_GELU_FIRST_ORDER) dphi = Q(1.703125f * dphi);
+                else dphi = Q(Q(1.59375f + Q(0.2138671875f * Q(sv * sv))) * dphi);
+                d = Q(ax + Q(sv * dphi));
+            }
+        }
+        return Q(d * g);
+    };
+
+    const bool two = p.act >= ACT_SILU;                      // a second saved tensor
+    const u32x4* grad = reinterpret_cast<const u32x4*>(grad_);
+    const u32x4* saved = reinterpret_cast<const u32x4*>(saved_);
+    const u32x4* aux = reinterpret_cast<const u32x4*>(aux_);
+    u32x4* out = reinterpret_cast<u32x4*>(out_);
+    const int64_t n_vec = n / EPV;
+    const int64_t stride = (int64_t)gridDim.x * TPB;
+    for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n_vec; i += stride) {
+        const u32x4 gv = grad[i], sv = saved[i];
+        const u32x4 av = two ? aux[i] : u32x4{0, 0, 0, 0};
+        u32x4 o;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            float r[2];
+#pragma unroll
+            for (int h = 0; h < PD; ++h)
+                r[h] = eval(Pack<DT>::get(gv[d], h), Pack<DT>::get(sv[d], h), Pack<DT>::get(av[d], h));
+            o[d] = Pack<DT>::put(r[0], r[PD - 1]);
+        }
+        __builtin_nontemporal_store(o, &out[i]);
+    }
+    const int64_t t0 = n_vec * EPV;
+    const int64_t gi = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (gi < n - t0) {
+        const float r = eval(load_scalar<DT>(grad_, t0 + gi), load_scalar<DT>(saved_, t0 + gi),
+                             two ? load_scalar<DT>(aux_, t0 + gi) : 0.0f);
+        store_scalar<DT>(out_, t0 + gi, mxq_round_dt<ADT>(r));
+    }
+}
+
+// SoftmaxFunction.backward (mx/softmax.py:56-88) over the last axis, same work mapping as the
+// forward kernel:  g = Q(grad); s = Q(sum Q(g y)); grad_input = Q(y Q(g - s)) (, Q(. * ln2) for
+// softmax_exp2, with ln2 at bfloat16 precision).
+template <int DT, int RMODE, int QMODE, int VPL>
+__global__ __launch_bounds__(TPB) void softmax_backward_row_kernel(const void* __restrict__ grad_,
+                                                                   const void* __restrict__ y_,
+                                                                   void* __restrict__ out_, int64_t rows,
+                                                                   int n, SoftmaxParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int EPV = 4 * PD;
+    constexpr int EPL = VPL * EPV;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.q.zone_row]);
+
+    auto Qd = [&](float v) {
+        if (QMODE == SMQ_IDENT) return v;
+        if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, p.q.fmt.nan_from);
+        return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
+                                                          p.q.allow_denorm != 0, zone, ZS);
+    };
+    auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
+
+    const int lane = threadIdx.x & 63;
+    const int nvec = n / EPV;
+    const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
+    for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows; row += waves) {
+        const u32x4* gin = reinterpret_cast<const u32x4*>(grad_) + row * nvec;
+        const u32x4* yin = reinterpret_cast<const u32x4*>(y_) + row * nvec;
+        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec;
+        float g[EPL];
+        u32x4 yraw[VPL];
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const bool valid = j * 64 + lane < nvec;
+            u32x4 graw = {0, 0, 0, 0};
+            yraw[j] = u32x4{0, 0, 0, 0};
+            if (valid) {
+                graw = gin[j * 64 + lane];
+                yraw[j] = yin[j * 64 + lane];
+            }
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const int e = (j * 4 + d) * PD + h;
+                    g[e] = valid ? Qd(Pack<DT>::get(graw[d], h)) : 0.0f;
+                    sum += valid ? Q(g[e] * Pack<DT>::get(yraw[j][d], h)) : 0.0f;
+                }
+        }
+        sum = Q(wave_reduce<SumOp>(sum));
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            u32x4 o;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                float q[2];
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const float t = Q(Pack<DT>::get(yraw[j][d], h) * Q(g[(j * 4 + d) * PD + h] - sum));
+                    q[h] = p.exp_mode == 1 ? Q(t * 0.69140625f) : t;
+                }
+                o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+            }
+            if (j * 64 + lane < nvec) __builtin_nontemporal_store(o, &out[j * 64 + lane]);
+        }
+    }
+}
+
+}  // namespace

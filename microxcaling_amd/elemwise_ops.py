@@ -111,6 +111,33 @@ def elemwise_plan(mx_specs, round=None):
     return ("identity",)
 
 
+_CHAIN_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
+
+
+def fused_chain_args(x, mx_specs, round=None):
+    """For the kernels that run a whole chain of "tensor op, then quantize_elemwise_op" steps on a
+    GPU tensor: (x, dtype code, (bits, exp_bits, max_norm, rounding code, allow_denorm)) with x
+    cast to bf16 where the chain's first quantization would do that, or None when such a kernel
+    cannot stand in for the chain (CPU or fp16 tensors, fused kernels switched off,
+    round-half-even to a wide format on a bf16 tensor).  bits == 0 means "no format"."""
+    from . import gemm
+    if not (gemm.fused_enabled() and x.is_cuda):
+        return None
+    rnd = mx_specs['round'] if round is None else round
+    plan = elemwise_plan(mx_specs, rnd)
+    if plan[0] == "to_bf16":
+        x = x.to(torch.bfloat16)
+        plan = ("identity",)
+    if x.dtype not in _CHAIN_DTYPE_CODE:
+        return None
+    if plan[0] == "identity":
+        return x, _CHAIN_DTYPE_CODE[x.dtype], (0, 0, 1.0, 0, 1)
+    _, bits, exp_bits, max_norm, denorm = plan
+    if x.dtype == torch.bfloat16 and bits >= 9 and rnd == 'even':
+        return None
+    return x, _CHAIN_DTYPE_CODE[x.dtype], (bits, exp_bits, max_norm, _native_round(rnd), int(denorm))
+
+
 def quantize_elemwise_op(A, mx_specs, round=None):
     """Elementwise quantization selected by mx_specs['bfloat'] / ['fp']
     (mx/elemwise_ops.py:233-267)."""

@@ -10,7 +10,6 @@ from .vector_ops import (vec_add, vec_mul, vec_quantize, vec_recip, vec_reduce_m
 torch_layer_norm = F.layer_norm
 
 
-_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
 MAX_FUSED_ROW = 4096
 
 
@@ -20,28 +19,20 @@ def _fused_forward(x, bf_weight, bf_bias, eps, mx_specs, rms):
     statistic) or None when the kernel does not cover the case (CPU tensors, rows longer than 4096
     or not a multiple of 16 bytes, fp16, mixed dtypes, vec_use_recip, round-half-even to a wide
     format on bf16 tensors)."""
-    from . import _lib, gemm
+    from . import _lib
     from .custom_extensions import _flags_value
-    from .elemwise_ops import _native_round, elemwise_plan
-    if not (gemm.fused_enabled() and x.is_cuda) or mx_specs['vec_use_recip']:
+    from .elemwise_ops import fused_chain_args
+    if mx_specs['vec_use_recip']:
         return None
-    rnd = mx_specs['round']
-    plan = elemwise_plan(mx_specs, rnd)
-    if plan[0] == "to_bf16":                   # what the first quantization of the chain does
-        x = x.to(torch.bfloat16)
-        plan = ("identity",)
-    if x.dtype not in _DTYPE_CODE or bf_weight.dtype != x.dtype or bf_bias.dtype != x.dtype:
+    args = fused_chain_args(x, mx_specs)
+    if args is None:
+        return None
+    x, code, (bits, exp_bits, max_norm, rmode, denorm) = args
+    if bf_weight.dtype != x.dtype or bf_bias.dtype != x.dtype:
         return None
     n = x.shape[-1]
     if n == 0 or n > MAX_FUSED_ROW or n % (16 // x.element_size()) != 0 or bf_weight.numel() != n:
         return None
-    if plan[0] == "identity":
-        bits, exp_bits, max_norm, denorm, rmode = 0, 0, 1.0, True, 0
-    else:
-        _, bits, exp_bits, max_norm, denorm = plan
-        rmode = _native_round(rnd)
-        if x.dtype == torch.bfloat16 and bits >= 9 and rnd == 'even':
-            return None
     x = x.contiguous()
     w, b = bf_weight.contiguous(), bf_bias.contiguous()
     out, x_norm = torch.empty_like(x), torch.empty_like(x)
@@ -49,9 +40,9 @@ def _fused_forward(x, bf_weight, bf_bias, eps, mx_specs, rms):
     lib = _lib.gpu()
     with torch.cuda.device(x.device):
         rc = lib.mxq_norm_lastdim(x.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(),
-                                  x_norm.data_ptr(), stat.data_ptr(), _DTYPE_CODE[x.dtype],
+                                  x_norm.data_ptr(), stat.data_ptr(), code,
                                   x.numel() // n, n, float(eps), int(rms), bits, exp_bits, max_norm,
-                                  rmode, int(denorm), _flags_value(),
+                                  rmode, denorm, _flags_value(),
                                   torch.cuda.current_stream(x.device).cuda_stream)
     _lib.check(rc, lib)
     return out, x_norm, stat

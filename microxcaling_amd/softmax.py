@@ -10,48 +10,66 @@ from .vector_ops import (vec_div, vec_exp, vec_exp2, vec_mul, vec_quantize, vec_
 f_softmax = F.softmax
 LN_2_BF16 = 0.69140625           # ln(2) at bfloat16 precision
 
-_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
 MAX_FUSED_ROW = 4096
 
 
 def _fused_forward(input, dim, mx_specs):
     """The whole forward chain as one kernel launch (mxq_softmax_lastdim), or None when the kernel
-    does not cover the case: CPU tensors, another axis than the last, rows longer than 4096 or not
-    a multiple of 16 bytes, fp16 tensors, round-half-even to a wide format on a bf16 tensor."""
-    from . import _lib, gemm
-    from .elemwise_ops import _native_round, elemwise_plan
-    if not (gemm.fused_enabled() and input.is_cuda and dim == input.dim() - 1):
+    does not cover the case: another axis than the last, rows longer than 4096 or not a multiple
+    of 16 bytes, and what fused_chain_args excludes."""
+    from . import _lib
+    from .custom_extensions import _flags_value
+    from .elemwise_ops import fused_chain_args
+    if dim != input.dim() - 1:
         return None
-    rnd = mx_specs['round']
-    plan = elemwise_plan(mx_specs, rnd)
-    if plan[0] == "to_bf16":
-        input = input.to(torch.bfloat16)       # the first quantization of the chain does this
-        plan = ("identity",)
-    if input.dtype not in _DTYPE_CODE:
+    args = fused_chain_args(input, mx_specs)
+    if args is None:
         return None
-    n = input.shape[-1]
-    if n == 0 or n > MAX_FUSED_ROW or n % (16 // input.element_size()) != 0:
+    x, code, (bits, exp_bits, max_norm, rmode, denorm) = args
+    n = x.shape[-1]
+    if n == 0 or n > MAX_FUSED_ROW or n % (16 // x.element_size()) != 0:
         return None
-    if plan[0] == "identity":
-        bits, exp_bits, max_norm, denorm, rmode = 0, 0, 1.0, True, 0
-    else:
-        _, bits, exp_bits, max_norm, denorm = plan
-        rmode = _native_round(rnd)
-        if input.dtype == torch.bfloat16 and bits >= 9 and rnd == 'even':
-            return None
     if mx_specs.get('softmax_exp2', False):
         exp_mode = 1
     else:
         exp_mode = 2 if mx_specs['vec_use_exp2'] else 0
-    x = input.contiguous()
+    x = x.contiguous()
     out = torch.empty_like(x)
     lib = _lib.gpu()
-    from .custom_extensions import _flags_value
     with torch.cuda.device(x.device):
-        rc = lib.mxq_softmax_lastdim(x.data_ptr(), out.data_ptr(), _DTYPE_CODE[x.dtype],
-                                     x.numel() // n, n, bits, exp_bits, max_norm, rmode, int(denorm),
-                                     exp_mode, int(bool(mx_specs['vec_use_recip'])), _flags_value(),
+        rc = lib.mxq_softmax_lastdim(x.data_ptr(), out.data_ptr(), code, x.numel() // n, n, bits,
+                                     exp_bits, max_norm, rmode, denorm, exp_mode,
+                                     int(bool(mx_specs['vec_use_recip'])), _flags_value(),
                                      torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check(rc, lib)
+    return out
+
+
+def _fused_backward(grad_output, output, dim, mx_specs):
+    """The backward chain as one kernel launch (mxq_softmax_backward_lastdim), under the same
+    conditions as _fused_forward; None otherwise."""
+    from . import _lib
+    from .custom_extensions import _flags_value
+    from .elemwise_ops import fused_chain_args
+    if dim != grad_output.dim() - 1:
+        return None
+    args = fused_chain_args(grad_output, mx_specs)
+    if args is None:
+        return None
+    g, code, (bits, exp_bits, max_norm, rmode, denorm) = args
+    n = g.shape[-1]
+    if n == 0 or n > MAX_FUSED_ROW or n % (16 // g.element_size()) != 0:
+        return None
+    if output.dtype != g.dtype or output.shape != g.shape or output.device != g.device:
+        return None
+    g, y = g.contiguous(), output.contiguous()
+    out = torch.empty_like(g)
+    lib = _lib.gpu()
+    with torch.cuda.device(g.device):
+        rc = lib.mxq_softmax_backward_lastdim(g.data_ptr(), y.data_ptr(), out.data_ptr(), code,
+                                              g.numel() // n, n, bits, exp_bits, max_norm, rmode, denorm,
+                                              int(bool(mx_specs.get('softmax_exp2', False))), _flags_value(),
+                                              torch.cuda.current_stream(g.device).cuda_stream)
     _lib.check(rc, lib)
     return out
 
@@ -88,6 +106,9 @@ class SoftmaxFunction(torch.autograd.Function):
         output, = ctx.saved_tensors
         specs = ctx.mx_specs
         rnd = specs['round']
+        fused = _fused_backward(grad_output, output, ctx.dim, specs)
+        if fused is not None:
+            return (fused, None, None, None)
         grad_output = vec_quantize(grad_output, mx_specs=specs, round=rnd)
         dot = vec_mul(grad_output, output, mx_specs=specs, round=rnd)
         dot = vec_reduce_sum(dot, ctx.dim, keepdim=True, mx_specs=specs, round=rnd)

@@ -519,3 +519,62 @@ def test_fused_activation_special_values(dev, act, dtype):
     got = _ACTS[act](A, x.to(dev), specs)
     want = _ACTS[act](A, x, specs)
     _one_step_apart(got, want, 0.2)
+
+
+@pytest.mark.parametrize("act", sorted(_ACTS))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=12), dict(bfloat=16, round="floor"),
+                                  dict(bfloat=16, quantize_backprop=False)],
+                         ids=["bfloat16", "bfloat12", "bfloat16-floor", "no-backprop-quantization"])
+def test_fused_activation_backward_equals_chain(dev, act, dtype, spec):
+    """The backward kernel has only exact arithmetic and the quantizer in it: from the same saved
+    tensors it must give the chain of vec_* ops bit for bit (special values included)."""
+    from microxcaling_amd import activations as A, gemm
+    specs = _specs(**spec)
+    g = torch.Generator().manual_seed(len(act))
+    x = (torch.randn(130, 257, generator=g) * 3).to(dtype)
+    x[0, :8] = torch.tensor([0.0, -0.0, float("inf"), float("-inf"), float("nan"), 1e-30, 88.0, -88.0]).to(dtype)
+    grad = (torch.randn(130, 257, generator=g) * torch.exp2(torch.randint(-20, 20, (130, 257), generator=g).float())).to(dtype)
+    grad[1, :3] = torch.tensor([float("inf"), float("nan"), 0.0]).to(dtype)
+    xi = x.to(dev).requires_grad_(True)
+    y = _ACTS[act](A, xi, specs)
+    grads = []
+    for fused in (True, False):
+        gemm.set_fused(fused)
+        try:
+            xi.grad = None
+            y.backward(grad.to(dev), retain_graph=True)
+            grads.append(xi.grad.clone())
+        finally:
+            gemm.set_fused(True)
+    assert_bits_equal(grads[0].cpu(), grads[1].cpu(), act)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, softmax_exp2=True), dict(bfloat=12)],
+                         ids=["bfloat16", "bfloat16-exp2", "bfloat12"])
+@pytest.mark.parametrize("shape", [(3, 5, 2048), (64, 1000), (33, 264)])
+def test_fused_softmax_backward_against_chain(dev, dtype, spec, shape):
+    """One-kernel softmax backward against the chain of vec_* ops on the same saved output; only the
+    order of the row sum differs."""
+    from microxcaling_amd import gemm
+    from microxcaling_amd.softmax import softmax
+    specs = _specs(**spec)
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g) * 3).to(dtype).to(dev).requires_grad_(True)
+    grad = torch.randn(*shape, generator=g).to(dtype).to(dev)
+    y = softmax(x, dim=-1, mx_specs=specs)
+    grads = []
+    for fused in (True, False):
+        gemm.set_fused(fused)
+        try:
+            x.grad = None
+            y.backward(grad, retain_graph=True)
+            grads.append(x.grad.clone())
+        finally:
+            gemm.set_fused(True)
+    got, want = grads[0].float().cpu(), grads[1].float().cpu()
+    scale = want.abs().max().item()
+    d = (got - want).abs()
+    assert d.max().item() <= 2.0 ** -6 * scale
+    assert (d > 0).float().mean().item() <= 0.05
