@@ -221,6 +221,31 @@ def make_workload(name):
                     launches=1 if fused else 12,
                     desc="%s, bfloat16 quantization after every step, %s" % (what, "one kernel" if fused else
                                                                              "separate tensor passes"))
+    if name in ("layernorm_bf16_train", "layernorm_bf16_train_unfused"):
+        # LayerNorm forward + backward over bf16 [32768, 4096]: two row kernels + the parameter
+        # gradients (column sums, separate steps either way)
+        from microxcaling_amd import gemm
+        from microxcaling_amd.layernorm import LayerNorm
+        from microxcaling_amd.specs import finalize_mx_specs
+        specs = finalize_mx_specs({"bfloat": 16})
+        fused = not name.endswith("unfused")
+        x = (torch.randn(32768, 4096, generator=torch.Generator().manual_seed(6)) * 2 + 0.5).to(torch.bfloat16)
+        ln = {}
+
+        def run(xd):
+            if "m" not in ln:
+                ln["m"] = LayerNorm(4096, eps=1e-5, mx_specs=specs).to(torch.bfloat16).to(xd.device)
+                ln["g"] = torch.randn(xd.shape, generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(xd.device)
+            gemm.set_fused(fused)
+            xi = xd.requires_grad_(True)
+            xi.grad = None
+            ln["m"](xi).backward(ln["g"])
+            return xi.grad
+        cpu_ln = LayerNorm(4096, eps=1e-5, mx_specs=specs).to(torch.bfloat16)
+        return dict(x=x, gpu=run, cpu=lambda t: cpu_ln(t), bytes=x.numel() * (6 + 8 + 6), dtype="bf16", sample_axis=0,
+                    launches=9 if fused else 50,
+                    desc="LayerNorm forward + backward, bf16 [32768,4096], bfloat16 quantization after every step, %s"
+                         % ("row kernels + separate parameter gradients" if fused else "separate tensor passes"))
     if name in ("gelu_bf16_train", "gelu_bf16_train_unfused", "softmax_bf16_train", "softmax_bf16_train_unfused"):
         # forward + backward of one bfloat16 layer: the fused forward kernel writes what the fused
         # backward kernel reads

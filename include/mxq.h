@@ -127,6 +127,16 @@ int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void*
                      int bits, int exp_bits, float max_norm, int rmode, int allow_denorm, int flags,
                      void* hip_stream);
 
+/* The gradient with respect to the input of the same two layers (LayerNormFunction.backward via
+ * _norm_backward_LN, mx/norm_utils.py:188-258; RMSNormFunction.backward, mx/layernorm.py:150-168)
+ * from what mxq_norm_lastdim wrote: x_norm and row_stat.  weight: the n values the layer saved.
+ * The gradients of weight and bias are column sums and stay separate steps.  Agrees with the
+ * reference's chain up to the order of the row sums. */
+int mxq_norm_backward_lastdim(const void* grad_out, const void* weight, const void* x_norm,
+                              const void* row_stat, void* grad_in, int dtype, int64_t rows, int64_t n,
+                              int rms_norm, int bits, int exp_bits, float max_norm, int rmode,
+                              int allow_denorm, int flags, void* hip_stream);
+
 /* The forward passes of SigmoidFunction, TanhFunction, SiLUFunction and GELUFunction
  * (mx/activations.py:237-297, 418-557) on a contiguous fp32 or bf16 tensor of n elements, as one
  * kernel, with the elementwise quantizer (bits / exp_bits / max_norm as in mxq_softmax_lastdim,

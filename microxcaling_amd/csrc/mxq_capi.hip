@@ -530,6 +530,41 @@ int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void*
     return check_launch(who);
 }
 
+int mxq_norm_backward_lastdim(const void* grad_out, const void* weight, const void* x_norm,
+                              const void* row_stat, void* grad_in, int dtype, int64_t rows, int64_t n,
+                              int rms_norm, int bits, int exp_bits, float max_norm, int rmode,
+                              int allow_denorm, int flags, void* hip_stream) {
+    const char* who = "mxq_norm_backward_lastdim";
+    NormParams p;
+    bool ident, closed;
+    int rc = chain_params(dtype, bits, exp_bits, max_norm, rmode, allow_denorm, flags, &p.q, &ident, &closed, who);
+    if (rc) return rc;
+    p.eps = 0.0f;
+    p.rms = rms_norm ? 1 : 0;
+    const int epv = dtype == MXQ_DTYPE_F32 ? 4 : 8;
+    if (rows < 0 || n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (n > 4096 || n % epv != 0)
+        return fail(MXQ_ERR_ARGUMENT, "%s: row length %lld must be a multiple of %d and at most 4096",
+                    who, (long long)n, epv);
+    if (rows == 0 || n == 0) return MXQ_OK;
+    if (!grad_out || !weight || !x_norm || !row_stat || !grad_in) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(grad_out) || !aligned16(weight) || !aligned16(x_norm) || !aligned16(grad_in))
+        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int grid = grid_for(ceil_div(rows, kThreads / 64));
+    const int64_t nvec = n / epv;
+#define MXQ_NMB(DT, RM, QM)                                                                        \
+    do {                                                                                           \
+        constexpr int V = (DT == MXQ_F32) ? 2 : 1;                                                 \
+        if (nvec <= 128 * V) norm_backward_row_kernel<DT, RM, QM, 2 * V><<<grid, kThreads, 0, s>>>(grad_out, weight, x_norm, row_stat, grad_in, rows, (int)n, p);      \
+        else if (nvec <= 256 * V) norm_backward_row_kernel<DT, RM, QM, 4 * V><<<grid, kThreads, 0, s>>>(grad_out, weight, x_norm, row_stat, grad_in, rows, (int)n, p); \
+        else norm_backward_row_kernel<DT, RM, QM, 8 * V><<<grid, kThreads, 0, s>>>(grad_out, weight, x_norm, row_stat, grad_in, rows, (int)n, p);                     \
+    } while (0)
+    MXQ_CHAIN_DISPATCH(MXQ_NMB);
+#undef MXQ_NMB
+    return check_launch(who);
+}
+
 int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t rows, int64_t K,
                 int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
                 int flush_fp32_subnorms, int rmode, int flags, void* hip_stream) {

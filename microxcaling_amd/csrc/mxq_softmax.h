@@ -485,4 +485,116 @@ __global__ __launch_bounds__(TPB) void softmax_backward_row_kernel(const void* _
     }
 }
 
+// Gradient with respect to the input of LayerNorm / RMSNorm over the last axis from what the
+// forward pass saved (mx/norm_utils.py:188-258 with axes = -1, mx/layernorm.py:150-168), same work
+// mapping as norm_row_kernel.  With g = Q(grad_output), d = Q(g w), n = row length:
+//   LayerNorm: sd = Q(sqrt v), si = Q(1 / sd)                                 (v = saved var + eps)
+//              t = Q(Q(Q(sum Q(Q(d z) sd)) / n) Q(1 / v))                     (z = saved normalized input)
+//              dx = Q(Q(d si) + Q(-t z));  grad_input = Q(dx - Q(Q(sum dx) / n))
+//   RMSNorm:   d1 = Q(d r), proj = Q(Q(sum Q(d1 z)) / n)                      (r = saved 1 / rms)
+//              grad_input = d1 - Q(z proj), rounded to the tensor dtype only
+template <int DT, int RMODE, int QMODE, int VPL>
+__global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __restrict__ grad_,
+                                                                const void* __restrict__ weight_,
+                                                                const void* __restrict__ znorm_,
+                                                                const void* __restrict__ stat_,
+                                                                void* __restrict__ out_, int64_t rows, int n,
+                                                                NormParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int EPV = 4 * PD;
+    constexpr int EPL = VPL * EPV;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.q.zone_row]);
+
+    auto Qd = [&](float v) {
+        if (QMODE == SMQ_IDENT) return v;
+        if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, p.q.fmt.nan_from);
+        return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
+                                                          p.q.allow_denorm != 0, zone, ZS);
+    };
+    auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
+
+    const int lane = threadIdx.x & 63;
+    const int nvec = n / EPV;
+    const float count = (float)n;
+    const u32x4* wv = reinterpret_cast<const u32x4*>(weight_);
+    const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
+    for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows; row += waves) {
+        const u32x4* gin = reinterpret_cast<const u32x4*>(grad_) + row * nvec;
+        const u32x4* zin = reinterpret_cast<const u32x4*>(znorm_) + row * nvec;
+        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec;
+        const float stat = load_scalar<DT>(stat_, row);
+        // row scalars
+        const float sd = p.rms ? 0.0f : Q(sqrtf(stat));
+        const float si = p.rms ? stat : Q(1.0f / sd);
+        float d[EPL];                                        // Q(g w), then Q(d si)
+        u32x4 zraw[VPL];
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const bool valid = j * 64 + lane < nvec;
+            u32x4 graw = {0, 0, 0, 0}, wraw = {0, 0, 0, 0};
+            zraw[j] = u32x4{0, 0, 0, 0};
+            if (valid) {
+                graw = gin[j * 64 + lane];
+                wraw = wv[j * 64 + lane];
+                zraw[j] = zin[j * 64 + lane];
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const int e = (j * 4 + k) * PD + h;
+                    const float z = Pack<DT>::get(zraw[j][k], h);
+                    const float dn = Q(Qd(Pack<DT>::get(graw[k], h)) * Pack<DT>::get(wraw[k], h));
+                    if (p.rms) {
+                        d[e] = Q(dn * si);
+                        sum += valid ? Q(d[e] * z) : 0.0f;
+                    } else {
+                        d[e] = Q(dn * si);
+                        sum += valid ? Q(Q(dn * z) * sd) : 0.0f;
+                    }
+                }
+        }
+        float t = Q(Q(wave_reduce<SumOp>(sum)) / count);
+        if (!p.rms) t = -Q(t * Q(1.0f / stat));
+        float sum2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const bool valid = j * 64 + lane < nvec;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const int e = (j * 4 + k) * PD + h;
+                    const float z = Pack<DT>::get(zraw[j][k], h);
+                    if (p.rms) {
+                        d[e] = mxq_round_dt<ADT>(d[e] - Q(z * t));
+                    } else {
+                        d[e] = Q(d[e] + Q(t * z));
+                        sum2 += valid ? d[e] : 0.0f;
+                    }
+                }
+        }
+        const float dm = p.rms ? 0.0f : -Q(Q(wave_reduce<SumOp>(sum2)) / count);
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            u32x4 o;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                float q[2];
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const float v = d[(j * 4 + k) * PD + h];
+                    q[h] = p.rms ? v : Q(v + dm);
+                }
+                o[k] = Pack<DT>::put(q[0], q[PD - 1]);
+            }
+            if (j * 64 + lane < nvec) __builtin_nontemporal_store(o, &out[j * 64 + lane]);
+        }
+    }
+}
+
 }  // namespace

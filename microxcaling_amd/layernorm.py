@@ -52,6 +52,38 @@ def _leading_axes(t):
     return list(range(t.ndim - 1))
 
 
+def _fused_grad_input(grad_output, weight, x_norm, stat, mx_specs, rms):
+    """The gradient with respect to the input as one kernel launch (mxq_norm_backward_lastdim) from
+    the saved normalized input and row statistic, under the conditions of _fused_forward; None
+    otherwise."""
+    from . import _lib
+    from .custom_extensions import _flags_value
+    from .elemwise_ops import fused_chain_args
+    if mx_specs['vec_use_recip']:
+        return None
+    args = fused_chain_args(grad_output, mx_specs)
+    if args is None:
+        return None
+    g, code, (bits, exp_bits, max_norm, rmode, denorm) = args
+    n = g.shape[-1]
+    if n == 0 or n > MAX_FUSED_ROW or n % (16 // g.element_size()) != 0 or weight.numel() != n:
+        return None
+    rows = g.numel() // n
+    if any(t.dtype != g.dtype or t.device != g.device for t in (weight, x_norm, stat)) \
+            or x_norm.shape != g.shape or stat.numel() != rows:
+        return None
+    g, w, z, st = g.contiguous(), weight.contiguous(), x_norm.contiguous(), stat.contiguous()
+    out = torch.empty_like(g)
+    lib = _lib.gpu()
+    with torch.cuda.device(g.device):
+        rc = lib.mxq_norm_backward_lastdim(g.data_ptr(), w.data_ptr(), z.data_ptr(), st.data_ptr(),
+                                           out.data_ptr(), code, rows, n, int(rms), bits, exp_bits,
+                                           max_norm, rmode, denorm, _flags_value(),
+                                           torch.cuda.current_stream(g.device).cuda_stream)
+    _lib.check(rc, lib)
+    return out
+
+
 def _param_grads(grad_output, x_norm, specs):
     """grad_bias = sum(g), grad_weight = sum(g * x_norm) over every axis but the last."""
     axes = _leading_axes(grad_output)
@@ -84,7 +116,9 @@ class LayerNormFunction(torch.autograd.Function):
         s = ctx.mx_specs
         grad_output = vec_quantize(grad_output, mx_specs=s)
         grad_weight, grad_bias = _param_grads(grad_output, x_norm, s)
-        grad_input = _norm_backward_LN(grad_output, -1, weight, x_norm, x_vare, s)
+        grad_input = _fused_grad_input(grad_output, weight, x_norm, x_vare, s, rms=False)
+        if grad_input is None:
+            grad_input = _norm_backward_LN(grad_output, -1, weight, x_norm, x_vare, s)
         return (grad_input, grad_weight, grad_bias, None, None, None)
 
 
@@ -116,6 +150,9 @@ class RMSNormFunction(torch.autograd.Function):
         s = ctx.mx_specs
         grad_output = vec_quantize(grad_output, mx_specs=s)
         grad_weight, grad_bias = _param_grads(grad_output, x_norm, s)
+        fused = _fused_grad_input(grad_output, weight, x_norm, rms_inv, s, rms=True)
+        if fused is not None:
+            return (fused, grad_weight, grad_bias, None, None, None)
         dx1 = vec_mul(vec_mul(grad_output, weight, mx_specs=s), rms_inv, mx_specs=s)
         proj = vec_reduce_mean(vec_mul(dx1, x_norm, mx_specs=s), -1, keepdim=True, mx_specs=s)
         # the last subtraction carries no mx_specs in the reference (mx/layernorm.py:166): unquantized

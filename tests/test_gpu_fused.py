@@ -578,3 +578,40 @@ def test_fused_softmax_backward_against_chain(dev, dtype, spec, shape):
     d = (got - want).abs()
     assert d.max().item() <= 2.0 ** -6 * scale
     assert (d > 0).float().mean().item() <= 0.05
+
+
+@pytest.mark.parametrize("kind", ["layernorm", "rmsnorm"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=12)], ids=["bfloat16", "bfloat12"])
+@pytest.mark.parametrize("shape", [(6, 40, 1024), (257, 264), (9, 4096)])
+def test_fused_norm_backward_against_chain(dev, kind, dtype, spec, shape):
+    """One-kernel gradient with respect to the input of LayerNorm / RMSNorm against the chain of
+    vec_* ops from the same saved tensors; only the order of the two row sums differs.  The
+    parameter gradients come from the same separate steps either way."""
+    from microxcaling_amd import gemm, layernorm as L
+    specs = _specs(**spec)
+    g = torch.Generator().manual_seed(sum(shape))
+    n = shape[-1]
+    mod = (L.LayerNorm if kind == "layernorm" else L.RMSNorm)(n, eps=1e-5, mx_specs=specs)
+    with torch.no_grad():
+        mod.weight.copy_(1 + 0.3 * torch.randn(n, generator=g))
+        mod.bias.copy_(0.1 * torch.randn(n, generator=g))
+    mod = mod.to(dtype).to(dev)
+    x = (torch.randn(*shape, generator=g) * 2 + 0.5).to(dtype).to(dev).requires_grad_(True)
+    grad = torch.randn(*shape, generator=g).to(dtype).to(dev)
+    y = mod(x)
+    res = []
+    for fused in (True, False):
+        gemm.set_fused(fused)
+        try:
+            x.grad = None
+            mod.weight.grad = None
+            y.backward(grad, retain_graph=True)
+            res.append((x.grad.clone(), mod.weight.grad.clone()))
+        finally:
+            gemm.set_fused(True)
+    assert torch.equal(res[0][1], res[1][1])
+    got, want = res[0][0].float().cpu(), res[1][0].float().cpu()
+    d = (got - want).abs()
+    assert d.max().item() <= 2.0 ** -5 * want.abs().max().item()
+    assert (d > 0).float().mean().item() <= 0.08
