@@ -6,8 +6,10 @@
 Usage:  python -m microxcaling_amd.build_ext
 hipcc cross-compiles, so no GPU is needed to build.
 """
+import concurrent.futures
 import os
 import subprocess
+import tempfile
 import sys
 
 PKG = os.path.dirname(os.path.abspath(__file__))
@@ -35,12 +37,24 @@ def _run(cmd, verbose):
         print(out, flush=True)
 
 
+GPU_SOURCES = ["mxq_capi.hip", "mxq_capi_gemm.hip", "mxq_capi_chain.hip"]
+
+
 def build_gpu(verbose=True):
-    cmd = [os.path.join(ROCM, "bin", "hipcc"), "--offload-arch=gfx950",
-           # keep fp32 math scalar: packed fp32 instructions are not used by these kernels
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           *COMMON, "-o", GPU_LIB, os.path.join(CSRC, "mxq_capi.hip")]
-    _run(cmd, verbose)
+    """Compiles the translation units side by side, then links them."""
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    flags = ["--offload-arch=gfx950",
+             # keep fp32 math scalar: packed fp32 instructions are not used by these kernels
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             *[f for f in COMMON if f != "-shared"]]
+    with tempfile.TemporaryDirectory(prefix="mxq_build_") as tmp:
+        objects = [os.path.join(tmp, os.path.splitext(src)[0] + ".o") for src in GPU_SOURCES]
+        with concurrent.futures.ThreadPoolExecutor(max_workers=len(GPU_SOURCES)) as pool:
+            jobs = [pool.submit(_run, [hipcc, *flags, "-c", "-o", obj, os.path.join(CSRC, src)], verbose)
+                    for src, obj in zip(GPU_SOURCES, objects)]
+            for job in jobs:
+                job.result()
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", GPU_LIB, *objects], verbose)
     return GPU_LIB
 
 

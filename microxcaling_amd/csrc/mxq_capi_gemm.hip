@@ -1,0 +1,243 @@
+// C ABI of libmxq_gfx950.so, continued: packed MX tensors and the scaled-MFMA GEMM.
+#include "mxq_capi_common.h"
+#include "mxq_gemm.h"
+
+namespace {
+
+template <int DT, int RMODE, bool ZE, bool LEAN>
+struct LaunchPack {
+    static void run(const void* in, void* codes, void* scales, int64_t n_vec, int kind, MxParams p,
+                    hipStream_t s) {
+        const int grid = grid_for(ceil_div(n_vec, (int64_t)kThreads * 4));
+        const u32x4* i4 = reinterpret_cast<const u32x4*>(in);
+        unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
+        if (kind == 1) mx_pack_kernel<DT, RMODE, ZE, 1, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+        else if (kind == 4) mx_pack_kernel<DT, RMODE, ZE, 4, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+        else mx_pack_kernel<DT, RMODE, ZE, 0, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+    }
+};
+
+template <int DT, int RMODE, bool ZE, bool LEAN>
+struct LaunchPackT {
+    static void run(const void* in, void* codes, void* scales, int64_t items, int64_t n_tiles,
+                    int64_t pv, int kind, MxParams p, hipStream_t s) {
+        const unsigned grid = (unsigned)ceil_div(items, kThreads);
+        const u32x2* i2 = reinterpret_cast<const u32x2*>(in);
+        unsigned char* c = reinterpret_cast<unsigned char*>(codes);
+        unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
+        if (kind == 1) mx_pack_t_kernel<DT, RMODE, ZE, 1><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+        else if (kind == 4) mx_pack_t_kernel<DT, RMODE, ZE, 4><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+        else mx_pack_t_kernel<DT, RMODE, ZE, 0><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+    }
+};
+
+template <int CB, int BL, int ODT>
+int launch_gemm_dt(int64_t batch, const GemmArgs& g, hipStream_t s) {
+    // large problems: persistent 256 x 256 tile kernel (144 KB of dynamic LDS, one workgroup per CU);
+    // it fetches 16 scale bytes per row at a time, hence K % 512
+    const int64_t tiles_m = ceil_div(g.M, G2_BM), tiles_n = ceil_div(g.N, G2_BN);
+    const int64_t total = tiles_m * tiles_n * batch;
+    if (g.M >= 512 && g.N >= 512 && g.K % 512 == 0 && (int64_t)256 * g.kbytes < ((int64_t)1 << 31) &&
+        total < ((int64_t)1 << 30)) {
+        static bool configured = false;               // raising the dynamic-LDS limit is per kernel
+        static int cus = 0;
+        if (!configured) {
+            hipError_t e = hipFuncSetAttribute(
+                reinterpret_cast<const void*>(&mx_gemm_nt_kernel_256p<CB, BL, ODT>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, G3_LDS_BYTES);
+            int dev = 0;
+            if (e == hipSuccess) e = hipGetDevice(&dev);
+            if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            if (e != hipSuccess || cus <= 0)
+                return fail(MXQ_ERR_LAUNCH, "mxq_gemm_mx_nt: cannot configure the tile kernel (%d bytes of LDS): %s",
+                            G3_LDS_BYTES, hipGetErrorString(e));
+            cus -= cus % 8;                           // a workgroup must stay on its XCD from tile to tile
+            if (cus < 8) cus = 8;
+            configured = true;
+        }
+        const unsigned grid = (unsigned)(total < cus ? total : cus);
+        mx_gemm_nt_kernel_256p<CB, BL, ODT><<<grid, 512, G3_LDS_BYTES, s>>>(g, (int)tiles_m, (int)tiles_n, (int)total);
+    } else {
+        dim3 grid((unsigned)(ceil_div(g.N, GEMM_BN) * ceil_div(g.M, GEMM_BM)), (unsigned)batch);
+        mx_gemm_nt_kernel<CB, BL, ODT><<<grid, kThreads, 0, s>>>(g);
+    }
+    return MXQ_OK;
+}
+
+template <int CB, int BL>
+int launch_gemm(int c_dtype, int64_t batch, const GemmArgs& g, hipStream_t s) {
+    if (c_dtype == MXQ_DTYPE_F32) return launch_gemm_dt<CB, BL, MXQ_F32>(batch, g, s);
+    if (c_dtype == MXQ_DTYPE_BF16) return launch_gemm_dt<CB, BL, MXQ_BF16>(batch, g, s);
+    return launch_gemm_dt<CB, BL, MXQ_F16>(batch, g, s);
+}
+
+// splits of the outer axis for the two-pass outer reduction
+int code_kind(int ebits, int mbits, int flags, const char* who) {
+    const bool fp4 = ebits == 2 && mbits == 3;
+    if (flags & MXQ_FLAG_PACK_NIBBLES) {
+        if (!fp4) {
+            fail(MXQ_ERR_ARGUMENT, "%s: 4-bit codes exist for the e2m1 format only", who);
+            return -1;
+        }
+        return MXQ_CODES_E2M1;
+    }
+    if (ebits == 5 && mbits <= 4) return MXQ_CODES_E5M2;
+    if (ebits >= 2 && ebits <= 4 && mbits <= 5) return MXQ_CODES_E4M3;
+    fail(MXQ_ERR_ARGUMENT, "%s: element format e%dm%d has no 8-bit float code (supported: up to "
+         "e4m3, and e5m2)", who, ebits, mbits - 2);
+    return -1;
+}
+
+}  // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t rows, int64_t K,
+                int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                int flush_fp32_subnorms, int rmode, int flags, void* hip_stream) {
+    const char* who = "mxq_pack_mx";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    const int kind = code_kind(elem_ebits, elem_mbits, flags, who);
+    if (kind < 0) return MXQ_ERR_ARGUMENT;
+    if (rows < 0 || K < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (K % 32 != 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be a multiple of the block size 32", who);
+    int64_t total;
+    if (mul_overflows(rows, K, 1, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !codes || !scales) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(in) || !aligned16(codes))
+        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    dispatch<LaunchPack>(dtype, rmode, ze, true, in, codes, scales, total / (16 / elem_size(dtype)), kind,
+                         p, (hipStream_t)hip_stream);
+    return check_launch(who);
+}
+
+int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t batch, int64_t R,
+                  int64_t C, int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                  int flush_fp32_subnorms, int rmode, int flags, void* hip_stream) {
+    const char* who = "mxq_pack_mx_t";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    const int kind = code_kind(elem_ebits, elem_mbits, flags, who);
+    if (kind < 0) return MXQ_ERR_ARGUMENT;
+    if (batch < 0 || R < 0 || C < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    const int vw = 8 / elem_size(dtype);                 // columns in the 8 bytes a lane owns
+    if (R % 32 != 0 || C % vw != 0)
+        return fail(MXQ_ERR_ARGUMENT, "%s: R must be a multiple of 32 and C of %d", who, vw);
+    int64_t total;
+    if (mul_overflows(batch, R, C, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !codes || !scales) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if ((reinterpret_cast<uintptr_t>(in) & 7) || !aligned16(codes))
+        return fail(MXQ_ERR_ARGUMENT, "%s: input must be 8-byte and codes 16-byte aligned", who);
+    const int64_t n_tiles = R / 32, pv = C / vw, items = batch * n_tiles * pv;
+    if (ceil_div(items, kThreads) > 0x7FFFFFFF) return fail(MXQ_ERR_ARGUMENT, "%s: tensor too large", who);
+    dispatch<LaunchPackT>(dtype, rmode, ze, true, in, codes, scales, items, n_tiles, pv, kind, p,
+                          (hipStream_t)hip_stream);
+    return check_launch(who);
+}
+
+int mxq_unpack_mx(const void* codes, const void* scales, int code_kind, void* out, int dtype,
+                  int64_t rows, int64_t K, void* hip_stream) {
+    const char* who = "mxq_unpack_mx";
+    if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
+    if (code_kind != MXQ_CODES_E4M3 && code_kind != MXQ_CODES_E5M2 && code_kind != MXQ_CODES_E2M1)
+        return fail(MXQ_ERR_ARGUMENT, "%s: unknown code kind %d", who, code_kind);
+    if (rows < 0 || K < 0 || K % 32 != 0) return fail(MXQ_ERR_ARGUMENT, "%s: bad size", who);
+    const int64_t n = rows * K;
+    if (n == 0) return MXQ_OK;
+    if (!codes || !scales || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    const unsigned char* cd = reinterpret_cast<const unsigned char*>(codes);
+    const unsigned char* sc = reinterpret_cast<const unsigned char*>(scales);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int grid = grid_for(ceil_div(n, kThreads * 4));
+#define MXQ_UNPACK(DT)                                                                       \
+    if (code_kind == 1) mx_unpack_kernel<DT, 1><<<grid, kThreads, 0, s>>>(cd, sc, out, n);      \
+    else if (code_kind == 4) mx_unpack_kernel<DT, 4><<<grid, kThreads, 0, s>>>(cd, sc, out, n); \
+    else mx_unpack_kernel<DT, 0><<<grid, kThreads, 0, s>>>(cd, sc, out, n);
+    if (dtype == MXQ_DTYPE_F32) { MXQ_UNPACK(MXQ_F32) }
+    else if (dtype == MXQ_DTYPE_BF16) { MXQ_UNPACK(MXQ_BF16) }
+    else { MXQ_UNPACK(MXQ_F16) }
+#undef MXQ_UNPACK
+    return check_launch(who);
+}
+
+int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const void* b_codes,
+                   const void* b_scales, int b_kind, const void* bias, void* c, int c_dtype,
+                   int64_t batch, int64_t M, int64_t N, int64_t K, int epilogue_quant,
+                   void* hip_stream) {
+    const char* who = "mxq_gemm_mx_nt";
+    if (c_dtype < 0 || c_dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, c_dtype);
+    if (epilogue_quant != 0 && (epilogue_quant != 1 || c_dtype != MXQ_DTYPE_BF16))
+        return fail(MXQ_ERR_ARGUMENT, "%s: epilogue_quant must be 0, or 1 with a bf16 output", who);
+    if (batch < 0 || M < 0 || N < 0 || K < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    const bool nib = a_kind == MXQ_CODES_E2M1;
+    if ((a_kind != MXQ_CODES_E4M3 && a_kind != MXQ_CODES_E5M2 && a_kind != MXQ_CODES_E2M1) ||
+        (b_kind != MXQ_CODES_E4M3 && b_kind != MXQ_CODES_E5M2 && b_kind != MXQ_CODES_E2M1))
+        return fail(MXQ_ERR_ARGUMENT, "%s: unknown code kind %d / %d", who, a_kind, b_kind);
+    if (nib != (b_kind == MXQ_CODES_E2M1))
+        return fail(MXQ_ERR_ARGUMENT, "%s: e2m1 nibble codes need both operands in that form", who);
+    const int kstep = nib ? 2 * GEMM_BK : GEMM_BK;      // elements in a 128-byte K step
+    if (K % kstep != 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be a multiple of %d", who, kstep);
+    if (batch == 0 || M == 0 || N == 0) return MXQ_OK;
+    if (K == 0) return fail(MXQ_ERR_ARGUMENT, "%s: K must be positive", who);
+    if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF || batch > 65535)
+        return fail(MXQ_ERR_ARGUMENT, "%s: size too large", who);
+    if (!a_codes || !a_scales || !b_codes || !b_scales || !c) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(a_codes) || !aligned16(b_codes) || (reinterpret_cast<uintptr_t>(a_scales) & 3) ||
+        (reinterpret_cast<uintptr_t>(b_scales) & 3))
+        return fail(MXQ_ERR_ARGUMENT, "%s: codes must be 16-byte and scales 4-byte aligned", who);
+    GemmArgs g;
+    g.a = reinterpret_cast<const unsigned char*>(a_codes);
+    g.sa = reinterpret_cast<const unsigned char*>(a_scales);
+    g.b = reinterpret_cast<const unsigned char*>(b_codes);
+    g.sb = reinterpret_cast<const unsigned char*>(b_scales);
+    g.c = c;
+    g.bias = bias;
+    g.q_nan_from = 0u;
+    if (epilogue_quant) {                               // bfloat16, nearest: only the NaN threshold is needed
+        ElemParams q;
+        int rc = make_elem_params(MXQ_DTYPE_BF16, 9, 8, 3.3895313892515355e38f, MXQ_ROUND_NEAREST, 0, 1, 0, &q, who);
+        if (rc) return rc;
+        g.q_nan_from = q.fmt.nan_from;
+    }
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.kbytes = (int)(nib ? K / 2 : K);
+    g.batch_a = M * g.kbytes; g.batch_sa = M * (K / 32);
+    g.batch_b = N * g.kbytes; g.batch_sb = N * (K / 32);
+    g.batch_c = M * N;
+    hipStream_t s = (hipStream_t)hip_stream;
+    int rc;
+    if (nib) rc = launch_gemm<4, 4>(c_dtype, batch, g, s);
+    else if (!a_kind && !b_kind) rc = launch_gemm<0, 0>(c_dtype, batch, g, s);
+    else if (a_kind && !b_kind) rc = launch_gemm<1, 0>(c_dtype, batch, g, s);
+    else if (!a_kind && b_kind) rc = launch_gemm<0, 1>(c_dtype, batch, g, s);
+    else rc = launch_gemm<1, 1>(c_dtype, batch, g, s);
+    if (rc) return rc;
+    return check_launch(who);
+}
+
+int mxq_probe_mfma_rate(int64_t workgroups, int iters, int code_kind, void* sink, void* hip_stream) {
+    const char* who = "mxq_probe_mfma_rate";
+    if (workgroups <= 0 || workgroups > 0x7FFFFFFF || iters <= 0 || !sink ||
+        (code_kind != MXQ_CODES_E4M3 && code_kind != MXQ_CODES_E2M1))
+        return fail(MXQ_ERR_ARGUMENT, "%s: bad argument", who);
+    if (code_kind == MXQ_CODES_E2M1)
+        mfma_rate_probe_kernel<4><<<(unsigned)workgroups, kThreads, 0, (hipStream_t)hip_stream>>>(
+            iters, reinterpret_cast<float*>(sink));
+    else
+        mfma_rate_probe_kernel<0><<<(unsigned)workgroups, kThreads, 0, (hipStream_t)hip_stream>>>(
+            iters, reinterpret_cast<float*>(sink));
+    return check_launch(who);
+}
+
+}  // extern "C"
+#pragma GCC visibility pop

@@ -1,4 +1,4 @@
-// Host-side parameter preparation shared by the GPU entry points (mxq_capi.hip) and the host
+// Host-side parameter preparation shared by the GPU entry points (mxq_capi*.hip) and the host
 // build (mxq_host.cpp): argument checks, element-format constants, choice of round-up-zone table.
 #pragma once
 #include <stdarg.h>
