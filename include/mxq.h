@@ -127,6 +127,15 @@ int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void*
                      int bits, int exp_bits, float max_norm, int rmode, int allow_denorm, int flags,
                      void* hip_stream);
 
+/* vec_add / vec_sub / vec_mul / vec_div / vec_recip (mx/vector_ops.py:38-75): `a op b` on contiguous
+ * fp32 or bf16 tensors of n elements, rounded to the tensor dtype, then the elementwise quantizer
+ * (as in mxq_quantize_elemwise; bits == 0: none) -- one pass instead of two.  op: 0 add, 1 sub,
+ * 2 mul, 3 div.  mode 0: b is a tensor; 1: a op scalar; 2: scalar op a (b is ignored in modes 1, 2).
+ * Bit-identical to the tensor op followed by quantize_elemwise_op. */
+int mxq_binary_elemwise(const void* a, const void* b, float scalar, int mode, void* out, int dtype,
+                        int64_t n, int op, int bits, int exp_bits, float max_norm, int rmode,
+                        int allow_denorm, int flags, void* hip_stream);
+
 /* The gradient with respect to the input of the same two layers (LayerNormFunction.backward via
  * _norm_backward_LN, mx/norm_utils.py:188-258; RMSNormFunction.backward, mx/layernorm.py:150-168)
  * from what mxq_norm_lastdim wrote: x_norm and row_stat.  weight: the n values the layer saved.

@@ -166,6 +166,33 @@ int mxq_softmax_backward_lastdim(const void* grad_out, const void* y, void* grad
     return check_launch(who);
 }
 
+int mxq_binary_elemwise(const void* a, const void* b, float scalar, int mode, void* out, int dtype,
+                        int64_t n, int op, int bits, int exp_bits, float max_norm, int rmode,
+                        int allow_denorm, int flags, void* hip_stream) {
+    const char* who = "mxq_binary_elemwise";
+    BinaryParams p;
+    bool ident, closed;
+    int rc = chain_params(dtype, bits, exp_bits, max_norm, rmode, allow_denorm, flags, &p.q, &ident, &closed, who);
+    if (rc) return rc;
+    if (op < BIN_ADD || op > BIN_DIV) return fail(MXQ_ERR_ARGUMENT, "%s: unknown operation %d", who, op);
+    if (mode < BIN_TENSOR_TENSOR || mode > BIN_SCALAR_TENSOR) return fail(MXQ_ERR_ARGUMENT, "%s: unknown mode %d", who, mode);
+    p.op = op;
+    p.mode = mode;
+    p.scalar = scalar;
+    if (n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (n == 0) return MXQ_OK;
+    if (!a || !out || (mode == BIN_TENSOR_TENSOR && !b)) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    if (!aligned16(a) || !aligned16(out) || (mode == BIN_TENSOR_TENSOR && !aligned16(b)))
+        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int epv = dtype == MXQ_DTYPE_F32 ? 4 : 8;
+    const int grid = grid_for(ceil_div(ceil_div(n, epv), (int64_t)kThreads * 2));
+#define MXQ_BIN(DT, RM, QM) binary_kernel<DT, RM, QM><<<grid, kThreads, 0, s>>>(a, b, out, n, p)
+    MXQ_CHAIN_DISPATCH(MXQ_BIN);
+#undef MXQ_BIN
+    return check_launch(who);
+}
+
 int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void* out, void* x_norm,
                      void* row_stat, int dtype, int64_t rows, int64_t n, float eps, int rms_norm,
                      int bits, int exp_bits, float max_norm, int rmode, int allow_denorm, int flags,

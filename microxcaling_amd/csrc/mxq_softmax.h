@@ -597,4 +597,87 @@ __global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __re
     }
 }
 
+// a op b followed by the elementwise quantizer (vec_add / vec_sub / vec_mul / vec_div / vec_recip,
+// mx/vector_ops.py:38-75): one pass instead of torch's op plus a quantization pass.  The second
+// operand may be a scalar, on either side.  Only correctly rounded arithmetic: bit-identical to the
+// two steps.
+enum { BIN_ADD = 0, BIN_SUB = 1, BIN_MUL = 2, BIN_DIV = 3 };
+enum { BIN_TENSOR_TENSOR = 0, BIN_TENSOR_SCALAR = 1, BIN_SCALAR_TENSOR = 2 };
+
+struct BinaryParams {
+    ElemParams q;
+    int op;
+    int mode;
+    float scalar;
+};
+
+template <int DT, int RMODE, int QMODE>
+__global__ __launch_bounds__(TPB) void binary_kernel(const void* __restrict__ a_, const void* __restrict__ b_,
+                                                     void* __restrict__ out_, int64_t n, BinaryParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int EPV = 4 * PD;
+    constexpr int UNROLL = 2;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.q.zone_row]);
+
+    auto Q = [&](float v) {
+        v = mxq_round_dt<ADT>(v);
+        if (QMODE == SMQ_IDENT) return v;
+        if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, p.q.fmt.nan_from);
+        return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
+                                                          p.q.allow_denorm != 0, zone, ZS);
+    };
+    const bool tensor_b = p.mode == BIN_TENSOR_TENSOR;
+    const bool swap = p.mode == BIN_SCALAR_TENSOR;
+    auto eval = [&](float x, float y) {
+        if (!tensor_b) y = p.scalar;
+        const float l = swap ? y : x, r = swap ? x : y;
+        switch (p.op) {
+            case BIN_ADD: return Q(l + r);
+            case BIN_SUB: return Q(l - r);
+            case BIN_MUL: return Q(l * r);
+            default:
+                // scalar / tensor is torch's Tensor.__rtruediv__: reciprocal(), then times the scalar
+                return swap ? Q(mxq_round_dt<ADT>(1.0f / r) * l) : Q(l / r);
+        }
+    };
+
+    const u32x4* a = reinterpret_cast<const u32x4*>(a_);
+    const u32x4* b = reinterpret_cast<const u32x4*>(b_);
+    u32x4* out = reinterpret_cast<u32x4*>(out_);
+    const int64_t n_vec = n / EPV;
+    const int64_t stride = (int64_t)gridDim.x * TPB * UNROLL;
+    for (int64_t base = (int64_t)blockIdx.x * TPB * UNROLL + threadIdx.x; base - threadIdx.x < n_vec;
+         base += stride) {
+        u32x4 va[UNROLL], vb[UNROLL];
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            const int64_t i = base + (int64_t)j * TPB;
+            va[j] = (i < n_vec) ? a[i] : u32x4{0, 0, 0, 0};
+            vb[j] = (tensor_b && i < n_vec) ? b[i] : u32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            const int64_t i = base + (int64_t)j * TPB;
+            u32x4 o;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                float r[2];
+#pragma unroll
+                for (int h = 0; h < PD; ++h) r[h] = eval(Pack<DT>::get(va[j][d], h), Pack<DT>::get(vb[j][d], h));
+                o[d] = Pack<DT>::put(r[0], r[PD - 1]);
+            }
+            if (i < n_vec) __builtin_nontemporal_store(o, &out[i]);
+        }
+    }
+    const int64_t t0 = n_vec * EPV;
+    const int64_t gi = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (gi < n - t0) {
+        const float r = eval(load_scalar<DT>(a_, t0 + gi), tensor_b ? load_scalar<DT>(b_, t0 + gi) : 0.0f);
+        store_scalar<DT>(out_, t0 + gi, r);
+    }
+}
+
 }  // namespace

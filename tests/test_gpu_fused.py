@@ -615,3 +615,40 @@ def test_fused_norm_backward_against_chain(dev, kind, dtype, spec, shape):
     d = (got - want).abs()
     assert d.max().item() <= 2.0 ** -5 * want.abs().max().item()
     assert (d > 0).float().mean().item() <= 0.08
+
+
+@pytest.mark.parametrize("op,mode", [(o, m) for o in ("add", "sub", "mul", "div")
+                                     for m in ("tensor", "scalar_right", "scalar_left")] + [("recip", "scalar_left")])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=12, round="floor"), dict(fp=16, round="even")],
+                         ids=["bfloat16", "bfloat12-floor", "fp16-even"])
+def test_fused_vec_ops_equal_the_two_steps(dev, op, mode, dtype, spec):
+    """vec_add / vec_sub / vec_mul / vec_div / vec_recip as one kernel against the same function on
+    CPU tensors (torch's op, then the quantizer): bit for bit, special values included."""
+    from microxcaling_amd import vector_ops as V
+    from microxcaling_amd.specs import apply_mx_specs
+    specs = _specs(**spec)
+    g = torch.Generator().manual_seed(len(op) + len(mode))
+    shape = (37, 131)                                              # 4847 elements: a ragged tail
+    a = (torch.randn(*shape, generator=g) * torch.exp2(torch.randint(-30, 30, shape, generator=g).float())).to(dtype)
+    b = (torch.randn(*shape, generator=g) * torch.exp2(torch.randint(-30, 30, shape, generator=g).float())).to(dtype)
+    special = torch.tensor([0.0, -0.0, float("inf"), float("-inf"), float("nan"), 1e-39, 3e38, -3e38]).to(dtype)
+    a[0, :8] = special
+    b[0, :8] = special.flip(0)
+    b[1, :8] = special
+    fn = {"add": V.vec_add, "sub": V.vec_sub, "mul": V.vec_mul, "div": V.vec_div}.get(op)
+
+    def run(x, y):
+        if op == "recip":
+            return V.vec_recip(x, mx_specs=specs)
+        if mode == "tensor":
+            return fn(x, y, mx_specs=specs)
+        if mode == "scalar_right":
+            return fn(x, 1.703125, mx_specs=specs)
+        return fn(3, x, mx_specs=specs)
+    want = run(a, b)
+    with torch.no_grad():
+        got = run(a.to(dev), b.to(dev))
+    unfusable = dtype == torch.bfloat16 and spec.get("round") == "even"      # wide format, half-even, bf16 tensor
+    assert (V._fused_binary(a.to(dev), b.to(dev), V._ADD, apply_mx_specs(specs), None) is None) == unfusable
+    assert_bits_equal(got.cpu(), want, "%s %s" % (op, mode))
