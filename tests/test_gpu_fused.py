@@ -652,3 +652,44 @@ def test_fused_vec_ops_equal_the_two_steps(dev, op, mode, dtype, spec):
     unfusable = dtype == torch.bfloat16 and spec.get("round") == "even"      # wide format, half-even, bf16 tensor
     assert (V._fused_binary(a.to(dev), b.to(dev), V._ADD, apply_mx_specs(specs), None) is None) == unfusable
     assert_bits_equal(got.cpu(), want, "%s %s" % (op, mode))
+
+
+def test_layers_replay_from_a_hip_graph(dev):
+    """The kernels take torch's current stream and allocate nothing themselves, so a block of MX
+    layers can be captured once and replayed: linear (packed GEMM) -> GELU -> LayerNorm -> softmax.
+    Every replay, with fresh input contents and eager work in between, must equal the eager result
+    bit for bit."""
+    from microxcaling_amd import activations as A, layernorm as L
+    from microxcaling_amd.linear import linear
+    from microxcaling_amd.softmax import softmax
+    specs = _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32, bfloat=16)
+    g = torch.Generator().manual_seed(5)
+    w = (torch.randn(1024, 512, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    b = torch.randn(1024, generator=g).to(torch.bfloat16).to(dev)
+    ln = L.LayerNorm(1024, eps=1e-5, mx_specs=specs).to(torch.bfloat16).to(dev)
+
+    def block(x):
+        with torch.no_grad():
+            h = linear(x, w, b, mx_specs=specs)
+            h = A.gelu(h, mx_specs=specs)
+            h = ln(h)
+            return softmax(h, dim=-1, mx_specs=specs)
+
+    static_x = torch.randn(512, 512, generator=g).to(torch.bfloat16).to(dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                      # warm-up outside the capture (kernel attributes, caches)
+        for _ in range(2):
+            block(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = block(static_x)
+    for i in range(3):
+        x = (torch.randn(512, 512, generator=g) * (i + 1)).to(torch.bfloat16).to(dev)
+        want = block(x)                                # eager work between the replays
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y.view(torch.int16), want.view(torch.int16)), i
