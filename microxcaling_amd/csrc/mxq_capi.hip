@@ -111,9 +111,19 @@ int reduce_outer(const float* in, float* out, void* workspace, int64_t outer, in
     const bool vec = (inner % 4 == 0) && aligned16(in) && aligned16(out) && (splits == 1 || aligned16(workspace));
     const int64_t rows_per_split = ceil_div(outer > 0 ? outer : 1, splits);
     float* partial = splits == 1 ? out : reinterpret_cast<float*>(workspace);
-    dim3 grid((unsigned)ceil_div(ceil_div(inner, vec ? 4 : 1), kThreads), (unsigned)splits);
-    if (vec) reduce_outer_kernel<OP, 4><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
-    else reduce_outer_kernel<OP, 1><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
+    if (vec) {
+        // column groups of a row per block: as many as it takes to cover the row, up to 8 x 256
+        const int64_t groups = ceil_div(inner / 4, (int64_t)kThreads);
+        const int kg = groups >= 8 ? 8 : groups >= 4 ? 4 : groups >= 2 ? 2 : 1;
+        dim3 grid((unsigned)ceil_div(groups, kg), (unsigned)splits);
+        if (kg == 8) reduce_outer_kernel<OP, 4, 8><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
+        else if (kg == 4) reduce_outer_kernel<OP, 4, 4><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
+        else if (kg == 2) reduce_outer_kernel<OP, 4, 2><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
+        else reduce_outer_kernel<OP, 4, 1><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
+    } else {
+        dim3 grid((unsigned)ceil_div(inner, kThreads), (unsigned)splits);
+        reduce_outer_kernel<OP, 1, 1><<<grid, kThreads, 0, s>>>(in, partial, outer, inner, rows_per_split);
+    }
     int rc = check_launch(who);
     if (rc || splits == 1) return rc;
     reduce_outer_final_kernel<OP><<<(unsigned)ceil_div(inner, 64), kThreads, 0, s>>>(partial, out, splits, inner);

@@ -497,44 +497,71 @@ __global__ __launch_bounds__(TPB) void reduce_inner_wave_kernel(const float* __r
     }
 }
 
-// outer axis: (outer, inner) -> partial (splits, inner); lane owns 4 (or 1) consecutive columns
-template <class OP, int VW>
+// outer axis: (outer, inner) -> partial (splits, inner).  VW = 4: a lane owns KG groups of 4
+// consecutive columns, 1024 columns apart, so that a block reads KG * 4 KB of contiguous memory per
+// row -- whole rows when inner <= 8192, and then its rows_per_split rows are one contiguous chunk.
+// VW = 1: one column per lane (unaligned shapes).  Rows are accumulated in order.
+template <class OP, int VW, int KG>
 __global__ __launch_bounds__(TPB) void reduce_outer_kernel(const float* __restrict__ in,
                                                            float* __restrict__ partial,
                                                            int64_t outer, int64_t inner,
                                                            int64_t rows_per_split) {
-    const int64_t cg = (int64_t)blockIdx.x * TPB + threadIdx.x;   // column group
-    if (cg * VW >= inner) return;
     const int64_t r0 = (int64_t)blockIdx.y * rows_per_split;
     const int64_t r1 = (r0 + rows_per_split < outer) ? r0 + rows_per_split : outer;
-    float acc[VW];
-#pragma unroll
-    for (int k = 0; k < VW; ++k) acc[k] = OP::init();
     if constexpr (VW == 4) {
-        const u32x4* p = reinterpret_cast<const u32x4*>(in) + cg;
-        const int64_t pv = inner / 4;
+        const int64_t pv = inner / 4;                     // column groups per row
+        const int64_t cg0 = (int64_t)blockIdx.x * TPB * KG + threadIdx.x;
+        float acc[KG][4];
+#pragma unroll
+        for (int g = 0; g < KG; ++g)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) acc[g][k] = OP::init();
+        const u32x4* p = reinterpret_cast<const u32x4*>(in);
+        constexpr int RU = 16 / KG;                       // rows in flight: 16 loads (256 bytes) per lane
         int64_t r = r0;
-        for (; r + 8 <= r1; r += 8) {                 // eight rows (128 bytes per lane) in flight
-            u32x4 w[8];
+        for (; r + RU <= r1; r += RU) {
+            u32x4 w[RU][KG];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) w[u] = p[(r + u) * pv];
+            for (int u = 0; u < RU; ++u)
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
+                for (int g = 0; g < KG; ++g) {
+                    const int64_t cg = cg0 + (int64_t)g * TPB;
+                    w[u][g] = cg < pv ? p[(r + u) * pv + cg] : u32x4{0, 0, 0, 0};
+                }
 #pragma unroll
-                for (int k = 0; k < 4; ++k) acc[k] = OP::apply(acc[k], mxq_float(w[u][k]));
+            for (int u = 0; u < RU; ++u)
+#pragma unroll
+                for (int g = 0; g < KG; ++g)
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) acc[g][k] = OP::apply(acc[g][k], mxq_float(w[u][g][k]));
         }
         for (; r < r1; ++r) {
-            u32x4 w = p[r * pv];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) acc[k] = OP::apply(acc[k], mxq_float(w[k]));
+            for (int g = 0; g < KG; ++g) {
+                const int64_t cg = cg0 + (int64_t)g * TPB;
+                if (cg < pv) {
+                    const u32x4 w = p[r * pv + cg];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) acc[g][k] = OP::apply(acc[g][k], mxq_float(w[k]));
+                }
+            }
         }
-        u32x4 o;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) o[k] = mxq_bits(acc[k]);
-        reinterpret_cast<u32x4*>(partial + (int64_t)blockIdx.y * inner)[cg] = o;
+        for (int g = 0; g < KG; ++g) {
+            const int64_t cg = cg0 + (int64_t)g * TPB;
+            if (cg < pv) {
+                u32x4 o;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) o[k] = mxq_bits(acc[g][k]);
+                reinterpret_cast<u32x4*>(partial + (int64_t)blockIdx.y * inner)[cg] = o;
+            }
+        }
     } else {
-        for (int64_t r = r0; r < r1; ++r) acc[0] = OP::apply(acc[0], in[r * inner + cg]);
-        partial[(int64_t)blockIdx.y * inner + cg] = acc[0];
+        const int64_t cg = (int64_t)blockIdx.x * TPB + threadIdx.x;
+        if (cg >= inner) return;
+        float acc = OP::init();
+        for (int64_t r = r0; r < r1; ++r) acc = OP::apply(acc, in[r * inner + cg]);
+        partial[(int64_t)blockIdx.y * inner + cg] = acc;
     }
 }
 
