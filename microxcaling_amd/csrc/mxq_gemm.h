@@ -4,15 +4,20 @@
 //   codes  uint8 (rows, K)      one OCP 8-bit float per element: e4m3 ("fn") for the element
 //                               formats fp8_e4m3 / fp6_e3m2 / fp6_e2m3 / fp4_e2m1 (all of whose
 //                               values e4m3 represents exactly), e5m2 for fp8_e5m2
+//          or uint8 (rows, K/2) fp4_e2m1 elements as OCP e2m1 nibbles, the element with the lower K
+//                               index in the low nibble
 //   scales uint8 (rows, K/32)   E8M0: shared exponent + 127, 255 = NaN block
 // codes[i][k] * 2^(scales[i][k/32] - 127) is bit-for-bit the value the fake-quantizing kernels
 // return (before their final rounding to a 16-bit tensor dtype).
 //
 // v_mfma_scale_f32_16x16x128_f8f6f4 multiplies a 16x128 by a 128x16 tile of such codes.  Lane
-// (row = lane % 16, g = lane / 16) supplies 32 codes of its row: K = 16g .. 16g+15 in its first four
-// registers and K = 64+16g .. 64+16g+15 in the last four.  The E8M0 byte of K block j (32
-// consecutive K) of a row is taken from the scale register of lane row + 16j -- so each lane passes
-// the scale of block g, and block scaling costs nothing extra.
+// (row = lane % 16, g = lane / 16) supplies 32 8-bit codes of its row: K = 16g .. 16g+15 in its
+// first four registers and K = 64+16g .. 64+16g+15 in the last four -- or 32 nibbles, K = 32g ..
+// 32g+31, in four registers.  The E8M0 byte of K block j (32 consecutive K) of a row is taken
+// from the scale register of lane row + 16j -- so each lane passes the scale of block g, and block
+// scaling costs nothing extra.  v_mfma_scale_f32_32x32x64_f8f6f4 (the large-tile kernel) is the
+// same with lane (row = lane % 32, g = lane / 32): K = 16g .. and 32+16g .., or nibbles 32g ..,
+// scale of block j from lane row + 32j.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
