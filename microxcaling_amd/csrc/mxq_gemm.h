@@ -272,6 +272,9 @@ __device__ __forceinline__ v16f mx_mfma32(const Frag& b, const Frag& a, v16f c, 
     }
 }
 
+// Output tiles are written once and not read again by the kernel: streaming stores keep them from
+// displacing the operand panels in L2 (3-5 % on the large shapes).
+#define MXQ_C_STORE(ptr, val) __builtin_nontemporal_store(val, ptr)
 // The MFMAs are issued with the B fragment as the first operand, i.e. they compute 16 x 16 blocks
 // of C^T: a lane then holds four *consecutive columns* n = 4 * (lane / 16) + r of one row
 // m = lane % 16, which it can store with a single 8- or 16-byte access.
@@ -306,13 +309,13 @@ __device__ __forceinline__ void store_c4(void* c, const void* bias, uint32_t q_n
     if (tile_inside) {                                       // uniform per workgroup
         const int64_t idx = base + (int64_t)m * N + n;
         if (OUT_DT == MXQ_F32) {
-            *reinterpret_cast<v4f*>(reinterpret_cast<float*>(c) + idx) = v;
+            MXQ_C_STORE(reinterpret_cast<v4f*>(reinterpret_cast<float*>(c) + idx), v);
         } else if (OUT_DT == MXQ_BF16) {
-            *reinterpret_cast<u32x2*>(reinterpret_cast<unsigned short*>(c) + idx) =
-                u32x2{Pack<MXQ_BF16>::put(v[0], v[1]), Pack<MXQ_BF16>::put(v[2], v[3])};
+            MXQ_C_STORE(reinterpret_cast<u32x2*>(reinterpret_cast<unsigned short*>(c) + idx),
+                        (u32x2{Pack<MXQ_BF16>::put(v[0], v[1]), Pack<MXQ_BF16>::put(v[2], v[3])}));
         } else {
-            *reinterpret_cast<u32x2*>(reinterpret_cast<unsigned short*>(c) + idx) =
-                u32x2{Pack<MXQ_F16>::put(v[0], v[1]), Pack<MXQ_F16>::put(v[2], v[3])};
+            MXQ_C_STORE(reinterpret_cast<u32x2*>(reinterpret_cast<unsigned short*>(c) + idx),
+                        (u32x2{Pack<MXQ_F16>::put(v[0], v[1]), Pack<MXQ_F16>::put(v[2], v[3])}));
         }
     } else if (m < M) {
 #pragma unroll
@@ -338,9 +341,9 @@ __device__ __forceinline__ void store_c8(void* c, const void* bias, uint32_t q_n
 #pragma unroll
             for (int r = 0; r < 8; ++r) v[r] = epilogue_value<OUT_DT>(v[r], false, 0.0f, q_nan_from);
         }
-        *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned short*>(c) + base + (int64_t)m * N + n) =
-            u32x4{Pack<OUT_DT>::put(v[0], v[1]), Pack<OUT_DT>::put(v[2], v[3]),
-                  Pack<OUT_DT>::put(v[4], v[5]), Pack<OUT_DT>::put(v[6], v[7])};
+        MXQ_C_STORE(reinterpret_cast<u32x4*>(reinterpret_cast<unsigned short*>(c) + base + (int64_t)m * N + n),
+                    (u32x4{Pack<OUT_DT>::put(v[0], v[1]), Pack<OUT_DT>::put(v[2], v[3]),
+                           Pack<OUT_DT>::put(v[4], v[5]), Pack<OUT_DT>::put(v[6], v[7])}));
     } else if (m < M) {
 #pragma unroll
         for (int r = 0; r < 8; ++r)
@@ -761,8 +764,8 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
                         swap_with_lane16(p[0], p[1]);
                         unsigned short* out = reinterpret_cast<unsigned short*>(g.c) + cbase +
                                               (int64_t)(mt + m16) * g.N + nt + 8 * (2 * half + fg);
-                        *reinterpret_cast<u32x4*>(out) = p[0];
-                        *reinterpret_cast<u32x4*>(out + (int64_t)16 * g.N) = p[1];
+                        MXQ_C_STORE(reinterpret_cast<u32x4*>(out), p[0]);
+                        MXQ_C_STORE(reinterpret_cast<u32x4*>(out + (int64_t)16 * g.N), p[1]);
                     } else {
 #pragma unroll
                         for (int h = 0; h < 2; ++h)
@@ -782,8 +785,8 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
                             swap_with_lane16(p[0], p[1]);
                             float* out = reinterpret_cast<float*>(g.c) + cbase + (int64_t)(mt + m16) * g.N + nt +
                                          8 * q + 4 * (2 * half + fg);
-                            *reinterpret_cast<u32x4*>(out) = p[0];
-                            *reinterpret_cast<u32x4*>(out + (int64_t)16 * g.N) = p[1];
+                            MXQ_C_STORE(reinterpret_cast<u32x4*>(out), p[0]);
+                            MXQ_C_STORE(reinterpret_cast<u32x4*>(out + (int64_t)16 * g.N), p[1]);
                         }
                     } else {
 #pragma unroll
