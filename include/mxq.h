@@ -107,7 +107,7 @@ int mxq_reduce_max_outer(const float* in, float* out, void* workspace, int64_t o
  * bfloat / fp, and for bfloat16 with round-half-even on a bf16 tensor).
  * exp_mode 0: exp(x); 1: 2^x (mx_specs['softmax_exp2']); 2: 2^Q(x * 1.4453125) (['vec_use_exp2']).
  * use_recip: e * Q(1 / sum) instead of e / sum (['vec_use_recip']).
- * n must be a multiple of 16 bytes worth of elements and at most 4096.  The reference has no native
+ * n must be a multiple of 16 bytes worth of elements and at most 16384.  The reference has no native
  * counterpart (it runs ten tensor ops); results agree with that chain up to the last-bit
  * differences of exp and of the summation order. */
 int mxq_softmax_lastdim(const void* in, void* out, int dtype, int64_t rows, int64_t n, int bits,
@@ -120,7 +120,7 @@ int mxq_softmax_lastdim(const void* in, void* out, int dtype, int64_t rows, int6
  * bits == 0: none) after every step.  weight, bias: n values of the tensor dtype, already quantized.
  * out: (rows, n).  x_norm (may be NULL): (rows, n), the normalized input the layer saves for its
  * backward pass.  row_stat: rows values, var + eps (LayerNorm) or 1 / rms (RMSNorm), also saved.
- * n: multiple of 16 bytes worth of elements, at most 4096.  Agrees with the reference's chain of
+ * n: multiple of 16 bytes worth of elements, at most 16384.  Agrees with the reference's chain of
  * tensor ops up to the order of the two row sums. */
 int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void* out, void* x_norm,
                      void* row_stat, int dtype, int64_t rows, int64_t n, float eps, int rms_norm,

@@ -1,45 +1,6 @@
 // C ABI of libmxq_gfx950.so, continued: kernels that run a whole chain of "tensor op, then
-// elementwise quantizer" steps -- softmax, LayerNorm / RMSNorm, activations, forward and backward.
-#include "mxq_capi_common.h"
-#include "mxq_softmax.h"
-
-namespace {
-
-int chain_params(int dtype, int bits, int exp_bits, float max_norm, int rmode, int allow_denorm,
-                        int flags, ElemParams* q, bool* ident, bool* closed, const char* who) {
-    *ident = bits == 0;
-    if (dtype != MXQ_DTYPE_F32 && dtype != MXQ_DTYPE_BF16)
-        return fail(MXQ_ERR_ARGUMENT, "%s: dtype code %d (fp32 and bf16 tensors only)", who, dtype);
-    int rc = make_elem_params(dtype, *ident ? 9 : bits, *ident ? 8 : exp_bits, *ident ? 1.0f : max_norm,
-                              *ident ? MXQ_ROUND_NEAREST : rmode, 0, allow_denorm, flags, q, who);
-    if (rc) return rc;
-    if (!*ident && !lean_ok(dtype, q->fmt, rmode, true))
-        return fail(MXQ_ERR_ARGUMENT, "%s: round-half-even to %d fraction bits on a bf16 tensor is "
-                    "only available through the separate elementwise steps", who, q->fmt.t);
-    *closed = !*ident && dtype == MXQ_DTYPE_BF16 && bits == 9 && exp_bits == 8 &&
-              rmode == MXQ_ROUND_NEAREST && allow_denorm && q->fmt.max_bits == 0x7F7F0000u;
-    return MXQ_OK;
-}
-// LAUNCH(DT, RMODE, QMODE) for the instance that serves (dtype, ident, closed, rmode)
-#define MXQ_CHAIN_DISPATCH(LAUNCH)                                                   \
-    do {                                                                             \
-        if (dtype == MXQ_DTYPE_F32) {                                                \
-            if (ident) LAUNCH(MXQ_F32, MXQ_NEAREST, SMQ_IDENT);                      \
-            else if (rmode == MXQ_ROUND_FLOOR) LAUNCH(MXQ_F32, MXQ_FLOOR, SMQ_GENERIC);     \
-            else if (rmode == MXQ_ROUND_NEAREST) LAUNCH(MXQ_F32, MXQ_NEAREST, SMQ_GENERIC); \
-            else LAUNCH(MXQ_F32, MXQ_EVEN, SMQ_GENERIC);                             \
-        } else {                                                                     \
-            if (ident) LAUNCH(MXQ_BF16, MXQ_NEAREST, SMQ_IDENT);                     \
-            else if (closed) LAUNCH(MXQ_BF16, MXQ_NEAREST, SMQ_BF16);                \
-            else if (rmode == MXQ_ROUND_FLOOR) LAUNCH(MXQ_BF16, MXQ_FLOOR, SMQ_GENERIC);     \
-            else if (rmode == MXQ_ROUND_NEAREST) LAUNCH(MXQ_BF16, MXQ_NEAREST, SMQ_GENERIC); \
-            else LAUNCH(MXQ_BF16, MXQ_EVEN, SMQ_GENERIC);                            \
-        }                                                                            \
-    } while (0)
-
-// Which code the element format packs to: MXQ_CODES_E4M3 / _E5M2 bytes, or _E2M1 nibbles when the
-// caller asks for them (MXQ_FLAG_PACK_NIBBLES, fp4 only); -1 = no packed form.
-}  // namespace
+// elementwise quantizer" steps -- softmax forward and backward, activations, single vector ops.
+#include "mxq_capi_chain.h"
 
 #pragma GCC visibility push(default)
 extern "C" {
@@ -57,23 +18,16 @@ int mxq_softmax_lastdim(const void* in, void* out, int dtype, int64_t rows, int6
     p.use_recip = use_recip ? 1 : 0;
     const int epv = dtype == MXQ_DTYPE_F32 ? 4 : 8;
     if (rows < 0 || n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
-    if (n > 4096 || n % epv != 0)
-        return fail(MXQ_ERR_ARGUMENT, "%s: row length %lld must be a multiple of %d and at most 4096",
-                    who, (long long)n, epv);
+    if (n > kMaxRow || n % epv != 0)
+        return fail(MXQ_ERR_ARGUMENT, "%s: row length %lld must be a multiple of %d and at most %lld",
+                    who, (long long)n, epv, (long long)kMaxRow);
     if (rows == 0 || n == 0) return MXQ_OK;
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     if (!aligned16(in) || !aligned16(out))
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
     hipStream_t s = (hipStream_t)hip_stream;
-    const int grid = grid_for(ceil_div(rows, kThreads / 64));
     const int64_t nvec = n / epv;                       // 16-byte vectors per row, 64 lanes
-#define MXQ_SM(DT, RM, QM)                                                                         \
-    do {                                                                                           \
-        constexpr int V = (DT == MXQ_F32) ? 2 : 1;                                                 \
-        if (nvec <= 128 * V) softmax_row_kernel<DT, RM, QM, 2 * V><<<grid, kThreads, 0, s>>>(in, out, rows, (int)n, p);      \
-        else if (nvec <= 256 * V) softmax_row_kernel<DT, RM, QM, 4 * V><<<grid, kThreads, 0, s>>>(in, out, rows, (int)n, p); \
-        else softmax_row_kernel<DT, RM, QM, 8 * V><<<grid, kThreads, 0, s>>>(in, out, rows, (int)n, p);                     \
-    } while (0)
+#define MXQ_SM(DT, RM, QM) MXQ_ROW_CASES(softmax_row_kernel, DT, RM, QM, in, out, rows, (int)n, p)
     MXQ_CHAIN_DISPATCH(MXQ_SM);
 #undef MXQ_SM
     return check_launch(who);
@@ -144,23 +98,16 @@ int mxq_softmax_backward_lastdim(const void* grad_out, const void* y, void* grad
     p.use_recip = 0;
     const int epv = dtype == MXQ_DTYPE_F32 ? 4 : 8;
     if (rows < 0 || n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
-    if (n > 4096 || n % epv != 0)
-        return fail(MXQ_ERR_ARGUMENT, "%s: row length %lld must be a multiple of %d and at most 4096",
-                    who, (long long)n, epv);
+    if (n > kMaxRow || n % epv != 0)
+        return fail(MXQ_ERR_ARGUMENT, "%s: row length %lld must be a multiple of %d and at most %lld",
+                    who, (long long)n, epv, (long long)kMaxRow);
     if (rows == 0 || n == 0) return MXQ_OK;
     if (!grad_out || !y || !grad_in) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     if (!aligned16(grad_out) || !aligned16(y) || !aligned16(grad_in))
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
     hipStream_t s = (hipStream_t)hip_stream;
-    const int grid = grid_for(ceil_div(rows, kThreads / 64));
     const int64_t nvec = n / epv;
-#define MXQ_SMB(DT, RM, QM)                                                                         \
-    do {                                                                                            \
-        constexpr int V = (DT == MXQ_F32) ? 2 : 1;                                                  \
-        if (nvec <= 128 * V) softmax_backward_row_kernel<DT, RM, QM, 2 * V><<<grid, kThreads, 0, s>>>(grad_out, y, grad_in, rows, (int)n, p);      \
-        else if (nvec <= 256 * V) softmax_backward_row_kernel<DT, RM, QM, 4 * V><<<grid, kThreads, 0, s>>>(grad_out, y, grad_in, rows, (int)n, p); \
-        else softmax_backward_row_kernel<DT, RM, QM, 8 * V><<<grid, kThreads, 0, s>>>(grad_out, y, grad_in, rows, (int)n, p);                     \
-    } while (0)
+#define MXQ_SMB(DT, RM, QM) MXQ_ROW_CASES(softmax_backward_row_kernel, DT, RM, QM, grad_out, y, grad_in, rows, (int)n, p)
     MXQ_CHAIN_DISPATCH(MXQ_SMB);
 #undef MXQ_SMB
     return check_launch(who);
@@ -190,76 +137,6 @@ int mxq_binary_elemwise(const void* a, const void* b, float scalar, int mode, vo
 #define MXQ_BIN(DT, RM, QM) binary_kernel<DT, RM, QM><<<grid, kThreads, 0, s>>>(a, b, out, n, p)
     MXQ_CHAIN_DISPATCH(MXQ_BIN);
 #undef MXQ_BIN
-    return check_launch(who);
-}
-
-int mxq_norm_lastdim(const void* in, const void* weight, const void* bias, void* out, void* x_norm,
-                     void* row_stat, int dtype, int64_t rows, int64_t n, float eps, int rms_norm,
-                     int bits, int exp_bits, float max_norm, int rmode, int allow_denorm, int flags,
-                     void* hip_stream) {
-    const char* who = "mxq_norm_lastdim";
-    NormParams p;
-    bool ident, closed;
-    int rc = chain_params(dtype, bits, exp_bits, max_norm, rmode, allow_denorm, flags, &p.q, &ident, &closed, who);
-    if (rc) return rc;
-    p.eps = eps;
-    p.rms = rms_norm ? 1 : 0;
-    const int epv = dtype == MXQ_DTYPE_F32 ? 4 : 8;
-    if (rows < 0 || n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
-    if (n > 4096 || n % epv != 0)
-        return fail(MXQ_ERR_ARGUMENT, "%s: row length %lld must be a multiple of %d and at most 4096",
-                    who, (long long)n, epv);
-    if (rows == 0 || n == 0) return MXQ_OK;
-    if (!in || !out || !weight || !bias || !row_stat) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
-    if (!aligned16(in) || !aligned16(out) || !aligned16(weight) || !aligned16(bias) || !aligned16(x_norm))
-        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
-    hipStream_t s = (hipStream_t)hip_stream;
-    const int grid = grid_for(ceil_div(rows, kThreads / 64));
-    const int64_t nvec = n / epv;
-#define MXQ_NM(DT, RM, QM)                                                                         \
-    do {                                                                                           \
-        constexpr int V = (DT == MXQ_F32) ? 2 : 1;                                                 \
-        if (nvec <= 128 * V) norm_row_kernel<DT, RM, QM, 2 * V><<<grid, kThreads, 0, s>>>(in, weight, bias, out, x_norm, row_stat, rows, (int)n, p);      \
-        else if (nvec <= 256 * V) norm_row_kernel<DT, RM, QM, 4 * V><<<grid, kThreads, 0, s>>>(in, weight, bias, out, x_norm, row_stat, rows, (int)n, p); \
-        else norm_row_kernel<DT, RM, QM, 8 * V><<<grid, kThreads, 0, s>>>(in, weight, bias, out, x_norm, row_stat, rows, (int)n, p);                     \
-    } while (0)
-    MXQ_CHAIN_DISPATCH(MXQ_NM);
-#undef MXQ_NM
-    return check_launch(who);
-}
-
-int mxq_norm_backward_lastdim(const void* grad_out, const void* weight, const void* x_norm,
-                              const void* row_stat, void* grad_in, int dtype, int64_t rows, int64_t n,
-                              int rms_norm, int bits, int exp_bits, float max_norm, int rmode,
-                              int allow_denorm, int flags, void* hip_stream) {
-    const char* who = "mxq_norm_backward_lastdim";
-    NormParams p;
-    bool ident, closed;
-    int rc = chain_params(dtype, bits, exp_bits, max_norm, rmode, allow_denorm, flags, &p.q, &ident, &closed, who);
-    if (rc) return rc;
-    p.eps = 0.0f;
-    p.rms = rms_norm ? 1 : 0;
-    const int epv = dtype == MXQ_DTYPE_F32 ? 4 : 8;
-    if (rows < 0 || n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
-    if (n > 4096 || n % epv != 0)
-        return fail(MXQ_ERR_ARGUMENT, "%s: row length %lld must be a multiple of %d and at most 4096",
-                    who, (long long)n, epv);
-    if (rows == 0 || n == 0) return MXQ_OK;
-    if (!grad_out || !weight || !x_norm || !row_stat || !grad_in) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
-    if (!aligned16(grad_out) || !aligned16(weight) || !aligned16(x_norm) || !aligned16(grad_in))
-        return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
-    hipStream_t s = (hipStream_t)hip_stream;
-    const int grid = grid_for(ceil_div(rows, kThreads / 64));
-    const int64_t nvec = n / epv;
-#define MXQ_NMB(DT, RM, QM)                                                                        \
-    do {                                                                                           \
-        constexpr int V = (DT == MXQ_F32) ? 2 : 1;                                                 \
-        if (nvec <= 128 * V) norm_backward_row_kernel<DT, RM, QM, 2 * V><<<grid, kThreads, 0, s>>>(grad_out, weight, x_norm, row_stat, grad_in, rows, (int)n, p);      \
-        else if (nvec <= 256 * V) norm_backward_row_kernel<DT, RM, QM, 4 * V><<<grid, kThreads, 0, s>>>(grad_out, weight, x_norm, row_stat, grad_in, rows, (int)n, p); \
-        else norm_backward_row_kernel<DT, RM, QM, 8 * V><<<grid, kThreads, 0, s>>>(grad_out, weight, x_norm, row_stat, grad_in, rows, (int)n, p);                     \
-    } while (0)
-    MXQ_CHAIN_DISPATCH(MXQ_NMB);
-#undef MXQ_NMB
     return check_launch(who);
 }
 

@@ -438,6 +438,25 @@ __device__ __forceinline__ float wave_reduce(float v) {
     return v;
 }
 
+// The same over the WPR consecutive waves of a workgroup that share a row: wave results combined in
+// wave order through `part` (one float per wave of the workgroup).  Every wave of the workgroup
+// must take part.
+template <class OP, int WPR>
+__device__ __forceinline__ float row_reduce(float v, float* part) {
+    v = wave_reduce<OP>(v);
+    if constexpr (WPR > 1) {
+        const int wib = threadIdx.x >> 6;
+        __syncthreads();                                     // the previous round has been read
+        if ((threadIdx.x & 63) == 0) part[wib] = v;
+        __syncthreads();
+        const int first = wib - wib % WPR;
+        v = part[first];
+#pragma unroll
+        for (int k = 1; k < WPR; ++k) v = OP::apply(v, part[first + k]);
+    }
+    return v;
+}
+
 // one block of 256 lanes per row (inner large) ...
 template <class OP>
 __global__ __launch_bounds__(TPB) void reduce_inner_block_kernel(const float* __restrict__ in,

@@ -11,15 +11,16 @@ struct SoftmaxParams {
 
 namespace {
 
-// One wave per row; a lane keeps VPL 16-byte vectors of the row in registers from the load to the
-// store (vector j of lane l is vector 64 j + l of the row), so the row is read once and written
-// once.  QMODE: SMQ_GENERIC = the elementwise quantizer with the format in p.q; SMQ_IDENT = the
+// WPR (1, 2 or 4) waves per row; a lane keeps VPL 16-byte vectors of the row in registers from the
+// load to the store (vector j of lane l of the row's 64 WPR lanes is vector 64 WPR j + l), so the
+// row is read once and written once.  Row reductions: shuffles inside a wave, then the waves of a
+// row in order through LDS.  QMODE: SMQ_GENERIC = the elementwise quantizer with the format in p.q; SMQ_IDENT = the
 // identity on values of the tensor dtype (no format configured, or bfloat16 with round-half-even on
 // a bf16 tensor); SMQ_BF16 = closed form for bf16 tensor -> bfloat16, round-half-away.
 // Every step rounds to the tensor dtype first, like the tensor op it stands for, then quantizes.
 enum { SMQ_GENERIC = 0, SMQ_IDENT = 1, SMQ_BF16 = 2 };
 
-template <int DT, int RMODE, int QMODE, int VPL>
+template <int DT, int RMODE, int QMODE, int VPL, int WPR>
 __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict__ in_,
                                                           void* __restrict__ out_, int64_t rows,
                                                           int n, SoftmaxParams p) {
@@ -46,16 +47,21 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
         return Q(v);
     };
 
-    const int lane = threadIdx.x & 63;
-    const int nvec = n / EPV;
-    const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
-    for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows; row += waves) {
-        const u32x4* in = reinterpret_cast<const u32x4*>(in_) + row * nvec;
-        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec;
+    constexpr int LPR = 64 * WPR;                            // lanes per row
+    constexpr int RPB = (TPB / 64) / WPR;                    // rows per block and iteration
+    __shared__ float part[TPB / 64];
+    const int wib = threadIdx.x >> 6;                        // wave in block
+    const int lane = (wib % WPR) * 64 + (threadIdx.x & 63);  // lane within the row
+    const int nvec_row = n / EPV;
+    for (int64_t row0 = (int64_t)blockIdx.x * RPB; row0 < rows; row0 += (int64_t)gridDim.x * RPB) {
+        const int64_t row = row0 + wib / WPR;
+        const int nvec = row < rows ? nvec_row : 0;          // a block's spare waves go through the motions
+        const u32x4* in = reinterpret_cast<const u32x4*>(in_) + row * nvec_row;
+        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec_row;
         u32x4 raw[VPL];
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
-            const int v = j * 64 + lane;
+            const int v = j * LPR + lane;
             if (v < nvec) raw[j] = in[v];
         }
         // positions past the end of the row behave like -inf: they drop out of the maximum and
@@ -64,7 +70,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
         float m = -__builtin_inff();
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
-            const bool valid = j * 64 + lane < nvec;
+            const bool valid = j * LPR + lane < nvec;
 #pragma unroll
             for (int d = 0; d < 4; ++d)
 #pragma unroll
@@ -74,7 +80,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
                     m = MaxOp::apply(m, x[e]);                 // NaN sticks, like torch.max
                 }
         }
-        m = wave_reduce<MaxOp>(m);
+        m = row_reduce<MaxOp, WPR>(m, part);
 
         float sum = 0.0f;
         if (p.exp_mode == 0) {                               // one loop per mode: no branch per element
@@ -96,7 +102,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
                 sum += x[e];
             }
         }
-        sum = Qp(wave_reduce<SumOp>(sum));
+        sum = Qp(row_reduce<SumOp, WPR>(sum, part));
         const bool recip = p.use_recip != 0;
         const float r = recip ? Qp(1.0f / sum) : 0.0f;
         // e / sum without a division per element: one refined reciprocal per row, then a product
@@ -124,7 +130,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
                 }
                 o[d] = Pack<DT>::put(q[0], q[PD - 1]);
             }
-            if (j * 64 + lane < nvec) __builtin_nontemporal_store(o, &out[j * 64 + lane]);
+            if (j * LPR + lane < nvec) __builtin_nontemporal_store(o, &out[j * LPR + lane]);
         }
     }
 }
@@ -150,7 +156,7 @@ struct NormParams {
 
 namespace {
 
-template <int DT, int RMODE, int QMODE, int VPL>
+template <int DT, int RMODE, int QMODE, int VPL, int WPR>
 __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ in_,
                                                        const void* __restrict__ weight_,
                                                        const void* __restrict__ bias_,
@@ -173,19 +179,24 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
     };
     auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
 
-    const int lane = threadIdx.x & 63;
-    const int nvec = n / EPV;
+    constexpr int LPR = 64 * WPR;                            // lanes per row
+    constexpr int RPB = (TPB / 64) / WPR;                    // rows per block and iteration
+    __shared__ float part[TPB / 64];
+    const int wib = threadIdx.x >> 6;                        // wave in block
+    const int lane = (wib % WPR) * 64 + (threadIdx.x & 63);  // lane within the row
+    const int nvec_row = n / EPV;
     const float count = (float)n;
-    const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
-    for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows; row += waves) {
-        const u32x4* in = reinterpret_cast<const u32x4*>(in_) + row * nvec;
+    for (int64_t row0 = (int64_t)blockIdx.x * RPB; row0 < rows; row0 += (int64_t)gridDim.x * RPB) {
+        const int64_t row = row0 + wib / WPR;
+        const int nvec = row < rows ? nvec_row : 0;          // a block's spare waves go through the motions
+        const u32x4* in = reinterpret_cast<const u32x4*>(in_) + row * nvec_row;
         float x[EPL];
         float sum = 0.0f;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
-            const bool valid = j * 64 + lane < nvec;
+            const bool valid = j * LPR + lane < nvec;
             u32x4 raw = {0, 0, 0, 0};
-            if (valid) raw = in[j * 64 + lane];
+            if (valid) raw = in[j * LPR + lane];
 #pragma unroll
             for (int d = 0; d < 4; ++d)
 #pragma unroll
@@ -196,10 +207,10 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
                 }
         }
         if (!p.rms) {
-            const float mean = Q(Q(wave_reduce<SumOp>(sum)) / count);
+            const float mean = Q(Q(row_reduce<SumOp, WPR>(sum, part)) / count);
 #pragma unroll
             for (int j = 0; j < VPL; ++j) {
-                const bool valid = j * 64 + lane < nvec;
+                const bool valid = j * LPR + lane < nvec;
 #pragma unroll
                 for (int k = 0; k < EPV; ++k) x[j * EPV + k] = valid ? Q(x[j * EPV + k] - mean) : 0.0f;
             }
@@ -207,18 +218,18 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
         float sq = 0.0f;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) sq += Q(x[e] * x[e]);
-        const float var = Q(Q(wave_reduce<SumOp>(sq)) / count);
+        const float var = Q(Q(row_reduce<SumOp, WPR>(sq, part)) / count);
         const float vare = Q(var + p.eps);
         const float rinv = Q(1.0f / Q(sqrtf(vare)));
-        if (lane == 0) store_scalar<DT>(stat_, row, p.rms ? rinv : vare);
+        if (lane == 0 && nvec != 0) store_scalar<DT>(stat_, row, p.rms ? rinv : vare);
 
         const u32x4* wv = reinterpret_cast<const u32x4*>(weight_);
         const u32x4* bv = reinterpret_cast<const u32x4*>(bias_);
-        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec;
+        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec_row;
         u32x4* zn = znorm_ ? reinterpret_cast<u32x4*>(znorm_) + row * nvec : nullptr;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
-            const int v = j * 64 + lane;
+            const int v = j * LPR + lane;
             if (v >= nvec) continue;
             const u32x4 w4 = wv[v], b4 = bv[v];
             u32x4 o, z4;
@@ -417,7 +428,7 @@ __global__ __launch_bounds__(TPB) void activation_backward_kernel(const void* __
 // SoftmaxFunction.backward (mx/softmax.py:56-88) over the last axis, same work mapping as the
 // forward kernel:  g = Q(grad); s = Q(sum Q(g y)); grad_input = Q(y Q(g - s)) (, Q(. * ln2) for
 // softmax_exp2, with ln2 at bfloat16 precision).
-template <int DT, int RMODE, int QMODE, int VPL>
+template <int DT, int RMODE, int QMODE, int VPL, int WPR>
 __global__ __launch_bounds__(TPB) void softmax_backward_row_kernel(const void* __restrict__ grad_,
                                                                    const void* __restrict__ y_,
                                                                    void* __restrict__ out_, int64_t rows,
@@ -438,24 +449,29 @@ __global__ __launch_bounds__(TPB) void softmax_backward_row_kernel(const void* _
     };
     auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
 
-    const int lane = threadIdx.x & 63;
-    const int nvec = n / EPV;
-    const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
-    for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows; row += waves) {
-        const u32x4* gin = reinterpret_cast<const u32x4*>(grad_) + row * nvec;
-        const u32x4* yin = reinterpret_cast<const u32x4*>(y_) + row * nvec;
-        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec;
+    constexpr int LPR = 64 * WPR;                            // lanes per row
+    constexpr int RPB = (TPB / 64) / WPR;                    // rows per block and iteration
+    __shared__ float part[TPB / 64];
+    const int wib = threadIdx.x >> 6;                        // wave in block
+    const int lane = (wib % WPR) * 64 + (threadIdx.x & 63);  // lane within the row
+    const int nvec_row = n / EPV;
+    for (int64_t row0 = (int64_t)blockIdx.x * RPB; row0 < rows; row0 += (int64_t)gridDim.x * RPB) {
+        const int64_t row = row0 + wib / WPR;
+        const int nvec = row < rows ? nvec_row : 0;          // a block's spare waves go through the motions
+        const u32x4* gin = reinterpret_cast<const u32x4*>(grad_) + row * nvec_row;
+        const u32x4* yin = reinterpret_cast<const u32x4*>(y_) + row * nvec_row;
+        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec_row;
         float g[EPL];
         u32x4 yraw[VPL];
         float sum = 0.0f;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
-            const bool valid = j * 64 + lane < nvec;
+            const bool valid = j * LPR + lane < nvec;
             u32x4 graw = {0, 0, 0, 0};
             yraw[j] = u32x4{0, 0, 0, 0};
             if (valid) {
-                graw = gin[j * 64 + lane];
-                yraw[j] = yin[j * 64 + lane];
+                graw = gin[j * LPR + lane];
+                yraw[j] = yin[j * LPR + lane];
             }
 #pragma unroll
             for (int d = 0; d < 4; ++d)
@@ -466,7 +482,7 @@ __global__ __launch_bounds__(TPB) void softmax_backward_row_kernel(const void* _
                     sum += valid ? Q(g[e] * Pack<DT>::get(yraw[j][d], h)) : 0.0f;
                 }
         }
-        sum = Q(wave_reduce<SumOp>(sum));
+        sum = Q(row_reduce<SumOp, WPR>(sum, part));
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
             u32x4 o;
@@ -480,7 +496,7 @@ __global__ __launch_bounds__(TPB) void softmax_backward_row_kernel(const void* _
                 }
                 o[d] = Pack<DT>::put(q[0], q[PD - 1]);
             }
-            if (j * 64 + lane < nvec) __builtin_nontemporal_store(o, &out[j * 64 + lane]);
+            if (j * LPR + lane < nvec) __builtin_nontemporal_store(o, &out[j * LPR + lane]);
         }
     }
 }
@@ -493,7 +509,7 @@ __global__ __launch_bounds__(TPB) void softmax_backward_row_kernel(const void* _
 //              dx = Q(Q(d si) + Q(-t z));  grad_input = Q(dx - Q(Q(sum dx) / n))
 //   RMSNorm:   d1 = Q(d r), proj = Q(Q(sum Q(d1 z)) / n)                      (r = saved 1 / rms)
 //              grad_input = d1 - Q(z proj), rounded to the tensor dtype only
-template <int DT, int RMODE, int QMODE, int VPL>
+template <int DT, int RMODE, int QMODE, int VPL, int WPR>
 __global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __restrict__ grad_,
                                                                 const void* __restrict__ weight_,
                                                                 const void* __restrict__ znorm_,
@@ -516,16 +532,21 @@ __global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __re
     };
     auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
 
-    const int lane = threadIdx.x & 63;
-    const int nvec = n / EPV;
+    constexpr int LPR = 64 * WPR;                            // lanes per row
+    constexpr int RPB = (TPB / 64) / WPR;                    // rows per block and iteration
+    __shared__ float part[TPB / 64];
+    const int wib = threadIdx.x >> 6;                        // wave in block
+    const int lane = (wib % WPR) * 64 + (threadIdx.x & 63);  // lane within the row
+    const int nvec_row = n / EPV;
     const float count = (float)n;
     const u32x4* wv = reinterpret_cast<const u32x4*>(weight_);
-    const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
-    for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows; row += waves) {
-        const u32x4* gin = reinterpret_cast<const u32x4*>(grad_) + row * nvec;
-        const u32x4* zin = reinterpret_cast<const u32x4*>(znorm_) + row * nvec;
-        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec;
-        const float stat = load_scalar<DT>(stat_, row);
+    for (int64_t row0 = (int64_t)blockIdx.x * RPB; row0 < rows; row0 += (int64_t)gridDim.x * RPB) {
+        const int64_t row = row0 + wib / WPR;
+        const int nvec = row < rows ? nvec_row : 0;          // a block's spare waves go through the motions
+        const u32x4* gin = reinterpret_cast<const u32x4*>(grad_) + row * nvec_row;
+        const u32x4* zin = reinterpret_cast<const u32x4*>(znorm_) + row * nvec_row;
+        u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec_row;
+        const float stat = nvec != 0 ? load_scalar<DT>(stat_, row) : 1.0f;
         // row scalars
         const float sd = p.rms ? 0.0f : Q(sqrtf(stat));
         const float si = p.rms ? stat : Q(1.0f / sd);
@@ -534,13 +555,13 @@ __global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __re
         float sum = 0.0f;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
-            const bool valid = j * 64 + lane < nvec;
+            const bool valid = j * LPR + lane < nvec;
             u32x4 graw = {0, 0, 0, 0}, wraw = {0, 0, 0, 0};
             zraw[j] = u32x4{0, 0, 0, 0};
             if (valid) {
-                graw = gin[j * 64 + lane];
-                wraw = wv[j * 64 + lane];
-                zraw[j] = zin[j * 64 + lane];
+                graw = gin[j * LPR + lane];
+                wraw = wv[j * LPR + lane];
+                zraw[j] = zin[j * LPR + lane];
             }
 #pragma unroll
             for (int k = 0; k < 4; ++k)
@@ -558,12 +579,12 @@ __global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __re
                     }
                 }
         }
-        float t = Q(Q(wave_reduce<SumOp>(sum)) / count);
+        float t = Q(Q(row_reduce<SumOp, WPR>(sum, part)) / count);
         if (!p.rms) t = -Q(t * Q(1.0f / stat));
         float sum2 = 0.0f;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
-            const bool valid = j * 64 + lane < nvec;
+            const bool valid = j * LPR + lane < nvec;
 #pragma unroll
             for (int k = 0; k < 4; ++k)
 #pragma unroll
@@ -578,7 +599,7 @@ __global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __re
                     }
                 }
         }
-        const float dm = p.rms ? 0.0f : -Q(Q(wave_reduce<SumOp>(sum2)) / count);
+        const float dm = p.rms ? 0.0f : -Q(Q(row_reduce<SumOp, WPR>(sum2, part)) / count);
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
             u32x4 o;
@@ -592,7 +613,7 @@ __global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __re
                 }
                 o[k] = Pack<DT>::put(q[0], q[PD - 1]);
             }
-            if (j * 64 + lane < nvec) __builtin_nontemporal_store(o, &out[j * 64 + lane]);
+            if (j * LPR + lane < nvec) __builtin_nontemporal_store(o, &out[j * LPR + lane]);
         }
     }
 }

@@ -10,13 +10,13 @@ from .vector_ops import (vec_add, vec_mul, vec_quantize, vec_recip, vec_reduce_m
 torch_layer_norm = F.layer_norm
 
 
-MAX_FUSED_ROW = 4096
+MAX_FUSED_ROW = 16384
 
 
 def _fused_forward(x, bf_weight, bf_bias, eps, mx_specs, rms):
     """The forward chain, including the quantization of the input x, as one kernel launch
     (mxq_norm_lastdim); weight and bias are already quantized.  Returns (output, x_norm, row
-    statistic) or None when the kernel does not cover the case (CPU tensors, rows longer than 4096
+    statistic) or None when the kernel does not cover the case (CPU tensors, rows longer than 16384
     or not a multiple of 16 bytes, fp16, mixed dtypes, vec_use_recip, round-half-even to a wide
     format on bf16 tensors)."""
     from . import _lib

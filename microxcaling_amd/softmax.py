@@ -10,12 +10,12 @@ from .vector_ops import (vec_div, vec_exp, vec_exp2, vec_mul, vec_quantize, vec_
 f_softmax = F.softmax
 LN_2_BF16 = 0.69140625           # ln(2) at bfloat16 precision
 
-MAX_FUSED_ROW = 4096
+MAX_FUSED_ROW = 16384
 
 
 def _fused_forward(input, dim, mx_specs):
     """The whole forward chain as one kernel launch (mxq_softmax_lastdim), or None when the kernel
-    does not cover the case: another axis than the last, rows longer than 4096 or not a multiple
+    does not cover the case: another axis than the last, rows longer than 16384 or not a multiple
     of 16 bytes, and what fused_chain_args excludes."""
     from . import _lib
     from .custom_extensions import _flags_value

@@ -302,7 +302,9 @@ def test_linear_backward_runs(dev):
 
 # ---- fused softmax kernel against the oracle's chain of tensor ops --------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(3, 5, 2048), (64, 1000), (7, 8), (2, 4096), (33, 264)])
+@pytest.mark.parametrize("shape", [(3, 5, 2048), (64, 1000), (7, 8), (2, 4096), (33, 264),
+                                   # two and four waves per row; row counts that leave waves of a block spare
+                                   (5, 8192), (3, 6000), (5, 16384), (2, 3, 12000)])
 @pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, softmax_exp2=True),
                                   dict(bfloat=16, vec_use_exp2=True, vec_use_recip=True),
                                   dict(bfloat=16, round="floor"), dict(bfloat=16, round="even"),
@@ -553,7 +555,7 @@ def test_fused_activation_backward_equals_chain(dev, act, dtype, spec):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, softmax_exp2=True), dict(bfloat=12)],
                          ids=["bfloat16", "bfloat16-exp2", "bfloat12"])
-@pytest.mark.parametrize("shape", [(3, 5, 2048), (64, 1000), (33, 264)])
+@pytest.mark.parametrize("shape", [(3, 5, 2048), (64, 1000), (33, 264), (5, 8192), (3, 16384)])
 def test_fused_softmax_backward_against_chain(dev, dtype, spec, shape):
     """One-kernel softmax backward against the chain of vec_* ops on the same saved output; only the
     order of the row sum differs."""
@@ -583,7 +585,7 @@ def test_fused_softmax_backward_against_chain(dev, dtype, spec, shape):
 @pytest.mark.parametrize("kind", ["layernorm", "rmsnorm"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=12)], ids=["bfloat16", "bfloat12"])
-@pytest.mark.parametrize("shape", [(6, 40, 1024), (257, 264), (9, 4096)])
+@pytest.mark.parametrize("shape", [(6, 40, 1024), (257, 264), (9, 4096), (5, 8192), (3, 16384)])
 def test_fused_norm_backward_against_chain(dev, kind, dtype, spec, shape):
     """One-kernel gradient with respect to the input of LayerNorm / RMSNorm against the chain of
     vec_* ops from the same saved tensors; only the order of the two row sums differs.  The

@@ -184,7 +184,7 @@ def test_lstm(dev):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("layer", ["layernorm", "rmsnorm"])
-@pytest.mark.parametrize("shape", [(64, 4096), (5, 7, 1000), (33, 264), (9, 8)])
+@pytest.mark.parametrize("shape", [(64, 4096), (5, 7, 1000), (33, 264), (9, 8), (5, 8192), (3, 16384)])
 @pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, round="floor"), dict(fp=16),
                                   dict(bfloat=16, round="even")])
 def test_fused_norm_kernel_against_the_separate_steps(dev, dtype, layer, shape, spec):
@@ -197,6 +197,8 @@ def test_fused_norm_kernel_against_the_separate_steps(dev, dtype, layer, shape, 
     specs = _specs(quantize_backprop=True, **spec)
     g = torch.Generator().manual_seed(sum(shape))
     x = (torch.randn(*shape, generator=g) * 2 + 0.3).to(dtype)
+    if "fp" in spec and shape[-1] > 4096:
+        x = x * 0.25                                   # keep the row sums inside the fp16 format's range
     go = torch.randn(*shape, generator=g).to(dtype)
     m = cls(shape[-1], eps=1e-5, mx_specs=specs).to(dtype)
     with torch.no_grad():
