@@ -33,11 +33,11 @@ struct LaunchPackT {
 
 template <int CB, int BL, int ODT>
 int launch_gemm_dt(int64_t batch, const GemmArgs& g, hipStream_t s) {
-    // large problems: persistent 256 x 256 tile kernel (144 KB of dynamic LDS, one workgroup per CU);
-    // it fetches 16 scale bytes per row at a time, hence K % 512
+    // large problems: persistent 256 x 256 tile kernel (152 KB of dynamic LDS, one workgroup per CU);
+    // it fetches 16 scale bytes (512 K) per row at a time, so a row must have at least that many
     const int64_t tiles_m = ceil_div(g.M, G2_BM), tiles_n = ceil_div(g.N, G2_BN);
     const int64_t total = tiles_m * tiles_n * batch;
-    if (g.M >= 512 && g.N >= 512 && g.K % 512 == 0 && (int64_t)256 * g.kbytes < ((int64_t)1 << 31) &&
+    if (g.M >= 512 && g.N >= 512 && g.K >= 512 && (int64_t)256 * g.kbytes < ((int64_t)1 << 31) &&
         total < ((int64_t)1 << 30)) {
         static bool configured = false;               // raising the dynamic-LDS limit is per kernel
         static int cus = 0;

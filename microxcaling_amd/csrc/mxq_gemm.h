@@ -541,8 +541,9 @@ constexpr int G2_BM = 256, G2_BN = 256;
 //
 // Scales: one byte per row and 32 K, i.e. 4 bytes per row and K step, each row in a different
 // cache line.  Fetching them per step would double the number of L2 requests of the kernel, so a
-// lane fetches 16 bytes = four K steps of one row at a time into a two-deep ring of scale groups.
-// This needs K % 512 == 0 and a K walk that starts at a multiple of four steps.
+// lane fetches 16 bytes = 512 K of one row at a time into a two-deep ring of scale groups.  What
+// is left of a row when K is not a multiple of 512 comes in per step, 4 bytes per row, into a
+// two-deep ring of its own.
 //
 // A workgroup walks over tiles w, w + G, w + 2 G, ... (G = grid size, a multiple of 8 so that a
 // workgroup stays on its XCD) in one flat sequence of K steps: the last step of a tile already
@@ -553,10 +554,18 @@ constexpr int G3_TILE_BYTES = 256 * 128;
 constexpr int G3_STAGE_BYTES = 2 * G3_TILE_BYTES;            // codes of A and B for one K step
 constexpr int G3_SCALE_OFF = 2 * G3_STAGE_BYTES;
 constexpr int G3_SCALE_GROUP = 512 * 16;                     // 512 rows x 4 K steps x 4 bytes
-constexpr int G3_LDS_BYTES = G3_SCALE_OFF + 2 * G3_SCALE_GROUP;
+constexpr int G3_TAIL_OFF = G3_SCALE_OFF + 2 * G3_SCALE_GROUP;
+constexpr int G3_TAIL_PLANE = 512 * 4;                       // 512 rows x 4 scale bytes
+constexpr int G3_TAIL_SLOT = 2 * G3_TAIL_PLANE;              // one K step: one plane (8-bit) or two (nibbles)
+constexpr int G3_LDS_BYTES = G3_TAIL_OFF + 2 * G3_TAIL_SLOT;
 
 __device__ __forceinline__ void dma16(uint32_t lds_base, uint32_t voff, const unsigned char* sbase) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_base), "v"(voff), "s"(sbase) : "memory");
+}
+// 4 bytes per lane, lane L lands at base + 4 L
+__device__ __forceinline__ void dma4(uint32_t lds_base, uint32_t voff, const unsigned char* sbase) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
                  :: "s"(lds_base), "v"(voff), "s"(sbase) : "memory");
 }
 
@@ -573,6 +582,7 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     constexpr int GS = 16 / SBY;                             // K steps covered by a 16-byte scale group
     const int KB = g.K >> 5;
     const int nk = g.kbytes / GEMM_BK;
+    const int nfull = nk - nk % GS;                          // K steps whose scales come in whole groups
     const int per_batch = tiles_m * tiles_n;
     const int G = gridDim.x;
 
@@ -621,10 +631,14 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
             offb[i] = (uint32_t)min(r, g.N - 1 - n0) * (uint32_t)g.kbytes + ((lane & 7) ^ key_b(r)) * 16;
         }
         offs = (uint32_t)min(s_row, (s_is_b ? g.N - n0 : g.M - m0) - 1) * (uint32_t)KB;
-        // Every tile walks K cyclically from its own starting step (a multiple of four), so that
-        // the K slices in flight at any moment are spread over the memory channels.
-        f_kstart = (int)(((unsigned)logical * 5u) % (unsigned)(nk / GS)) * GS;
+        // The tiles of an XCD walk K in step, so that the A and B panels they share are fetched
+        // into that XCD's L2 once (a start staggered per tile cost up to 30 % on long-K shapes, whose
+        // panels do not stay in L2 that long).  The eight XCDs start at eight different places of a
+        // cyclic walk, which spreads the slices in flight over the memory channels -- unless the
+        // last scale group of a row is a partial one: then everybody starts at K = 0.
+        f_kstart = nfull != nk ? 0 : (int)(((unsigned)(logical % 8) * (unsigned)(nk / GS)) / 8u) * GS;
     };
+    int f_groups = 0;                                        // scale groups fetched so far
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;     // LDS byte address of the array (normally 0)
     // load i (0..7 codes, 8 scales) of flat step t, which is K step fs of the fetch-side tile
     auto fetch_part = [&](int t, int fs, int i) {
@@ -636,9 +650,17 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
             dma16(st + (wave * 32 + i * 8) * 128, offa[i], fA + k0);
         } else if (i < 8) {
             dma16(st + G3_TILE_BYTES + (wave * 32 + (i - 4) * 8) * 128, offb[i - 4], fB + k0);
-        } else if (t % GS == 0) {                           // a new group of GS K steps
-            dma16(lds0 + G3_SCALE_OFF + ((t / GS) & 1) * G3_SCALE_GROUP + wave * 1024, offs,
-                  fS + ((k0 * EPB) >> 5));
+        } else if (fs < nfull) {
+            if (fs % GS == 0) {                              // a new group of GS K steps
+                dma16(lds0 + G3_SCALE_OFF + (f_groups & 1) * G3_SCALE_GROUP + wave * 1024, offs,
+                      fS + ((k0 * EPB) >> 5));
+                ++f_groups;
+            }
+        } else {                                             // past the last whole group: this step only
+#pragma unroll
+            for (int e = 0; e < EPB; ++e)
+                dma4(lds0 + G3_TAIL_OFF + (fs & 1) * G3_TAIL_SLOT + e * G3_TAIL_PLANE + wave * 256, offs,
+                     fS + ((k0 * EPB) >> 5) + 4 * e);
         }
     };
 
@@ -658,8 +680,8 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
         a_addr[q] = a_lane * 128 + ((fg ^ key_a(a_lane) ^ (2 * q)) * 16);
         b_addr[q] = G3_TILE_BYTES + b_lane * 128 + ((fg ^ key_b(b_lane) ^ (2 * q)) * 16);
     }
-    const int sa_off = G3_SCALE_OFF + a_lane * 16;
-    const int sb_off = G3_SCALE_OFF + 4096 + b_lane * 16;
+    const int sa_off = G3_SCALE_OFF + a_lane * 16, sa_tail = G3_TAIL_OFF + a_lane * 4;
+    const int sb_off = G3_SCALE_OFF + 4096 + b_lane * 16, sb_tail = G3_TAIL_OFF + (256 + b_lane) * 4;
     const int sshift = fg * 8;
     struct Frag { u32x4 r[4]; };
     auto frag = [&](const unsigned char* stage, const int* addr, int tile) {
@@ -669,33 +691,42 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
         return f;
     };
     struct Scales { int w[EPB]; };
-    auto scales = [&](const unsigned char* p) {              // the row's scale bytes, this lane's block first
-        Scales sc;
-#pragma unroll
-        for (int e = 0; e < EPB; ++e) sc.w[e] = (int)(reinterpret_cast<const uint32_t*>(p)[e] >> sshift);
-        return sc;
-    };
-    // flat step t: multiply the stage t & 1 while the tile copy fills the other one with K step
-    // fs of the fetch-side tile
-    auto step = [&](int t, int fs) {
+    int c_groups = 0, c_slot = 0;                            // scale groups started, the one in use
+    // flat step t, K step cs of the tile: multiply the stage t & 1 while the tile copy fills the
+    // other one with K step fs of the fetch-side tile
+    auto step = [&](int t, int cs, int fs) {
         const unsigned char* cur = lds + (t & 1) * G3_STAGE_BYTES;
-        const unsigned char* sc = lds + ((t / GS) & 1) * G3_SCALE_GROUP + (t % GS) * SBY;
+        const bool tail = cs >= nfull;
+        if (!tail && cs % GS == 0) c_slot = c_groups++ & 1;
+        // the scale bytes of this step: inside the current group (16 bytes per row), or the planes
+        // of a single step (4 bytes per row each)
+        const unsigned char* sc = tail ? lds + (cs & 1) * G3_TAIL_SLOT
+                                       : lds + c_slot * G3_SCALE_GROUP + (cs % GS) * SBY;
+        auto scales = [&](int in_group, int in_tail) {       // the row's scale bytes, this lane's block first
+            Scales r;
+#pragma unroll
+            for (int e = 0; e < EPB; ++e) {
+                const unsigned char* p = tail ? sc + in_tail + e * G3_TAIL_PLANE : sc + in_group + 4 * e;
+                r.w[e] = (int)(*reinterpret_cast<const uint32_t*>(p) >> sshift);
+            }
+            return r;
+        };
         Frag af[2];
         Scales sa[2];
 #pragma unroll
         for (int ti = 0; ti < 2; ++ti) {
             af[ti] = frag(cur, a_addr, ti);
-            sa[ti] = scales(sc + sa_off + ti * 512);
+            sa[ti] = scales(sa_off + ti * 512, sa_tail + ti * 128);
         }
         Frag bf = frag(cur, b_addr, 0);
-        Scales sb = scales(sc + sb_off);
+        Scales sb = scales(sb_off, sb_tail);
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) {
             Frag bf_next = bf;                               // the next B fragment is read in the
             Scales sb_next = sb;                             // shadow of this fragment's MFMAs
             if (tj + 1 < 4) {
                 bf_next = frag(cur, b_addr, tj + 1);
-                sb_next = scales(sc + sb_off + (tj + 1) * 512);
+                sb_next = scales(sb_off + (tj + 1) * 512, sb_tail + (tj + 1) * 128);
             }
 #pragma unroll
             for (int h = 0; h < NH; ++h)
@@ -726,12 +757,12 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
 
     int t = 0;
     while (true) {
-        for (int cs = 0; cs + 1 < nk; ++cs, ++t) step(t, cs + 1);
+        for (int cs = 0; cs + 1 < nk; ++cs, ++t) step(t, cs, cs + 1);
         // last K step of this tile: the tile copy moves on to the next tile (or, when there is none,
         // fetches this tile's first step once more; nobody reads it)
         const int next = logical + G;
         if (next < total) fetch_tile(next);
-        step(t, 0);
+        step(t, nk - 1, 0);
         ++t;
 
         const int bz = logical / per_batch;

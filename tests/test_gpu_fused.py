@@ -49,7 +49,10 @@ def test_pack_then_unpack_is_the_fake_quantized_tensor(dev, fmt, rnd, dtype):
                                          # the persistent 256 x 256 kernel (K % 512 == 0): one tile
                                          # per workgroup, ragged edges, several tiles per workgroup
                                          (512, 768, 512, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
-                                         (2048, 2048, 512, 5), (2050, 1800, 1024, 5)])
+                                         (2048, 2048, 512, 5), (2050, 1800, 1024, 5),
+                                         # ... with a partial last scale group (K % 512 != 0)
+                                         (600, 520, 640, 2), (1024, 768, 1152, 1), (2050, 1800, 1408, 3),
+                                         (512, 512, 896, 1)])
 @pytest.mark.parametrize("fa,fb", [("fp8_e4m3", "fp8_e4m3"), ("fp8_e5m2", "fp8_e4m3"),
                                    ("fp6_e2m3", "fp8_e5m2"), ("fp4_e2m1", "fp6_e3m2")])
 def test_scaled_mfma_gemm_against_fp64(dev, M, N, K, batch, fa, fb):
@@ -77,7 +80,7 @@ def test_scaled_mfma_gemm_against_fp64(dev, M, N, K, batch, fa, fb):
 
 
 @pytest.mark.parametrize("M,N,K,batch", [(128, 136, 256, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
-                                         (2050, 1800, 512, 5), (520, 777, 512, 1)])
+                                         (2050, 1800, 512, 5), (520, 777, 512, 1), (1030, 520, 1152, 2)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gemm_16bit_outputs_equal_rounded_fp32_output(dev, M, N, K, batch, dtype, with_bias):
@@ -187,7 +190,9 @@ def test_nibble_pack_is_the_fake_quantized_tensor(dev, rnd, dtype):
                                          (1, 5, 512, 1), (600, 520, 256, 2),
                                          # persistent kernel (K % 512 == 0)
                                          (512, 768, 512, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
-                                         (2050, 1800, 1536, 3)])
+                                         (2050, 1800, 1536, 3),
+                                         # ... with a partial last scale group (K % 512 != 0)
+                                         (600, 520, 768, 2), (1024, 768, 1280, 1), (2050, 1800, 2304, 2)])
 def test_fp4_gemm_on_nibbles_against_fp64(dev, M, N, K, batch):
     """Both operands as e2m1 nibbles at the 4-bit MFMA rate: against fp64 on the unpacked operands,
     with a 2^-3 .. 2^3 spread of block scales, and against the same GEMM on byte codes (same
