@@ -208,11 +208,17 @@ int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t 
  * both roundings to c_dtype, which is what "matmul, then add the bias" gives as tensor ops.
  * epilogue_quant = 1 (bf16 C only): additionally apply the elementwise quantization of the layers
  * with mx_specs['bfloat'] = 16 and round-half-away (quantize_elemwise_op, mx/linear.py:88-96,
- * mx/bmm.py:55-57) to the rounded product and again to the rounded sum with the bias. */
+ * mx/bmm.py:55-57) to the rounded product and again to the rounded sum with the bias.
+ * workspace (may be NULL): mxq_gemm_workspace_bytes(...) bytes of device memory, 16-byte aligned.
+ * Products with few output tiles (decode shapes: M <= 128) split K over several workgroups per
+ * tile and add the fp32 partial tiles up in a second launch, in a fixed order; without a workspace
+ * they run unsplit (same result up to the order of the additions, several times slower). */
 int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const void* b_codes,
                    const void* b_scales, int b_kind, const void* bias, void* c, int c_dtype,
                    int64_t batch, int64_t M, int64_t N, int64_t K, int epilogue_quant,
-                   void* hip_stream);
+                   void* workspace, int64_t workspace_bytes, void* hip_stream);
+/* 0 when the product would not be split. */
+int64_t mxq_gemm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int a_kind);
 
 /* Measurement aid (no counterpart in the reference): launches `workgroups` x 256 lanes, each wave
  * issuing iters x 16 scaled 16x16x128 MFMAs on register-resident operands of kind MXQ_CODES_E4M3 or

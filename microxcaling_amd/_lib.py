@@ -46,7 +46,8 @@ GPU_SYMBOLS = {
                                _c_int, _c_f32, _c_int, _c_int, _c_int, _c_ptr]),
     "mxq_unpack_mx": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_i64, _c_i64, _c_ptr]),
     "mxq_gemm_mx_nt": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int,
-                                _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr]),
+                                _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_i64, _c_ptr]),
+    "mxq_gemm_workspace_bytes": (_c_i64, [_c_i64, _c_i64, _c_i64, _c_i64, _c_int]),
     "mxq_probe_mfma_rate": (_c_int, [_c_i64, _c_int, _c_int, _c_ptr, _c_ptr]),
     "mxq_reduce_sum_inner": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),
     "mxq_reduce_max_inner": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),

@@ -31,8 +31,23 @@ struct LaunchPackT {
     }
 };
 
+// The small-tile kernel on few tiles leaves most CUs idle (a decode-shaped product, M <= 128, has
+// N / 128 of them): split the K steps of every tile over several workgroups until about two per CU
+// are in flight, each with at least two steps.  1 = no split.
+int gemm_k_splits(int64_t batch, int64_t M, int64_t N, int64_t K, bool nibbles) {
+    if (M >= 512 && N >= 512 && K >= 512) return 1;                       // the large-tile kernel
+    const int64_t tiles = ceil_div(M, GEMM_BM) * ceil_div(N, GEMM_BN) * batch;
+    const int64_t nk = K / (nibbles ? 2 * GEMM_BK : GEMM_BK);
+    if (tiles >= 256 || nk < 4) return 1;
+    int64_t splits = ceil_div(512, tiles);
+    if (splits > nk / 2) splits = nk / 2;
+    if (splits > 64) splits = 64;
+    const int64_t per = ceil_div(nk, splits);
+    return (int)ceil_div(nk, per);                                        // no empty split
+}
+
 template <int CB, int BL, int ODT>
-int launch_gemm_dt(int64_t batch, const GemmArgs& g, hipStream_t s) {
+int launch_gemm_dt(int64_t batch, const GemmArgs& g, void* workspace, int64_t workspace_bytes, hipStream_t s) {
     // large problems: persistent 256 x 256 tile kernel (152 KB of dynamic LDS, one workgroup per CU);
     // it fetches 16 scale bytes (512 K) per row at a time, so a row must have at least that many
     const int64_t tiles_m = ceil_div(g.M, G2_BM), tiles_n = ceil_div(g.N, G2_BN);
@@ -58,17 +73,31 @@ int launch_gemm_dt(int64_t batch, const GemmArgs& g, hipStream_t s) {
         const unsigned grid = (unsigned)(total < cus ? total : cus);
         mx_gemm_nt_kernel_256p<CB, BL, ODT><<<grid, 512, G3_LDS_BYTES, s>>>(g, (int)tiles_m, (int)tiles_n, (int)total);
     } else {
-        dim3 grid((unsigned)(ceil_div(g.N, GEMM_BN) * ceil_div(g.M, GEMM_BM)), (unsigned)batch);
-        mx_gemm_nt_kernel<CB, BL, ODT><<<grid, kThreads, 0, s>>>(g);
+        const int splits = gemm_k_splits(batch, g.M, g.N, g.K, CB == 4);
+        const int64_t need = (int64_t)splits * batch * g.M * g.N * (int64_t)sizeof(float);
+        const unsigned tiles = (unsigned)(ceil_div(g.N, GEMM_BN) * ceil_div(g.M, GEMM_BM));
+        if (splits > 1 && workspace != nullptr && workspace_bytes >= need && aligned16(workspace)) {
+            GemmArgs part = g;                        // fp32 partial tiles, no epilogue
+            part.c = workspace;
+            part.bias = nullptr;
+            part.q_nan_from = 0u;
+            part.k_splits = splits;
+            mx_gemm_nt_kernel<CB, BL, MXQ_F32><<<dim3(tiles, (unsigned)batch, (unsigned)splits), kThreads, 0, s>>>(part);
+            const int64_t rows = batch * g.M, items = rows * ceil_div(g.N, 4);
+            gemm_split_reduce_kernel<ODT><<<(unsigned)ceil_div(items, kThreads), kThreads, 0, s>>>(
+                reinterpret_cast<const float*>(workspace), g.c, g.bias, g.q_nan_from, splits, rows, g.N);
+        } else {
+            mx_gemm_nt_kernel<CB, BL, ODT><<<dim3(tiles, (unsigned)batch), kThreads, 0, s>>>(g);
+        }
     }
     return MXQ_OK;
 }
 
 template <int CB, int BL>
-int launch_gemm(int c_dtype, int64_t batch, const GemmArgs& g, hipStream_t s) {
-    if (c_dtype == MXQ_DTYPE_F32) return launch_gemm_dt<CB, BL, MXQ_F32>(batch, g, s);
-    if (c_dtype == MXQ_DTYPE_BF16) return launch_gemm_dt<CB, BL, MXQ_BF16>(batch, g, s);
-    return launch_gemm_dt<CB, BL, MXQ_F16>(batch, g, s);
+int launch_gemm(int c_dtype, int64_t batch, const GemmArgs& g, void* ws, int64_t ws_bytes, hipStream_t s) {
+    if (c_dtype == MXQ_DTYPE_F32) return launch_gemm_dt<CB, BL, MXQ_F32>(batch, g, ws, ws_bytes, s);
+    if (c_dtype == MXQ_DTYPE_BF16) return launch_gemm_dt<CB, BL, MXQ_BF16>(batch, g, ws, ws_bytes, s);
+    return launch_gemm_dt<CB, BL, MXQ_F16>(batch, g, ws, ws_bytes, s);
 }
 
 // splits of the outer axis for the two-pass outer reduction
@@ -173,7 +202,7 @@ int mxq_unpack_mx(const void* codes, const void* scales, int code_kind, void* ou
 int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const void* b_codes,
                    const void* b_scales, int b_kind, const void* bias, void* c, int c_dtype,
                    int64_t batch, int64_t M, int64_t N, int64_t K, int epilogue_quant,
-                   void* hip_stream) {
+                   void* workspace, int64_t workspace_bytes, void* hip_stream) {
     const char* who = "mxq_gemm_mx_nt";
     if (c_dtype < 0 || c_dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, c_dtype);
     if (epilogue_quant != 0 && (epilogue_quant != 1 || c_dtype != MXQ_DTYPE_BF16))
@@ -211,18 +240,27 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const 
     }
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.kbytes = (int)(nib ? K / 2 : K);
+    g.k_splits = 1;
     g.batch_a = M * g.kbytes; g.batch_sa = M * (K / 32);
     g.batch_b = N * g.kbytes; g.batch_sb = N * (K / 32);
     g.batch_c = M * N;
     hipStream_t s = (hipStream_t)hip_stream;
     int rc;
-    if (nib) rc = launch_gemm<4, 4>(c_dtype, batch, g, s);
-    else if (!a_kind && !b_kind) rc = launch_gemm<0, 0>(c_dtype, batch, g, s);
-    else if (a_kind && !b_kind) rc = launch_gemm<1, 0>(c_dtype, batch, g, s);
-    else if (!a_kind && b_kind) rc = launch_gemm<0, 1>(c_dtype, batch, g, s);
-    else rc = launch_gemm<1, 1>(c_dtype, batch, g, s);
+    if (nib) rc = launch_gemm<4, 4>(c_dtype, batch, g, workspace, workspace_bytes, s);
+    else if (!a_kind && !b_kind) rc = launch_gemm<0, 0>(c_dtype, batch, g, workspace, workspace_bytes, s);
+    else if (a_kind && !b_kind) rc = launch_gemm<1, 0>(c_dtype, batch, g, workspace, workspace_bytes, s);
+    else if (!a_kind && b_kind) rc = launch_gemm<0, 1>(c_dtype, batch, g, workspace, workspace_bytes, s);
+    else rc = launch_gemm<1, 1>(c_dtype, batch, g, workspace, workspace_bytes, s);
     if (rc) return rc;
     return check_launch(who);
+}
+
+int64_t mxq_gemm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int a_kind) {
+    if (batch <= 0 || M <= 0 || N <= 0 || K <= 0) return 0;
+    const bool nib = a_kind == MXQ_CODES_E2M1;
+    if (K % (nib ? 2 * GEMM_BK : GEMM_BK) != 0) return 0;
+    const int splits = gemm_k_splits(batch, M, N, K, nib);
+    return splits == 1 ? 0 : (int64_t)splits * batch * M * N * (int64_t)sizeof(float);
 }
 
 int mxq_probe_mfma_rate(int64_t workgroups, int iters, int code_kind, void* sink, void* hip_stream) {

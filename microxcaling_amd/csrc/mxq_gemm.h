@@ -202,6 +202,8 @@ struct GemmArgs {
                           // closed form mxq_quant_bf16_to_bfloat16_nearest with this threshold)
     int M, N, K;
     int kbytes;           // bytes of codes per row: K (8-bit codes) or K / 2 (e2m1 nibbles)
+    int k_splits;         // small-tile kernel: workgroups along gridDim.z share the K steps of a tile and
+                          // each write an fp32 partial tile (split z of batch b at ((z * batch + b) M N)
     int64_t batch_a, batch_sa, batch_b, batch_sb, batch_c;   // strides between batches (bytes / elements of C)
 };
 
@@ -456,10 +458,14 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
         for (int e = 0; e < EPB; ++e)
             *reinterpret_cast<uint32_t*>((s_is_a ? sAs : sBs) + srow * SBY + 4 * e) = sv[e];
     };
-    // K is walked cyclically from a per-workgroup starting step (see the 256 x 256 kernel)
-    const int nk = g.kbytes / GEMM_BK;
+    // this workgroup's K steps (all of them unless the tile is split over gridDim.z), walked
+    // cyclically from a per-workgroup starting step
+    const int nk_all = g.kbytes / GEMM_BK;
+    const int per_split = (nk_all + g.k_splits - 1) / g.k_splits;
+    const int kbeg = (int)blockIdx.z * per_split;
+    const int nk = min(per_split, nk_all - kbeg);
     const int kstart = (int)((blockIdx.x * 5u + blockIdx.y) % (unsigned)nk);
-    auto kof = [&](int step) { return ((kstart + step) % nk) * GEMM_BK; };
+    auto kof = [&](int step) { return (kbeg + (kstart + step) % nk) * GEMM_BK; };
     fetch(kof(0));
     stash();
     __syncthreads();
@@ -503,7 +509,7 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
         __syncthreads();
     }
 
-    const int64_t cbase = bz * g.batch_c;
+    const int64_t cbase = ((int64_t)blockIdx.z * gridDim.y + bz) * g.batch_c;
     const bool inside = m0 + GEMM_BM <= g.M && n0 + GEMM_BN <= g.N && (g.N & 3) == 0 &&
                         ((uintptr_t)g.c & 15) == 0;
     const bool inside8 = inside && (g.N & 7) == 0 && ((uintptr_t)g.bias & 15) == 0;
@@ -524,6 +530,33 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
 }
 
 constexpr int G2_BM = 256, G2_BN = 256;
+
+// Second pass of a split small-tile GEMM: C = epilogue(sum over splits, in order, of the fp32 partial
+// tiles); `rows` = batch * M rows of N columns, four columns per lane.
+template <int OUT_DT>
+__global__ __launch_bounds__(TPB) void gemm_split_reduce_kernel(const float* __restrict__ partial, void* c,
+                                                                const void* bias, uint32_t q_nan_from,
+                                                                int splits, int64_t rows, int N) {
+    const int groups = (N + 3) / 4;
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= rows * groups) return;
+    const int64_t m = i / groups;
+    const int n = (int)(i % groups) * 4;
+    const bool vec = (N & 3) == 0 && ((uintptr_t)c & 15) == 0;
+    const int64_t plane = rows * (int64_t)N;
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < splits; ++z) {
+        const float* p = partial + z * plane + m * N + n;
+        if (vec) {
+            acc += *reinterpret_cast<const v4f*>(p);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < N) acc[r] += p[r];
+        }
+    }
+    store_c4<OUT_DT>(c, bias, q_nan_from, 0, (int)m, n, (int)rows, N, vec, acc);
+}
 
 // ================================================================================================
 // Main GEMM kernel: persistent workgroups, tile 256 x 256 x 128 bytes of K, 512 lanes = 4 x 2 waves,

@@ -144,11 +144,14 @@ def gemm_nt(a_packed, b_packed, out_dtype=torch.float32, bias=None, epilogue_qua
             raise RuntimeError("%s: bias must hold N values of the output dtype" % who)
     out = torch.empty(ac.shape[:-2] + (M, N), dtype=out_dtype, device=ac.device)
     lib = _lib.gpu()
+    ws_bytes = lib.mxq_gemm_workspace_bytes(batch, M, N, K, int(ae))    # few tiles: K is split
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=ac.device) if ws_bytes else None
     with torch.cuda.device(ac.device):
         rc = lib.mxq_gemm_mx_nt(ac.data_ptr(), asc.data_ptr(), int(ae), bc.data_ptr(),
                                 bsc.data_ptr(), int(be), None if bias is None else bias.data_ptr(),
                                 out.data_ptr(), _DTYPE[out_dtype], batch, M, N, K,
-                                int(bool(epilogue_quant)), _stream(ac))
+                                int(bool(epilogue_quant)), None if ws is None else ws.data_ptr(),
+                                ws_bytes, _stream(ac))
     _lib.check(rc, lib)
     return out
 

@@ -52,7 +52,10 @@ def test_pack_then_unpack_is_the_fake_quantized_tensor(dev, fmt, rnd, dtype):
                                          (2048, 2048, 512, 5), (2050, 1800, 1024, 5),
                                          # ... with a partial last scale group (K % 512 != 0)
                                          (600, 520, 640, 2), (1024, 768, 1152, 1), (2050, 1800, 1408, 3),
-                                         (512, 512, 896, 1)])
+                                         (512, 512, 896, 1),
+                                         # few output tiles: K split over several workgroups per tile
+                                         (64, 1024, 2048, 1), (16, 2050, 4096, 2), (100, 520, 1152, 1),
+                                         (1, 128, 8192, 1)])
 @pytest.mark.parametrize("fa,fb", [("fp8_e4m3", "fp8_e4m3"), ("fp8_e5m2", "fp8_e4m3"),
                                    ("fp6_e2m3", "fp8_e5m2"), ("fp4_e2m1", "fp6_e3m2")])
 def test_scaled_mfma_gemm_against_fp64(dev, M, N, K, batch, fa, fb):
@@ -80,7 +83,8 @@ def test_scaled_mfma_gemm_against_fp64(dev, M, N, K, batch, fa, fb):
 
 
 @pytest.mark.parametrize("M,N,K,batch", [(128, 136, 256, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
-                                         (2050, 1800, 512, 5), (520, 777, 512, 1), (1030, 520, 1152, 2)])
+                                         (2050, 1800, 512, 5), (520, 777, 512, 1), (1030, 520, 1152, 2),
+                                         (64, 1032, 2048, 1), (30, 777, 1024, 2)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gemm_16bit_outputs_equal_rounded_fp32_output(dev, M, N, K, batch, dtype, with_bias):
@@ -102,7 +106,8 @@ def test_gemm_16bit_outputs_equal_rounded_fp32_output(dev, M, N, K, batch, dtype
     assert got.dtype == dtype and torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
-@pytest.mark.parametrize("M,N,K,batch", [(128, 136, 256, 1), (600, 520, 1024, 2), (2050, 1800, 512, 3)])
+@pytest.mark.parametrize("M,N,K,batch", [(128, 136, 256, 1), (600, 520, 1024, 2), (2050, 1800, 512, 3),
+                                         (64, 1032, 2048, 1)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gemm_epilogue_quantization_equals_separate_steps(dev, M, N, K, batch, with_bias):
     """epilogue_quant: the bfloat16 / round-half-away quantization after the product and after the
@@ -192,7 +197,9 @@ def test_nibble_pack_is_the_fake_quantized_tensor(dev, rnd, dtype):
                                          (512, 768, 512, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
                                          (2050, 1800, 1536, 3),
                                          # ... with a partial last scale group (K % 512 != 0)
-                                         (600, 520, 768, 2), (1024, 768, 1280, 1), (2050, 1800, 2304, 2)])
+                                         (600, 520, 768, 2), (1024, 768, 1280, 1), (2050, 1800, 2304, 2),
+                                         # few output tiles: K split over several workgroups per tile
+                                         (64, 1024, 2048, 1), (16, 2050, 4096, 2)])
 def test_fp4_gemm_on_nibbles_against_fp64(dev, M, N, K, batch):
     """Both operands as e2m1 nibbles at the 4-bit MFMA rate: against fp64 on the unpacked operands,
     with a 2^-3 .. 2^3 spread of block scales, and against the same GEMM on byte codes (same
@@ -700,3 +707,26 @@ def test_layers_replay_from_a_hip_graph(dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(static_y.view(torch.int16), want.view(torch.int16)), i
+
+
+def test_gemm_split_k_is_used_and_optional(dev):
+    """Few output tiles: the library asks for a workspace and splits K; without one the product
+    still comes out (unsplit), equal up to the order of the additions."""
+    from microxcaling_amd import _lib
+    from microxcaling_amd.fused import pack_mx, gemm_nt
+    lib = _lib.gpu()
+    assert lib.mxq_gemm_workspace_bytes(1, 64, 1024, 4096, 0) > 0
+    assert lib.mxq_gemm_workspace_bytes(1, 4096, 4096, 4096, 0) == 0          # large-tile kernel
+    assert lib.mxq_gemm_workspace_bytes(1, 64, 1024, 256, 0) == 0             # too few K steps
+    g = torch.Generator().manual_seed(3)
+    a, b = torch.randn(64, 4096, generator=g).to(dev), torch.randn(1024, 4096, generator=g).to(dev)
+    (ac, asc, ak), (bc, bsc, bk) = pack_mx(a, "fp8_e4m3"), pack_mx(b, "fp8_e4m3")
+    split = gemm_nt((ac, asc, ak), (bc, bsc, bk), torch.float32)
+    plain = torch.empty_like(split)
+    rc = lib.mxq_gemm_mx_nt(ac.data_ptr(), asc.data_ptr(), 0, bc.data_ptr(), bsc.data_ptr(), 0, None,
+                            plain.data_ptr(), 0, 1, 64, 1024, 4096, 0, None, 0,
+                            torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert rel_err(split, plain) < 1e-4
+
