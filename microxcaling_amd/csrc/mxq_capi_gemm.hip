@@ -31,11 +31,20 @@ struct LaunchPackT {
     }
 };
 
+// The persistent 256 x 256 tile kernel serves products with enough tiles to occupy half the CUs;
+// below that the small tiles, with K split, are two to five times faster (512 x 4096 x 8192: 329 ->
+// 745 TFLOP/s).
+constexpr int64_t kMinLargeTiles = 128;
+bool large_tiles(int64_t batch, int64_t M, int64_t N, int64_t K) {
+    const int64_t total = ceil_div(M, G2_BM) * ceil_div(N, G2_BN) * batch;
+    return M >= 512 && N >= 512 && K >= 512 && total >= kMinLargeTiles && total < ((int64_t)1 << 30);
+}
+
 // The small-tile kernel on few tiles leaves most CUs idle (a decode-shaped product, M <= 128, has
 // N / 128 of them): split the K steps of every tile over several workgroups until about two per CU
 // are in flight, each with at least two steps.  1 = no split.
 int gemm_k_splits(int64_t batch, int64_t M, int64_t N, int64_t K, bool nibbles) {
-    if (M >= 512 && N >= 512 && K >= 512) return 1;                       // the large-tile kernel
+    if (large_tiles(batch, M, N, K)) return 1;
     const int64_t tiles = ceil_div(M, GEMM_BM) * ceil_div(N, GEMM_BN) * batch;
     const int64_t nk = K / (nibbles ? 2 * GEMM_BK : GEMM_BK);
     if (tiles >= 256 || nk < 4) return 1;
@@ -52,8 +61,7 @@ int launch_gemm_dt(int64_t batch, const GemmArgs& g, void* workspace, int64_t wo
     // it fetches 16 scale bytes (512 K) per row at a time, so a row must have at least that many
     const int64_t tiles_m = ceil_div(g.M, G2_BM), tiles_n = ceil_div(g.N, G2_BN);
     const int64_t total = tiles_m * tiles_n * batch;
-    if (g.M >= 512 && g.N >= 512 && g.K >= 512 && (int64_t)256 * g.kbytes < ((int64_t)1 << 31) &&
-        total < ((int64_t)1 << 30)) {
+    if (large_tiles(batch, g.M, g.N, g.K) && (int64_t)256 * g.kbytes < ((int64_t)1 << 31)) {
         static bool configured = false;               // raising the dynamic-LDS limit is per kernel
         static int cus = 0;
         if (!configured) {

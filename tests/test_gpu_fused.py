@@ -46,13 +46,15 @@ def test_pack_then_unpack_is_the_fake_quantized_tensor(dev, fmt, rnd, dtype):
 @pytest.mark.parametrize("M,N,K,batch", [(128, 128, 128, 1), (256, 384, 512, 1), (100, 72, 256, 1),
                                          (130, 257, 128, 3), (16, 16, 128, 2), (1, 5, 384, 1),
                                          (512, 768, 256, 1), (600, 520, 128, 2),
-                                         # the persistent 256 x 256 kernel (K % 512 == 0): one tile
-                                         # per workgroup, ragged edges, several tiles per workgroup
+                                         # large shapes with few tiles: small tiles, K split
                                          (512, 768, 512, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
-                                         (2048, 2048, 512, 5), (2050, 1800, 1024, 5),
+                                         (600, 520, 640, 2), (1024, 768, 1152, 1), (512, 512, 896, 1),
+                                         # the persistent 256 x 256 kernel (at least 128 tiles): fewer
+                                         # tiles than CUs, several tiles per workgroup, ragged edges
+                                         (2048, 2048, 512, 2), (2048, 2048, 512, 5), (2050, 1800, 1024, 5),
+                                         (4096, 2048, 1024, 1), (530, 512, 512, 22),
                                          # ... with a partial last scale group (K % 512 != 0)
-                                         (600, 520, 640, 2), (1024, 768, 1152, 1), (2050, 1800, 1408, 3),
-                                         (512, 512, 896, 1),
+                                         (2050, 1800, 1408, 3), (2048, 4096, 640, 1), (1100, 1500, 1152, 5),
                                          # few output tiles: K split over several workgroups per tile
                                          (64, 1024, 2048, 1), (16, 2050, 4096, 2), (100, 520, 1152, 1),
                                          (1, 128, 8192, 1)])
@@ -84,7 +86,8 @@ def test_scaled_mfma_gemm_against_fp64(dev, M, N, K, batch, fa, fb):
 
 @pytest.mark.parametrize("M,N,K,batch", [(128, 136, 256, 1), (600, 520, 1024, 2), (1024, 512, 2048, 1),
                                          (2050, 1800, 512, 5), (520, 777, 512, 1), (1030, 520, 1152, 2),
-                                         (64, 1032, 2048, 1), (30, 777, 1024, 2)])
+                                         (64, 1032, 2048, 1), (30, 777, 1024, 2), (2050, 1800, 1152, 2),
+                                         (2048, 4104, 512, 1)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_gemm_16bit_outputs_equal_rounded_fp32_output(dev, M, N, K, batch, dtype, with_bias):
