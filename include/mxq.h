@@ -42,10 +42,13 @@ extern "C" {
 /* flags */
 #define MXQ_FLAG_EXACT_EXPONENT 1 /* bit-field exponents instead of torch's floor(log2(x)) */
 #define MXQ_FLAG_PACK_NIBBLES 4   /* mxq_pack_mx / _t, fp4 (e2m1) only: 4-bit codes, two per byte */
+#define MXQ_FLAG_PACK_SIXBIT 8    /* mxq_pack_mx / _t, fp6 (e2m3, e3m2) only: 6-bit codes, four in three bytes */
 
 /* kinds of packed element codes */
 #define MXQ_CODES_E4M3 0 /* one OCP e4m3 byte per element */
 #define MXQ_CODES_E5M2 1 /* one OCP e5m2 byte per element */
+#define MXQ_CODES_E2M3 2 /* OCP e2m3, 6 bits per element: element j of a row in bits 6 j .. 6 j + 5 of the row */
+#define MXQ_CODES_E3M2 3 /* OCP e3m2, 6 bits per element, same packing */
 #define MXQ_CODES_E2M1 4 /* one OCP e2m1 nibble per element, the lower K index in the low nibble */
 
 /* status codes */
@@ -185,6 +188,7 @@ int mxq_softmax_backward_lastdim(const void* grad_out, const void* y, void* grad
  *   codes  uint8 (rows, K)     OCP e4m3 for fp8_e4m3 / fp6_e3m2 / fp6_e2m3 / fp4_e2m1 elements (e4m3
  *                              holds all their values exactly), OCP e5m2 for fp8_e5m2 elements;
  *          or uint8 (rows, K/2) OCP e2m1 nibbles for fp4_e2m1 with MXQ_FLAG_PACK_NIBBLES
+ *          or uint8 (rows, 3K/4) OCP 6-bit codes for fp6_e2m3 / fp6_e3m2 with MXQ_FLAG_PACK_SIXBIT
  *   scales uint8 (rows, K/32)  E8M0 (shared exponent + 127; 255 = the block is NaN)
  * value = code * 2^(scale - 127), identical to what mxq_quantize_mx_by_tile returns. */
 int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t rows, int64_t K,

@@ -12,6 +12,8 @@ struct LaunchPack {
         const u32x4* i4 = reinterpret_cast<const u32x4*>(in);
         unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
         if (kind == 1) mx_pack_kernel<DT, RMODE, ZE, 1, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+        else if (kind == 2) mx_pack_kernel<DT, RMODE, ZE, 2, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+        else if (kind == 3) mx_pack_kernel<DT, RMODE, ZE, 3, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
         else if (kind == 4) mx_pack_kernel<DT, RMODE, ZE, 4, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
         else mx_pack_kernel<DT, RMODE, ZE, 0, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
     }
@@ -26,6 +28,8 @@ struct LaunchPackT {
         unsigned char* c = reinterpret_cast<unsigned char*>(codes);
         unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
         if (kind == 1) mx_pack_t_kernel<DT, RMODE, ZE, 1><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+        else if (kind == 2) mx_pack_t_kernel<DT, RMODE, ZE, 2><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+        else if (kind == 3) mx_pack_t_kernel<DT, RMODE, ZE, 3><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
         else if (kind == 4) mx_pack_t_kernel<DT, RMODE, ZE, 4><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
         else mx_pack_t_kernel<DT, RMODE, ZE, 0><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
     }
@@ -111,6 +115,12 @@ int launch_gemm(int c_dtype, int64_t batch, const GemmArgs& g, void* ws, int64_t
 // splits of the outer axis for the two-pass outer reduction
 int code_kind(int ebits, int mbits, int flags, const char* who) {
     const bool fp4 = ebits == 2 && mbits == 3;
+    if (flags & MXQ_FLAG_PACK_SIXBIT) {
+        if (ebits == 2 && mbits == 5) return MXQ_CODES_E2M3;
+        if (ebits == 3 && mbits == 4) return MXQ_CODES_E3M2;
+        fail(MXQ_ERR_ARGUMENT, "%s: 6-bit codes exist for the e2m3 and e3m2 formats only", who);
+        return -1;
+    }
     if (flags & MXQ_FLAG_PACK_NIBBLES) {
         if (!fp4) {
             fail(MXQ_ERR_ARGUMENT, "%s: 4-bit codes exist for the e2m1 format only", who);
@@ -186,7 +196,7 @@ int mxq_unpack_mx(const void* codes, const void* scales, int code_kind, void* ou
                   int64_t rows, int64_t K, void* hip_stream) {
     const char* who = "mxq_unpack_mx";
     if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
-    if (code_kind != MXQ_CODES_E4M3 && code_kind != MXQ_CODES_E5M2 && code_kind != MXQ_CODES_E2M1)
+    if (code_kind < MXQ_CODES_E4M3 || code_kind > MXQ_CODES_E2M1)
         return fail(MXQ_ERR_ARGUMENT, "%s: unknown code kind %d", who, code_kind);
     if (rows < 0 || K < 0 || K % 32 != 0) return fail(MXQ_ERR_ARGUMENT, "%s: bad size", who);
     const int64_t n = rows * K;
@@ -198,6 +208,8 @@ int mxq_unpack_mx(const void* codes, const void* scales, int code_kind, void* ou
     const int grid = grid_for(ceil_div(n, kThreads * 4));
 #define MXQ_UNPACK(DT)                                                                       \
     if (code_kind == 1) mx_unpack_kernel<DT, 1><<<grid, kThreads, 0, s>>>(cd, sc, out, n);      \
+    else if (code_kind == 2) mx_unpack_kernel<DT, 2><<<grid, kThreads, 0, s>>>(cd, sc, out, n); \
+    else if (code_kind == 3) mx_unpack_kernel<DT, 3><<<grid, kThreads, 0, s>>>(cd, sc, out, n); \
     else if (code_kind == 4) mx_unpack_kernel<DT, 4><<<grid, kThreads, 0, s>>>(cd, sc, out, n); \
     else mx_unpack_kernel<DT, 0><<<grid, kThreads, 0, s>>>(cd, sc, out, n);
     if (dtype == MXQ_DTYPE_F32) { MXQ_UNPACK(MXQ_F32) }

@@ -268,6 +268,24 @@ MXQ_HD float mxq_decode_e2m1(uint32_t c) {
     return (c & 0x8u) ? -v : v;
 }
 
+// OCP 6-bit codes of values the formats represent exactly.  e2m3: sign, 2 exponent bits (bias 1),
+// 3 fraction bits -- up to 7.5 in steps of 1/8 below 1.  e3m2: 3 exponent bits (bias 3), 2 fraction
+// bits -- up to 28, steps of 1/16 below 1/4.  MANT = fraction bits, BIAS = exponent bias.
+template <int MANT, int BIAS>
+MXQ_HD uint32_t mxq_encode_fp6(float y) {
+    const uint32_t u = mxq_bits(y), ua = u & 0x7FFFFFFFu;
+    const uint32_t normal = (ua >> (23 - MANT)) - ((uint32_t)(127 - BIAS) << MANT);
+    const uint32_t subnormal = (uint32_t)(mxq_float(ua) * (float)(1 << (BIAS - 1 + MANT)));
+    return ((u >> 26) & 0x20u) | (ua >= ((uint32_t)(128 - BIAS) << 23) ? normal : subnormal);
+}
+template <int MANT, int BIAS>
+MXQ_HD float mxq_decode_fp6(uint32_t c) {
+    const uint32_t e = (c >> MANT) & ((1u << (5 - MANT)) - 1u), m = c & ((1u << MANT) - 1u);
+    const float v = e ? ldexpf((float)((1u << MANT) + m), (int)e - BIAS - MANT)
+                      : ldexpf((float)m, 1 - BIAS - MANT);
+    return (c & 0x20u) ? -v : v;
+}
+
 // E8M0 byte of a block scale: exponent + 127, 255 for a NaN block (MxqScale.scale is NaN)
 MXQ_HD uint32_t mxq_encode_e8m0(float scale) {
     const uint32_t u = mxq_bits(scale);

@@ -29,14 +29,20 @@ namespace {
 // ================================================================================================
 // quantize + pack, shared axis innermost, block size 32
 // ================================================================================================
-// KIND of the codes: 0 = OCP e4m3 bytes, 1 = OCP e5m2 bytes, 4 = OCP e2m1 nibbles (two per byte, the
+// KIND of the codes (the operand format numbers of the scaled MFMA): 0 = OCP e4m3 bytes, 1 = OCP e5m2
+// bytes, 2 = OCP e2m3 and 3 = OCP e3m2 6-bit codes (a little-endian bit stream: element j of a row
+// in bits 6 j .. 6 j + 5, four elements in three bytes), 4 = OCP e2m1 nibbles (two per byte, the
 // element with the lower K index in the low nibble)
 template <int KIND>
 __device__ __forceinline__ uint32_t mx_encode(float y) {
     if (KIND == 1) return mxq_encode_e5m2(y);
+    if (KIND == 2) return mxq_encode_fp6<3, 1>(y);
+    if (KIND == 3) return mxq_encode_fp6<2, 3>(y);
     if (KIND == 4) return mxq_encode_e2m1(y);
     return mxq_encode_e4m3(y);
 }
+template <int KIND>
+constexpr int code_bits() { return KIND == 4 ? 4 : (KIND == 2 || KIND == 3) ? 6 : 8; }
 
 template <int DT, int RMODE, bool ZONE_ELEM, int KIND, int UNROLL>
 __global__ __launch_bounds__(TPB) void mx_pack_kernel(const u32x4* __restrict__ in,
@@ -66,6 +72,7 @@ __global__ __launch_bounds__(TPB) void mx_pack_kernel(const u32x4* __restrict__ 
             const uint32_t um = group_max<LPT>(vec_abs_max<DT>(v[j]));
             const MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, ZS);
             uint32_t out[PD] = {};
+            uint64_t six = 0;                              // 6-bit codes: 24 (fp32 in) or 48 bits per lane
 #pragma unroll
             for (int d = 0; d < 4; ++d)
 #pragma unroll
@@ -74,10 +81,34 @@ __global__ __launch_bounds__(TPB) void mx_pack_kernel(const u32x4* __restrict__ 
                         Pack<DT>::get(v[j][d], h), sc, p.fmt, zone, ZS);
                     const uint32_t c = mx_encode<KIND>(y);
                     const int e = d * PD + h;              // element index inside the vector
-                    if (KIND == 4) out[0] |= c << (4 * e);
+                    if (code_bits<KIND>() == 6) six |= (uint64_t)c << (6 * e);
+                    else if (KIND == 4) out[0] |= c << (4 * e);
                     else out[e / 4] |= c << (8 * (e % 4));
                 }
-            if (i < n_vec) {
+            if constexpr (code_bits<KIND>() == 6) {
+                // 16 elements = 12 bytes: the first of 2 (4) neighbouring lanes collects and stores them
+                uint32_t w0, w1, w2;
+                if (PD == 2) {
+                    const uint64_t hi = __shfl_down(six, 1, 64);
+                    w0 = (uint32_t)six;
+                    w1 = (uint32_t)(six >> 32) | ((uint32_t)hi << 16);
+                    w2 = (uint32_t)(hi >> 16);
+                } else {
+                    const uint32_t b0 = (uint32_t)six, b1 = (uint32_t)__shfl_down(six, 1, 64),
+                                   b2 = (uint32_t)__shfl_down(six, 2, 64), b3 = (uint32_t)__shfl_down(six, 3, 64);
+                    w0 = b0 | (b1 << 24);
+                    w1 = (b1 >> 8) | (b2 << 16);
+                    w2 = (b2 >> 16) | (b3 << 8);
+                }
+                if (i < n_vec && (threadIdx.x & (4 / PD - 1)) == 0) {
+                    uint32_t* dst = reinterpret_cast<uint32_t*>(reinterpret_cast<unsigned char*>(codes_) + i * (3 * PD));
+                    dst[0] = w0;
+                    dst[1] = w1;
+                    dst[2] = w2;
+                }
+                if (i < n_vec && (threadIdx.x & (LPT - 1)) == 0)
+                    scales[i / LPT] = (unsigned char)mxq_encode_e8m0(sc.scale);
+            } else if (i < n_vec) {
                 if (KIND == 4) {
                     if (PD == 1) reinterpret_cast<unsigned short*>(codes_)[i] = (unsigned short)out[0];
                     else reinterpret_cast<uint32_t*>(codes_)[i] = out[0];
@@ -143,12 +174,20 @@ __global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict_
             const float y = mxq_quant_mx_elem_unscaled<RMODE, ADT, ZONE_ELEM>(
                 Pack<DT>::get(raw[r][k / PD], k % PD), sc, p.fmt, zone, ZS);
             const uint32_t code = mx_encode<KIND>(y);
-            if (KIND == 4) out[r / 8] |= code << (4 * (r % 8));
+            if (code_bits<KIND>() == 6) {
+                out[(6 * r) >> 5] |= code << ((6 * r) & 31);
+                if (((6 * r) & 31) > 26) out[((6 * r) >> 5) + 1] |= code >> (32 - ((6 * r) & 31));
+            } else if (KIND == 4) out[r / 8] |= code << (4 * (r % 8));
             else out[r / 4] |= code << (8 * (r % 4));
         }
         if (live) {
             const int64_t col = c * VW + k;
-            if (KIND == 4) {
+            if (code_bits<KIND>() == 6) {
+                u32x2* dst = reinterpret_cast<u32x2*>(codes + ((pre_i * C + col) * R + tile_i * ROWS) / 4 * 3);
+                dst[0] = u32x2{out[0], out[1]};
+                dst[1] = u32x2{out[2], out[3]};
+                dst[2] = u32x2{out[4], out[5]};
+            } else if (KIND == 4) {
                 *reinterpret_cast<u32x4*>(codes + ((pre_i * C + col) * R + tile_i * ROWS) / 2) =
                     u32x4{out[0], out[1], out[2], out[3]};
             } else {
@@ -170,7 +209,12 @@ __global__ __launch_bounds__(TPB) void mx_unpack_kernel(const unsigned char* __r
     for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (int64_t)gridDim.x * TPB) {
         const uint32_t s = scales[i >> 5];
         float y;
-        if (KIND == 4) y = mxq_decode_e2m1((codes[i >> 1] >> (4 * (i & 1))) & 15u);
+        if (code_bits<KIND>() == 6) {
+            const int64_t bit = 6 * i;
+            const uint32_t two = codes[bit >> 3] | ((uint32_t)codes[(bit >> 3) + ((bit & 7) > 2)] << 8);
+            const uint32_t c6 = (two >> (bit & 7)) & 63u;
+            y = (KIND == 2) ? mxq_decode_fp6<3, 1>(c6) : mxq_decode_fp6<2, 3>(c6);
+        } else if (KIND == 4) y = mxq_decode_e2m1((codes[i >> 1] >> (4 * (i & 1))) & 15u);
         else y = (KIND == 1) ? mxq_decode_e5m2(codes[i]) : mxq_decode_e4m3(codes[i]);
         float v = y * ldexpf(1.0f, (int)s - 127);
         if (s == 255u) v = mxq_float(MXQ_QNAN_BITS);

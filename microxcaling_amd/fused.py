@@ -15,8 +15,8 @@ _PACKABLE = (ElemFormat.fp8_e4m3, ElemFormat.fp8_e5m2, ElemFormat.fp6_e3m2, Elem
              ElemFormat.fp4)
 GEMM_K_MULTIPLE = 128
 # kinds of element codes (include/mxq.h MXQ_CODES_*): e4m3 bytes, e5m2 bytes, e2m1 nibbles
-CODES_E4M3, CODES_E5M2, CODES_E2M1 = 0, 1, 4
-_FLAG_PACK_NIBBLES = 4
+CODES_E4M3, CODES_E5M2, CODES_E2M3, CODES_E3M2, CODES_E2M1 = 0, 1, 2, 3, 4
+_FLAG_PACK_NIBBLES, _FLAG_PACK_SIXBIT = 4, 8
 
 
 def _as_format(fmt):
@@ -26,18 +26,33 @@ def _as_format(fmt):
 
 
 def _code_kind(fmt, nibbles, who):
+    """`nibbles` = pack below 8 bits per element: fp4 as nibbles, fp6 as 6-bit codes."""
     if nibbles:
-        if fmt != ElemFormat.fp4:
-            raise RuntimeError("%s: only fp4 elements pack into nibbles (got %s)" % (who, fmt))
-        return CODES_E2M1
+        if fmt == ElemFormat.fp4:
+            return CODES_E2M1
+        if fmt in (ElemFormat.fp6_e2m3, ElemFormat.fp6_e3m2):
+            return CODES_E2M3 if fmt == ElemFormat.fp6_e2m3 else CODES_E3M2
+        raise RuntimeError("%s: only fp4 elements pack into nibbles and fp6 elements into 6-bit "
+                           "codes (got %s)" % (who, fmt))
     return CODES_E5M2 if fmt == ElemFormat.fp8_e5m2 else CODES_E4M3
+
+
+def _code_bytes(K, kind):
+    """Bytes of codes for K elements of a row."""
+    kind = int(kind)
+    return K // 2 if kind == CODES_E2M1 else K * 3 // 4 if kind in (CODES_E2M3, CODES_E3M2) else K
+
+
+def _pack_flag(kind):
+    return _FLAG_PACK_NIBBLES if kind == CODES_E2M1 else \
+        _FLAG_PACK_SIXBIT if kind in (CODES_E2M3, CODES_E3M2) else 0
 
 
 def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=False, nibbles=False):
     """MX-quantize A along its last axis (block 32) into (codes, scales, code_kind): codes uint8 of
-    A's shape (one e4m3 / e5m2 byte per element) or, with nibbles=True (fp4 only), of half the last
-    axis (two e2m1 codes per byte, the lower index in the low nibble); scales uint8 with the last
-    axis divided by 32."""
+    A's shape (one e4m3 / e5m2 byte per element) or, with nibbles=True, of half the last axis for
+    fp4 (two e2m1 codes per byte, the lower index in the low nibble) and of 3/4 of it for fp6 (6-bit
+    codes as a little-endian bit stream); scales uint8 with the last axis divided by 32."""
     who = "pack_mx"
     fmt = _as_format(elem_format)
     if fmt not in _PACKABLE:
@@ -51,14 +66,14 @@ def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=F
         raise RuntimeError("%s: the last axis must be a multiple of 32" % who)
     ebits, mbits, _, max_norm, _ = _get_format_params(fmt)
     rows = A.numel() // K if K else 0
-    codes = torch.empty(A.shape[:-1] + (K // 2 if nibbles else K,), dtype=torch.uint8, device=A.device)
+    codes = torch.empty(A.shape[:-1] + (_code_bytes(K, kind),), dtype=torch.uint8, device=A.device)
     scales = torch.empty(A.shape[:-1] + (K // 32,), dtype=torch.uint8, device=A.device)
     lib = _lib.gpu()
     with torch.cuda.device(A.device):
         rc = lib.mxq_pack_mx(A.data_ptr(), codes.data_ptr(), scales.data_ptr(), _DTYPE[A.dtype],
                              rows, K, scale_bits, ebits, mbits, max_norm,
                              int(bool(flush_fp32_subnorms)), int(RoundingMode[round]),
-                             _flags_value() | (_FLAG_PACK_NIBBLES if nibbles else 0), _stream(A))
+                             _flags_value() | _pack_flag(kind), _stream(A))
     _lib.check(rc, lib)
     return codes, scales, kind
 
@@ -83,14 +98,14 @@ def pack_mx_t(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms
                            "last one of 8 bytes" % (who, tuple(A.shape)))
     ebits, mbits, _, max_norm, _ = _get_format_params(fmt)
     batch = A.numel() // (R * C) if R * C else 0
-    codes = torch.empty(A.shape[:-2] + (C, R // 2 if nibbles else R), dtype=torch.uint8, device=A.device)
+    codes = torch.empty(A.shape[:-2] + (C, _code_bytes(R, kind)), dtype=torch.uint8, device=A.device)
     scales = torch.empty(A.shape[:-2] + (C, R // 32), dtype=torch.uint8, device=A.device)
     lib = _lib.gpu()
     with torch.cuda.device(A.device):
         rc = lib.mxq_pack_mx_t(A.data_ptr(), codes.data_ptr(), scales.data_ptr(), _DTYPE[A.dtype],
                                batch, R, C, scale_bits, ebits, mbits, max_norm,
                                int(bool(flush_fp32_subnorms)), int(RoundingMode[round]),
-                               _flags_value() | (_FLAG_PACK_NIBBLES if nibbles else 0), _stream(A))
+                               _flags_value() | _pack_flag(kind), _stream(A))
     _lib.check(rc, lib)
     return codes, scales, kind
 
@@ -98,7 +113,7 @@ def pack_mx_t(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms
 def _packed_k(codes, scales, kind, who):
     """Length of the quantized axis of a packed tensor, after checking that codes and scales fit."""
     K = scales.shape[-1] * 32
-    if codes.shape[:-1] != scales.shape[:-1] or codes.shape[-1] != (K // 2 if int(kind) == CODES_E2M1 else K):
+    if codes.shape[:-1] != scales.shape[:-1] or codes.shape[-1] != _code_bytes(K, kind):
         raise RuntimeError("%s: codes %s and scales %s do not belong together (code kind %d)"
                            % (who, tuple(codes.shape), tuple(scales.shape), int(kind)))
     return K

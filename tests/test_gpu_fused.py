@@ -191,7 +191,7 @@ def test_nibble_pack_is_the_fake_quantized_tensor(dev, rnd, dtype):
     got = unpack_mx(codes, scales, kind, dtype).transpose(-1, -2).contiguous()
     assert_bits_equal(got, want_t, "nibbles, transposed")
     with pytest.raises(RuntimeError, match="nibbles"):
-        pack_mx(x.to(dev), "fp6_e2m3", nibbles=True)
+        pack_mx(x.to(dev), "fp8_e4m3", nibbles=True)
 
 
 @pytest.mark.parametrize("M,N,K,batch", [(128, 128, 256, 1), (100, 72, 256, 1), (130, 257, 768, 3),
@@ -733,3 +733,47 @@ def test_gemm_split_k_is_used_and_optional(dev):
     torch.cuda.synchronize()
     assert rel_err(split, plain) < 1e-4
 
+
+
+@pytest.mark.parametrize("fmt", ["fp6_e2m3", "fp6_e3m2"])
+@pytest.mark.parametrize("rnd", ["nearest", "floor", "even"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_sixbit_pack_is_the_fake_quantized_tensor(dev, fmt, rnd, dtype):
+    """fp6 elements as 6-bit codes (four in three bytes, little-endian bit stream): unpacking gives
+    the oracle's _quantize_mx output bit for bit, for the row-wise and for the transposing pack, and
+    the codes are those of the byte form."""
+    from microxcaling_amd.fused import pack_mx, pack_mx_t, unpack_mx, CODES_E2M3, CODES_E3M2
+    g = torch.Generator().manual_seed(78)
+    x = torch.randn(96, 256, generator=g) * torch.exp(3 * torch.randn(96, 256, generator=g))
+    x[3, 40] = float("inf")
+    x[5, 70] = float("nan")
+    x[7, :64] *= 1e-38
+    x[9, :32] = 0.0
+    x[11, :32] = -1e-30 * torch.rand(32, generator=g)
+    x = x.to(dtype)
+    want = O.quantize_mx(x, 8, fmt, axes=[-1], block_size=32, round=rnd)
+    codes, scales, kind = pack_mx(x.to(dev), fmt, 8, rnd, nibbles=True)
+    assert codes.shape == (96, 192) and scales.shape == (96, 8)
+    assert kind == (CODES_E2M3 if fmt == "fp6_e2m3" else CODES_E3M2)
+    assert_bits_equal(unpack_mx(codes, scales, kind, dtype), want, "6-bit codes")
+    # the bit stream, decoded on the host, against the values of the byte codes at scale 1
+    bytes_, scales8, kind8 = pack_mx(x.to(dev), fmt, 8, rnd)
+    assert torch.equal(scales8, scales)
+    elems = unpack_mx(bytes_, torch.full_like(scales8, 127), kind8, torch.float32).cpu()
+    raw = codes.cpu().numpy().astype("uint64").reshape(96, 64, 3)
+    word = raw[..., 0] | (raw[..., 1] << 8) | (raw[..., 2] << 16)                 # four elements per 24 bits
+    import numpy as np
+    c6 = torch.from_numpy(((word[..., None] >> (6 * np.arange(4, dtype="uint64"))) & 63).astype("int64")).reshape(96, 256)
+    mant, bias = (3, 1) if fmt == "fp6_e2m3" else (2, 3)
+    e, m, s = (c6 >> mant) & ((1 << (5 - mant)) - 1), c6 & ((1 << mant) - 1), (c6 >> 5) & 1
+    val = torch.where(e > 0, ((1 << mant) + m).double() * torch.exp2((e - bias - mant).double()),
+                      m.double() * 2.0 ** (1 - bias - mant))
+    val = torch.where(s == 1, -val, val).float()
+    finite = (scales8 != 255).repeat_interleave(32, dim=-1).cpu()
+    assert torch.equal(val[finite], elems[finite])
+    # transposing pack
+    want_t = O.quantize_mx(x, 8, fmt, axes=[-2], block_size=32, round=rnd)
+    codes, scales, kind = pack_mx_t(x.to(dev), fmt, 8, rnd, nibbles=True)
+    assert codes.shape == (256, 72) and scales.shape == (256, 3)
+    got = unpack_mx(codes, scales, kind, dtype).transpose(-1, -2).contiguous()
+    assert_bits_equal(got, want_t, "6-bit codes, transposed")
