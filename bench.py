@@ -97,7 +97,8 @@ def make_workload(name):
         return dict(x=x, gpu=fn, cpu=cpu, bytes=x.numel() * 4, dtype="f32", sample_axis=0 if dim == -1 else 1,
                     launches=1 if dim == -1 else 2,
                     desc="reduce %s over axis %d, fp32 [16384,8192]" % (op, dim))
-    if name in ("mx_linear", "mx_linear_unfused", "mx_linear_fp4", "mx_linear_fp4_unfused"):
+    if name in ("mx_linear", "mx_linear_unfused", "mx_linear_fp4", "mx_linear_fp4_unfused",
+                "mx_linear_fp6", "mx_linear_fp6_unfused"):
         # config 4: mx.Linear forward, MXFP8 e4m3 (or MXFP4 e2m1) both operands, block 32 along K, bias
         from microxcaling_amd import gemm
         from microxcaling_amd.linear import linear
@@ -107,7 +108,7 @@ def make_workload(name):
         x = torch.randn(M, K, generator=g).to(torch.bfloat16)
         w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
         b = torch.randn(N, generator=g).to(torch.bfloat16)
-        ef = "fp4_e2m1" if "fp4" in name else "fp8_e4m3"
+        ef = "fp4_e2m1" if "fp4" in name else "fp6_e2m3" if "fp6" in name else "fp8_e4m3"
         specs = finalize_mx_specs({"w_elem_format": ef, "a_elem_format": ef, "block_size": 32})
         dev_extra = {}
         fused = not name.endswith("_unfused")
@@ -119,9 +120,9 @@ def make_workload(name):
             return linear(xd, dev_extra["w"], dev_extra["b"], mx_specs=specs)
         return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, ef, ef),
                     flops=2.0 * M * N * K, bytes=0, dtype="%s x %s -> f32 acc" % (ef, ef), sample_axis=0,
-                    cpu_rows=1024, launches=5, peak="fp4" if ef == "fp4_e2m1" else "fp8",
+                    cpu_rows=1024, launches=5, peak="fp4" if ef == "fp4_e2m1" else "fp8",   # fp6 runs on byte codes: fp8 rate
                     desc="mx.Linear forward: x bf16 [16384,4096], W bf16 [14336,4096] ~N(0,0.02), bias; %s "
-                         "block 32 along K, %s" % ("MXFP4 e2m1" if ef == "fp4_e2m1" else "MXFP8 e4m3",
+                         "block 32 along K, %s" % ({"fp4_e2m1": "MXFP4 e2m1", "fp6_e2m3": "MXFP6 e2m3"}.get(ef, "MXFP8 e4m3"),
                                                    ("packed codes + scaled-MFMA GEMM" if fused else
                                                     "fake-quantize kernels + torch (hipBLASLt) bf16 GEMM")))
     if name in ("mx_linear_train", "mx_linear_train_unfused"):
@@ -336,7 +337,8 @@ def cpu_baseline(wl, budget_s=15.0):
                          torch.__version__, cores)}
 
 
-# MI355X dense MFMA peaks, published: fp8 (e4m3 / e5m2 byte codes) and fp4 (e2m1 nibble codes)
+# MI355X dense MFMA peaks, published: fp8 (e4m3 / e5m2 byte codes, which also carry fp6 elements) and
+# fp4 (e2m1 nibble codes)
 MFMA_PEAK_TFLOPS = {"fp8": 5000.0, "fp4": 10100.0}
 
 

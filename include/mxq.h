@@ -207,7 +207,8 @@ int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t 
 /* C[b] (M, N) = A[b] (M, K) x B[b] (N, K)^T for b < batch, all tensors contiguous, fp32
  * accumulation on the scaled MFMA units; c_dtype is a MXQ_DTYPE_* code.  a_kind, b_kind:
  * MXQ_CODES_* of the operands; e4m3 and e5m2 bytes mix freely (K % 128 == 0), e2m1 nibbles need both
- * operands in that form (K % 256 == 0) and run at the 4-bit MFMA rate.
+ * operands in that form (K % 256 == 0) and run at the 4-bit MFMA rate.  6-bit codes (e2m3, e3m2)
+ * are a storage form only: the call rejects them, fp6 operands come as byte codes.
  * bias (optional, may be NULL): N values of dtype c_dtype; then C = round(round(A x B^T) + bias),
  * both roundings to c_dtype, which is what "matmul, then add the bias" gives as tensor ops.
  * epilogue_quant = 1 (bf16 C only): additionally apply the elementwise quantization of the layers

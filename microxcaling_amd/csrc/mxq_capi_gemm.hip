@@ -229,6 +229,10 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const 
         return fail(MXQ_ERR_ARGUMENT, "%s: epilogue_quant must be 0, or 1 with a bf16 output", who);
     if (batch < 0 || M < 0 || N < 0 || K < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
     const bool nib = a_kind == MXQ_CODES_E2M1;
+    auto sixbit = [](int kind) { return kind == MXQ_CODES_E2M3 || kind == MXQ_CODES_E3M2; };
+    if (sixbit(a_kind) || sixbit(b_kind))
+        return fail(MXQ_ERR_ARGUMENT, "%s: 6-bit codes are a storage form; the GEMM takes fp6 operands as "
+                    "byte codes (mxq_pack_mx without MXQ_FLAG_PACK_SIXBIT)", who);
     if ((a_kind != MXQ_CODES_E4M3 && a_kind != MXQ_CODES_E5M2 && a_kind != MXQ_CODES_E2M1) ||
         (b_kind != MXQ_CODES_E4M3 && b_kind != MXQ_CODES_E5M2 && b_kind != MXQ_CODES_E2M1))
         return fail(MXQ_ERR_ARGUMENT, "%s: unknown code kind %d / %d", who, a_kind, b_kind);
