@@ -395,7 +395,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: the quantization path has no multi-GPU part "
-                         "(blocks are independent; see DESIGN.md); run with --gpus 1")
+                         "(blocks are independent, so sharding needs no exchange step); run with --gpus 1")
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
 

@@ -4,36 +4,76 @@
 
 namespace {
 
+// max_code != 0: the element format is the format of the codes, which then come straight from the
+// rounded significands (mx_code_of); the round-up-zone variants always take the generic way
 template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchPack {
-    static void run(const void* in, void* codes, void* scales, int64_t n_vec, int kind, MxParams p,
-                    hipStream_t s) {
+    template <int KIND>
+    static void one(int grid, const u32x4* in, void* codes, unsigned char* sc, int64_t n_vec, MxParams p,
+                    uint32_t max_code, hipStream_t s) {
+        if constexpr (!ZE) {
+            if (max_code != 0u) {
+                mx_pack_kernel<DT, RMODE, ZE, KIND, 4, true><<<grid, kThreads, 0, s>>>(in, codes, sc, n_vec, p, max_code);
+                return;
+            }
+        }
+        mx_pack_kernel<DT, RMODE, ZE, KIND, 4, false><<<grid, kThreads, 0, s>>>(in, codes, sc, n_vec, p, 0u);
+    }
+    static void run(const void* in, void* codes, void* scales, int64_t n_vec, int kind, uint32_t max_code,
+                    MxParams p, hipStream_t s) {
         const int grid = grid_for(ceil_div(n_vec, (int64_t)kThreads * 4));
         const u32x4* i4 = reinterpret_cast<const u32x4*>(in);
         unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
-        if (kind == 1) mx_pack_kernel<DT, RMODE, ZE, 1, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
-        else if (kind == 2) mx_pack_kernel<DT, RMODE, ZE, 2, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
-        else if (kind == 3) mx_pack_kernel<DT, RMODE, ZE, 3, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
-        else if (kind == 4) mx_pack_kernel<DT, RMODE, ZE, 4, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
-        else mx_pack_kernel<DT, RMODE, ZE, 0, 4><<<grid, kThreads, 0, s>>>(i4, codes, sc, n_vec, p);
+        if (kind == 1) one<1>(grid, i4, codes, sc, n_vec, p, max_code, s);
+        else if (kind == 2) one<2>(grid, i4, codes, sc, n_vec, p, max_code, s);
+        else if (kind == 3) one<3>(grid, i4, codes, sc, n_vec, p, max_code, s);
+        else if (kind == 4) one<4>(grid, i4, codes, sc, n_vec, p, max_code, s);
+        else one<0>(grid, i4, codes, sc, n_vec, p, max_code, s);
     }
 };
 
 template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchPackT {
+    template <int KIND>
+    static void one(unsigned grid, const u32x2* in, unsigned char* c, unsigned char* sc, int64_t items,
+                    int64_t n_tiles, int64_t pv, MxParams p, uint32_t max_code, hipStream_t s) {
+        if constexpr (!ZE) {
+            if (max_code != 0u) {
+                mx_pack_t_kernel<DT, RMODE, ZE, KIND, true><<<grid, kThreads, 0, s>>>(in, c, sc, items, n_tiles, pv, p, max_code);
+                return;
+            }
+        }
+        mx_pack_t_kernel<DT, RMODE, ZE, KIND, false><<<grid, kThreads, 0, s>>>(in, c, sc, items, n_tiles, pv, p, 0u);
+    }
     static void run(const void* in, void* codes, void* scales, int64_t items, int64_t n_tiles,
-                    int64_t pv, int kind, MxParams p, hipStream_t s) {
+                    int64_t pv, int kind, uint32_t max_code, MxParams p, hipStream_t s) {
         const unsigned grid = (unsigned)ceil_div(items, kThreads);
         const u32x2* i2 = reinterpret_cast<const u32x2*>(in);
         unsigned char* c = reinterpret_cast<unsigned char*>(codes);
         unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
-        if (kind == 1) mx_pack_t_kernel<DT, RMODE, ZE, 1><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
-        else if (kind == 2) mx_pack_t_kernel<DT, RMODE, ZE, 2><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
-        else if (kind == 3) mx_pack_t_kernel<DT, RMODE, ZE, 3><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
-        else if (kind == 4) mx_pack_t_kernel<DT, RMODE, ZE, 4><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
-        else mx_pack_t_kernel<DT, RMODE, ZE, 0><<<grid, kThreads, 0, s>>>(i2, c, sc, items, n_tiles, pv, p);
+        if (kind == 1) one<1>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
+        else if (kind == 2) one<2>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
+        else if (kind == 3) one<3>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
+        else if (kind == 4) one<4>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
+        else one<0>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
     }
 };
+
+// max_code for the direct form, or 0: the element format must be the one the code kind stores
+uint32_t direct_max_code(int kind, int ebits, int mbits, const MxParams& p) {
+    const bool same = (kind == MXQ_CODES_E4M3 && ebits == 4 && mbits == 5) ||
+                      (kind == MXQ_CODES_E5M2 && ebits == 5 && mbits == 4) ||
+                      (kind == MXQ_CODES_E2M3 && ebits == 2 && mbits == 5) ||
+                      (kind == MXQ_CODES_E3M2 && ebits == 3 && mbits == 4) ||
+                      (kind == MXQ_CODES_E2M1 && ebits == 2 && mbits == 3);
+    if (!same) return 0u;
+    const uint32_t mc = mxq_max_code(p.fmt);
+    const uint32_t top = (1u << (kind == MXQ_CODES_E2M1 ? 3 : kind >= MXQ_CODES_E2M3 ? 5 : 7)) - 1u;
+    // e4m3 keeps its last code for NaN, e5m2 its last exponent for Inf / NaN: a max_norm beyond the
+    // largest finite code means a non-standard format
+    const uint32_t finite = kind == MXQ_CODES_E4M3 ? 0x7Eu : kind == MXQ_CODES_E5M2 ? 0x7Bu : top;
+    return mc <= finite ? mc : 0u;
+}
 
 // The persistent 256 x 256 tile kernel serves products with enough tiles to occupy half the CUs;
 // below that the small tiles, with K split, are two to five times faster (512 x 4096 x 8192: 329 ->
@@ -160,7 +200,7 @@ int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t ro
     if (!aligned16(in) || !aligned16(codes))
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
     dispatch<LaunchPack>(dtype, rmode, ze, true, in, codes, scales, total / (16 / elem_size(dtype)), kind,
-                         p, (hipStream_t)hip_stream);
+                         direct_max_code(kind, elem_ebits, elem_mbits, p), p, (hipStream_t)hip_stream);
     return check_launch(who);
 }
 
@@ -187,8 +227,8 @@ int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t 
         return fail(MXQ_ERR_ARGUMENT, "%s: input must be 8-byte and codes 16-byte aligned", who);
     const int64_t n_tiles = R / 32, pv = C / vw, items = batch * n_tiles * pv;
     if (ceil_div(items, kThreads) > 0x7FFFFFFF) return fail(MXQ_ERR_ARGUMENT, "%s: tensor too large", who);
-    dispatch<LaunchPackT>(dtype, rmode, ze, true, in, codes, scales, items, n_tiles, pv, kind, p,
-                          (hipStream_t)hip_stream);
+    dispatch<LaunchPackT>(dtype, rmode, ze, true, in, codes, scales, items, n_tiles, pv, kind,
+                          direct_max_code(kind, elem_ebits, elem_mbits, p), p, (hipStream_t)hip_stream);
     return check_launch(who);
 }
 

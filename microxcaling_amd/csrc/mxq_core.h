@@ -229,6 +229,44 @@ MXQ_HD float mxq_quant_mx_elem_unscaled(float x, const MxqScale& sc, const MxqFm
     return mxq_round_lean<RMODE, ZONE>(a, mxq_sign_source<DT>(a), f, true, zone, zshift);
 }
 
+// The same element as the code of its own format, without the detour over the float value: with
+// k = the rounded significand at exponent e (mxq_round_lean's r and ebc), the magnitude code is
+// ((e - min_exp) << t) + k -- for subnormals (e = min_exp, k < 2^t) that is k, for normals the
+// implicit one of k adds 1 to the exponent field, and a k that rounded up to 2^(t+1) carries into
+// the next exponent.  Codes grow with the magnitude, so saturation is a clamp of the code at
+// max_code, the code of max_norm.  SIGN_POS: bit of the sign in the code.  Not for the round-up
+// zone variant (there e can exceed the exponent of the value).  NaN inputs give an arbitrary code
+// (their block's scale byte says NaN).
+template <int RMODE, int DT, int SIGN_POS>
+MXQ_HD uint32_t mxq_quant_mx_code(float x, const MxqScale& sc, const MxqFmt& f, uint32_t max_code) {
+    const float a = x * sc.inv_scale;
+    const uint32_t ua = mxq_bits(a) & 0x7FFFFFFFu;
+    const uint32_t eb = ua >> 23;
+    const uint32_t ebc = eb > f.min_eb ? eb : f.min_eb;
+    const float s = ldexpf(mxq_float(ua), f.t127 - (int)ebc);   // exact
+    float r;
+    if (RMODE == MXQ_FLOOR) {
+        r = floorf(s);
+    } else if (RMODE == MXQ_NEAREST) {
+        r = floorf(s + f.half);
+    } else {
+        r = __builtin_rintf(s);
+        r = (s == f.tie_fix) ? 1.0f : r;
+    }
+    uint32_t mag = ((ebc - f.min_eb) << f.t) + (uint32_t)r;
+    mag = mag < max_code ? mag : max_code;
+    return mag | ((mxq_bits(mxq_sign_source<DT>(a)) >> 31) << SIGN_POS);
+}
+
+// max_code of the above for a format whose max_norm is one of its own values; 0 otherwise (then
+// the caller rounds to the float value and encodes that)
+inline uint32_t mxq_max_code(const MxqFmt& f) {
+    if (f.ebits == 0 || f.t > 22) return 0u;
+    const uint32_t eb = f.max_bits >> 23, frac = f.max_bits & 0x7FFFFFu;
+    if (eb < f.min_eb || eb >= 255u || (frac & ((1u << (23 - f.t)) - 1u)) != 0u) return 0u;
+    return ((eb - f.min_eb) << f.t) + (1u << f.t) + (frac >> (23 - f.t));
+}
+
 // OCP 8-bit float codes of a value that is exactly representable in the format (no rounding
 // happens here).  e4m3 is the "fn" variant: bias 7, subnormals m * 2^-9, no infinities.
 MXQ_HD uint32_t mxq_encode_e4m3(float y) {

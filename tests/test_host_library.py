@@ -285,3 +285,22 @@ def test_shared_exp_method_none_is_block_of_one():
     a = _quantize_mx(x, 8, "fp8_e4m3", shared_exp_method="none", axes=[-1], block_size=4)
     b = O.quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=1)
     assert_bits_equal(a, b)
+
+
+def test_direct_pack_codes_equal_the_encoded_rounded_values(tmp_path):
+    """The pack kernels' shortcut (code from the rounded significand, no float value in between)
+    against the long way, on the host, for all five code formats x fp32 / bf16 tensors x rounding
+    modes: tests/cpp/pack_code_check.cpp exits non-zero on the first mismatch."""
+    import shutil
+    import subprocess
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        pytest.skip("no host C++ compiler")
+    exe = str(tmp_path / "pack_code_check")
+    subprocess.run([cxx, "-O2", "-std=c++17", "-ffp-contract=off", "-I", os.path.join(ROOT_DIR, "include"),
+                    "-I", os.path.join(ROOT_DIR, "microxcaling_amd", "csrc"), "-o", exe,
+                    os.path.join(ROOT_DIR, "tests", "cpp", "pack_code_check.cpp")], check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True, timeout=300).stdout
+    assert out.count("inputs agree") == 30 and "MISMATCH" not in out
+    # nearest and even are served by the shortcut (floor takes the round-up-zone variant)
+    assert out.count("zone variant") == 10
