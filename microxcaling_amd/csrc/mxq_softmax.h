@@ -1,6 +1,8 @@
 // Softmax over the last axis with an elementwise quantization after every step
 // (mx/softmax.py:20-54 over mx/vector_ops.py:38-130): one kernel instead of ten tensor passes.
 #pragma once
+#include <type_traits>
+
 #include "mxq_kernels.h"
 
 struct SoftmaxParams {
@@ -39,6 +41,13 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
                                                           p.q.allow_denorm != 0, zone, ZS);
     };
     auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
+    // SMQ_BF16, values known to be +0 or normal and far from the top binade: the closed form without
+    // its special cases
+    auto Qplain_d = [](float v) {                            // v already is a value of the tensor dtype
+        const uint32_t u = mxq_bits(v);
+        return mxq_float(u + (u & 0x10000u));
+    };
+    auto Qplain = [&](float v) { return Qplain_d(mxq_round_dt<ADT>(v)); };
 
     // the quantizer for exponentials, their row sum and the quotients: all >= +0 and <= 4096 (or
     // NaN / +Inf), where the closed form needs no special cases
@@ -68,6 +77,13 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
         // contribute exp(-inf) = 0 to the sum
         float x[EPL];
         float m = -__builtin_inff();
+        // SMQ_BF16: the special cases of the quantizer (zero, subnormal, Inf, NaN, top binade) cost
+        // more than its arithmetic, and rows of logits rarely hold any.  A wave whose inputs all lie
+        // in 2^-100 <= |x| < 2^100 quantizes them with the plain closed form; if the row maximum
+        // lies there too, every x - m is +0 or a normal number below 2^101 (a multiple of 2^-108),
+        // and so is 1.4453125 (x - m): the plain form again.  Any other wave takes the general form.
+        bool plain = QMODE == SMQ_BF16;
+        auto in_plain_range = [](uint32_t ua) { return ua - 0x0D800000u < 0x64000000u; };   // [2^-100, 2^100)
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
             const bool valid = j * LPR + lane < nvec;
@@ -76,32 +92,58 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
 #pragma unroll
                 for (int h = 0; h < PD; ++h) {
                     const int e = (j * 4 + d) * PD + h;
-                    x[e] = valid ? Qd(Pack<DT>::get(raw[j][d], h)) : -__builtin_inff();
-                    m = MaxOp::apply(m, x[e]);                 // NaN sticks, like torch.max
+                    const float v = Pack<DT>::get(raw[j][d], h);
+                    if (QMODE == SMQ_BF16) {
+                        plain = plain && (!valid || in_plain_range(mxq_bits(v) & 0x7FFFFFFFu));
+                        x[e] = valid ? Qplain_d(v) : -__builtin_inff();
+                    } else {
+                        x[e] = valid ? Qd(v) : -__builtin_inff();
+                    }
                 }
         }
-        m = row_reduce<MaxOp, WPR>(m, part);
-
-        float sum = 0.0f;
-        if (p.exp_mode == 0) {                               // one loop per mode: no branch per element
+        if (QMODE == SMQ_BF16) {
+            plain = __all(plain);                            // wave-uniform from here on
+            if (!plain) {
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                x[e] = Qp(expf(Q(x[e] - m)));
-                sum += x[e];
-            }
-        } else if (p.exp_mode == 1) {
+                for (int j = 0; j < VPL; ++j)
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                x[e] = Qp(exp2f(Q(x[e] - m)));
-                sum += x[e];
-            }
-        } else {
+                    for (int d = 0; d < 4; ++d)
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) {
-                x[e] = Qp(exp2f(Q(1.4453125f * Q(x[e] - m))));
-                sum += x[e];
+                        for (int h = 0; h < PD; ++h)
+                            if (j * LPR + lane < nvec) x[(j * 4 + d) * PD + h] = Qd(Pack<DT>::get(raw[j][d], h));
             }
         }
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) m = MaxOp::apply(m, x[e]);     // NaN sticks, like torch.max
+        m = row_reduce<MaxOp, WPR>(m, part);
+        // m is the same in every lane of the row; the vote makes the branch below a scalar one
+        if (QMODE == SMQ_BF16) plain = __all(plain && in_plain_range(mxq_bits(m) & 0x7FFFFFFFu));
+
+        float sum = 0.0f;
+        auto exponentials = [&](auto plain_tag) {            // one loop per mode: no branch per element
+            auto Qs = [&](float v) { return decltype(plain_tag)::value ? Qplain(v) : Q(v); };
+            if (p.exp_mode == 0) {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    x[e] = Qp(expf(Qs(x[e] - m)));
+                    sum += x[e];
+                }
+            } else if (p.exp_mode == 1) {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    x[e] = Qp(exp2f(Qs(x[e] - m)));
+                    sum += x[e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    x[e] = Qp(exp2f(Qs(1.4453125f * Qs(x[e] - m))));
+                    sum += x[e];
+                }
+            }
+        };
+        if (QMODE == SMQ_BF16 && plain) exponentials(std::true_type{});
+        else exponentials(std::false_type{});
         sum = Qp(row_reduce<SumOp, WPR>(sum, part));
         const bool recip = p.use_recip != 0;
         const float r = recip ? Qp(1.0f / sum) : 0.0f;

@@ -376,6 +376,50 @@ def test_fused_softmax_special_rows(dev):
     assert (got[ok] - want[ok]).abs().max() <= 2.0 ** -8
 
 
+@pytest.mark.parametrize("shape", [(64, 2048), (9, 264), (6, 8192), (5, 16384)])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, softmax_exp2=True),
+                                  dict(bfloat=16, vec_use_exp2=True, vec_use_recip=True)])
+def test_fused_softmax_plain_and_general_forms_agree(dev, shape, spec):
+    """bf16 rows whose values all lie in [2^-100, 2^100) are quantized without the special cases of
+    the closed form; any other row takes the general form.  A row with one entry at -200 and the
+    same row with -inf there must come out bit-identical: both entries weigh exactly 0, and only
+    the second row holds a special value."""
+    from microxcaling_amd.softmax import softmax
+    g = torch.Generator().manual_seed(shape[1])
+    x = (torch.randn(*shape, generator=g) * 3).to(torch.bfloat16)
+    x[x == 0] = 1.0
+    y = x.clone()
+    cols = torch.arange(shape[0]) * 37 % shape[1]
+    x[torch.arange(shape[0]), cols] = -200.0
+    y[torch.arange(shape[0]), cols] = float("-inf")
+    specs = _specs(**spec)
+    got_plain = softmax(x.to(dev), dim=-1, mx_specs=specs).cpu()
+    got_general = softmax(y.to(dev), dim=-1, mx_specs=specs).cpu()
+    assert (got_plain[torch.arange(shape[0]), cols] == 0).all()
+    assert torch.equal(got_plain.view(torch.int16), got_general.view(torch.int16))
+
+
+def test_fused_softmax_bf16_rows_outside_the_plain_range(dev):
+    """Huge, tiny, zero and subnormal bf16 logits against the chain of tensor ops."""
+    from microxcaling_amd.softmax import softmax
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(8, 256, generator=g).to(torch.bfloat16)
+    x[0, 3] = 2.0 ** 101                                 # maximum beyond the plain range
+    x[1] = x[1] * 2.0 ** -110                            # every entry below it
+    x[2, 10:20] = 0.0
+    x[3, 7] = -0.0
+    x[4, 5] = 2.0 ** -130                                # bf16 subnormal
+    x[5, ::2] = 2.0 ** 100
+    x[6] = x[6] * 2.0 ** 99
+    specs = _specs(bfloat=16)
+    got = softmax(x.to(dev), dim=-1, mx_specs=specs).cpu()
+    want = O.softmax_forward(x, -1, bfloat=16)
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    ok = ~torch.isnan(want)
+    assert (got[ok].float() - want[ok].float()).abs().max() <= 2.0 ** -8
+    assert got[0, 3] == 1 and got[0].float().sum() == 1
+
+
 def test_softmax_unfused_path_still_matches(dev):
     from microxcaling_amd import gemm
     from microxcaling_amd.softmax import softmax
