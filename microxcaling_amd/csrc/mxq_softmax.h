@@ -331,16 +331,29 @@ __global__ __launch_bounds__(TPB) void activation_kernel(const void* __restrict_
         return mxq_quant_elemwise<RMODE, ADT, true, true>(v, p.q.fmt, p.q.saturate != 0,
                                                           p.q.allow_denorm != 0, zone, ZS);
     };
-    auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
     const bool via_exp2 = p.exp_mode == 2;
-    auto logistic = [&](float y) {
-        const float t = -y;
-        const float e = via_exp2 ? Q(exp2f(Q(1.4453125f * t))) : Q(expf(t));
-        return Q(1.0f / Q(e + 1.0f));
-    };
-    // one element: result, logistic factor (silu, gelu), quantized input
-    auto eval = [&](float x, float& aux, float& q) {
-        q = Qd(x);
+    // one element: result, logistic factor (silu, gelu), quantized input.
+    // plain_tag (SMQ_BF16 only): the input lies in 2^-20 <= |x| < 8.  Every intermediate value of
+    // the five chains is then a normal number, neither zero nor near the top binade (|arguments of
+    // exp| < 50, so the exponentials lie in 4e-22 .. 3e21 and the logistic factor in 4e-22 .. 1;
+    // sums add numbers of the same sign), and the closed form of the quantizer needs none of its
+    // special cases, which cost four times its arithmetic.
+    auto eval = [&](auto plain_tag, float x, float& aux, float& q) {
+        constexpr bool PLAIN = decltype(plain_tag)::value;
+        auto Qd_ = [&](float v) {
+            if (PLAIN) {
+                const uint32_t u = mxq_bits(v);
+                return mxq_float(u + (u & 0x10000u));
+            }
+            return Qd(v);
+        };
+        auto Q = [&](float v) { return Qd_(mxq_round_dt<ADT>(v)); };
+        auto logistic = [&](float y) {
+            const float t = -y;
+            const float e = via_exp2 ? Q(exp2f(Q(1.4453125f * t))) : Q(expf(t));
+            return Q(1.0f / Q(e + 1.0f));
+        };
+        q = Qd_(x);
         aux = 0.0f;
         switch (p.act) {
             case ACT_SIGMOID: return logistic(q);
@@ -355,6 +368,7 @@ __global__ __launch_bounds__(TPB) void activation_kernel(const void* __restrict_
             }
         }
     };
+    auto in_plain_range = [](uint32_t ua) { return ua - 0x35800000u < 0x0B800000u; };   // [2^-20, 8)
 
     const u32x4* in = reinterpret_cast<const u32x4*>(in_);
     u32x4* out = reinterpret_cast<u32x4*>(out_);
@@ -365,15 +379,28 @@ __global__ __launch_bounds__(TPB) void activation_kernel(const void* __restrict_
     for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n_vec; i += stride) {
         const u32x4 v = in[i];
         u32x4 o, a, qv;
+        auto vector = [&](auto plain_tag) {
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            float r[2], ax[2], qq[2];
+            for (int d = 0; d < 4; ++d) {
+                float r[2], ax[2], qq[2];
 #pragma unroll
-            for (int h = 0; h < PD; ++h) r[h] = eval(Pack<DT>::get(v[d], h), ax[h], qq[h]);
-            o[d] = Pack<DT>::put(r[0], r[PD - 1]);
-            a[d] = Pack<DT>::put(ax[0], ax[PD - 1]);
-            qv[d] = Pack<DT>::put(qq[0], qq[PD - 1]);
+                for (int h = 0; h < PD; ++h) r[h] = eval(plain_tag, Pack<DT>::get(v[d], h), ax[h], qq[h]);
+                o[d] = Pack<DT>::put(r[0], r[PD - 1]);
+                a[d] = Pack<DT>::put(ax[0], ax[PD - 1]);
+                qv[d] = Pack<DT>::put(qq[0], qq[PD - 1]);
+            }
+        };
+        bool plain = QMODE == SMQ_BF16;
+        if (QMODE == SMQ_BF16) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+#pragma unroll
+                for (int h = 0; h < PD; ++h)
+                    plain = plain && in_plain_range(mxq_bits(Pack<DT>::get(v[d], h)) & 0x7FFFFFFFu);
+            plain = __all(plain);                            // one branch per wave
         }
+        if (QMODE == SMQ_BF16 && plain) vector(std::true_type{});
+        else vector(std::false_type{});
         __builtin_nontemporal_store(o, &out[i]);
         if (auxv) __builtin_nontemporal_store(a, &auxv[i]);
         if (qinv) __builtin_nontemporal_store(qv, &qinv[i]);
@@ -383,7 +410,7 @@ __global__ __launch_bounds__(TPB) void activation_kernel(const void* __restrict_
     const int64_t gi = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (gi < n - t0) {
         float ax, qq;
-        const float r = eval(load_scalar<DT>(in_, t0 + gi), ax, qq);
+        const float r = eval(std::false_type{}, load_scalar<DT>(in_, t0 + gi), ax, qq);
         store_scalar<DT>(out_, t0 + gi, mxq_round_dt<ADT>(r));
         if (aux_) store_scalar<DT>(aux_, t0 + gi, mxq_round_dt<ADT>(ax));
         if (qin_) store_scalar<DT>(qin_, t0 + gi, qq);

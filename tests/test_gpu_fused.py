@@ -571,6 +571,32 @@ def test_fused_activation_against_chain(dev, act, dtype, spec):
 
 
 @pytest.mark.parametrize("act", sorted(_ACTS))
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, vec_use_exp2=True)], ids=["exp", "exp2"])
+def test_fused_activation_plain_and_general_forms_agree(dev, act, spec):
+    """bf16 inputs with 2^-20 <= |x| < 8 are quantized without the special cases of the closed form,
+    wave by wave; one value outside that range sends its wave through the general form.  The
+    results of all other elements must not depend on which form their wave took."""
+    from microxcaling_amd import activations as A
+    specs = _specs(**spec)
+    g = torch.Generator().manual_seed(len(act))
+    n = 512 * 300
+    x = (torch.randn(n, generator=g) * 2.5).clamp(-7.9, 7.9)
+    x[x.abs() < 2.0 ** -19] = 0.5
+    x[:4096] = torch.exp2(torch.linspace(-19.9, 2.99, 4096)) * (1 - 2 * (torch.arange(4096) % 2))   # the whole range
+    x = x.to(torch.bfloat16)
+    assert ((x.float().abs() >= 2.0 ** -20) & (x.float().abs() < 8)).all()
+    y = x.clone()
+    hit = torch.arange(300) * 512 + torch.arange(300) * 7 % 512      # one per wave and iteration
+    y[hit] = torch.tensor([0.0, float("inf"), 100.0, 2.0 ** -30, -8.0, float("nan")]).to(torch.bfloat16).repeat(50)
+    got_plain = _ACTS[act](A, x.to(dev), specs).cpu()
+    got_general = _ACTS[act](A, y.to(dev), specs).cpu()
+    keep = torch.ones(n, dtype=torch.bool)
+    keep[hit] = False
+    assert torch.equal(got_plain[keep].view(torch.int16), got_general[keep].view(torch.int16))
+    _one_step_apart(got_plain, _ACTS[act](A, x, specs), 0.03)
+
+
+@pytest.mark.parametrize("act", sorted(_ACTS))
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_fused_activation_special_values(dev, act, dtype):
     from microxcaling_amd import activations as A
