@@ -10,6 +10,7 @@ HOST_LIB_PATH = os.path.join(PKG, "libmxq_host.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 FLAG_EXACT_EXPONENT = 1
+FLAG_GENERAL_FORM = 16
 HOST_FLAG_ROUND_EVERY_OP = 2
 
 _c_int, _c_i64, _c_f32, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p

@@ -28,6 +28,7 @@ struct ElemParams {
     int allow_denorm;
     int zone_row;
     int zshift;
+    int general_only;   // chain kernels: MXQ_FLAG_GENERAL_FORM
 };
 
 namespace mxq_detail {
@@ -141,6 +142,7 @@ inline int make_elem_params(int dtype, int bits, int exp_bits, float max_norm, i
     if (rc) return rc;
     p->saturate = saturate ? 1 : 0;
     p->allow_denorm = allow_denorm ? 1 : 0;
+    p->general_only = (flags & MXQ_FLAG_GENERAL_FORM) ? 1 : 0;
     zone_for(dtype, flags, &p->zone_row, &p->zshift);
     // the top binade's round-up zone: floor(log2|x|) = 128 there
     static const unsigned char top_count[3] = {zone_rows[0][276], zone_rows[1][276], 0};

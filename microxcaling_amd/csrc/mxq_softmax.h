@@ -82,7 +82,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
         // in 2^-100 <= |x| < 2^100 quantizes them with the plain closed form; if the row maximum
         // lies there too, every x - m is +0 or a normal number below 2^101 (a multiple of 2^-108),
         // and so is 1.4453125 (x - m): the plain form again.  Any other wave takes the general form.
-        bool plain = QMODE == SMQ_BF16;
+        bool plain = QMODE == SMQ_BF16 && !p.q.general_only;
         auto in_plain_range = [](uint32_t ua) { return ua - 0x0D800000u < 0x64000000u; };   // [2^-100, 2^100)
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
@@ -220,6 +220,26 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
                                                           p.q.allow_denorm != 0, zone, ZS);
     };
     auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
+    // SMQ_BF16: the closed form without its special cases, for values that are normal numbers far
+    // from the top binade, or zero (a -0 stays -0 here; see below where that can happen).  A wave
+    // uses it for the per-element steps of a row while everything those steps see lies in a range
+    // that keeps them there:
+    //   inputs 2^-20 <= |x| < 2^20 (every lane of the wave), |mean| < 2^21
+    //     => x - mean is +0 or at least 2^-35 in magnitude (both are multiples of 2^-35 when the
+    //        mean is not negligible), its square +0 or at least 2^-70;
+    //   2^-30 <= 1 / sqrt(var + eps) < 2^30 => the normalized value is +0 or within 2^-65 .. 2^51;
+    //   weights 2^-20 <= |w| < 2^20, bias +0 or 2^-40 <= |b| < 2^40 (this lane's columns)
+    //     => w z is normal or +-0, and w z + b is normal, +0 (exact cancellation), b or w z.  A -0
+    //        product (z = +0, w < 0) gives the same sum as the +0 the general form turns it into.
+    // The per-row scalars always take the general form.
+    auto Qplain_d = [](float v) {
+        const uint32_t u = mxq_bits(v);
+        return mxq_float(u + (u & 0x10000u));
+    };
+    auto Qplain = [&](float v) { return Qplain_d(mxq_round_dt<ADT>(v)); };
+    auto within = [](float v, uint32_t lo, uint32_t hi) {    // lo <= |v| < hi as bit patterns
+        return (mxq_bits(v) & 0x7FFFFFFFu) - lo < hi - lo;
+    };
 
     constexpr int LPR = 64 * WPR;                            // lanes per row
     constexpr int RPB = (TPB / 64) / WPR;                    // rows per block and iteration
@@ -228,12 +248,35 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
     const int lane = (wib % WPR) * 64 + (threadIdx.x & 63);  // lane within the row
     const int nvec_row = n / EPV;
     const float count = (float)n;
+    const u32x4* wv = reinterpret_cast<const u32x4*>(weight_);
+    const u32x4* bv = reinterpret_cast<const u32x4*>(bias_);
+
+    // this lane's columns are the same in every row: are their weights and biases in range?
+    bool wb_plain = QMODE == SMQ_BF16 && !p.q.general_only;
+    if (QMODE == SMQ_BF16) {
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const int v = j * LPR + lane;
+            if (v >= nvec_row) continue;
+            const u32x4 w4 = wv[v], b4 = bv[v];
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const float w = Pack<DT>::get(w4[d], h), b = Pack<DT>::get(b4[d], h);
+                    wb_plain = wb_plain && within(w, 0x35800000u, 0x49800000u) &&               // [2^-20, 2^20)
+                               (mxq_bits(b) == 0u || within(b, 0x2B800000u, 0x53800000u));      // +0, [2^-40, 2^40)
+                }
+        }
+        wb_plain = __all(wb_plain);
+    }
+
     for (int64_t row0 = (int64_t)blockIdx.x * RPB; row0 < rows; row0 += (int64_t)gridDim.x * RPB) {
         const int64_t row = row0 + wib / WPR;
         const int nvec = row < rows ? nvec_row : 0;          // a block's spare waves go through the motions
         const u32x4* in = reinterpret_cast<const u32x4*>(in_) + row * nvec_row;
         float x[EPL];
-        float sum = 0.0f;
+        bool plain = QMODE == SMQ_BF16 && !p.q.general_only;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
             const bool valid = j * LPR + lane < nvec;
@@ -244,51 +287,87 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
 #pragma unroll
                 for (int h = 0; h < PD; ++h) {
                     const int e = (j * 4 + d) * PD + h;
-                    x[e] = valid ? Qd(Pack<DT>::get(raw[d], h)) : 0.0f;   // zeros add nothing to the sums
-                    sum += p.rms ? 0.0f : x[e];
+                    const float v = Pack<DT>::get(raw[d], h);
+                    if (QMODE == SMQ_BF16) {
+                        plain = plain && (!valid || within(v, 0x35800000u, 0x49800000u));
+                        x[e] = valid ? Qplain_d(v) : 0.0f;   // zeros add nothing to the sums
+                    } else {
+                        x[e] = valid ? Qd(v) : 0.0f;
+                    }
                 }
         }
-        if (!p.rms) {
-            const float mean = Q(Q(row_reduce<SumOp, WPR>(sum, part)) / count);
+        if (QMODE == SMQ_BF16) {
+            plain = __all(plain);                            // wave-uniform from here on
+            if (!plain) {                                    // rare: read the row once more
 #pragma unroll
-            for (int j = 0; j < VPL; ++j) {
-                const bool valid = j * LPR + lane < nvec;
+                for (int j = 0; j < VPL; ++j) {
+                    if (j * LPR + lane >= nvec) continue;
+                    const u32x4 raw = in[j * LPR + lane];
 #pragma unroll
-                for (int k = 0; k < EPV; ++k) x[j * EPV + k] = valid ? Q(x[j * EPV + k] - mean) : 0.0f;
+                    for (int d = 0; d < 4; ++d)
+#pragma unroll
+                        for (int h = 0; h < PD; ++h) x[(j * 4 + d) * PD + h] = Qd(Pack<DT>::get(raw[d], h));
+                }
             }
         }
-        float sq = 0.0f;
+        float sum = 0.0f;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) sq += Q(x[e] * x[e]);
+        for (int e = 0; e < EPL; ++e) sum += p.rms ? 0.0f : x[e];
+        float sq = 0.0f;
+        float mean = 0.0f;
+        if (!p.rms) {
+            mean = Q(Q(row_reduce<SumOp, WPR>(sum, part)) / count);
+            if (QMODE == SMQ_BF16) plain = __all(plain && within(mean, 0u, 0x4A000000u));    // |mean| < 2^21
+        }
+        auto centre_and_square = [&](auto plain_tag) {
+            auto Qs = [&](float v) { return decltype(plain_tag)::value ? Qplain(v) : Q(v); };
+            if (!p.rms) {
+#pragma unroll
+                for (int j = 0; j < VPL; ++j) {
+                    const bool valid = j * LPR + lane < nvec;
+#pragma unroll
+                    for (int k = 0; k < EPV; ++k) x[j * EPV + k] = valid ? Qs(x[j * EPV + k] - mean) : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) sq += Qs(x[e] * x[e]);
+        };
+        if (QMODE == SMQ_BF16 && plain) centre_and_square(std::true_type{});
+        else centre_and_square(std::false_type{});
         const float var = Q(Q(row_reduce<SumOp, WPR>(sq, part)) / count);
         const float vare = Q(var + p.eps);
         const float rinv = Q(1.0f / Q(sqrtf(vare)));
         if (lane == 0 && nvec != 0) store_scalar<DT>(stat_, row, p.rms ? rinv : vare);
+        if (QMODE == SMQ_BF16)
+            plain = __all(plain && wb_plain && mxq_bits(rinv) - 0x30800000u < 0x1E000000u);   // [2^-30, 2^30)
 
-        const u32x4* wv = reinterpret_cast<const u32x4*>(weight_);
-        const u32x4* bv = reinterpret_cast<const u32x4*>(bias_);
         u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec_row;
         u32x4* zn = znorm_ ? reinterpret_cast<u32x4*>(znorm_) + row * nvec : nullptr;
+        auto scale_and_shift = [&](auto plain_tag) {
+            auto Qs = [&](float v) { return decltype(plain_tag)::value ? Qplain(v) : Q(v); };
 #pragma unroll
-        for (int j = 0; j < VPL; ++j) {
-            const int v = j * LPR + lane;
-            if (v >= nvec) continue;
-            const u32x4 w4 = wv[v], b4 = bv[v];
-            u32x4 o, z4;
+            for (int j = 0; j < VPL; ++j) {
+                const int v = j * LPR + lane;
+                if (v >= nvec) continue;
+                const u32x4 w4 = wv[v], b4 = bv[v];
+                u32x4 o, z4;
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                float q[2], z[2];
+                for (int d = 0; d < 4; ++d) {
+                    float q[2], z[2];
 #pragma unroll
-                for (int h = 0; h < PD; ++h) {
-                    z[h] = Q(x[(j * 4 + d) * PD + h] * rinv);
-                    q[h] = Q(Q(Pack<DT>::get(w4[d], h) * z[h]) + Pack<DT>::get(b4[d], h));
+                    for (int h = 0; h < PD; ++h) {
+                        z[h] = Qs(x[(j * 4 + d) * PD + h] * rinv);
+                        q[h] = Qs(Qs(Pack<DT>::get(w4[d], h) * z[h]) + Pack<DT>::get(b4[d], h));
+                    }
+                    o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+                    z4[d] = Pack<DT>::put(z[0], z[PD - 1]);
                 }
-                o[d] = Pack<DT>::put(q[0], q[PD - 1]);
-                z4[d] = Pack<DT>::put(z[0], z[PD - 1]);
+                __builtin_nontemporal_store(o, &out[v]);
+                if (zn) __builtin_nontemporal_store(z4, &zn[v]);
             }
-            __builtin_nontemporal_store(o, &out[v]);
-            if (zn) __builtin_nontemporal_store(z4, &zn[v]);
-        }
+        };
+        if (QMODE == SMQ_BF16 && plain) scale_and_shift(std::true_type{});
+        else scale_and_shift(std::false_type{});
     }
 }
 
@@ -390,7 +469,7 @@ __global__ __launch_bounds__(TPB) void activation_kernel(const void* __restrict_
                 qv[d] = Pack<DT>::put(qq[0], qq[PD - 1]);
             }
         };
-        bool plain = QMODE == SMQ_BF16;
+        bool plain = QMODE == SMQ_BF16 && !p.q.general_only;
         if (QMODE == SMQ_BF16) {
 #pragma unroll
             for (int d = 0; d < 4; ++d)

@@ -31,6 +31,14 @@ def set_exponent_mode(mode):
         raise ValueError("exponent mode must be 'torch' or 'exact'")
 
 
+def set_general_form(on):
+    """The softmax, norm and activation kernels skip the special cases of the bfloat16 quantizer for
+    waves whose values all lie in a range where none can occur.  on=True switches that shortcut off
+    (same results, slower): what the tests compare the shortcut with."""
+    global _flags
+    _flags = (_flags | _lib.FLAG_GENERAL_FORM) if on else (_flags & ~_lib.FLAG_GENERAL_FORM)
+
+
 def _flags_value():
     return _flags
 

@@ -898,3 +898,108 @@ def test_fp6_gemm_on_sixbit_codes_against_fp64(dev, M, N, K, batch, fa, fb):
     assert torch.equal(got16.view(torch.int16), want16.view(torch.int16))
     with pytest.raises(RuntimeError, match="both operands"):
         gemm_nt(pa, pack_mx(b.to(dev), fb), torch.float32)
+
+
+# ---- the plain-range shortcut of the bfloat16 quantizer against the general form ---------------------
+def _general_form():
+    """Context: the chain kernels never take the shortcut."""
+    import contextlib
+    from microxcaling_amd import custom_extensions as CE
+
+    @contextlib.contextmanager
+    def ctx():
+        CE.set_general_form(True)
+        try:
+            yield
+        finally:
+            CE.set_general_form(False)
+    return ctx()
+
+
+def _edge_rows(rows, n, g, lo, hi):
+    """bf16 rows that sit on the edges of a plain range [2^lo, 2^hi): both ends, alternating signs,
+    constant rows (no spread at all), rows of two values one step apart, and random rows of every
+    magnitude in between."""
+    x = torch.randn(rows, n, generator=g) * torch.exp2(torch.randint(lo + 2, hi - 3, (rows, 1), generator=g).float())
+    x[0] = 2.0 ** lo
+    x[1] = -(2.0 ** lo)
+    x[2] = 2.0 ** hi * (1 - 2.0 ** -8)
+    x[3] = torch.where(torch.arange(n) % 2 == 0, 2.0 ** lo, -(2.0 ** hi) * (1 - 2.0 ** -8))
+    x[4] = 1.0
+    x[5] = torch.where(torch.arange(n) % 2 == 0, 1.0, 1.0 + 2.0 ** -7)
+    x[6] = torch.where(torch.arange(n) % 3 == 0, 3.0, 2.0 ** lo)
+    x[7] = torch.exp2(torch.linspace(lo, hi - 0.01, n)) * (1 - 2 * (torch.arange(n) % 2))
+    x = x.to(torch.bfloat16)
+    tiny = x.float().abs() < 2.0 ** lo
+    x[tiny] = 2.0 ** lo
+    x[x.float().abs() >= 2.0 ** hi] = 2.0 ** (hi - 1)
+    return x
+
+
+@pytest.mark.parametrize("n", [264, 2048, 8192, 16384])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, softmax_exp2=True),
+                                  dict(bfloat=16, vec_use_exp2=True, vec_use_recip=True)])
+def test_softmax_shortcut_equals_general_form(dev, n, spec):
+    from microxcaling_amd.softmax import softmax
+    g = torch.Generator().manual_seed(n)
+    x = _edge_rows(24, n, g, -100, 100)
+    x[8:16] = (torch.randn(8, n, generator=g) * 3).to(torch.bfloat16)     # ordinary logits
+    x[x == 0] = 1.0
+    specs = _specs(**spec)
+    got = softmax(x.to(dev), dim=-1, mx_specs=specs).cpu()
+    with _general_form():
+        want = softmax(x.to(dev), dim=-1, mx_specs=specs).cpu()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("layer", ["layernorm", "rmsnorm"])
+@pytest.mark.parametrize("n", [264, 4096, 8192, 16384])
+@pytest.mark.parametrize("eps", [1e-5, 1e-12, 0.0])
+def test_norm_shortcut_equals_general_form(dev, layer, n, eps):
+    """Inputs, weights and biases on the edges of their plain ranges, constant rows (variance 0:
+    with eps = 0 the row scale is Inf and the wave must leave the shortcut), products that cancel
+    the bias exactly, zero and negative-zero biases, weights of both signs."""
+    from microxcaling_amd import layernorm as L
+    from microxcaling_amd.specs import apply_mx_specs
+    g = torch.Generator().manual_seed(n + len(layer))
+    x = _edge_rows(40, n, g, -20, 20)
+    w = torch.exp2(torch.linspace(-20, 19.99, n)) * (1 - 2 * (torch.arange(n) % 2).float())
+    b = torch.randn(n, generator=g) * torch.exp2(torch.randint(-39, 39, (n,), generator=g).float())
+    b = torch.sign(b) * b.abs().clamp(2.0 ** -39.5, 2.0 ** 39.5)
+    b[::5] = 0.0
+    w, b = w.to(torch.bfloat16), b.to(torch.bfloat16)
+    specs = apply_mx_specs(_specs(bfloat=16))
+    outs = []
+    for wi, bi in ((w, b), (torch.ones_like(w), torch.zeros_like(b)), (-w, -b.abs())):
+        for general in (False, True):
+            if general:
+                with _general_form():
+                    r = L._fused_forward(x.to(dev), wi.to(dev), bi.to(dev), eps, specs, layer == "rmsnorm")
+            else:
+                r = L._fused_forward(x.to(dev), wi.to(dev), bi.to(dev), eps, specs, layer == "rmsnorm")
+            assert r is not None
+            outs.append([t.cpu() for t in r])
+        for a, c, what in zip(outs[-2], outs[-1], ("output", "normalized input", "row statistic")):
+            same = (a.view(torch.int16) == c.view(torch.int16)) | (torch.isnan(a) & torch.isnan(c))
+            assert same.all(), what
+
+
+@pytest.mark.parametrize("act", sorted(_ACTS))
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, vec_use_exp2=True)], ids=["exp", "exp2"])
+def test_activation_shortcut_equals_general_form(dev, act, spec):
+    from microxcaling_amd import activations as A
+    g = torch.Generator().manual_seed(len(act) + 1)
+    x = _edge_rows(64, 2048, g, -20, 3).reshape(-1)
+    specs = _specs(**spec)
+    got = _ACTS[act](A, x.to(dev), specs).cpu()
+    with _general_form():
+        want = _ACTS[act](A, x.to(dev), specs).cpu()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # every bf16 value of the range, both signs
+    codes = torch.arange(0x3580, 0x4100, dtype=torch.int32)
+    allv = torch.cat([codes, codes + 0x8000]).to(torch.int16).view(torch.bfloat16)
+    allv = allv.repeat(2)[: (2 * allv.numel()) // 512 * 512]
+    got = _ACTS[act](A, allv.to(dev), specs).cpu()
+    with _general_form():
+        want = _ACTS[act](A, allv.to(dev), specs).cpu()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
