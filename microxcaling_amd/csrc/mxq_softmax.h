@@ -448,6 +448,63 @@ __global__ __launch_bounds__(TPB) void activation_kernel(const void* __restrict_
         }
     };
     auto in_plain_range = [](uint32_t ua) { return ua - 0x35800000u < 0x0B800000u; };   // [2^-20, 8)
+    // The plain form on the two bf16 values of a dword at once: one conversion rounds both to bf16,
+    // one add moves both odd significands up (no carry leaves the low half: 0xFFFF is a NaN).
+    // dword in: the pair as loaded; dwords out: result, logistic factor, quantized input.
+    auto eval_pair = [&](uint32_t w, uint32_t& aux_w, uint32_t& q_w) {
+        struct Pair { float a, b; };
+        auto packed = [](float a, float b) {
+            const uint32_t r = Pack<MXQ_BF16>::put(a, b);
+            return r + (r & 0x00010001u);
+        };
+        auto unpack = [](uint32_t r) { return Pair{mxq_float(r << 16), mxq_float(r & 0xFFFF0000u)}; };
+        auto Q2 = [&](float a, float b) { return unpack(packed(a, b)); };
+        auto logistic = [&](Pair y) {                        // packed
+            Pair e;
+            if (via_exp2) {
+                const Pair t = Q2(1.4453125f * -y.a, 1.4453125f * -y.b);
+                e = Q2(exp2f(t.a), exp2f(t.b));
+            } else {
+                e = Q2(expf(-y.a), expf(-y.b));
+            }
+            const Pair s = Q2(e.a + 1.0f, e.b + 1.0f);
+            // 1 / s for s with an 8-bit significand, 1 <= s < 2^72: a refined hardware reciprocal
+            // and one residual correction give the correctly rounded fp32 quotient (what the
+            // division of the general form gives) for a third of its instructions
+            auto recip = [](float d) {
+                const float r0 = __builtin_amdgcn_rcpf(d);
+                const float r1 = fmaf(fmaf(-d, r0, 1.0f), r0, r0);
+                return fmaf(fmaf(-r1, d, 1.0f), r1, r1);
+            };
+            return packed(recip(s.a), recip(s.b));
+        };
+        q_w = w + (w & 0x00010001u);
+        const Pair q = unpack(q_w);
+        aux_w = 0u;
+        switch (p.act) {
+            case ACT_SIGMOID: return logistic(q);
+            case ACT_TANH: return packed(tanhf(q.a), tanhf(q.b));
+            case ACT_SILU: {
+                aux_w = logistic(q);
+                const Pair s = unpack(aux_w);
+                return packed(q.a * s.a, q.b * s.b);
+            }
+            case ACT_GELU_FIRST_ORDER: {
+                aux_w = logistic(Q2(1.703125f * q.a, 1.703125f * q.b));
+                const Pair s = unpack(aux_w);
+                return packed(q.a * s.a, q.b * s.b);
+            }
+            default: {
+                const Pair sq = Q2(q.a * q.a, q.b * q.b);
+                const Pair cube = Q2(sq.a * q.a, sq.b * q.b);
+                const Pair c = Q2(0.044677734375f * cube.a, 0.044677734375f * cube.b);
+                const Pair in = Q2(c.a + q.a, c.b + q.b);
+                aux_w = logistic(Q2(1.59375f * in.a, 1.59375f * in.b));
+                const Pair s = unpack(aux_w);
+                return packed(q.a * s.a, q.b * s.b);
+            }
+        }
+    };
 
     const u32x4* in = reinterpret_cast<const u32x4*>(in_);
     u32x4* out = reinterpret_cast<u32x4*>(out_);
@@ -461,12 +518,19 @@ __global__ __launch_bounds__(TPB) void activation_kernel(const void* __restrict_
         auto vector = [&](auto plain_tag) {
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-                float r[2], ax[2], qq[2];
+                if constexpr (decltype(plain_tag)::value && DT == MXQ_BF16) {
+                    uint32_t aw, qw;
+                    o[d] = eval_pair(v[d], aw, qw);
+                    a[d] = aw;
+                    qv[d] = qw;
+                } else {
+                    float r[2], ax[2], qq[2];
 #pragma unroll
-                for (int h = 0; h < PD; ++h) r[h] = eval(plain_tag, Pack<DT>::get(v[d], h), ax[h], qq[h]);
-                o[d] = Pack<DT>::put(r[0], r[PD - 1]);
-                a[d] = Pack<DT>::put(ax[0], ax[PD - 1]);
-                qv[d] = Pack<DT>::put(qq[0], qq[PD - 1]);
+                    for (int h = 0; h < PD; ++h) r[h] = eval(plain_tag, Pack<DT>::get(v[d], h), ax[h], qq[h]);
+                    o[d] = Pack<DT>::put(r[0], r[PD - 1]);
+                    a[d] = Pack<DT>::put(ax[0], ax[PD - 1]);
+                    qv[d] = Pack<DT>::put(qq[0], qq[PD - 1]);
+                }
             }
         };
         bool plain = QMODE == SMQ_BF16 && !p.q.general_only;
