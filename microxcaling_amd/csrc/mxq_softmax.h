@@ -240,6 +240,14 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
     auto within = [](float v, uint32_t lo, uint32_t hi) {    // lo <= |v| < hi as bit patterns
         return (mxq_bits(v) & 0x7FFFFFFFu) - lo < hi - lo;
     };
+    // the plain form on two values at once: one conversion rounds both to bf16, one add moves both
+    // odd significands up (no carry leaves the low half: 0xFFFF is a NaN)
+    auto plain_packed = [](float a, float b) {
+        const uint32_t r = Pack<MXQ_BF16>::put(a, b);
+        return r + (r & 0x00010001u);
+    };
+    auto low_of = [](uint32_t r) { return mxq_float(r << 16); };
+    auto high_of = [](uint32_t r) { return mxq_float(r & 0xFFFF0000u); };
 
     constexpr int LPR = 64 * WPR;                            // lanes per row
     constexpr int RPB = (TPB / 64) / WPR;                    // rows per block and iteration
@@ -320,17 +328,37 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
             if (QMODE == SMQ_BF16) plain = __all(plain && within(mean, 0u, 0x4A000000u));    // |mean| < 2^21
         }
         auto centre_and_square = [&](auto plain_tag) {
-            auto Qs = [&](float v) { return decltype(plain_tag)::value ? Qplain(v) : Q(v); };
-            if (!p.rms) {
+            if constexpr (decltype(plain_tag)::value && DT == MXQ_BF16) {
+                if (!p.rms) {
 #pragma unroll
-                for (int j = 0; j < VPL; ++j) {
-                    const bool valid = j * LPR + lane < nvec;
+                    for (int j = 0; j < VPL; ++j) {
+                        const bool valid = j * LPR + lane < nvec;
 #pragma unroll
-                    for (int k = 0; k < EPV; ++k) x[j * EPV + k] = valid ? Qs(x[j * EPV + k] - mean) : 0.0f;
+                        for (int k = 0; k < EPV; k += 2) {
+                            const uint32_t r = plain_packed(x[j * EPV + k] - mean, x[j * EPV + k + 1] - mean);
+                            x[j * EPV + k] = valid ? low_of(r) : 0.0f;
+                            x[j * EPV + k + 1] = valid ? high_of(r) : 0.0f;
+                        }
+                    }
                 }
-            }
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) sq += Qs(x[e] * x[e]);
+                for (int e = 0; e < EPL; e += 2) {           // same order of additions as one by one
+                    const uint32_t r = plain_packed(x[e] * x[e], x[e + 1] * x[e + 1]);
+                    sq += low_of(r);
+                    sq += high_of(r);
+                }
+            } else {
+                if (!p.rms) {
+#pragma unroll
+                    for (int j = 0; j < VPL; ++j) {
+                        const bool valid = j * LPR + lane < nvec;
+#pragma unroll
+                        for (int k = 0; k < EPV; ++k) x[j * EPV + k] = valid ? Q(x[j * EPV + k] - mean) : 0.0f;
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) sq += Q(x[e] * x[e]);
+            }
         };
         if (QMODE == SMQ_BF16 && plain) centre_and_square(std::true_type{});
         else centre_and_square(std::false_type{});
@@ -344,7 +372,6 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
         u32x4* out = reinterpret_cast<u32x4*>(out_) + row * nvec_row;
         u32x4* zn = znorm_ ? reinterpret_cast<u32x4*>(znorm_) + row * nvec : nullptr;
         auto scale_and_shift = [&](auto plain_tag) {
-            auto Qs = [&](float v) { return decltype(plain_tag)::value ? Qplain(v) : Q(v); };
 #pragma unroll
             for (int j = 0; j < VPL; ++j) {
                 const int v = j * LPR + lane;
@@ -353,14 +380,22 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
                 u32x4 o, z4;
 #pragma unroll
                 for (int d = 0; d < 4; ++d) {
-                    float q[2], z[2];
+                    if constexpr (decltype(plain_tag)::value && DT == MXQ_BF16) {
+                        const int e = (j * 4 + d) * 2;
+                        const uint32_t zr = plain_packed(x[e] * rinv, x[e + 1] * rinv);
+                        const uint32_t wz = plain_packed(low_of(w4[d]) * low_of(zr), high_of(w4[d]) * high_of(zr));
+                        o[d] = plain_packed(low_of(wz) + low_of(b4[d]), high_of(wz) + high_of(b4[d]));
+                        z4[d] = zr;
+                    } else {
+                        float q[2], z[2];
 #pragma unroll
-                    for (int h = 0; h < PD; ++h) {
-                        z[h] = Qs(x[(j * 4 + d) * PD + h] * rinv);
-                        q[h] = Qs(Qs(Pack<DT>::get(w4[d], h) * z[h]) + Pack<DT>::get(b4[d], h));
+                        for (int h = 0; h < PD; ++h) {
+                            z[h] = Q(x[(j * 4 + d) * PD + h] * rinv);
+                            q[h] = Q(Q(Pack<DT>::get(w4[d], h) * z[h]) + Pack<DT>::get(b4[d], h));
+                        }
+                        o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+                        z4[d] = Pack<DT>::put(z[0], z[PD - 1]);
                     }
-                    o[d] = Pack<DT>::put(q[0], q[PD - 1]);
-                    z4[d] = Pack<DT>::put(z[0], z[PD - 1]);
                 }
                 __builtin_nontemporal_store(o, &out[v]);
                 if (zn) __builtin_nontemporal_store(z4, &zn[v]);
