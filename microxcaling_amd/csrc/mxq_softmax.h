@@ -643,6 +643,71 @@ __global__ __launch_bounds__(TPB) void activation_backward_kernel(const void* __
     };
 
     const bool two = p.act >= ACT_SILU;                      // a second saved tensor
+
+    // SMQ_BF16, plain range (see activation_kernel): a wave whose three inputs lie in
+    //   grad 2^-30 <= |g| < 2^40;
+    //   saved: sigmoid 2^-60 <= s <= 1; tanh 2^-20 <= |t| <= 1; silu 2^-40 <= |y| < 2^20;
+    //          gelu 2^-20 <= |x| < 8;       logistic factor (silu, gelu) 2^-60 <= s <= 1
+    // sees only normal numbers and zeros in its chain: 1 - s is +0 (a saturated logistic, which is
+    // common) or at least 2^-8, the products are zero or stay above 2^-80, and the sum "s + ..." of
+    // silu and gelu can cancel, exactly (+0) or down to one unit of its smaller term (at least
+    // 2^-87, so that d g stays above 2^-117).  A zero only ever meets a product (which stays a zero of some sign) or the sum with
+    // s > 0 (which ignores its sign), so the derivative d is +0 or normal; d g is then normal or
+    // +-0, and adding +0.0 before the last quantization turns a -0 into the +0 the general form gives.
+    // Both values of a dword go through the plain form at once (see eval_pair there).
+    const uint32_t s_lo = p.act == ACT_SIGMOID ? 0x2180u : p.act == ACT_SILU ? 0x2B80u : 0x3580u;
+    const uint32_t s_hi = p.act == ACT_SIGMOID ? 0x3F81u : p.act == ACT_TANH ? 0x3F81u
+                        : p.act == ACT_SILU ? 0x4980u : 0x4100u;
+    const uint32_t s_mask = p.act == ACT_SIGMOID ? 0xFFFFu : 0x7FFFu;   // the sigmoid must be positive
+    auto halves_within = [](uint32_t w, uint32_t mask, uint32_t lo, uint32_t hi) {   // both bf16 halves
+        return ((w & mask) - lo < hi - lo) && (((w >> 16) & mask) - lo < hi - lo);
+    };
+    auto eval_pair = [&](uint32_t gw, uint32_t sw, uint32_t aw) {
+        struct Pair { float a, b; };
+        auto packed = [](float a, float b) {
+            const uint32_t r = Pack<MXQ_BF16>::put(a, b);
+            return r + (r & 0x00010001u);
+        };
+        auto unpack = [](uint32_t r) { return Pair{mxq_float(r << 16), mxq_float(r & 0xFFFF0000u)}; };
+        auto Q2 = [&](float a, float b) { return unpack(packed(a, b)); };
+        const Pair g = unpack(gw + (gw & 0x00010001u));
+        const Pair sv = unpack(sw), ax = unpack(aw);
+        Pair d;
+        switch (p.act) {
+            case ACT_SIGMOID: {
+                const Pair t = Q2(1.0f - sv.a, 1.0f - sv.b);
+                d = Q2(sv.a * t.a, sv.b * t.b);
+                break;
+            }
+            case ACT_TANH: {
+                const Pair t = Q2(sv.a * sv.a, sv.b * sv.b);
+                d = Q2(1.0f - t.a, 1.0f - t.b);
+                break;
+            }
+            case ACT_SILU: {
+                const Pair t = Q2(1.0f - ax.a, 1.0f - ax.b);
+                const Pair u = Q2(sv.a * t.a, sv.b * t.b);
+                d = Q2(ax.a + u.a, ax.b + u.b);
+                break;
+            }
+            default: {
+                const Pair t = Q2(1.0f - ax.a, 1.0f - ax.b);
+                Pair dphi = Q2(ax.a * t.a, ax.b * t.b);
+                if (p.act == ACT_GELU_FIRST_ORDER) {
+                    dphi = Q2(1.703125f * dphi.a, 1.703125f * dphi.b);
+                } else {
+                    const Pair sq = Q2(sv.a * sv.a, sv.b * sv.b);
+                    const Pair c = Q2(0.2138671875f * sq.a, 0.2138671875f * sq.b);
+                    const Pair e = Q2(1.59375f + c.a, 1.59375f + c.b);
+                    dphi = Q2(e.a * dphi.a, e.b * dphi.b);
+                }
+                const Pair u = Q2(sv.a * dphi.a, sv.b * dphi.b);
+                d = Q2(ax.a + u.a, ax.b + u.b);
+            }
+        }
+        return packed(d.a * g.a + 0.0f, d.b * g.b + 0.0f);
+    };
+
     const u32x4* grad = reinterpret_cast<const u32x4*>(grad_);
     const u32x4* saved = reinterpret_cast<const u32x4*>(saved_);
     const u32x4* aux = reinterpret_cast<const u32x4*>(aux_);
@@ -653,13 +718,30 @@ __global__ __launch_bounds__(TPB) void activation_backward_kernel(const void* __
         const u32x4 gv = grad[i], sv = saved[i];
         const u32x4 av = two ? aux[i] : u32x4{0, 0, 0, 0};
         u32x4 o;
+        bool plain = false;
+        if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
+            plain = !p.q.general_only;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            float r[2];
+            for (int d = 0; d < 4; ++d)
+                plain = plain && halves_within(gv[d], 0x7FFFu, 0x3080u, 0x5380u) &&
+                        halves_within(sv[d], s_mask, s_lo, s_hi) &&
+                        (!two || halves_within(av[d], 0xFFFFu, 0x2180u, 0x3F81u));
+            plain = __all(plain);                            // one branch per wave
+        }
+        if (plain) {
+            if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
 #pragma unroll
-            for (int h = 0; h < PD; ++h)
-                r[h] = eval(Pack<DT>::get(gv[d], h), Pack<DT>::get(sv[d], h), Pack<DT>::get(av[d], h));
-            o[d] = Pack<DT>::put(r[0], r[PD - 1]);
+                for (int d = 0; d < 4; ++d) o[d] = eval_pair(gv[d], sv[d], av[d]);
+            }
+        } else {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                float r[2];
+#pragma unroll
+                for (int h = 0; h < PD; ++h)
+                    r[h] = eval(Pack<DT>::get(gv[d], h), Pack<DT>::get(sv[d], h), Pack<DT>::get(av[d], h));
+                o[d] = Pack<DT>::put(r[0], r[PD - 1]);
+            }
         }
         __builtin_nontemporal_store(o, &out[i]);
     }

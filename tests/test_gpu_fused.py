@@ -1003,3 +1003,36 @@ def test_activation_shortcut_equals_general_form(dev, act, spec):
     with _general_form():
         want = _ACTS[act](A, allv.to(dev), specs).cpu()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("act", sorted(_ACTS))
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, vec_use_exp2=True)], ids=["exp", "exp2"])
+def test_activation_backward_shortcut_equals_general_form(dev, act, spec):
+    """Saved tensors and gradients inside the plain ranges of the backward kernel (and a few waves
+    outside: saturated sigmoids, large inputs), including the inputs around which the derivative of
+    silu and gelu changes sign, where the last sum of the chain cancels."""
+    from microxcaling_amd import activations as A
+    g = torch.Generator().manual_seed(len(act) + 7)
+    n = 512 * 400
+    x = (torch.randn(n, generator=g) * 1.5).clamp(-5, 5)
+    x[: 512 * 64] = torch.linspace(-1.5, -0.5, 512 * 64)          # the zeros of silu' and gelu'
+    x[512 * 64: 512 * 72] = torch.linspace(5.0, 9.0, 512 * 8)     # saturating
+    x[x.abs() < 2.0 ** -19] = 0.25
+    x = x.to(torch.bfloat16)
+    x[512 * 72: 512 * 80] = torch.linspace(-9.0, -4.0, 512 * 8)   # tiny logistic factors
+    x = x.to(torch.bfloat16)
+    grad = torch.randn(n, generator=g) * torch.exp2(torch.randint(-28, 38, (n,), generator=g).float())
+    grad = (torch.sign(grad) * grad.abs().clamp(2.0 ** -29.5, 2.0 ** 39.5)).to(torch.bfloat16)
+    grad[512 * 300:] = (grad[512 * 300:].float() * 2.0 ** -12).to(torch.bfloat16)     # partly below the range
+    specs = _specs(**spec)
+    grads = []
+    for general in (False, True):
+        xi = x.to(dev).requires_grad_(True)
+        if general:
+            with _general_form():
+                _ACTS[act](A, xi, specs).backward(grad.to(dev))
+        else:
+            _ACTS[act](A, xi, specs).backward(grad.to(dev))
+        grads.append(xi.grad.cpu())
+    assert torch.equal(grads[0].view(torch.int16), grads[1].view(torch.int16))
+    assert (grads[0].float() == 0).float().mean() < 0.2
