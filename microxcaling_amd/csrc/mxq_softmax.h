@@ -793,37 +793,96 @@ __global__ __launch_bounds__(TPB) void softmax_backward_row_kernel(const void* _
         float g[EPL];
         u32x4 yraw[VPL];
         float sum = 0.0f;
+        // SMQ_BF16, plain range (see softmax_row_kernel): gradients 2^-30 <= |g| < 2^30 and saved
+        // outputs 2^-60 <= y <= 1 in every lane of the wave, and |s| < 2^30 for the row sum, keep
+        // every per-element value a normal number or +0 (g - s cancels to +0 or to no less than
+        // 2^-46, and y > 0 keeps the sign of a zero): both bf16 values of a dword then go through
+        // the plain form of the quantizer at once.
+        bool plain = false;
+        if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) plain = !p.q.general_only;
+        auto plain_packed = [](float a, float b) {
+            const uint32_t r = Pack<MXQ_BF16>::put(a, b);
+            return r + (r & 0x00010001u);
+        };
+        auto low_of = [](uint32_t r) { return mxq_float(r << 16); };
+        auto high_of = [](uint32_t r) { return mxq_float(r & 0xFFFF0000u); };
+        auto halves_within = [](uint32_t w, uint32_t mask, uint32_t lo, uint32_t hi) {
+            return ((w & mask) - lo < hi - lo) && (((w >> 16) & mask) - lo < hi - lo);
+        };
+        if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
 #pragma unroll
-        for (int j = 0; j < VPL; ++j) {
-            const bool valid = j * LPR + lane < nvec;
-            u32x4 graw = {0, 0, 0, 0};
-            yraw[j] = u32x4{0, 0, 0, 0};
-            if (valid) {
-                graw = gin[j * LPR + lane];
-                yraw[j] = yin[j * LPR + lane];
-            }
-#pragma unroll
-            for (int d = 0; d < 4; ++d)
-#pragma unroll
-                for (int h = 0; h < PD; ++h) {
-                    const int e = (j * 4 + d) * PD + h;
-                    g[e] = valid ? Qd(Pack<DT>::get(graw[d], h)) : 0.0f;
-                    sum += valid ? Q(g[e] * Pack<DT>::get(yraw[j][d], h)) : 0.0f;
+            for (int j = 0; j < VPL; ++j) {
+                const bool valid = j * LPR + lane < nvec;
+                u32x4 graw = {0, 0, 0, 0};
+                yraw[j] = u32x4{0, 0, 0, 0};
+                if (valid) {
+                    graw = gin[j * LPR + lane];
+                    yraw[j] = yin[j * LPR + lane];
                 }
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    plain = plain && (!valid || (halves_within(graw[d], 0x7FFFu, 0x3080u, 0x4E80u) &&
+                                                 halves_within(yraw[j][d], 0xFFFFu, 0x2180u, 0x3F81u)));
+                    const uint32_t gq = graw[d] + (graw[d] & 0x00010001u);
+                    const int e = (j * 4 + d) * 2;
+                    g[e] = valid ? low_of(gq) : 0.0f;
+                    g[e + 1] = valid ? high_of(gq) : 0.0f;
+                    const uint32_t prod = plain_packed(g[e] * low_of(yraw[j][d]), g[e + 1] * high_of(yraw[j][d]));
+                    sum += valid ? low_of(prod) : 0.0f;
+                    sum += valid ? high_of(prod) : 0.0f;
+                }
+            }
+            plain = __all(plain);                            // wave-uniform from here on
+        }
+        if (!plain) {                                        // (for SMQ_BF16: rare, reads the gradient again)
+            sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) {
+                const bool valid = j * LPR + lane < nvec;
+                u32x4 graw = {0, 0, 0, 0};
+                yraw[j] = u32x4{0, 0, 0, 0};
+                if (valid) {
+                    graw = gin[j * LPR + lane];
+                    yraw[j] = yin[j * LPR + lane];
+                }
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+#pragma unroll
+                    for (int h = 0; h < PD; ++h) {
+                        const int e = (j * 4 + d) * PD + h;
+                        g[e] = valid ? Qd(Pack<DT>::get(graw[d], h)) : 0.0f;
+                        sum += valid ? Q(g[e] * Pack<DT>::get(yraw[j][d], h)) : 0.0f;
+                    }
+            }
         }
         sum = Q(row_reduce<SumOp, WPR>(sum, part));
+        if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16)
+            plain = __all(plain && (mxq_bits(sum) & 0x7FFFFFFFu) < 0x4E800000u);       // |s| < 2^30, the same in every lane
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
             u32x4 o;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-                float q[2];
-#pragma unroll
-                for (int h = 0; h < PD; ++h) {
-                    const float t = Q(Pack<DT>::get(yraw[j][d], h) * Q(g[(j * 4 + d) * PD + h] - sum));
-                    q[h] = p.exp_mode == 1 ? Q(t * 0.69140625f) : t;
+                bool done = false;
+                if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
+                    if (plain) {
+                        const int e = (j * 4 + d) * 2;
+                        const uint32_t diff = plain_packed(g[e] - sum, g[e + 1] - sum);
+                        uint32_t r = plain_packed(low_of(yraw[j][d]) * low_of(diff), high_of(yraw[j][d]) * high_of(diff));
+                        if (p.exp_mode == 1) r = plain_packed(low_of(r) * 0.69140625f, high_of(r) * 0.69140625f);
+                        o[d] = r;
+                        done = true;
+                    }
                 }
-                o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+                if (!done) {
+                    float q[2];
+#pragma unroll
+                    for (int h = 0; h < PD; ++h) {
+                        const float t = Q(Pack<DT>::get(yraw[j][d], h) * Q(g[(j * 4 + d) * PD + h] - sum));
+                        q[h] = p.exp_mode == 1 ? Q(t * 0.69140625f) : t;
+                    }
+                    o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+                }
             }
             if (j * LPR + lane < nvec) __builtin_nontemporal_store(o, &out[j * LPR + lane]);
         }

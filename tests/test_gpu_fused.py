@@ -1036,3 +1036,37 @@ def test_activation_backward_shortcut_equals_general_form(dev, act, spec):
         grads.append(xi.grad.cpu())
     assert torch.equal(grads[0].view(torch.int16), grads[1].view(torch.int16))
     assert (grads[0].float() == 0).float().mean() < 0.2
+
+
+@pytest.mark.parametrize("n", [264, 2048, 4096, 16384])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=16, softmax_exp2=True)], ids=["exp", "exp2"])
+def test_softmax_backward_shortcut_equals_general_form(dev, n, spec):
+    """Gradients and saved outputs inside the plain ranges (rows of ordinary logits), gradients on
+    the edges of their range, a constant gradient (g - s cancels everywhere), rows with outputs that
+    underflowed to zero and gradients outside the range (general form)."""
+    from microxcaling_amd.softmax import softmax
+    g = torch.Generator().manual_seed(n + 3)
+    rows = 48
+    x = (torch.randn(rows, n, generator=g) * 3).to(torch.bfloat16)
+    x[40:44, ::7] = -200.0                                       # outputs that are exactly zero
+    grad = torch.randn(rows, n, generator=g) * torch.exp2(torch.randint(-27, 27, (rows, 1), generator=g).float())
+    grad[0] = 2.0 ** -30
+    grad[1] = -(2.0 ** 30) * (1 - 2.0 ** -8)
+    grad[2] = torch.where(torch.arange(n) % 2 == 0, 2.0 ** -30, 2.0 ** 29)
+    grad[3] = 0.75
+    grad[4] = torch.where(torch.arange(n) % 2 == 0, 1.0, 1.0 + 2.0 ** -7)
+    grad[44:] = grad[44:] * 2.0 ** -40                           # below the range
+    grad = torch.sign(grad) * grad.abs().clamp(min=2.0 ** -80)
+    grad[:44] = torch.sign(grad[:44]) * grad[:44].abs().clamp(2.0 ** -30, 2.0 ** 29.9)
+    grad = grad.to(torch.bfloat16)
+    specs = _specs(**spec)
+    grads = []
+    for general in (False, True):
+        xi = x.to(dev).requires_grad_(True)
+        if general:
+            with _general_form():
+                softmax(xi, dim=-1, mx_specs=specs).backward(grad.to(dev))
+        else:
+            softmax(xi, dim=-1, mx_specs=specs).backward(grad.to(dev))
+        grads.append(xi.grad.cpu())
+    assert torch.equal(grads[0].view(torch.int16), grads[1].view(torch.int16))
