@@ -928,6 +928,46 @@ __global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __re
     const int nvec_row = n / EPV;
     const float count = (float)n;
     const u32x4* wv = reinterpret_cast<const u32x4*>(weight_);
+
+    // SMQ_BF16, plain range (see norm_row_kernel).  A wave takes the plain form of the quantizer, on
+    // both bf16 values of a dword at once, for the per-element steps while what they see stays in
+    //   gradients 2^-30 <= |g| < 2^30, weights 2^-20 <= |w| < 2^20 (this lane's columns),
+    //   normalized inputs +0 or 2^-30 <= |z| < 2^10, 2^-30 <= sd, si (r) < 2^30:
+    //     g w, its products with si, with z, and that with sd are normal or zero (above 2^-110);
+    //   then the row scalar t: +-0 or 2^-40 <= |t| < 2^30: t z is +-0 or above 2^-70, and
+    //     d + t z is +0 (exact cancellation) or at least one unit of the smaller term;
+    //   then the row mean dm: +-0 or 2^-60 <= |dm| < 2^80, likewise.
+    // A zero of either sign only ever meets a row sum (which starts at +0 and is quantized in the
+    // general form) or a sum with a nonzero number.  The row scalars always take the general form.
+    constexpr bool CAN_PLAIN = QMODE == SMQ_BF16 && DT == MXQ_BF16;
+    auto plain_packed = [](float a, float b) {
+        const uint32_t r = Pack<MXQ_BF16>::put(a, b);
+        return r + (r & 0x00010001u);
+    };
+    auto low_of = [](uint32_t r) { return mxq_float(r << 16); };
+    auto high_of = [](uint32_t r) { return mxq_float(r & 0xFFFF0000u); };
+    auto half_within = [](uint32_t h, uint32_t lo, uint32_t hi) { return (h & 0x7FFFu) - lo < hi - lo; };
+    auto halves_within = [&](uint32_t w, uint32_t lo, uint32_t hi) {
+        return half_within(w & 0xFFFFu, lo, hi) && half_within(w >> 16, lo, hi);
+    };
+    auto scalar_within = [](float v, uint32_t lo, uint32_t hi, bool or_zero) {
+        const uint32_t ua = mxq_bits(v) & 0x7FFFFFFFu;
+        return (or_zero && ua == 0u) || ua - lo < hi - lo;
+    };
+    bool w_plain = false;
+    if constexpr (CAN_PLAIN) {
+        w_plain = !p.q.general_only;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            const int v = j * LPR + lane;
+            if (v >= nvec_row) continue;
+            const u32x4 w4 = wv[v];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) w_plain = w_plain && halves_within(w4[k], 0x3580u, 0x4980u);
+        }
+        w_plain = __all(w_plain);
+    }
+
     for (int64_t row0 = (int64_t)blockIdx.x * RPB; row0 < rows; row0 += (int64_t)gridDim.x * RPB) {
         const int64_t row = row0 + wib / WPR;
         const int nvec = row < rows ? nvec_row : 0;          // a block's spare waves go through the motions
@@ -941,65 +981,143 @@ __global__ __launch_bounds__(TPB) void norm_backward_row_kernel(const void* __re
         float d[EPL];                                        // Q(g w), then Q(d si)
         u32x4 zraw[VPL];
         float sum = 0.0f;
+        bool plain = false;
+        if constexpr (CAN_PLAIN) {
+            plain = w_plain && mxq_bits(si) - 0x30800000u < 0x1E000000u &&                   // [2^-30, 2^30), positive
+                    (p.rms || mxq_bits(sd) - 0x30800000u < 0x1E000000u);
 #pragma unroll
-        for (int j = 0; j < VPL; ++j) {
-            const bool valid = j * LPR + lane < nvec;
-            u32x4 graw = {0, 0, 0, 0}, wraw = {0, 0, 0, 0};
-            zraw[j] = u32x4{0, 0, 0, 0};
-            if (valid) {
-                graw = gin[j * LPR + lane];
-                wraw = wv[j * LPR + lane];
-                zraw[j] = zin[j * LPR + lane];
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-#pragma unroll
-                for (int h = 0; h < PD; ++h) {
-                    const int e = (j * 4 + k) * PD + h;
-                    const float z = Pack<DT>::get(zraw[j][k], h);
-                    const float dn = Q(Qd(Pack<DT>::get(graw[k], h)) * Pack<DT>::get(wraw[k], h));
-                    if (p.rms) {
-                        d[e] = Q(dn * si);
-                        sum += valid ? Q(d[e] * z) : 0.0f;
-                    } else {
-                        d[e] = Q(dn * si);
-                        sum += valid ? Q(Q(dn * z) * sd) : 0.0f;
-                    }
+            for (int j = 0; j < VPL; ++j) {
+                const bool valid = j * LPR + lane < nvec;
+                u32x4 graw = {0, 0, 0, 0}, wraw = {0, 0, 0, 0};
+                zraw[j] = u32x4{0, 0, 0, 0};
+                if (valid) {
+                    graw = gin[j * LPR + lane];
+                    wraw = wv[j * LPR + lane];
+                    zraw[j] = zin[j * LPR + lane];
                 }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t zw = zraw[j][k];
+                    plain = plain && (!valid || (halves_within(graw[k], 0x3080u, 0x4E80u) &&
+                                                 ((zw & 0xFFFFu) == 0u || half_within(zw & 0xFFFFu, 0x3080u, 0x4480u)) &&
+                                                 ((zw >> 16) == 0u || half_within(zw >> 16, 0x3080u, 0x4480u))));
+                    const int e = (j * 4 + k) * 2;
+                    const uint32_t gq = graw[k] + (graw[k] & 0x00010001u);
+                    const uint32_t dn = plain_packed(low_of(gq) * low_of(wraw[k]), high_of(gq) * high_of(wraw[k]));
+                    const uint32_t dd = plain_packed(low_of(dn) * si, high_of(dn) * si);
+                    d[e] = low_of(dd);
+                    d[e + 1] = high_of(dd);
+                    uint32_t ps;
+                    if (p.rms) {
+                        ps = plain_packed(d[e] * low_of(zw), d[e + 1] * high_of(zw));
+                    } else {
+                        const uint32_t pz = plain_packed(low_of(dn) * low_of(zw), high_of(dn) * high_of(zw));
+                        ps = plain_packed(low_of(pz) * sd, high_of(pz) * sd);
+                    }
+                    sum += valid ? low_of(ps) : 0.0f;
+                    sum += valid ? high_of(ps) : 0.0f;
+                }
+            }
+            plain = __all(plain);                            // wave-uniform from here on
+        }
+        if (!plain) {                                        // (for SMQ_BF16: rare, reads the row again)
+            sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) {
+                const bool valid = j * LPR + lane < nvec;
+                u32x4 graw = {0, 0, 0, 0}, wraw = {0, 0, 0, 0};
+                zraw[j] = u32x4{0, 0, 0, 0};
+                if (valid) {
+                    graw = gin[j * LPR + lane];
+                    wraw = wv[j * LPR + lane];
+                    zraw[j] = zin[j * LPR + lane];
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+#pragma unroll
+                    for (int h = 0; h < PD; ++h) {
+                        const int e = (j * 4 + k) * PD + h;
+                        const float z = Pack<DT>::get(zraw[j][k], h);
+                        const float dn = Q(Qd(Pack<DT>::get(graw[k], h)) * Pack<DT>::get(wraw[k], h));
+                        if (p.rms) {
+                            d[e] = Q(dn * si);
+                            sum += valid ? Q(d[e] * z) : 0.0f;
+                        } else {
+                            d[e] = Q(dn * si);
+                            sum += valid ? Q(Q(dn * z) * sd) : 0.0f;
+                        }
+                    }
+            }
         }
         float t = Q(Q(row_reduce<SumOp, WPR>(sum, part)) / count);
         if (!p.rms) t = -Q(t * Q(1.0f / stat));
+        if constexpr (CAN_PLAIN) plain = __all(plain && scalar_within(t, 0x2B800000u, 0x4E800000u, true));
         float sum2 = 0.0f;
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
             const bool valid = j * LPR + lane < nvec;
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-#pragma unroll
-                for (int h = 0; h < PD; ++h) {
-                    const int e = (j * 4 + k) * PD + h;
-                    const float z = Pack<DT>::get(zraw[j][k], h);
-                    if (p.rms) {
-                        d[e] = mxq_round_dt<ADT>(d[e] - Q(z * t));
-                    } else {
-                        d[e] = Q(d[e] + Q(t * z));
-                        sum2 += valid ? d[e] : 0.0f;
+            for (int k = 0; k < 4; ++k) {
+                bool done = false;
+                if constexpr (CAN_PLAIN) {
+                    if (plain) {
+                        const int e = (j * 4 + k) * 2;
+                        const uint32_t zw = zraw[j][k];
+                        const uint32_t tz = plain_packed(t * low_of(zw), t * high_of(zw));
+                        uint32_t nd;
+                        if (p.rms) {
+                            nd = Pack<MXQ_BF16>::put(d[e] - low_of(tz), d[e + 1] - high_of(tz));   // rounded only
+                        } else {
+                            nd = plain_packed(d[e] + low_of(tz), d[e + 1] + high_of(tz));
+                        }
+                        d[e] = low_of(nd);
+                        d[e + 1] = high_of(nd);
+                        if (!p.rms) {
+                            sum2 += valid ? d[e] : 0.0f;
+                            sum2 += valid ? d[e + 1] : 0.0f;
+                        }
+                        done = true;
                     }
                 }
+                if (!done) {
+#pragma unroll
+                    for (int h = 0; h < PD; ++h) {
+                        const int e = (j * 4 + k) * PD + h;
+                        const float z = Pack<DT>::get(zraw[j][k], h);
+                        if (p.rms) {
+                            d[e] = mxq_round_dt<ADT>(d[e] - Q(z * t));
+                        } else {
+                            d[e] = Q(d[e] + Q(t * z));
+                            sum2 += valid ? d[e] : 0.0f;
+                        }
+                    }
+                }
+            }
         }
         const float dm = p.rms ? 0.0f : -Q(Q(row_reduce<SumOp, WPR>(sum2, part)) / count);
+        if constexpr (CAN_PLAIN) plain = __all(plain && (p.rms || scalar_within(dm, 0x21800000u, 0x67800000u, true)));
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
             u32x4 o;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                float q[2];
-#pragma unroll
-                for (int h = 0; h < PD; ++h) {
-                    const float v = d[(j * 4 + k) * PD + h];
-                    q[h] = p.rms ? v : Q(v + dm);
+                bool done = false;
+                if constexpr (CAN_PLAIN) {
+                    if (plain && !p.rms) {
+                        const int e = (j * 4 + k) * 2;
+                        o[k] = plain_packed(d[e] + dm, d[e + 1] + dm);
+                        done = true;
+                    }
                 }
-                o[k] = Pack<DT>::put(q[0], q[PD - 1]);
+                if (!done) {
+                    float q[2];
+#pragma unroll
+                    for (int h = 0; h < PD; ++h) {
+                        const float v = d[(j * 4 + k) * PD + h];
+                        q[h] = p.rms ? v : Q(v + dm);
+                    }
+                    o[k] = Pack<DT>::put(q[0], q[PD - 1]);
+                }
             }
             if (j * LPR + lane < nvec) __builtin_nontemporal_store(o, &out[j * LPR + lane]);
         }
