@@ -84,6 +84,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
         // and so is 1.4453125 (x - m): the plain form again.  Any other wave takes the general form.
         bool plain = QMODE == SMQ_BF16 && !p.q.general_only;
         auto in_plain_range = [](uint32_t ua) { return ua - 0x0D800000u < 0x64000000u; };   // [2^-100, 2^100)
+        float lowest = __builtin_inff();                     // of this lane's quantized inputs
 #pragma unroll
         for (int j = 0; j < VPL; ++j) {
             const bool valid = j * LPR + lane < nvec;
@@ -96,6 +97,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
                     if (QMODE == SMQ_BF16) {
                         plain = plain && (!valid || in_plain_range(mxq_bits(v) & 0x7FFFFFFFu));
                         x[e] = valid ? Qplain_d(v) : -__builtin_inff();
+                        lowest = fminf(lowest, valid ? x[e] : __builtin_inff());
                     } else {
                         x[e] = valid ? Qd(v) : -__builtin_inff();
                     }
@@ -142,9 +144,46 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
                 }
             }
         };
-        if (QMODE == SMQ_BF16 && plain) exponentials(std::true_type{});
-        else exponentials(std::false_type{});
+        // Closer still: when no input of the wave lies more than 85 below the row maximum, the
+        // exponentials are normal numbers (2^-123 .. 1; exactly 0 past the end of the row), and when
+        // the smallest of them, divided by the row sum, is one too (checked below with a factor 2 to
+        // spare), so are the quotients: their quantizer needs no special cases either, and both bf16
+        // values of a pair go through it in packed form.
+        auto packed = [](float a, float b) {
+            const uint32_t w = Pack<MXQ_BF16>::put(a, b);
+            return w + (w & 0x00010001u);
+        };
+        auto low_of = [](uint32_t w) { return mxq_float(w << 16); };
+        auto high_of = [](uint32_t w) { return mxq_float(w & 0xFFFF0000u); };
+        bool close = false;
+        if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) close = __all(plain && lowest - m >= -85.0f);
+        if (close) {
+            if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
+#pragma unroll
+                for (int e = 0; e < EPL; e += 2) {
+                    uint32_t dw = packed(x[e] - m, x[e + 1] - m);
+                    if (p.exp_mode == 2) dw = packed(1.4453125f * low_of(dw), 1.4453125f * high_of(dw));
+                    const uint32_t ew = p.exp_mode == 0 ? packed(expf(low_of(dw)), expf(high_of(dw)))
+                                                        : packed(exp2f(low_of(dw)), exp2f(high_of(dw)));
+                    x[e] = low_of(ew);
+                    x[e + 1] = high_of(ew);
+                    sum += x[e];
+                    sum += x[e + 1];
+                }
+            }
+        } else if (QMODE == SMQ_BF16 && plain) {
+            exponentials(std::true_type{});
+        } else {
+            exponentials(std::false_type{});
+        }
         sum = Qp(row_reduce<SumOp, WPR>(sum, part));
+        if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
+            const float below = lowest - m;                  // +inf in a lane past the end of the row
+            const float smallest = p.exp_mode == 0 ? expf(below)
+                                                   : exp2f(p.exp_mode == 2 ? 1.4453125f * below : below);
+            close = __all(close && mxq_bits(sum) - 0x3F800000u < 0x0A000000u &&      // 1 <= sum < 2^20
+                          0.5f * smallest >= sum * 1.17549435e-38f);                 // quotients >= 2^-125
+        }
         const bool recip = p.use_recip != 0;
         const float r = recip ? Qp(1.0f / sum) : 0.0f;
         // e / sum without a division per element: one refined reciprocal per row, then a product
@@ -164,13 +203,23 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
             u32x4 o;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-                float q[2];
-#pragma unroll
-                for (int h = 0; h < PD; ++h) {
-                    const float e = x[(j * 4 + d) * PD + h];
-                    q[h] = Qp(recip ? e * r : quotient(e));
+                bool done = false;
+                if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
+                    if (close) {
+                        const float e0 = x[(j * 4 + d) * 2], e1 = x[(j * 4 + d) * 2 + 1];
+                        o[d] = recip ? packed(e0 * r, e1 * r) : packed(quotient(e0), quotient(e1));
+                        done = true;
+                    }
                 }
-                o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+                if (!done) {
+                    float q[2];
+#pragma unroll
+                    for (int h = 0; h < PD; ++h) {
+                        const float e = x[(j * 4 + d) * PD + h];
+                        q[h] = Qp(recip ? e * r : quotient(e));
+                    }
+                    o[d] = Pack<DT>::put(q[0], q[PD - 1]);
+                }
             }
             if (j * LPR + lane < nvec) __builtin_nontemporal_store(o, &out[j * LPR + lane]);
         }

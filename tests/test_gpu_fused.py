@@ -944,6 +944,17 @@ def test_softmax_shortcut_equals_general_form(dev, n, spec):
     g = torch.Generator().manual_seed(n)
     x = _edge_rows(24, n, g, -100, 100)
     x[8:16] = (torch.randn(8, n, generator=g) * 3).to(torch.bfloat16)     # ordinary logits
+    # around the limits of the form without any special case: spreads of 83 .. 86 below the
+    # maximum, smallest quotients next to the smallest normal number
+    even = torch.arange(n) % 2 == 0
+    x[16] = 1.0
+    x[17] = torch.where(even, 1.0, -82.0).to(torch.bfloat16)
+    x[18] = torch.where(even, 1.0, -83.5).to(torch.bfloat16)
+    x[19] = torch.where(even, 1.0, -85.0).to(torch.bfloat16)
+    x[20] = torch.where(torch.arange(n) == 5, 3.0, -80.0).to(torch.bfloat16)
+    x[21] = torch.linspace(-80, 5, n).to(torch.bfloat16)
+    x[22] = torch.where(torch.arange(n) < n // 2, 3.0, -75.0).to(torch.bfloat16)
+    x[23] = torch.where(torch.arange(n) < 4, 2.0, -70.0).to(torch.bfloat16)
     x[x == 0] = 1.0
     specs = _specs(**spec)
     got = softmax(x.to(dev), dim=-1, mx_specs=specs).cpu()
