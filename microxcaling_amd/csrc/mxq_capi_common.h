@@ -29,7 +29,7 @@ int grid_for(int64_t work_items_per_block_iter_total) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-int elem_size(int dtype) { return dtype == MXQ_DTYPE_F32 ? 4 : 2; }
+[[maybe_unused]] int elem_size(int dtype) { return dtype == MXQ_DTYPE_F32 ? 4 : 2; }
 
 // ---- dispatch over (dtype, rounding mode, element zone, lean) ------------------------------------
 // F is a functor template: F<DT, RMODE, ZONE_ELEM, LEAN>::run(args...).  The op-by-op form always

@@ -285,7 +285,6 @@ __global__ __launch_bounds__(TPB) void norm_row_kernel(const void* __restrict__ 
         const uint32_t u = mxq_bits(v);
         return mxq_float(u + (u & 0x10000u));
     };
-    auto Qplain = [&](float v) { return Qplain_d(mxq_round_dt<ADT>(v)); };
     auto within = [](float v, uint32_t lo, uint32_t hi) {    // lo <= |v| < hi as bit patterns
         return (mxq_bits(v) & 0x7FFFFFFFu) - lo < hi - lo;
     };
@@ -777,12 +776,15 @@ __global__ __launch_bounds__(TPB) void activation_backward_kernel(const void* __
                         (!two || halves_within(av[d], 0xFFFFu, 0x2180u, 0x3F81u));
             plain = __all(plain);                            // one branch per wave
         }
-        if (plain) {
-            if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
+        bool done = false;
+        if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
+            if (plain) {
 #pragma unroll
                 for (int d = 0; d < 4; ++d) o[d] = eval_pair(gv[d], sv[d], av[d]);
+                done = true;
             }
-        } else {
+        }
+        if (!done) {
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
                 float r[2];
