@@ -151,6 +151,22 @@ int mxq_norm_backward_lastdim(const void* grad_out, const void* weight, const vo
                               int rms_norm, int bits, int exp_bits, float max_norm, int rmode,
                               int allow_denorm, int flags, void* hip_stream);
 
+/* The gradients of the weight and the bias of the same two layers (LayerNormFunction.backward,
+ * mx/layernorm.py:51-59; RMSNormFunction.backward, mx/layernorm.py:148-156):
+ *   grad_bias = Q(sum over rows of g),  grad_weight = Q(sum over rows of Q(g * x_norm))
+ * for contiguous [rows, n] fp32 or bf16 tensors x_norm and g = Q(grad_out) (quantized on the way in,
+ * like mxq_norm_backward_lastdim does: the caller need not run that pass), Q the elementwise
+ * quantizer as in mxq_quantize_elemwise (bits == 0: none).  Sums are accumulated in fp32
+ * in a fixed order and rounded to the tensor dtype once, like torch.sum; agrees with the reference's
+ * steps up to that order.  grad_weight, grad_bias: n elements of the tensor dtype.  n must be a
+ * multiple of 16 bytes of elements.  workspace: mxq_norm_param_grads_workspace_bytes(dtype, rows, n)
+ * bytes of device memory, 16-byte aligned.  Two launches; g and x_norm are read once. */
+int64_t mxq_norm_param_grads_workspace_bytes(int dtype, int64_t rows, int64_t n);
+int mxq_norm_param_grads(const void* grad_out, const void* x_norm, void* grad_weight, void* grad_bias,
+                         void* workspace, int64_t workspace_bytes, int dtype, int64_t rows, int64_t n,
+                         int bits, int exp_bits, float max_norm, int rmode, int allow_denorm, int flags,
+                         void* hip_stream);
+
 /* The forward passes of SigmoidFunction, TanhFunction, SiLUFunction and GELUFunction
  * (mx/activations.py:237-297, 418-557) on a contiguous fp32 or bf16 tensor of n elements, as one
  * kernel, with the elementwise quantizer (bits / exp_bits / max_norm as in mxq_softmax_lastdim,

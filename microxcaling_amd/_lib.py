@@ -39,6 +39,9 @@ GPU_SYMBOLS = {
                                               _c_int, _c_f32, _c_int, _c_int, _c_int, _c_int, _c_ptr]),
     "mxq_norm_backward_lastdim": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64,
                                            _c_int, _c_int, _c_int, _c_f32, _c_int, _c_int, _c_int, _c_ptr]),
+    "mxq_norm_param_grads_workspace_bytes": (_c_i64, [_c_int, _c_i64, _c_i64]),
+    "mxq_norm_param_grads": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_i64, _c_i64,
+                                      _c_int, _c_int, _c_f32, _c_int, _c_int, _c_int, _c_ptr]),
     "mxq_binary_elemwise": (_c_int, [_c_ptr, _c_ptr, _c_f32, _c_int, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
                                      _c_int, _c_f32, _c_int, _c_int, _c_int, _c_ptr]),
     "mxq_pack_mx": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_int, _c_int, _c_int,

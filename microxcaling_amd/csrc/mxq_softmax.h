@@ -1258,4 +1258,137 @@ __global__ __launch_bounds__(TPB) void binary_kernel(const void* __restrict__ a_
     }
 }
 
+// Gradients of the weight and the bias of LayerNorm / RMSNorm over the last axis
+// (mx/layernorm.py:51-59, 148-156): with g = Q(output gradient) -- quantized here, which changes
+// nothing when the caller already has -- and z = the saved normalized input, both [rows, n],
+//   grad_bias[c] = Q(sum over rows of g[r, c]),  grad_weight[c] = Q(sum over rows of Q(g[r, c] z[r, c]))
+// where a sum is accumulated in fp32 and rounded to the tensor dtype once, as torch.sum does.
+// Two launches that read g and z once: column sums of a chunk of rows per block (fp32 partials in a
+// workspace), then the partials of a column added in a fixed order and quantized.
+//
+// norm_param_grad_partial_kernel: grid (column groups, row chunks).  A lane owns one 16-byte vector
+// of columns; the four waves of a block take every fourth row of the chunk and add their sums up
+// through LDS.  partial[(chunk * 2 + k) * n + c]: k = 0 weight, 1 bias.
+template <int DT, int RMODE, int QMODE>
+__global__ __launch_bounds__(TPB) void norm_param_grad_partial_kernel(const void* __restrict__ grad_,
+                                                                      const void* __restrict__ znorm_,
+                                                                      float* __restrict__ partial,
+                                                                      int64_t rows, int n,
+                                                                      int64_t rows_per_chunk, ElemParams q) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int PD = Pack<DT>::PER_DWORD;
+    constexpr int EPV = 4 * PD;
+    constexpr int WAVES = TPB / 64;
+    constexpr int UNROLL = 4;
+    __shared__ unsigned char zone[ZONE_PAD];
+    __shared__ float red[WAVES][2 * EPV][64];
+    load_zone(zone, g_zone_tables[q.zone_row]);
+
+    auto Qd = [&](float v) {                                 // v: a value of the tensor dtype
+        if (QMODE == SMQ_IDENT) return v;
+        if (QMODE == SMQ_BF16) return mxq_quant_bf16_to_bfloat16_nearest(v, q.fmt.nan_from);
+        return mxq_quant_elemwise<RMODE, ADT, true, true>(v, q.fmt, q.saturate != 0, q.allow_denorm != 0,
+                                                          zone, ZS);
+    };
+    auto Q = [&](float v) { return Qd(mxq_round_dt<ADT>(v)); };
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nvec_row = n / EPV;
+    const int cv = blockIdx.x * 64 + lane;
+    const bool live = cv < nvec_row;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_chunk;
+    const int64_t r1 = (r0 + rows_per_chunk < rows) ? r0 + rows_per_chunk : rows;
+    const u32x4* g = reinterpret_cast<const u32x4*>(grad_) + cv;
+    const u32x4* z = reinterpret_cast<const u32x4*>(znorm_) + cv;
+
+    float acc_w[EPV], acc_b[EPV];
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) acc_w[e] = acc_b[e] = 0.0f;
+
+    for (int64_t r = r0 + wave; r < r1; r += WAVES * UNROLL) {
+        u32x4 vg[UNROLL], vz[UNROLL];
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            const int64_t rr = r + j * WAVES;
+            const bool ok = live && rr < r1;
+            vg[j] = ok ? __builtin_nontemporal_load(&g[rr * nvec_row]) : u32x4{0, 0, 0, 0};
+            vz[j] = ok ? __builtin_nontemporal_load(&z[rr * nvec_row]) : u32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d)                    // rows past the chunk were read as +0
+#pragma unroll
+                for (int h = 0; h < PD; ++h) {
+                    const float gv = Qd(Pack<DT>::get(vg[j][d], h)), zv = Pack<DT>::get(vz[j][d], h);
+                    acc_w[d * PD + h] += Q(gv * zv);
+                    acc_b[d * PD + h] += gv;
+                }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+        red[wave][e][lane] = acc_w[e];
+        red[wave][EPV + e][lane] = acc_b[e];
+    }
+    __syncthreads();
+    if (!live) return;
+    // wave w adds up and stores entries k = w, w + WAVES, ... of this lane's 2 * EPV sums
+    float* dst = partial + (int64_t)blockIdx.y * 2 * n + (int64_t)cv * EPV;
+    for (int k = wave; k < 2 * EPV; k += WAVES) {
+        float s = red[0][k][lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) s += red[w][k][lane];
+        dst[(k / EPV) * (int64_t)n + (k % EPV)] = s;
+    }
+}
+
+// norm_param_grad_final_kernel: one lane per (k, column) pair, 64 pairs per block; wave w adds the
+// partials of its quarter of the chunks in order, the four quarter sums are added in order, the
+// result is rounded to the tensor dtype and quantized.  out_w / out_b: n elements each.
+template <int DT, int RMODE, int QMODE>
+__global__ __launch_bounds__(TPB) void norm_param_grad_final_kernel(const float* __restrict__ partial,
+                                                                    int chunks, int n,
+                                                                    void* __restrict__ out_w,
+                                                                    void* __restrict__ out_b, ElemParams q) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int WAVES = TPB / 64;
+    __shared__ unsigned char zone[ZONE_PAD];
+    __shared__ float red[WAVES][64];
+    load_zone(zone, g_zone_tables[q.zone_row]);
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t j = (int64_t)blockIdx.x * 64 + lane;         // k * n + column
+    const bool live = j < 2 * (int64_t)n;
+    const int per = (chunks + WAVES - 1) / WAVES;
+    const int c0 = wave * per, c1 = (c0 + per < chunks) ? c0 + per : chunks;
+    float s = 0.0f;
+    if (live) {
+        const float* src = partial + j;
+        const int64_t step = 2 * (int64_t)n;
+        int c = c0;
+        for (; c + 8 <= c1; c += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = src[(c + u) * step];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; c < c1; ++c) s += src[c * step];
+    }
+    red[wave][lane] = s;
+    __syncthreads();
+    if (wave != 0 || !live) return;
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) s += red[w][lane];       // +0 from a wave without chunks
+    float y = mxq_round_dt<ADT>(s);
+    if (QMODE == SMQ_BF16) y = mxq_quant_bf16_to_bfloat16_nearest(y, q.fmt.nan_from);
+    else if (QMODE != SMQ_IDENT)
+        y = mxq_quant_elemwise<RMODE, ADT, true, true>(y, q.fmt, q.saturate != 0, q.allow_denorm != 0, zone, ZS);
+    if (j < n) store_scalar<DT>(out_w, j, y);
+    else store_scalar<DT>(out_b, j - n, y);
+}
+
 }  // namespace

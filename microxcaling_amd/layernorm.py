@@ -84,8 +84,60 @@ def _fused_grad_input(grad_output, weight, x_norm, stat, mx_specs, rms):
     return out
 
 
+def _fused_param_grads(grad_output, x_norm, mx_specs):
+    """(grad_weight, grad_bias) as two kernel launches that read grad_output and x_norm once
+    (mxq_norm_param_grads), under the conditions of the other fused kernels; None otherwise."""
+    from . import _lib
+    from .custom_extensions import _flags_value
+    from .elemwise_ops import fused_chain_args
+    args = fused_chain_args(grad_output, mx_specs)
+    if args is None:
+        return None
+    g, code, (bits, exp_bits, max_norm, rmode, denorm) = args
+    n = g.shape[-1] if g.ndim else 0
+    if g.ndim < 2 or n == 0 or n % (16 // g.element_size()) != 0:
+        return None
+    rows = g.numel() // n
+    if rows == 0 or x_norm.dtype != g.dtype or x_norm.device != g.device or x_norm.shape != g.shape:
+        return None
+    g, z = g.contiguous(), x_norm.contiguous()
+    grad_weight = torch.empty(n, dtype=g.dtype, device=g.device)
+    grad_bias = torch.empty(n, dtype=g.dtype, device=g.device)
+    lib = _lib.gpu()
+    ws_bytes = lib.mxq_norm_param_grads_workspace_bytes(code, rows, n)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=g.device)
+    with torch.cuda.device(g.device):
+        rc = lib.mxq_norm_param_grads(g.data_ptr(), z.data_ptr(), grad_weight.data_ptr(),
+                                      grad_bias.data_ptr(), ws.data_ptr(), ws_bytes, code, rows, n,
+                                      bits, exp_bits, max_norm, rmode, denorm, _flags_value(),
+                                      torch.cuda.current_stream(g.device).cuda_stream)
+    _lib.check(rc, lib)
+    return grad_weight, grad_bias
+
+
+def _fused_backward(grad_output, weight, x_norm, stat, mx_specs, rms):
+    """(grad_input, grad_weight, grad_bias) from the output gradient as it arrives: both kernels
+    quantize it on the way in, so the separate quantization pass is not run.  None unless both
+    kernels cover the case."""
+    from .elemwise_ops import fused_chain_args
+    args = fused_chain_args(grad_output, mx_specs)
+    if args is None:
+        return None
+    g = args[0]                          # cast to bf16 once where the quantization is that cast
+    params = _fused_param_grads(g, x_norm, mx_specs)
+    if params is None:
+        return None
+    grad_input = _fused_grad_input(g, weight, x_norm, stat, mx_specs, rms)
+    if grad_input is None:
+        return None
+    return grad_input, params[0], params[1]
+
+
 def _param_grads(grad_output, x_norm, specs):
     """grad_bias = sum(g), grad_weight = sum(g * x_norm) over every axis but the last."""
+    fused = _fused_param_grads(grad_output, x_norm, specs)
+    if fused is not None:
+        return fused
     axes = _leading_axes(grad_output)
     grad_bias = vec_reduce_sum(grad_output, axes, mx_specs=specs)
     grad_weight = vec_reduce_sum(vec_mul(grad_output, x_norm, mx_specs=specs), axes, mx_specs=specs)
@@ -114,6 +166,9 @@ class LayerNormFunction(torch.autograd.Function):
     def backward(ctx, grad_output):
         x_norm, x_vare, weight = ctx.saved_tensors
         s = ctx.mx_specs
+        fused = _fused_backward(grad_output, weight, x_norm, x_vare, s, rms=False)
+        if fused is not None:
+            return fused + (None, None, None)
         grad_output = vec_quantize(grad_output, mx_specs=s)
         grad_weight, grad_bias = _param_grads(grad_output, x_norm, s)
         grad_input = _fused_grad_input(grad_output, weight, x_norm, x_vare, s, rms=False)
@@ -148,6 +203,9 @@ class RMSNormFunction(torch.autograd.Function):
     def backward(ctx, grad_output):
         x_norm, rms_inv, weight = ctx.saved_tensors
         s = ctx.mx_specs
+        fused = _fused_backward(grad_output, weight, x_norm, rms_inv, s, rms=True)
+        if fused is not None:
+            return fused + (None, None, None)
         grad_output = vec_quantize(grad_output, mx_specs=s)
         grad_weight, grad_bias = _param_grads(grad_output, x_norm, s)
         fused = _fused_grad_input(grad_output, weight, x_norm, rms_inv, s, rms=True)

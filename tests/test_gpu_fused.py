@@ -697,11 +697,56 @@ def test_fused_norm_backward_against_chain(dev, kind, dtype, spec, shape):
             res.append((x.grad.clone(), mod.weight.grad.clone()))
         finally:
             gemm.set_fused(True)
-    assert torch.equal(res[0][1], res[1][1])
+    step = 2.0 ** -7 if spec["bfloat"] == 16 else 2.0 ** -3        # one step of the format, relative
+    gw, gw_want = res[0][1].float().cpu(), res[1][1].float().cpu()
+    assert ((gw - gw_want).abs() <= step * gw_want.abs() + 1e-4 * gw_want.abs().max()).all()
     got, want = res[0][0].float().cpu(), res[1][0].float().cpu()
     d = (got - want).abs()
     assert d.max().item() <= 2.0 ** -5 * want.abs().max().item()
     assert (d > 0).float().mean().item() <= 0.08
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("spec", [dict(bfloat=16), dict(bfloat=12), dict(bfloat=14, round="floor")],
+                         ids=["bfloat16", "bfloat12", "bfloat14-floor"])
+@pytest.mark.parametrize("shape", [(1, 8), (5, 264), (257, 264), (6, 40, 1024), (4099, 520), (3, 16384),
+                                   (2048, 4096), (70000, 64)])
+def test_fused_norm_param_grads(dev, dtype, spec, shape):
+    """Weight and bias gradients of LayerNorm / RMSNorm as column-sum kernels against (a) the separate
+    steps (vec_mul, torch.sum, quantizer) on the GPU and (b) column sums in fp64 of the same quantized
+    products, quantized on the CPU: the order of an fp32 sum is all that differs, so a result is the
+    same number or, where the sum lies at a rounding boundary, the neighbouring one."""
+    from microxcaling_amd import gemm, layernorm as L
+    from microxcaling_amd.specs import apply_mx_specs
+    from microxcaling_amd.vector_ops import vec_mul, vec_quantize
+    specs = apply_mx_specs(_specs(**spec))
+    gen = torch.Generator().manual_seed(sum(shape))
+    g = vec_quantize((torch.randn(*shape, generator=gen) * 0.7 + 0.05).to(dtype).to(dev), mx_specs=specs)
+    z = (torch.randn(*shape, generator=gen) * 1.5).to(dtype).to(dev)
+    fused = L._fused_param_grads(g, z, specs)
+    assert fused is not None
+    gemm.set_fused(False)
+    try:
+        assert L._fused_param_grads(g, z, specs) is None
+        want_w, want_b = L._param_grads(g, z, specs)
+        prod = vec_mul(g, z, mx_specs=specs)
+    finally:
+        gemm.set_fused(True)
+    n = shape[-1]
+    bits = spec["bfloat"]
+    step = 2.0 ** -(bits - 9)                                 # one step of the format, relative
+    for got, want, terms in ((fused[0], want_w, prod), (fused[1], want_b, g)):
+        assert got.dtype == want.dtype and got.shape == want.shape == (n,)
+        got, want = got.double().cpu(), want.double().cpu()
+        terms = terms.double().reshape(-1, n)
+        slack = 1e-6 * terms.abs().sum(0).cpu()               # fp32 accumulation, any order
+        exact = terms.sum(0).cpu()
+        assert ((got - want).abs() <= step * want.abs() + slack).all()
+        # against the exact sum: the rounding to the tensor dtype and the quantizer's own (which on
+        # bf16 tensors moves odd significands up) stack to at most two steps
+        assert ((got - exact).abs() <= 2 * step * exact.abs() + slack).all()
+        if spec.get("round") != "floor":                      # every result is a value of the format
+            assert torch.equal(vec_quantize(got.to(dtype), mx_specs=specs).double(), got)
 
 
 @pytest.mark.parametrize("op,mode", [(o, m) for o in ("add", "sub", "mul", "div")
