@@ -35,27 +35,28 @@ struct LaunchPack {
 template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchPackT {
     template <int KIND>
-    static void one(unsigned grid, const u32x2* in, unsigned char* c, unsigned char* sc, int64_t items,
+    static void one(unsigned grid, const u32x2* in, unsigned char* c, unsigned char* sc, int64_t n_cgroups,
                     int64_t n_tiles, int64_t pv, MxParams p, uint32_t max_code, hipStream_t s) {
         if constexpr (!ZE) {
             if (max_code != 0u) {
-                mx_pack_t_kernel<DT, RMODE, ZE, KIND, true><<<grid, kThreads, 0, s>>>(in, c, sc, items, n_tiles, pv, p, max_code);
+                mx_pack_t_kernel<DT, RMODE, ZE, KIND, true><<<grid, kThreads, 0, s>>>(in, c, sc, n_cgroups, n_tiles, pv, p, max_code);
                 return;
             }
         }
-        mx_pack_t_kernel<DT, RMODE, ZE, KIND, false><<<grid, kThreads, 0, s>>>(in, c, sc, items, n_tiles, pv, p, 0u);
+        mx_pack_t_kernel<DT, RMODE, ZE, KIND, false><<<grid, kThreads, 0, s>>>(in, c, sc, n_cgroups, n_tiles, pv, p, 0u);
     }
-    static void run(const void* in, void* codes, void* scales, int64_t items, int64_t n_tiles,
+    static void run(const void* in, void* codes, void* scales, int64_t n_blocks, int64_t n_tiles,
                     int64_t pv, int kind, uint32_t max_code, MxParams p, hipStream_t s) {
-        const unsigned grid = (unsigned)ceil_div(items, kThreads);
+        const unsigned grid = (unsigned)n_blocks;
+        const int64_t n_cgroups = ceil_div(pv, 64);
         const u32x2* i2 = reinterpret_cast<const u32x2*>(in);
         unsigned char* c = reinterpret_cast<unsigned char*>(codes);
         unsigned char* sc = reinterpret_cast<unsigned char*>(scales);
-        if (kind == 1) one<1>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
-        else if (kind == 2) one<2>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
-        else if (kind == 3) one<3>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
-        else if (kind == 4) one<4>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
-        else one<0>(grid, i2, c, sc, items, n_tiles, pv, p, max_code, s);
+        if (kind == 1) one<1>(grid, i2, c, sc, n_cgroups, n_tiles, pv, p, max_code, s);
+        else if (kind == 2) one<2>(grid, i2, c, sc, n_cgroups, n_tiles, pv, p, max_code, s);
+        else if (kind == 3) one<3>(grid, i2, c, sc, n_cgroups, n_tiles, pv, p, max_code, s);
+        else if (kind == 4) one<4>(grid, i2, c, sc, n_cgroups, n_tiles, pv, p, max_code, s);
+        else one<0>(grid, i2, c, sc, n_cgroups, n_tiles, pv, p, max_code, s);
     }
 };
 
@@ -225,9 +226,11 @@ int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t 
     if (!in || !codes || !scales) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     if ((reinterpret_cast<uintptr_t>(in) & 7) || !aligned16(codes))
         return fail(MXQ_ERR_ARGUMENT, "%s: input must be 8-byte and codes 16-byte aligned", who);
-    const int64_t n_tiles = R / 32, pv = C / vw, items = batch * n_tiles * pv;
-    if (ceil_div(items, kThreads) > 0x7FFFFFFF) return fail(MXQ_ERR_ARGUMENT, "%s: tensor too large", who);
-    dispatch<LaunchPackT>(dtype, rmode, ze, true, in, codes, scales, items, n_tiles, pv, kind,
+    const int64_t n_tiles = R / 32, pv = C / vw;
+    // a workgroup: PACKT_TILES blocks of 32 rows x 64 column strips of 8 bytes
+    const int64_t n_blocks = batch * ceil_div(n_tiles, PACKT_TILES) * ceil_div(pv, 64);
+    if (n_blocks > 0x7FFFFFFF) return fail(MXQ_ERR_ARGUMENT, "%s: tensor too large", who);
+    dispatch<LaunchPackT>(dtype, rmode, ze, true, in, codes, scales, n_blocks, n_tiles, pv, kind,
                           direct_max_code(kind, elem_ebits, elem_mbits, p), p, (hipStream_t)hip_stream);
     return check_launch(who);
 }

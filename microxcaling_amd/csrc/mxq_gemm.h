@@ -139,27 +139,43 @@ __global__ __launch_bounds__(TPB) void mx_pack_kernel(const u32x4* __restrict__ 
 // quantize + pack + transpose: input (pre, R, C) with the shared axis = R (blocks of 32 rows, the
 // second-to-last axis), output codes (pre, C, R) and scales (pre, C, R / 32) -- the K-major operand
 // the GEMM wants when the contraction runs over R (gradients: x^T, grad_output^T, W^T).
-// A lane keeps a 32-row x 8-byte column strip in registers (like mx_strided_tile_kernel) and writes,
-// per column, the 32 codes of the block as 32 contiguous bytes.
+// A lane keeps a 32-row x 8-byte column strip in registers (like mx_strided_tile_kernel), which
+// gives, per column, the 32 codes of one block: 32 (16, 24) contiguous bytes of the output.  The
+// four waves of a workgroup take four consecutive blocks of the same 64 column strips and hand
+// their codes over through LDS, so that a column leaves as one 128 (64, 96) byte piece and its four
+// scale bytes as one word.
+// Work: blockIdx.x = (pre_i * n_tgroups + tile group) * n_cgroups + column group.
 // ================================================================================================
+constexpr int PACKT_TILES = TPB / 64;                   // blocks of 32 rows per workgroup
+static_assert(PACKT_TILES == 4, "the scale bytes of a column's blocks travel as one 32-bit word");
+
 template <int DT, int RMODE, bool ZONE_ELEM, int KIND, bool DIRECT>
 __global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict__ in,
                                                         unsigned char* __restrict__ codes,
                                                         unsigned char* __restrict__ scales,
-                                                        int64_t items, int64_t n_tiles, int64_t pv,
+                                                        int64_t n_cgroups, int64_t n_tiles, int64_t pv,
                                                         MxParams p, uint32_t max_code) {
     constexpr int ADT = Arith<DT>::DT_;
     constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
     constexpr int VW = Col8<DT>::VW;
     constexpr int PD = Pack<DT>::PER_DWORD;
     constexpr int ROWS = 32;
+    constexpr int NCOL = 64 * VW;                        // columns of a workgroup
+    constexpr int UPT = ROWS * code_bits<KIND>() / 64;   // 8-byte units of codes per block and column
+    constexpr int UPC = PACKT_TILES * UPT;               // ... per column of the workgroup
+    constexpr int LDC = UPC + 1;                         // padded column pitch in LDS
     __shared__ unsigned char zone[ZONE_PAD];
+    __shared__ u32x2 stage[NCOL * LDC];
+    __shared__ uint32_t stage_scales[NCOL];
 
-    const int64_t w = (int64_t)blockIdx.x * TPB + threadIdx.x;     // (pre_i, tile_i, column group)
-    const bool live = w < items;
-    const int64_t c = live ? w % pv : 0;
-    const int64_t pt = live ? w / pv : 0;                           // pre_i * n_tiles + tile_i
-    const int64_t off0 = pt * ROWS * pv + c;                        // in units of 8 bytes
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t n_tgroups = (n_tiles + PACKT_TILES - 1) / PACKT_TILES;
+    const int64_t cg = blockIdx.x % n_cgroups, rest = blockIdx.x / n_cgroups;
+    const int64_t tg = rest % n_tgroups, pre_i = rest / n_tgroups;
+    const int64_t c = cg * 64 + lane;                               // column strip
+    const int64_t tile_i = tg * PACKT_TILES + wave;
+    const bool live = c < pv && tile_i < n_tiles;
+    const int64_t off0 = live ? ((pre_i * n_tiles + tile_i) * ROWS) * pv + c : 0;   // in units of 8 bytes
 
     u32x2 raw[ROWS];
 #pragma unroll
@@ -177,8 +193,7 @@ __global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict_
             for (int h = 0; h < PD; ++h)
                 um[d * PD + h] = max(um[d * PD + h], abs_bits(Pack<DT>::get(raw[r][d], h)));
 
-    const int64_t pre_i = pt / n_tiles, tile_i = pt % n_tiles;
-    const int64_t C = pv * VW, R = n_tiles * ROWS;
+    uint32_t scale_bytes[VW];
 #pragma unroll
     for (int k = 0; k < VW; ++k) {
         const MxqScale sc = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, ZS);
@@ -193,22 +208,40 @@ __global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict_
             } else if (KIND == 4) out[r / 8] |= code << (4 * (r % 8));
             else out[r / 4] |= code << (8 * (r % 4));
         }
-        if (live) {
-            const int64_t col = c * VW + k;
-            if (code_bits<KIND>() == 6) {
-                u32x2* dst = reinterpret_cast<u32x2*>(codes + ((pre_i * C + col) * R + tile_i * ROWS) / 4 * 3);
-                dst[0] = u32x2{out[0], out[1]};
-                dst[1] = u32x2{out[2], out[3]};
-                dst[2] = u32x2{out[4], out[5]};
-            } else if (KIND == 4) {
-                *reinterpret_cast<u32x4*>(codes + ((pre_i * C + col) * R + tile_i * ROWS) / 2) =
-                    u32x4{out[0], out[1], out[2], out[3]};
+        u32x2* dst = stage + (lane * VW + k) * LDC + wave * UPT;
+#pragma unroll
+        for (int u = 0; u < UPT; ++u) dst[u] = u32x2{out[2 * u], out[2 * u + 1]};
+        scale_bytes[k] = mxq_encode_e8m0(sc.scale);
+    }
+#pragma unroll
+    for (int k = 0; k < VW; ++k)
+        reinterpret_cast<unsigned char*>(stage_scales)[(lane * VW + k) * PACKT_TILES + wave] =
+            (unsigned char)scale_bytes[k];
+    __syncthreads();
+
+    // hand-over: consecutive lanes write consecutive 8-byte units of a column
+    const int64_t C = pv * VW;
+    const int64_t col0 = cg * NCOL;
+    const int64_t t0 = tg * PACKT_TILES;
+    const int live_tiles = (n_tiles - t0 < PACKT_TILES) ? (int)(n_tiles - t0) : PACKT_TILES;
+    const int live_units = live_tiles * UPT;
+    const int64_t col_bytes = n_tiles * (UPT * 8);                  // bytes of codes per output column
+    for (int q = threadIdx.x; q < NCOL * UPC; q += TPB) {
+        const int cb = q / UPC, u = q % UPC;
+        if (u < live_units && col0 + cb < C) {
+            u32x2* dst = reinterpret_cast<u32x2*>(codes + (pre_i * C + col0 + cb) * col_bytes + t0 * (UPT * 8));
+            dst[u] = stage[cb * LDC + u];
+        }
+    }
+    for (int cb = threadIdx.x; cb < NCOL; cb += TPB) {
+        if (col0 + cb < C) {
+            unsigned char* dst = scales + (pre_i * C + col0 + cb) * n_tiles + t0;
+            const uint32_t word = stage_scales[cb];
+            if (live_tiles == PACKT_TILES && (reinterpret_cast<uintptr_t>(dst) & 3) == 0) {
+                *reinterpret_cast<uint32_t*>(dst) = word;
             } else {
-                u32x4* dst = reinterpret_cast<u32x4*>(codes + (pre_i * C + col) * R + tile_i * ROWS);
-                dst[0] = u32x4{out[0], out[1], out[2], out[3]};
-                dst[1] = u32x4{out[4], out[5], out[6], out[7]};
+                for (int t = 0; t < live_tiles; ++t) dst[t] = (unsigned char)(word >> (8 * t));
             }
-            scales[(pre_i * C + col) * n_tiles + tile_i] = (unsigned char)mxq_encode_e8m0(sc.scale);
         }
     }
 }

@@ -138,7 +138,7 @@ def test_gemm_epilogue_quantization_equals_separate_steps(dev, M, N, K, batch, w
 @pytest.mark.parametrize("fmt", PACKABLE)
 @pytest.mark.parametrize("rnd", ["nearest", "floor", "even"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(64, 40), (3, 96, 264), (128, 8)])
+@pytest.mark.parametrize("shape", [(64, 40), (3, 96, 264), (128, 8), (160, 1032), (2, 288, 520), (1024, 64)])
 def test_transposing_pack_equals_axis_minus2_quantization(dev, fmt, rnd, dtype, shape):
     """pack_mx_t = quantize along the second-to-last axis, transposed: bit for bit, including
     blocks with zeros, subnormals and NaN."""
