@@ -140,7 +140,10 @@ int launch_gemm_dt(int64_t batch, const GemmArgs& g, void* workspace, int64_t wo
             gemm_split_reduce_kernel<ODT><<<(unsigned)ceil_div(items, kThreads), kThreads, 0, s>>>(
                 reinterpret_cast<const float*>(workspace), g.c, g.bias, g.q_nan_from, splits, rows, g.N);
         } else {
-            mx_gemm_nt_kernel<CB, BL, ODT><<<dim3(tiles, (unsigned)batch), kThreads, 0, s>>>(g);
+            if (g.kbytes == GEMM_BK)
+                mx_gemm_nt_kernel<CB, BL, ODT, true><<<dim3(tiles, (unsigned)batch), kThreads, 0, s>>>(g);
+            else
+                mx_gemm_nt_kernel<CB, BL, ODT><<<dim3(tiles, (unsigned)batch), kThreads, 0, s>>>(g);
         }
     }
     return MXQ_OK;

@@ -478,7 +478,9 @@ __device__ __forceinline__ void swap_with_lane16(u32x4& a, u32x4& b) {
     }
 }
 
-template <int CBSZ, int BLGP, int OUT_DT>
+// ONE_STEP: K is a single 128-byte step (attention-shaped products, head_dim 128 or 256 nibbles):
+// no second fetch to wait for, no second hand-over through LDS.
+template <int CBSZ, int BLGP, int OUT_DT, bool ONE_STEP = false>
 __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     constexpr bool PAIR = OUT_DT != MXQ_F32;
     constexpr int EPB = (CBSZ == 4) ? 2 : 1;                 // elements per byte of codes
@@ -562,7 +564,7 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     for (int step = 0; step < nk; ++step) {
         // next tile (the last step fetches one it does not use: no branches in the loop body, so
         // the instruction order below survives compilation); it arrives while this step computes
-        fetch(kof(step + 1));
+        if constexpr (!ONE_STEP) fetch(kof(step + 1));
         __builtin_amdgcn_sched_barrier(0);
 
         v8i bf[4];
@@ -594,9 +596,11 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
             }
         }
         __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();                                     // every wave is done with this tile
-        stash();
-        __syncthreads();
+        if constexpr (!ONE_STEP) {
+            __syncthreads();                                 // every wave is done with this tile
+            stash();
+            __syncthreads();
+        }
     }
 
     const int64_t cbase = ((int64_t)blockIdx.z * gridDim.y + bz) * g.batch_c;
