@@ -73,6 +73,19 @@ int mxq_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre, i
                             float elem_max_norm, int64_t tile_size, int flush_fp32_subnorms,
                             int rmode, int flags, void* hip_stream);
 
+/* _quantize_mx with one exponent shared over the blocks of two or three axes at once, e.g. tiles of
+ * 32 x 32 elements (mx/mx_ops.py:226-298 with len(axes) > 1, blocks built by _reshape_to_blocks,
+ * mx/mx_ops.py:95-154).  The reference serves this case on its pure-PyTorch path only, its extension
+ * takes a single axis (mx/mx_ops.py:240-246).  The contiguous tensor is described by
+ * extents[0 .. 2 * n_axes]: outer_0, shared_0, outer_1, shared_1, ..., outer_n, where outer_i is the
+ * product of the axes between two shared ones (1 if there is none); n_axes in 1..3.  A tile takes
+ * tile_size consecutive positions of every shared axis (shorter at the end of an axis;
+ * tile_size <= 0: the whole axis). */
+int mxq_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, const int64_t* extents,
+                         int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                         int64_t tile_size, int flush_fp32_subnorms, int rmode, int flags,
+                         void* hip_stream);
+
 /* quantize_mx_func_cuda (mx/cpp/funcs.cpp:154-175, mx/cpp/mx.cu:12-110).
  * As above, but the shared exponent of element (i, k, j) comes from max_values[i * post + j]
  * (the keepdim abs-max over the middle axis, same dtype as `in`). */
@@ -254,7 +267,7 @@ int mxq_probe_mfma_rate(int64_t workgroups, int iters, int code_kind, void* sink
  * (mx/cpp/funcs.cpp:117-149) take CPU tensors; these are their stand-ins.  Pointers are host
  * pointers and the calls run synchronously on the calling thread.  The by-tile variant has no
  * CPU counterpart in the reference; it mirrors mxq_quantize_mx_by_tile so the kernel arithmetic
- * can be checked on a machine without a GPU. */
+ * can be checked on a machine without a GPU.  mxq_host_quantize_mx_axes mirrors mxq_quantize_mx_axes. */
 #define MXQ_HOST_FLAG_ROUND_EVERY_OP 2 /* bf16: round to bf16 after every op, no shortcuts */
 #define MXQ_HOST_FLAG_CLOSED_FORM 4    /* elementwise, bf16 tensor -> bfloat16, nearest: the closed
                                           form the fused softmax kernel uses (else: an error) */
@@ -270,6 +283,9 @@ int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t p
                                  int64_t axis_size, int64_t post, int scale_bits, int elem_ebits,
                                  int elem_mbits, float elem_max_norm, int64_t tile_size,
                                  int flush_fp32_subnorms, int rmode, int flags);
+int mxq_host_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, const int64_t* extents,
+                              int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                              int64_t tile_size, int flush_fp32_subnorms, int rmode, int flags);
 int mxq_host_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int bits,
                                int exp_bits, float max_norm, int rmode, int saturate_normals,
                                int allow_denorm, int flags);

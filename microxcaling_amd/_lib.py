@@ -22,6 +22,8 @@ GPU_SYMBOLS = {
     "mxq_quantize_mx_by_tile": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int,
                                          _c_int, _c_int, _c_f32, _c_i64, _c_int, _c_int, _c_int,
                                          _c_ptr]),
+    "mxq_quantize_mx_axes": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_f32,
+                                      _c_i64, _c_int, _c_int, _c_int, _c_ptr]),
     "mxq_quantize_mx_given_max": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64,
                                            _c_int, _c_int, _c_int, _c_f32, _c_int, _c_int, _c_int,
                                            _c_ptr]),
@@ -67,6 +69,8 @@ HOST_SYMBOLS = {
     "mxq_host_quantize_mx_by_tile": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64,
                                               _c_int, _c_int, _c_int, _c_f32, _c_i64, _c_int,
                                               _c_int, _c_int]),
+    "mxq_host_quantize_mx_axes": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int,
+                                           _c_f32, _c_i64, _c_int, _c_int, _c_int]),
     "mxq_host_quantize_elemwise": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_f32,
                                             _c_int, _c_int, _c_int, _c_int]),
 }

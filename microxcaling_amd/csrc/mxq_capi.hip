@@ -53,6 +53,14 @@ struct LaunchStrided {
 };
 
 template <int DT, int RMODE, bool ZE, bool LEAN>
+struct LaunchAxes {
+    static void run(const void* in, void* out, MxqAxes a, int64_t n_tiles, MxParams p, hipStream_t s) {
+        const int64_t grid = n_tiles < 8 * kMaxBlocks ? n_tiles : 8 * kMaxBlocks;
+        mx_axes_kernel<DT, RMODE, ZE, LEAN><<<(unsigned)grid, kThreads, 0, s>>>(in, out, a, n_tiles, p);
+    }
+};
+
+template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchGivenMax {
     static void run(const void* in, void* out, const void* maxv, int64_t total, int64_t axis,
                     int64_t post, MxParams p, hipStream_t s) {
@@ -168,6 +176,27 @@ int mxq_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre, i
         }
     }
     dispatch<LaunchStrided>(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, pre, axis_size, post, tile, ptr_ok, p, s);
+    return check_launch(who);
+}
+
+int mxq_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, const int64_t* extents,
+                         int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                         int64_t tile_size, int flush_fp32_subnorms, int rmode, int flags,
+                         void* hip_stream) {
+    const char* who = "mxq_quantize_mx_axes";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    MxqAxes a;
+    int64_t total;
+    rc = make_mx_axes(n_axes, extents, tile_size, &a, &total, who);
+    if (rc) return rc;
+    if (total == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    dispatch<LaunchAxes>(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, a, mxq_axes_tiles(a), p,
+                         (hipStream_t)hip_stream);
     return check_launch(who);
 }
 

@@ -50,6 +50,45 @@ MXQ_HD float mxq_round_dt(float f) {
     return f;
 }
 
+// ---- exponent shared over the blocks of several axes ----------------------------------------------
+// A contiguous tensor seen as (o[0], s[0], o[1], s[1], o[2], s[2], o[3]): up to three shared axes s
+// with the products o of the axes around them; unused places have extent 1.  A tile takes t[i]
+// consecutive positions of every shared axis (the last tile of an axis may be shorter) and one
+// position of every other axis (mx/mx_ops.py:95-154 with several axes).
+struct MxqAxes {
+    int64_t o[4];
+    int64_t s[3];
+    int64_t t[3];       // tile extent along each shared axis
+    int64_t nb[3];      // tiles along each shared axis
+};
+MXQ_HD int64_t mxq_axes_tiles(const MxqAxes& a) {
+    return a.o[0] * a.nb[0] * a.o[1] * a.nb[1] * a.o[2] * a.nb[2] * a.o[3];
+}
+// tile number -> offset of its first element, its extents len[] and the element strides st[] of
+// the shared axes
+MXQ_HD void mxq_axes_tile(const MxqAxes& a, int64_t tile, int64_t* base, int64_t len[3], int64_t st[3]) {
+    st[2] = a.o[3];
+    const int64_t st_o2 = a.s[2] * st[2];
+    st[1] = a.o[2] * st_o2;
+    const int64_t st_o1 = a.s[1] * st[1];
+    st[0] = a.o[1] * st_o1;
+    const int64_t st_o0 = a.s[0] * st[0];
+    int64_t r = tile;
+    const int64_t i3 = r % a.o[3]; r /= a.o[3];
+    const int64_t b2 = r % a.nb[2]; r /= a.nb[2];
+    const int64_t i2 = r % a.o[2]; r /= a.o[2];
+    const int64_t b1 = r % a.nb[1]; r /= a.nb[1];
+    const int64_t i1 = r % a.o[1]; r /= a.o[1];
+    const int64_t b0 = r % a.nb[0]; r /= a.nb[0];
+    *base = r * st_o0 + b0 * a.t[0] * st[0] + i1 * st_o1 + b1 * a.t[1] * st[1] + i2 * st_o2 +
+            b2 * a.t[2] * st[2] + i3;
+    const int64_t b[3] = {b0, b1, b2};
+    for (int k = 0; k < 3; ++k) {
+        const int64_t left = a.s[k] - b[k] * a.t[k];
+        len[k] = left < a.t[k] ? left : a.t[k];
+    }
+}
+
 // ---- element format ----------------------------------------------------------------------------
 struct MxqFmt {
     int ebits;          // exponent bits, 0 for integer formats

@@ -102,6 +102,43 @@ int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t p
     return MXQ_OK;
 }
 
+int mxq_host_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, const int64_t* extents,
+                              int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
+                              int64_t tile_size, int flush_fp32_subnorms, int rmode, int flags) {
+    const char* who = "mxq_host_quantize_mx_axes";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, rmode, flags, &p, &ze, who);
+    if (rc) return rc;
+    MxqAxes a;
+    int64_t total;
+    rc = make_mx_axes(n_axes, extents, tile_size, &a, &total, who);
+    if (rc) return rc;
+    if (total == 0) return MXQ_OK;
+    if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    const unsigned char* zone = kZone[p.zone_row];
+    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
+    const int64_t n_tiles = mxq_axes_tiles(a);
+    for (int64_t tile = 0; tile < n_tiles; ++tile) {
+        int64_t base, len[3], st[3];
+        mxq_axes_tile(a, tile, &base, len, st);
+        uint32_t um = 0;
+        for (int64_t i = 0; i < len[0]; ++i)
+            for (int64_t j = 0; j < len[1]; ++j)
+                for (int64_t k = 0; k < len[2]; ++k)
+                    um = std::max(um, mxq_bits(load_as_float(in, dtype, base + i * st[0] + j * st[1] + k * st[2])) & 0x7FFFFFFFu);
+        MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+        for (int64_t i = 0; i < len[0]; ++i)
+            for (int64_t j = 0; j < len[1]; ++j)
+                for (int64_t k = 0; k < len[2]; ++k) {
+                    const int64_t idx = base + i * st[0] + j * st[1] + k * st[2];
+                    store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift));
+                }
+    }
+    return MXQ_OK;
+}
+
 int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_values, int dtype,
                                    int64_t pre, int64_t axis_size, int64_t post, int scale_bits,
                                    int elem_ebits, int elem_mbits, float elem_max_norm,

@@ -338,6 +338,45 @@ __global__ __launch_bounds__(TPB) void mx_strided_kernel(const void* __restrict_
 }
 
 // ================================================================================================
+// MX quantization with the exponent shared over the blocks of two or three axes at once (tiles of
+// e.g. 32 x 32 elements): one workgroup per tile, two passes over the tile (the second reads it
+// from cache).  Serves the general case at any shape; the single-axis kernels above are the
+// fast path.
+// ================================================================================================
+template <int DT, int RMODE, bool ZONE_ELEM, bool LEAN>
+__global__ __launch_bounds__(TPB) void mx_axes_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                      MxqAxes a, int64_t n_tiles, MxParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    __shared__ unsigned char zone[ZONE_PAD];
+    __shared__ uint32_t wave_max[TPB / 64];
+    load_zone(zone, g_zone_tables[p.zone_row]);
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        int64_t base, len[3], st[3];
+        mxq_axes_tile(a, tile, &base, len, st);
+        const int64_t count = len[0] * len[1] * len[2], l12 = len[1] * len[2];
+        auto offset = [&](int64_t e) {
+            const int64_t i0 = e / l12, r = e % l12;
+            return base + i0 * st[0] + (r / len[2]) * st[1] + (r % len[2]) * st[2];
+        };
+        uint32_t um = 0;
+        for (int64_t e = threadIdx.x; e < count; e += TPB) um = max(um, abs_bits(load_scalar<DT>(in, offset(e))));
+        for (int d = 32; d >= 1; d >>= 1) um = max(um, (uint32_t)__shfl_xor((int)um, d, 64));
+        if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = um;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < TPB / 64; ++w) um = max(um, wave_max[w]);
+        const MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+        for (int64_t e = threadIdx.x; e < count; e += TPB) {
+            const int64_t off = offset(e);
+            store_scalar<DT>(out, off, mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, LEAN>(load_scalar<DT>(in, off), sc,
+                                                                                      p.fmt, zone, ZS));
+        }
+        __syncthreads();                                     // wave_max is reused by the next tile
+    }
+}
+
+// ================================================================================================
 // MX quantization with the block maximum supplied by the caller: element (i, k, j) uses
 // max_values[i * post + j].
 // ================================================================================================

@@ -61,6 +61,30 @@ inline bool mul_overflows(int64_t a, int64_t b, int64_t c, int64_t* out) {
     return false;
 }
 
+// extents: o0, s0, o1, ..., s(n-1), o(n): 2 * n_axes + 1 values.  tile_size <= 0: whole axes.
+inline int make_mx_axes(int n_axes, const int64_t* extents, int64_t tile_size, MxqAxes* a, int64_t* total,
+                        const char* who) {
+    if (n_axes < 1 || n_axes > 3) return fail(MXQ_ERR_ARGUMENT, "%s: %d shared axes (1 to 3 supported)", who, n_axes);
+    if (!extents) return fail(MXQ_ERR_ARGUMENT, "%s: null extents", who);
+    for (int k = 0; k < 4; ++k) a->o[k] = 1;
+    for (int k = 0; k < 3; ++k) a->s[k] = a->t[k] = a->nb[k] = 1;
+    __int128 n = 1;
+    for (int k = 0; k <= 2 * n_axes; ++k) {
+        if (extents[k] < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+        n *= extents[k];
+        if (n > (__int128)INT64_MAX) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+        if (k % 2 == 0) a->o[k / 2] = extents[k];
+        else a->s[k / 2] = extents[k];
+    }
+    *total = (int64_t)n;
+    if (*total == 0) return MXQ_OK;
+    for (int k = 0; k < n_axes; ++k) {
+        a->t[k] = (tile_size <= 0 || tile_size > a->s[k]) ? a->s[k] : tile_size;
+        a->nb[k] = ceil_div(a->s[k], a->t[k]);
+    }
+    return MXQ_OK;
+}
+
 inline int make_fmt(int dtype, int ebits, int mbits, float max_norm, MxqFmt* fmt, const char* who) {
     if (ebits < 0 || ebits > 8) return fail(MXQ_ERR_ARGUMENT, "%s: exponent bits %d outside [0, 8]", who, ebits);
     if (mbits < 2 || mbits > 24)

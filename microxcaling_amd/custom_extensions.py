@@ -5,6 +5,7 @@ with the same names, positional order, defaults and error type (RuntimeError).  
 take contiguous tensors on a HIP device and launch on torch's current stream for that device;
 the two ``*_cpp`` functions take CPU tensors.  Outputs are new tensors; inputs are not modified.
 """
+import math
 import types
 
 import torch
@@ -244,6 +245,54 @@ def quantize_mx_by_tile_func_cpp(A, scale_bits, elem_ebits, elem_mbits, elem_max
     return out
 
 
+def _axes_extents(shape, axes, who):
+    """(outer_0, shared_0, outer_1, ..., shared_n-1, outer_n) for sorted, distinct axes, as a ctypes
+    int64 array."""
+    import ctypes
+    axes = list(axes)
+    if not 1 <= len(axes) <= 3 or sorted(set(axes)) != axes or not all(0 <= a < len(shape) for a in axes):
+        raise RuntimeError("%s: axes must be one to three distinct, sorted, valid dimensions" % who)
+    ext, lo = [], 0
+    for a in axes:
+        ext += [math.prod(shape[lo:a]), int(shape[a])]
+        lo = a + 1
+    ext.append(math.prod(shape[lo:]))
+    return (ctypes.c_int64 * len(ext))(*ext)
+
+
+def quantize_mx_axes_func_cuda(A, scale_bits, elem_ebits, elem_mbits, elem_max_norm, tile_size, axes,
+                               flush_fp32_subnorms=False, rmode=0):
+    """MX quantization with the exponent shared over the blocks of several axes at once (tiles of
+    tile_size positions of every axis in `axes`; tile_size <= 0: whole axes).  Not in the
+    reference's extension, which takes one axis (mx/mx_ops.py:240-246)."""
+    who = "quantize_mx_axes_func_cuda"
+    _check_gpu_input(A, "A", who)
+    ext = _axes_extents(A.shape, axes, who)
+    out = torch.empty_like(A)
+    lib = _lib.gpu()
+    with torch.cuda.device(A.device):
+        rc = lib.mxq_quantize_mx_axes(A.data_ptr(), out.data_ptr(), _dtype_code(A, who), len(axes), ext,
+                                      scale_bits, elem_ebits, elem_mbits, elem_max_norm, tile_size,
+                                      int(bool(flush_fp32_subnorms)), int(rmode), _flags, _stream(A))
+    _lib.check(rc, lib)
+    return out
+
+
+def quantize_mx_axes_func_cpp(A, scale_bits, elem_ebits, elem_mbits, elem_max_norm, tile_size, axes,
+                              flush_fp32_subnorms=False, rmode=0):
+    """CPU twin of quantize_mx_axes_func_cuda."""
+    who = "quantize_mx_axes_func_cpp"
+    _check_cpu_input(A, "A", who)
+    ext = _axes_extents(A.shape, axes, who)
+    out = torch.empty_like(A)
+    lib = _lib.host()
+    rc = lib.mxq_host_quantize_mx_axes(A.data_ptr(), out.data_ptr(), _dtype_code(A, who), len(axes), ext,
+                                       scale_bits, elem_ebits, elem_mbits, elem_max_norm, tile_size,
+                                       int(bool(flush_fp32_subnorms)), int(rmode), _flags)
+    _lib.check(rc, lib, "mxq_host_last_error")
+    return out
+
+
 funcs = types.SimpleNamespace(
     quantize_mx_func_cpp=quantize_mx_func_cpp,
     quantize_elemwise_func_cpp=quantize_elemwise_func_cpp,
@@ -256,4 +305,6 @@ funcs = types.SimpleNamespace(
     quantize_mx_by_tile_func_cpp=quantize_mx_by_tile_func_cpp,
     reduce_sum_outer_dim=reduce_sum_outer_dim,
     reduce_max_outer_dim=reduce_max_outer_dim,
+    quantize_mx_axes_func_cuda=quantize_mx_axes_func_cuda,
+    quantize_mx_axes_func_cpp=quantize_mx_axes_func_cpp,
 )

@@ -5,11 +5,12 @@ One shared 2^k scale per `block_size` consecutive elements along one axis; eleme
 `elem_format` relative to that scale and returned in the input dtype ("fake quantization").
 
 Differences from the reference, on purpose:
-  * every single-axis case -- any axis, any block size, ragged last block -- is one kernel launch
-    (the reference reshapes, pads and takes a separate max for block sizes above 32 on the last
-    axis, mx/mx_ops.py:226-263); results are bit-identical to its pure-PyTorch path either way,
-    so ``custom_cuda`` is accepted but does not change the result;
-  * sharing an exponent across more than one axis and ``round='dither'`` raise.
+  * every case -- any axis, any block size, ragged last block, an exponent shared over the blocks
+    of up to three axes at once -- is one kernel launch (the reference reshapes, pads and takes a
+    separate max for block sizes above 32 on the last axis, and serves several axes on its
+    pure-PyTorch path only, mx/mx_ops.py:226-263); results are bit-identical to its pure-PyTorch
+    path either way, so ``custom_cuda`` is accepted but does not change the result;
+  * ``round='dither'`` raises.
 """
 import torch
 
@@ -29,9 +30,11 @@ def _quantize_mx(A, scale_bits, elem_format, shared_exp_method="max", axes=None,
                         "block size to")
     axes = [axes] if type(axes) == int else list(axes)
     axes = [x + A.ndim if x < 0 else x for x in axes]
-    if len(axes) != 1:
-        raise NotImplementedError("the native kernels share exponents along exactly one axis")
-    axis = axes[0]
+    axes = sorted(axes)
+    if len(axes) == 0 or len(set(axes)) != len(axes):
+        raise ValueError("axes must name at least one dimension, each once")
+    if len(axes) > 3:
+        raise NotImplementedError("the native kernels share an exponent over at most three axes")
     rmode = _native_round(round)
     ebits, mbits, _, max_norm, _ = _get_format_params(elem_format)
 
@@ -44,6 +47,12 @@ def _quantize_mx(A, scale_bits, elem_format, shared_exp_method="max", axes=None,
 
     from . import custom_extensions as ce
     A = A.contiguous()
+    if len(axes) > 1 and tile != 1:          # one exponent per tile of tile x tile (x tile) elements
+        fn = {"cuda": ce.funcs.quantize_mx_axes_func_cuda, "cpu": ce.funcs.quantize_mx_axes_func_cpp}.get(A.device.type)
+        if fn is None:
+            raise ValueError("Unrecognized device type %s" % A.device.type)
+        return fn(A, scale_bits, ebits, mbits, max_norm, tile, axes, flush_fp32_subnorms, rmode)
+    axis = axes[-1]                          # blocks of one element: any axis serves
     if A.device.type == "cuda":
         return ce.funcs.quantize_mx_by_tile_func_cuda(
             A, scale_bits, ebits, mbits, max_norm, tile, axis, flush_fp32_subnorms, rmode)

@@ -211,6 +211,24 @@ def test_mx_shapes(dev, shape, axis, bs, dtype):
         assert_bits_equal(got, want, "%s %s %s" % (shape, fmt, rnd))
 
 
+@pytest.mark.parametrize("shape,axes,bs", [((70, 45), [-2, -1], 32), ((3, 40, 5, 33), [1, 3], 8),
+                                           ((6, 10, 12), [0, 1, 2], 4), ((5, 64, 64), [1, 2], 0),
+                                           ((4, 7, 9), [2, 0], 32), ((2, 3, 4, 5, 6), [1, 2, 4], 2),
+                                           ((256, 384), [0, 1], 32), ((3, 100, 300), [1, 2], 64)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mx_several_axes(dev, shape, axes, bs, dtype):
+    """One exponent per tile of bs x bs (x bs) elements over two or three axes (mx/mx_ops.py:95-154,
+    226-298 with len(axes) > 1), against the oracle's restatement of the pure path."""
+    g = torch.Generator().manual_seed(sum(shape) + bs)
+    x = (torch.randn(*shape, generator=g) * torch.exp2(torch.randint(-12, 12, shape, generator=g).float())).to(dtype)
+    x.view(-1)[3] = 0.0
+    x.view(-1)[-1] = float("nan")
+    for fmt, rnd in (("fp8_e4m3", "nearest"), ("fp6_e3m2", "floor"), ("fp4_e2m1", "even"), ("int8", "nearest")):
+        want = O.quantize_mx(x, 8, fmt, axes=axes, block_size=bs, round=rnd)
+        got = mx_gpu(x.to(dev), 8, fmt, axes=axes, block_size=bs, round=rnd)
+        assert_bits_equal(got, want, "%s %s %s" % (shape, fmt, rnd))
+
+
 def test_mx_given_max_entry_point(dev):
     """quantize_mx_func_cuda: the caller reshapes to blocks and supplies the abs-max
     (mx/mx_ops.py:226-256)."""

@@ -80,7 +80,9 @@ def test_host_functions_reject_gpu_only_misuse():
     with pytest.raises(NotImplementedError):
         _quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=2, round="dither")
     with pytest.raises(NotImplementedError):
-        _quantize_mx(x, 8, "fp8_e4m3", axes=[0, 1], block_size=2)
+        _quantize_mx(torch.zeros(2, 2, 2, 2), 8, "fp8_e4m3", axes=[0, 1, 2, 3], block_size=2)
+    with pytest.raises(ValueError):
+        _quantize_mx(x, 8, "fp8_e4m3", axes=[1, -1], block_size=2)           # the same axis twice
 
 
 # ---- round-up zones against torch's own log2 ----------------------------------------------------
@@ -278,6 +280,55 @@ def test_mx_shapes_on_host(shape, axis, bs):
         x = (torch.randn(*shape, generator=g) * torch.exp(torch.randn(*shape, generator=g))).to(dtype)
         want = O.quantize_mx(x, 8, "fp8_e4m3", axes=[axis], block_size=bs)
         assert_bits_equal(_quantize_mx(x, 8, "fp8_e4m3", axes=[axis], block_size=bs), want)
+
+
+MULTI_AXIS_CASES = [((70, 45), [-2, -1], 32), ((3, 40, 5, 33), [1, 3], 8), ((6, 10, 12), [0, 1, 2], 4),
+                    ((5, 64, 64), [1, 2], 0), ((4, 7, 9), [2, 0], 32), ((2, 3, 4, 5, 6), [1, 2, 4], 2),
+                    ((64, 96), [0, 1], 32)]
+
+
+def tiles_as_rows(x, bs):
+    """A 2-D tensor cut into bs x bs tiles (zero padded), one tile per row, and the way back."""
+    R, C = x.shape
+    Rp, Cp = -(-R // bs) * bs, -(-C // bs) * bs
+    xp = torch.zeros(Rp, Cp, dtype=x.dtype)
+    xp[:R, :C] = x
+    rows = xp.reshape(Rp // bs, bs, Cp // bs, bs).permute(0, 2, 1, 3).reshape(-1, bs * bs)
+
+    def back(y):
+        return y.reshape(Rp // bs, Cp // bs, bs, bs).permute(0, 2, 1, 3).reshape(Rp, Cp)[:R, :C]
+    return rows, back
+
+
+@pytest.mark.parametrize("shape", [(64, 96), (70, 45), (31, 33)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_two_axis_blocks_are_single_axis_blocks_of_the_flattened_tile(shape, dtype):
+    """An exponent shared over 32 x 32 tiles (mx/mx_ops.py:95-154 with two axes) is the single-axis
+    quantization of each tile laid out as one row of 1024: pins the oracle's multi-axis blocking, and
+    the host library's, to the single-axis path that the golden vectors cover."""
+    g = torch.Generator().manual_seed(sum(shape))
+    x = (torch.randn(*shape, generator=g) * torch.exp2(torch.randint(-15, 15, shape, generator=g).float())).to(dtype)
+    rows, back = tiles_as_rows(x, 32)
+    for fmt, rnd in (("fp8_e4m3", "nearest"), ("fp4_e2m1", "even"), ("int8", "floor")):
+        want = back(O.quantize_mx(rows, 8, fmt, axes=[-1], block_size=1024, round=rnd))
+        assert_bits_equal(O.quantize_mx(x, 8, fmt, axes=[0, 1], block_size=32, round=rnd), want, "oracle")
+        assert_bits_equal(_quantize_mx(x, 8, fmt, axes=[0, 1], block_size=32, round=rnd), want, "host library")
+
+
+@pytest.mark.parametrize("shape,axes,bs", MULTI_AXIS_CASES)
+def test_mx_several_axes_on_host(shape, axes, bs):
+    g = torch.Generator().manual_seed(sum(shape))
+    for dtype in (torch.float32, torch.bfloat16):
+        x = (torch.randn(*shape, generator=g) * torch.exp2(torch.randint(-12, 12, shape, generator=g).float())).to(dtype)
+        x.view(-1)[3] = 0.0
+        x.view(-1)[-1] = float("nan")
+        for fmt, rnd in (("fp8_e4m3", "nearest"), ("fp6_e3m2", "floor"), ("fp4_e2m1", "even"), ("int8", "nearest")):
+            want = O.quantize_mx(x, 8, fmt, axes=axes, block_size=bs, round=rnd)
+            assert_bits_equal(_quantize_mx(x, 8, fmt, axes=axes, block_size=bs, round=rnd), want,
+                              "%s %s %s" % (shape, fmt, rnd))
+    # an exponent per element: the axes do not matter
+    a = _quantize_mx(x, 8, "fp8_e4m3", shared_exp_method="none", axes=axes, block_size=bs)
+    assert_bits_equal(a, O.quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=1))
 
 
 def test_shared_exp_method_none_is_block_of_one():
