@@ -86,6 +86,19 @@ int mxq_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, const
                          int64_t tile_size, int flush_fp32_subnorms, int rmode, int flags,
                          void* hip_stream);
 
+/* round='dither' (_round_mantissa, mx/elemwise_ops.py:57-59): the scaled value is rounded as
+ * floor(|s| + noise[i]) with noise in [0, 1), one value per element in the tensor's dtype, drawn by
+ * the caller (the reference draws it with torch.rand_like and serves this mode on its pure-PyTorch
+ * path only, mx/mx_ops.py:196-197).  Otherwise as mxq_quantize_mx_by_tile / mxq_quantize_elemwise.
+ * Given the same noise the result is that of the pure path, bit for bit. */
+int mxq_quantize_mx_dither_by_tile(const void* in, const void* noise, void* out, int dtype, int64_t pre,
+                                   int64_t axis_size, int64_t post, int scale_bits, int elem_ebits,
+                                   int elem_mbits, float elem_max_norm, int64_t tile_size,
+                                   int flush_fp32_subnorms, int flags, void* hip_stream);
+int mxq_quantize_elemwise_dither(const void* in, const void* noise, void* out, int dtype, int64_t n, int bits,
+                                 int exp_bits, float max_norm, int saturate_normals, int allow_denorm,
+                                 int flags, void* hip_stream);
+
 /* quantize_mx_func_cuda (mx/cpp/funcs.cpp:154-175, mx/cpp/mx.cu:12-110).
  * As above, but the shared exponent of element (i, k, j) comes from max_values[i * post + j]
  * (the keepdim abs-max over the middle axis, same dtype as `in`). */
@@ -286,6 +299,13 @@ int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t p
 int mxq_host_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, const int64_t* extents,
                               int scale_bits, int elem_ebits, int elem_mbits, float elem_max_norm,
                               int64_t tile_size, int flush_fp32_subnorms, int rmode, int flags);
+int mxq_host_quantize_mx_dither_by_tile(const void* in, const void* noise, void* out, int dtype, int64_t pre,
+                                        int64_t axis_size, int64_t post, int scale_bits, int elem_ebits,
+                                        int elem_mbits, float elem_max_norm, int64_t tile_size,
+                                        int flush_fp32_subnorms, int flags);
+int mxq_host_quantize_elemwise_dither(const void* in, const void* noise, void* out, int dtype, int64_t n,
+                                      int bits, int exp_bits, float max_norm, int saturate_normals,
+                                      int allow_denorm, int flags);
 int mxq_host_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int bits,
                                int exp_bits, float max_norm, int rmode, int saturate_normals,
                                int allow_denorm, int flags);

@@ -24,6 +24,10 @@ GPU_SYMBOLS = {
                                          _c_ptr]),
     "mxq_quantize_mx_axes": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_f32,
                                       _c_i64, _c_int, _c_int, _c_int, _c_ptr]),
+    "mxq_quantize_mx_dither_by_tile": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int,
+                                                _c_int, _c_int, _c_f32, _c_i64, _c_int, _c_int, _c_ptr]),
+    "mxq_quantize_elemwise_dither": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_f32,
+                                              _c_int, _c_int, _c_int, _c_ptr]),
     "mxq_quantize_mx_given_max": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64,
                                            _c_int, _c_int, _c_int, _c_f32, _c_int, _c_int, _c_int,
                                            _c_ptr]),
@@ -71,6 +75,10 @@ HOST_SYMBOLS = {
                                               _c_int, _c_int]),
     "mxq_host_quantize_mx_axes": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int,
                                            _c_f32, _c_i64, _c_int, _c_int, _c_int]),
+    "mxq_host_quantize_mx_dither_by_tile": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64,
+                                                     _c_int, _c_int, _c_int, _c_f32, _c_i64, _c_int, _c_int]),
+    "mxq_host_quantize_elemwise_dither": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int,
+                                                   _c_f32, _c_int, _c_int, _c_int]),
     "mxq_host_quantize_elemwise": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_int, _c_int, _c_f32,
                                             _c_int, _c_int, _c_int, _c_int]),
 }

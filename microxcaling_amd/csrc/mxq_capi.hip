@@ -200,6 +200,53 @@ int mxq_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, const
     return check_launch(who);
 }
 
+int mxq_quantize_mx_dither_by_tile(const void* in, const void* noise, void* out, int dtype, int64_t pre,
+                                   int64_t axis_size, int64_t post, int scale_bits, int elem_ebits,
+                                   int elem_mbits, float elem_max_norm, int64_t tile_size,
+                                   int flush_fp32_subnorms, int flags, void* hip_stream) {
+    const char* who = "mxq_quantize_mx_dither_by_tile";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, MXQ_ROUND_NEAREST, flags, &p, &ze, who);
+    if (rc) return rc;
+    if (pre < 0 || axis_size < 0 || post < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    int64_t total;
+    if (mul_overflows(pre, axis_size, post, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !out || !noise) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    const int64_t tile = (tile_size <= 0 || tile_size > axis_size) ? axis_size : tile_size;
+    const int64_t num_tiles = ceil_div(axis_size, tile);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int grid = grid_for(ceil_div(pre * num_tiles * post, kThreads));
+    if (dtype == MXQ_DTYPE_F32)
+        mx_dither_kernel<MXQ_F32><<<grid, kThreads, 0, s>>>(in, noise, out, pre, axis_size, post, tile, num_tiles, p);
+    else if (dtype == MXQ_DTYPE_BF16)
+        mx_dither_kernel<MXQ_BF16><<<grid, kThreads, 0, s>>>(in, noise, out, pre, axis_size, post, tile, num_tiles, p);
+    else
+        mx_dither_kernel<MXQ_F16><<<grid, kThreads, 0, s>>>(in, noise, out, pre, axis_size, post, tile, num_tiles, p);
+    return check_launch(who);
+}
+
+int mxq_quantize_elemwise_dither(const void* in, const void* noise, void* out, int dtype, int64_t n, int bits,
+                                 int exp_bits, float max_norm, int saturate_normals, int allow_denorm,
+                                 int flags, void* hip_stream) {
+    const char* who = "mxq_quantize_elemwise_dither";
+    ElemParams p;
+    int rc = make_elem_params(dtype, bits, exp_bits, max_norm, MXQ_ROUND_NEAREST, saturate_normals, allow_denorm,
+                              flags, &p, who);
+    if (rc) return rc;
+    if (n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (n == 0) return MXQ_OK;
+    if (!in || !out || !noise) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    hipStream_t s = (hipStream_t)hip_stream;
+    const int grid = grid_for(ceil_div(n, kThreads));
+    if (dtype == MXQ_DTYPE_F32) elemwise_dither_kernel<MXQ_F32><<<grid, kThreads, 0, s>>>(in, noise, out, n, p);
+    else if (dtype == MXQ_DTYPE_BF16) elemwise_dither_kernel<MXQ_BF16><<<grid, kThreads, 0, s>>>(in, noise, out, n, p);
+    else elemwise_dither_kernel<MXQ_F16><<<grid, kThreads, 0, s>>>(in, noise, out, n, p);
+    return check_launch(who);
+}
+
 int mxq_quantize_mx_given_max(const void* in, void* out, const void* max_values, int dtype,
                               int64_t pre, int64_t axis_size, int64_t post, int scale_bits,
                               int elem_ebits, int elem_mbits, float elem_max_norm,

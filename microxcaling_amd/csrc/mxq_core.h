@@ -22,6 +22,9 @@
 
 enum MxqDtype { MXQ_F32 = 0, MXQ_F16 = 1, MXQ_BF16 = 2 };
 enum MxqRound { MXQ_NEAREST = 0, MXQ_FLOOR = 1, MXQ_EVEN = 2 };   // mx/formats.py:12-19
+// round='dither' (mx/elemwise_ops.py:57-59) is not in that enum: floor(s + u) with u in [0, 1) drawn
+// by the caller, one per element.  Only the op-by-op form of the rounding knows it.
+#define MXQ_DITHER 3
 
 #define MXQ_QNAN_BITS 0x7FC00000u
 #define MXQ_INF_BITS 0x7F800000u
@@ -202,7 +205,7 @@ MXQ_HD float mxq_sign_source(float a) {
 // tensors with wide element formats (t >= 7) and, on the host, to cross-check the lean form.
 template <int RMODE, int DT>
 MXQ_HD float mxq_round_every_op(float a, const MxqFmt& f, bool saturate, const unsigned char* zone,
-                                int zshift) {
+                                int zshift, float noise = 0.0f) {
     const uint32_t ba = mxq_bits(a);
     const uint32_t ua = ba & 0x7FFFFFFFu;
     int e = 0;
@@ -222,6 +225,8 @@ MXQ_HD float mxq_round_every_op(float a, const MxqFmt& f, bool saturate, const u
         r = floorf(s);
     } else if (RMODE == MXQ_NEAREST) {
         r = floorf(mxq_round_dt<DT>(s + 0.5f));
+    } else if (RMODE == MXQ_DITHER) {
+        r = floorf(mxq_round_dt<DT>(s + noise));
     } else {
         float d = mxq_round_dt<DT>(s - 0.5f);
         float h = d * 0.5f;
@@ -240,7 +245,7 @@ MXQ_HD float mxq_round_every_op(float a, const MxqFmt& f, bool saturate, const u
 // LEAN: see mxq_round_lean for when it may be used.
 template <int RMODE, int DT, bool ZONE, bool LEAN>
 MXQ_HD float mxq_quant_mx_elem_raw(float x, const MxqScale& sc, const MxqFmt& f,
-                                   const unsigned char* zone, int zshift) {
+                                   const unsigned char* zone, int zshift, float noise = 0.0f) {
     const float a = x * sc.inv_scale;
     float y;
     if (LEAN) {
@@ -248,14 +253,14 @@ MXQ_HD float mxq_quant_mx_elem_raw(float x, const MxqScale& sc, const MxqFmt& f,
         // format either way, only its sign needs the bf16 view (mxq_sign_source)
         y = mxq_round_lean<RMODE, ZONE>(a, mxq_sign_source<DT>(a), f, true, zone, zshift);
     } else {
-        y = mxq_round_every_op<RMODE, DT>(mxq_round_dt<DT>(a), f, true, zone, zshift);
+        y = mxq_round_every_op<RMODE, DT>(mxq_round_dt<DT>(a), f, true, zone, zshift, noise);
     }
     return y * sc.scale;
 }
 template <int RMODE, int DT, bool ZONE, bool LEAN>
 MXQ_HD float mxq_quant_mx_elem(float x, const MxqScale& sc, const MxqFmt& f,
-                               const unsigned char* zone, int zshift) {
-    return mxq_round_dt<DT>(mxq_quant_mx_elem_raw<RMODE, DT, ZONE, LEAN>(x, sc, f, zone, zshift));
+                               const unsigned char* zone, int zshift, float noise = 0.0f) {
+    return mxq_round_dt<DT>(mxq_quant_mx_elem_raw<RMODE, DT, ZONE, LEAN>(x, sc, f, zone, zshift, noise));
 }
 
 // The same element, but as (value relative to the block scale): what a packed MX tensor stores.
@@ -394,11 +399,11 @@ MXQ_HD float mxq_quant_bf16_to_bfloat16_nearest_nonneg(float x) {
 // One element of the elementwise quantizer (mx/elemwise_ops.py:127-163).
 template <int RMODE, int DT, bool ZONE, bool LEAN>
 MXQ_HD float mxq_quant_elemwise(float x, const MxqFmt& f, bool saturate, bool allow_denorm,
-                                const unsigned char* zone, int zshift) {
+                                const unsigned char* zone, int zshift, float noise = 0.0f) {
     const uint32_t ux = mxq_bits(x) & 0x7FFFFFFFu;
     float y;
     if (LEAN) y = mxq_round_lean<RMODE, ZONE, DT == MXQ_BF16>(x, x + 0.0f, f, saturate || f.ebits == 0, zone, zshift);
-    else y = mxq_round_every_op<RMODE, DT>(ux < MXQ_INF_BITS ? x : 0.0f, f, saturate, zone, zshift);
+    else y = mxq_round_every_op<RMODE, DT>(ux < MXQ_INF_BITS ? x : 0.0f, f, saturate, zone, zshift, noise);
     // (|A| >= min_norm) * A is +-0, and sign(+-0) is 0
     if (!allow_denorm && f.ebits > 0 && (ux >> 23) < f.min_eb) y = 0.0f;
     // exponent 128: 2**128 = inf and the value turns into 0 * inf.  +-Inf is restored after the

@@ -35,8 +35,8 @@ void store_from_float(void* p, int dtype, int64_t i, float v) {
 }
 
 // element kernels selected once per call
-typedef float (*MxElemFn)(float, const MxqScale&, const MxqFmt&, const unsigned char*, int);
-typedef float (*ElemFn)(float, const MxqFmt&, bool, bool, const unsigned char*, int);
+typedef float (*MxElemFn)(float, const MxqScale&, const MxqFmt&, const unsigned char*, int, float);
+typedef float (*ElemFn)(float, const MxqFmt&, bool, bool, const unsigned char*, int, float);
 
 template <int DT, bool LEAN>
 MxElemFn pick_mx(int rmode, bool ze) {
@@ -96,7 +96,7 @@ int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t p
                 MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
                 for (int64_t k = k0; k < k1; ++k) {
                     const int64_t idx = (i * axis_size + k) * post + j;
-                    store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift));
+                    store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift, 0.0f));
                 }
             }
     return MXQ_OK;
@@ -133,9 +133,67 @@ int mxq_host_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, 
             for (int64_t j = 0; j < len[1]; ++j)
                 for (int64_t k = 0; k < len[2]; ++k) {
                     const int64_t idx = base + i * st[0] + j * st[1] + k * st[2];
-                    store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift));
+                    store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift, 0.0f));
                 }
     }
+    return MXQ_OK;
+}
+
+// round='dither': floor(scaled value + noise), noise[i] in [0, 1) drawn by the caller in the tensor
+// dtype, one per element (mx/elemwise_ops.py:57-59)
+int mxq_host_quantize_mx_dither_by_tile(const void* in, const void* noise, void* out, int dtype, int64_t pre,
+                                        int64_t axis_size, int64_t post, int scale_bits, int elem_ebits,
+                                        int elem_mbits, float elem_max_norm, int64_t tile_size,
+                                        int flush_fp32_subnorms, int flags) {
+    const char* who = "mxq_host_quantize_mx_dither_by_tile";
+    MxParams p;
+    bool ze;
+    int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
+                            flush_fp32_subnorms, MXQ_ROUND_NEAREST, flags, &p, &ze, who);
+    if (rc) return rc;
+    if (pre < 0 || axis_size < 0 || post < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    int64_t total;
+    if (mul_overflows(pre, axis_size, post, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
+    if (total == 0) return MXQ_OK;
+    if (!in || !out || !noise) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    const int64_t tile = (tile_size <= 0 || tile_size > axis_size) ? axis_size : tile_size;
+    const unsigned char* zone = kZone[p.zone_row];
+    MxElemFn fn = dtype == MXQ_DTYPE_BF16 ? mxq_quant_mx_elem<MXQ_DITHER, MXQ_BF16, true, false>
+                                          : mxq_quant_mx_elem<MXQ_DITHER, MXQ_F32, true, false>;
+    for (int64_t i = 0; i < pre; ++i)
+        for (int64_t k0 = 0; k0 < axis_size; k0 += tile)
+            for (int64_t j = 0; j < post; ++j) {
+                const int64_t k1 = std::min(k0 + tile, axis_size);
+                uint32_t um = 0;
+                for (int64_t k = k0; k < k1; ++k)
+                    um = std::max(um, mxq_bits(load_as_float(in, dtype, (i * axis_size + k) * post + j)) & 0x7FFFFFFFu);
+                MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+                for (int64_t k = k0; k < k1; ++k) {
+                    const int64_t idx = (i * axis_size + k) * post + j;
+                    store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift,
+                                                         load_as_float(noise, dtype, idx)));
+                }
+            }
+    return MXQ_OK;
+}
+
+int mxq_host_quantize_elemwise_dither(const void* in, const void* noise, void* out, int dtype, int64_t n,
+                                      int bits, int exp_bits, float max_norm, int saturate_normals,
+                                      int allow_denorm, int flags) {
+    const char* who = "mxq_host_quantize_elemwise_dither";
+    ElemParams p;
+    int rc = make_elem_params(dtype, bits, exp_bits, max_norm, MXQ_ROUND_NEAREST, saturate_normals, allow_denorm,
+                              flags, &p, who);
+    if (rc) return rc;
+    if (n < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    if (n == 0) return MXQ_OK;
+    if (!in || !out || !noise) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
+    const unsigned char* zone = kZone[p.zone_row];
+    ElemFn fn = dtype == MXQ_DTYPE_BF16 ? mxq_quant_elemwise<MXQ_DITHER, MXQ_BF16, true, false>
+                                        : mxq_quant_elemwise<MXQ_DITHER, MXQ_F32, true, false>;
+    for (int64_t i = 0; i < n; ++i)
+        store_from_float(out, dtype, i, fn(load_as_float(in, dtype, i), p.fmt, p.saturate != 0, p.allow_denorm != 0,
+                                           zone, p.zshift, load_as_float(noise, dtype, i)));
     return MXQ_OK;
 }
 
@@ -162,7 +220,7 @@ int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_va
             MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
             for (int64_t k = 0; k < axis_size; ++k) {
                 const int64_t idx = (i * axis_size + k) * post + j;
-                store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift));
+                store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift, 0.0f));
             }
         }
     return MXQ_OK;
@@ -196,7 +254,7 @@ int mxq_host_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, 
                            lean_ok(dtype, p.fmt, rmode, true) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < n; ++i)
         store_from_float(out, dtype, i,
-                         fn(load_as_float(in, dtype, i), p.fmt, p.saturate != 0, p.allow_denorm != 0, zone, p.zshift));
+                         fn(load_as_float(in, dtype, i), p.fmt, p.saturate != 0, p.allow_denorm != 0, zone, p.zshift, 0.0f));
     return MXQ_OK;
 }
 

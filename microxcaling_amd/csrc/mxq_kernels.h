@@ -457,6 +457,56 @@ __global__ __launch_bounds__(TPB) void elemwise_kernel(const void* __restrict__ 
 }
 
 // ================================================================================================
+// round='dither' (mx/elemwise_ops.py:57-59): floor(scaled value + noise) with noise in [0, 1) drawn
+// by the caller in the tensor dtype, one per element.  A training-time option off the hot path:
+// one element per lane, op-by-op form of the rounding.
+// ================================================================================================
+template <int DT>
+__global__ __launch_bounds__(TPB) void elemwise_dither_kernel(const void* __restrict__ in,
+                                                              const void* __restrict__ noise,
+                                                              void* __restrict__ out, int64_t n, ElemParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.zone_row]);
+    for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (int64_t)gridDim.x * TPB)
+        store_scalar<DT>(out, i, mxq_quant_elemwise<MXQ_DITHER, ADT, true, false>(
+                                     load_scalar<DT>(in, i), p.fmt, p.saturate != 0, p.allow_denorm != 0, zone, ZS,
+                                     load_scalar<DT>(noise, i)));
+}
+
+// tensor (pre, axis, post), tiles of `tile` positions of the middle axis; a lane owns one tile at one
+// `post` position
+template <int DT>
+__global__ __launch_bounds__(TPB) void mx_dither_kernel(const void* __restrict__ in,
+                                                        const void* __restrict__ noise,
+                                                        void* __restrict__ out, int64_t pre, int64_t axis_size,
+                                                        int64_t post, int64_t tile, int64_t num_tiles,
+                                                        MxParams p) {
+    constexpr int ADT = Arith<DT>::DT_;
+    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    __shared__ unsigned char zone[ZONE_PAD];
+    load_zone(zone, g_zone_tables[p.zone_row]);
+    const int64_t total = pre * num_tiles * post;
+    for (int64_t w = (int64_t)blockIdx.x * TPB + threadIdx.x; w < total; w += (int64_t)gridDim.x * TPB) {
+        const int64_t c = w % post;
+        const int64_t ti = (w / post) % num_tiles;
+        const int64_t pi = w / (post * num_tiles);
+        const int64_t row0 = ti * tile;
+        const int64_t rows = (row0 + tile > axis_size) ? (axis_size - row0) : tile;
+        const int64_t off0 = (pi * axis_size + row0) * post + c;
+        uint32_t um = 0;
+        for (int64_t r = 0; r < rows; ++r) um = max(um, abs_bits(load_scalar<DT>(in, off0 + r * post)));
+        const MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+        for (int64_t r = 0; r < rows; ++r) {
+            const int64_t i = off0 + r * post;
+            store_scalar<DT>(out, i, mxq_quant_mx_elem<MXQ_DITHER, ADT, true, false>(
+                                         load_scalar<DT>(in, i), sc, p.fmt, zone, ZS, load_scalar<DT>(noise, i)));
+        }
+    }
+}
+
+// ================================================================================================
 // Reductions (fp32).  max propagates NaN like torch.max; sums are accumulated in a fixed order.
 // ================================================================================================
 struct SumOp {

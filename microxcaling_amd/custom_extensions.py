@@ -293,6 +293,61 @@ def quantize_mx_axes_func_cpp(A, scale_bits, elem_ebits, elem_mbits, elem_max_no
     return out
 
 
+def _check_noise(A, noise, who):
+    if noise.dtype != A.dtype or noise.shape != A.shape or noise.device != A.device or not noise.is_contiguous():
+        raise RuntimeError("%s: noise must be a contiguous tensor like A (same shape, dtype, device)" % who)
+
+
+def quantize_elemwise_dither_func(A, noise, bits, exp_bits, max_norm, saturate_normals=False,
+                                  allow_denorm=True):
+    """round='dither' (mx/elemwise_ops.py:57-59) for CPU or GPU tensors: floor(scaled value + noise),
+    noise in [0, 1) like torch.rand_like(A).  Not in the reference's extension (pure path only)."""
+    who = "quantize_elemwise_dither_func"
+    out = torch.empty_like(A)
+    args = (_dtype_code(A, who), A.numel(), bits, exp_bits, max_norm, int(bool(saturate_normals)),
+            int(bool(allow_denorm)), _flags)
+    if A.is_cuda:
+        _check_gpu_input(A, "A", who)
+        _check_noise(A, noise, who)
+        lib = _lib.gpu()
+        with torch.cuda.device(A.device):
+            rc = lib.mxq_quantize_elemwise_dither(A.data_ptr(), noise.data_ptr(), out.data_ptr(), *args, _stream(A))
+        _lib.check(rc, lib)
+    else:
+        _check_cpu_input(A, "A", who)
+        _check_noise(A, noise, who)
+        lib = _lib.host()
+        rc = lib.mxq_host_quantize_elemwise_dither(A.data_ptr(), noise.data_ptr(), out.data_ptr(), *args)
+        _lib.check(rc, lib, "mxq_host_last_error")
+    return out
+
+
+def quantize_mx_dither_by_tile_func(A, noise, scale_bits, elem_ebits, elem_mbits, elem_max_norm, tile_size,
+                                    axis, flush_fp32_subnorms=False):
+    """MX quantization with round='dither' for CPU or GPU tensors; see quantize_elemwise_dither_func."""
+    who = "quantize_mx_dither_by_tile_func"
+    if not (0 <= axis < A.dim()):
+        raise RuntimeError("%s: axis exceeds input dimensions" % who)
+    pre, n, post = _collapse(A.shape, axis)
+    out = torch.empty_like(A)
+    args = (_dtype_code(A, who), pre, n, post, scale_bits, elem_ebits, elem_mbits, elem_max_norm, tile_size,
+            int(bool(flush_fp32_subnorms)), _flags)
+    if A.is_cuda:
+        _check_gpu_input(A, "A", who)
+        _check_noise(A, noise, who)
+        lib = _lib.gpu()
+        with torch.cuda.device(A.device):
+            rc = lib.mxq_quantize_mx_dither_by_tile(A.data_ptr(), noise.data_ptr(), out.data_ptr(), *args, _stream(A))
+        _lib.check(rc, lib)
+    else:
+        _check_cpu_input(A, "A", who)
+        _check_noise(A, noise, who)
+        lib = _lib.host()
+        rc = lib.mxq_host_quantize_mx_dither_by_tile(A.data_ptr(), noise.data_ptr(), out.data_ptr(), *args)
+        _lib.check(rc, lib, "mxq_host_last_error")
+    return out
+
+
 funcs = types.SimpleNamespace(
     quantize_mx_func_cpp=quantize_mx_func_cpp,
     quantize_elemwise_func_cpp=quantize_elemwise_func_cpp,
@@ -307,4 +362,6 @@ funcs = types.SimpleNamespace(
     reduce_max_outer_dim=reduce_max_outer_dim,
     quantize_mx_axes_func_cuda=quantize_mx_axes_func_cuda,
     quantize_mx_axes_func_cpp=quantize_mx_axes_func_cpp,
+    quantize_elemwise_dither_func=quantize_elemwise_dither_func,
+    quantize_mx_dither_by_tile_func=quantize_mx_dither_by_tile_func,
 )

@@ -5,7 +5,9 @@ Differences from the reference, on purpose:
   * there is one implementation per device -- HIP kernels for GPU tensors, the host library for CPU
     tensors -- and its results are bit-identical to the reference's pure-PyTorch path, so the
     ``custom_cuda`` switch is accepted but does not change the result;
-  * ``round='dither'`` (stochastic) is not implemented and raises.
+  * ``round='dither'`` (stochastic, mx/elemwise_ops.py:57-59) runs natively too: the noise is drawn
+    with torch.rand_like, as the reference does, and handed to the kernel; the kernels that run a
+    whole chain of steps do not take it (those layers run their separate steps).
 """
 import torch
 
@@ -25,7 +27,7 @@ def _quantize_elemwise_core(A, bits, exp_bits, max_norm, round='nearest',
     """Round every element of A to a format with `bits` = sign + implicit one + fraction bits and
     `exp_bits` exponent bits (0 = integer), overflowing to +-Inf or, if `saturate_normals`,
     clamping to +-max_norm.  Same contract as mx/elemwise_ops.py:82-170."""
-    rmode = _native_round(round)
+    rmode = None if round == "dither" else _native_round(round)
     if A.is_sparse:
         if A.layout != torch.sparse_coo:
             raise NotImplementedError("Only COO layout sparse tensors are currently supported.")
@@ -44,6 +46,13 @@ def _quantize_elemwise_core(A, bits, exp_bits, max_norm, round='nearest',
                                        saturate_normals=saturate_normals, allow_denorm=allow_denorm,
                                        custom_cuda=custom_cuda).transpose(-1, -2)
     A = A.contiguous()
+    if round == "dither":
+        # stochastic rounding: the noise comes from torch's generator, as in the reference
+        # (torch.rand_like, mx/elemwise_ops.py:58), so torch.manual_seed governs it
+        if A.device.type not in ("cuda", "cpu"):
+            raise ValueError("Unrecognized device type %s" % A.device.type)
+        return custom_extensions.funcs.quantize_elemwise_dither_func(
+            A, torch.rand_like(A, requires_grad=False), bits, exp_bits, max_norm, saturate_normals, allow_denorm)
     if A.device.type == "cuda":
         return custom_extensions.funcs.quantize_elemwise_func_cuda(
             A, bits, exp_bits, max_norm, rmode, saturate_normals, allow_denorm)

@@ -10,7 +10,8 @@ Differences from the reference, on purpose:
     separate max for block sizes above 32 on the last axis, and serves several axes on its
     pure-PyTorch path only, mx/mx_ops.py:226-263); results are bit-identical to its pure-PyTorch
     path either way, so ``custom_cuda`` is accepted but does not change the result;
-  * ``round='dither'`` raises.
+  * ``round='dither'`` draws its noise with torch.rand_like like the reference and runs natively
+    (single axis).
 """
 import torch
 
@@ -35,7 +36,7 @@ def _quantize_mx(A, scale_bits, elem_format, shared_exp_method="max", axes=None,
         raise ValueError("axes must name at least one dimension, each once")
     if len(axes) > 3:
         raise NotImplementedError("the native kernels share an exponent over at most three axes")
-    rmode = _native_round(round)
+    rmode = None if round == "dither" else _native_round(round)
     ebits, mbits, _, max_norm, _ = _get_format_params(elem_format)
 
     if shared_exp_method == "none":          # an exponent per element = blocks of one
@@ -47,6 +48,15 @@ def _quantize_mx(A, scale_bits, elem_format, shared_exp_method="max", axes=None,
 
     from . import custom_extensions as ce
     A = A.contiguous()
+    if round == "dither":
+        # stochastic rounding: floor(scaled value + u), u from torch's generator like the reference's
+        # torch.rand_like (mx/elemwise_ops.py:58)
+        if len(axes) > 1 and tile != 1:
+            raise NotImplementedError("round='dither' with an exponent shared over several axes")
+        if A.device.type not in ("cuda", "cpu"):
+            raise ValueError("Unrecognized device type %s" % A.device.type)
+        return ce.funcs.quantize_mx_dither_by_tile_func(A, torch.rand_like(A, requires_grad=False), scale_bits,
+                                                        ebits, mbits, max_norm, tile, axes[-1], flush_fp32_subnorms)
     if len(axes) > 1 and tile != 1:          # one exponent per tile of tile x tile (x tile) elements
         fn = {"cuda": ce.funcs.quantize_mx_axes_func_cuda, "cpu": ce.funcs.quantize_mx_axes_func_cpp}.get(A.device.type)
         if fn is None:

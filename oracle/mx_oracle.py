@@ -81,9 +81,12 @@ def ieee_max_norm(ebits, mbits):
 # ---------------------------------------------------------------------------------------------
 # element rounding
 # ---------------------------------------------------------------------------------------------
-def _round_scaled(v, mode):
-    """Integer rounding of a pre-scaled tensor.  mx/elemwise_ops.py:45-76 (dither excluded: the
-    native path never takes it, mx/mx_ops.py:197)."""
+def _round_scaled(v, mode, noise=None):
+    """Integer rounding of a pre-scaled tensor.  mx/elemwise_ops.py:45-76.  dither: `noise` stands in
+    for the reference's torch.rand_like(v) so that a test can hand both sides the same draw."""
+    if mode == "dither":
+        rand = torch.rand_like(v, requires_grad=False) if noise is None else noise.reshape(v.shape)
+        return torch.sign(v) * torch.floor(torch.abs(v) + rand)
     if mode == "floor":
         return torch.sign(v) * torch.floor(torch.abs(v))
     if mode == "nearest":
@@ -96,7 +99,7 @@ def _round_scaled(v, mode):
 
 
 def quantize_elemwise_core(A, bits, exp_bits, max_norm, round="nearest",
-                           saturate_normals=False, allow_denorm=True):
+                           saturate_normals=False, allow_denorm=True, noise=None):
     """Round every element of A to a (bits, exp_bits, max_norm) format.
     mx/elemwise_ops.py:82-170, pure branch (127-163)."""
     if not allow_denorm and exp_bits > 0:                                  # 128-130
@@ -113,7 +116,7 @@ def quantize_elemwise_core(A, bits, exp_bits, max_norm, round="nearest",
         private_exp = None
         out = out * (2 ** (bits - 2))
 
-    out = _round_scaled(out, round)                                        # 147
+    out = _round_scaled(out, round, noise)                                 # 147
 
     if private_exp is None:                                                # 150, 38-42
         out = out / (2 ** (bits - 2))
@@ -207,7 +210,7 @@ def _from_blocks(A, axes, unpadded, padded):
 
 
 def quantize_mx(A, scale_bits, elem_format, axes, block_size=0, round="nearest",
-                flush_fp32_subnorms=False):
+                flush_fp32_subnorms=False, noise=None):
     """MX fake-quantization of A.  mx/mx_ops.py:173-298, pure branch (265-292),
     shared_exp_method='max'."""
     if elem_format is None:
@@ -233,7 +236,7 @@ def quantize_mx(A, scale_bits, elem_format, axes, block_size=0, round="nearest",
 
     A = A / (2 ** se)                                                      # 285
     A = quantize_elemwise_core(A, mbits, ebits, max_norm, round=round,
-                               allow_denorm=True, saturate_normals=True)   # 287-290
+                               allow_denorm=True, saturate_normals=True, noise=noise)   # 287-290
     A = A * (2 ** se)                                                      # 292
 
     if block_size > 0:

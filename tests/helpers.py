@@ -67,3 +67,32 @@ def golden_inputs_module():
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     return mod
+
+
+_dither = None
+
+
+def dither_golden():
+    """Arrays written by tests/golden/gen_reference_dither_vectors.py, and its case tables."""
+    global _dither
+    if _dither is None:
+        import importlib.util
+        here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+        spec = importlib.util.spec_from_file_location("gen_reference_dither_vectors",
+                                                      os.path.join(here, "gen_reference_dither_vectors.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _dither = (np.load(os.path.join(here, "reference_dither_vectors.npz")), mod)
+    return _dither
+
+
+def dither_cases():
+    """(kind, dtype name, torch dtype, case number, seed, parameters, input tensor, expected output) for
+    every stored case."""
+    z, mod = dither_golden()
+    for name, dtype in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+        x = from_bits(z["x_" + name], dtype)
+        for n, case in enumerate(mod.MX_CASES):
+            yield "mx", name, dtype, n, 1000 + n, case, x, from_bits(z["mx_%s_%d" % (name, n)], dtype)
+        for n, case in enumerate(mod.ELEM_CASES):
+            yield "elem", name, dtype, n, 2000 + n, case, x, from_bits(z["elem_%s_%d" % (name, n)], dtype)

@@ -229,6 +229,37 @@ def test_mx_several_axes(dev, shape, axes, bs, dtype):
         assert_bits_equal(got, want, "%s %s %s" % (shape, fmt, rnd))
 
 
+def test_dither_with_the_reference_noise(dev):
+    """round='dither' on the GPU with the noise the reference drew (torch.rand_like under the stored
+    seed, regenerated on the CPU and copied over): the reference's outputs bit for bit."""
+    from helpers import dither_cases
+    from microxcaling_amd.custom_extensions import funcs
+    from microxcaling_amd.formats import _get_format_params
+    for kind, name, dtype, case_no, seed, case, x, want in dither_cases():
+        torch.manual_seed(seed)
+        noise = torch.rand_like(x).to(dev)
+        if kind == "mx":
+            fmt, axis, bs = case
+            ebits, mbits, _, max_norm, _ = _get_format_params(fmt)
+            got = funcs.quantize_mx_dither_by_tile_func(x.to(dev), noise, 8, ebits, mbits, max_norm, bs,
+                                                        axis % x.ndim, False)
+        else:
+            bits, eb, mn, sat = case
+            got = funcs.quantize_elemwise_dither_func(x.to(dev), noise, bits, eb, mn, sat, True)
+        torch.cuda.synchronize()
+        assert_bits_equal(got, want, "%s %s %d" % (kind, name, case_no))
+    # through the public call: the noise comes from torch's generator for the device
+    xs = torch.linspace(-3.9, 3.9, 4001, device=dev)
+    from microxcaling_amd.elemwise_ops import _quantize_elemwise_core
+    draws = torch.stack([_quantize_elemwise_core(xs, 5, 4, 448.0, round="dither") for _ in range(200)])
+    lo = _quantize_elemwise_core(xs, 5, 4, 448.0, round="floor")
+    step = torch.exp2(torch.floor(torch.log2(xs.abs().clamp_min(2.0 ** -6))) - 3)
+    assert ((draws == lo) | (draws == lo + torch.sign(xs) * step)).all()
+    assert ((draws.mean(0) - xs).abs() <= 0.3 * step).all()
+    got = mx_gpu(torch.randn(64, 64, device=dev), 8, "fp4_e2m1", axes=[-1], block_size=32, round="dither")
+    assert torch.isfinite(got).all()
+
+
 def test_mx_given_max_entry_point(dev):
     """quantize_mx_func_cuda: the caller reshapes to blocks and supplies the abs-max
     (mx/mx_ops.py:226-256)."""

@@ -78,7 +78,9 @@ def test_host_functions_reject_gpu_only_misuse():
         funcs.quantize_mx_func_cpp(torch.zeros(2, 2, 2, 2, 2, 2), 8, 4, 5, 448.0,
                                    torch.zeros(1), 0, False)                  # ndim > 5
     with pytest.raises(NotImplementedError):
-        _quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=2, round="dither")
+        _quantize_mx(x, 8, "fp8_e4m3", axes=[0, 1], block_size=2, round="dither")
+    with pytest.raises(NotImplementedError):
+        _quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=2, round="stochastic")
     with pytest.raises(NotImplementedError):
         _quantize_mx(torch.zeros(2, 2, 2, 2), 8, "fp8_e4m3", axes=[0, 1, 2, 3], block_size=2)
     with pytest.raises(ValueError):
@@ -355,3 +357,32 @@ def test_direct_pack_codes_equal_the_encoded_rounded_values(tmp_path):
     assert out.count("inputs agree") == 30 and "MISMATCH" not in out
     # nearest and even are served by the shortcut (floor takes the round-up-zone variant)
     assert out.count("zone variant") == 10
+
+
+def test_dither_reproduces_the_reference_under_the_same_seed():
+    """round='dither' on CPU tensors: the package draws its noise like the reference
+    (torch.rand_like under torch's generator) and the host library rounds floor(s + noise): the
+    reference's seeded outputs (tests/golden/reference_dither_vectors.npz) come out bit for bit."""
+    from helpers import dither_cases
+    from microxcaling_amd.elemwise_ops import _quantize_elemwise_core
+    for kind, name, dtype, case_no, seed, case, x, want in dither_cases():
+        torch.manual_seed(seed)
+        if kind == "mx":
+            fmt, axis, bs = case
+            got = _quantize_mx(x.clone(), 8, fmt, axes=[axis], block_size=bs, round="dither")
+        else:
+            bits, eb, mn, sat = case
+            got = _quantize_elemwise_core(x.clone(), bits, eb, mn, round="dither", saturate_normals=sat)
+        assert_bits_equal(got, want, "%s %s %d" % (kind, name, case_no))
+
+
+def test_dither_is_floor_or_ceiling_and_unbiased():
+    x = torch.linspace(-3.9, 3.9, 4001)
+    from microxcaling_amd.elemwise_ops import _quantize_elemwise_core
+    torch.manual_seed(0)
+    draws = torch.stack([_quantize_elemwise_core(x, 5, 4, 448.0, round="dither") for _ in range(400)])
+    lo = _quantize_elemwise_core(x, 5, 4, 448.0, round="floor")              # toward zero
+    step = torch.exp2(torch.floor(torch.log2(x.abs().clamp_min(2.0 ** -6))) - 3)
+    hi = lo + torch.sign(x) * step
+    assert ((draws == lo) | (draws == hi)).all()
+    assert ((draws.mean(0) - x).abs() <= 0.2 * step).all()

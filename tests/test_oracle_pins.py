@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import assert_bits_equal, canon_bits, from_bits, golden, golden_inputs_module
+from helpers import assert_bits_equal, canon_bits, dither_cases, from_bits, golden, golden_inputs_module
 from oracle import c_oracle as C
 from oracle import mx_oracle as O
 
@@ -378,3 +378,21 @@ def test_golden_exhaustive_bf16_digests():
             for rnd in ROUNDS:
                 y = O.quantize_mx(blk.clone(), 8, fmt, axes=[-1], block_size=32, round=rnd)
                 assert _digest(y) == meta["bf16_exhaustive_digests"]["%d.%s.%s" % (Mexp, fmt, rnd)]
+
+
+def test_golden_dither():
+    """round='dither' (mx/elemwise_ops.py:57-59): under the same torch seed the torch oracle draws
+    the noise the reference drew and reproduces its outputs bit for bit (no test of the reference
+    covers this mode; the C oracle has no generator and does not take it)."""
+    n = 0
+    for kind, name, dtype, case_no, seed, case, x, want in dither_cases():
+        torch.manual_seed(seed)
+        if kind == "mx":
+            fmt, axis, bs = case
+            got = O.quantize_mx(x.clone(), 8, fmt, axes=[axis], block_size=bs, round="dither")
+        else:
+            bits, eb, mn, sat = case
+            got = O.quantize_elemwise_core(x.clone(), bits, eb, mn, round="dither", saturate_normals=sat)
+        assert_bits_equal(got, want, "%s %s %d" % (kind, name, case_no))
+        n += 1
+    assert n == 26
