@@ -300,6 +300,42 @@ def make_workload(name):
                     launches=1 if fused else (22 if is_gelu else 12),
                     desc="%s forward, bf16 [16384,8192], bfloat16 quantization after every step, %s"
                          % ("GELU (cubic)" if is_gelu else "SiLU", "one kernel" if fused else "separate tensor passes"))
+    if name == "norm_param_grads_bf16":
+        # weight and bias gradients of LayerNorm over bf16 [32768, 4096] on their own: column sums of
+        # Q(g z) and of g; algorithmic bytes = g and z read once
+        from microxcaling_amd.layernorm import _fused_param_grads, _param_grads
+        from microxcaling_amd.specs import apply_mx_specs, finalize_mx_specs
+        specs = apply_mx_specs(finalize_mx_specs({"bfloat": 16}))
+        g = torch.Generator().manual_seed(9)
+        x = torch.randn(32768, 4096, generator=g).to(torch.bfloat16)
+        z = {}
+
+        def run(xd):
+            if "z" not in z:
+                z["z"] = (torch.randn(xd.shape, generator=torch.Generator().manual_seed(10)) * 1.5).to(torch.bfloat16).to(xd.device)
+            return _fused_param_grads(xd, z["z"], specs)
+        zc = (torch.randn(x.shape, generator=torch.Generator().manual_seed(10)) * 1.5).to(torch.bfloat16)
+        return dict(x=x, gpu=run, cpu=lambda t: _param_grads(t, zc[:t.shape[0], :t.shape[1]].contiguous(), specs), bytes=x.numel() * 4,
+                    dtype="bf16", sample_axis=0, launches=2,
+                    desc="LayerNorm weight and bias gradients, bf16 [32768,4096], bfloat16 quantization: "
+                         "two column-sum launches (CPU leg: this package's separate steps on CPU tensors)")
+    if name == "pack_t_bf16":
+        # quantize along axis -2 + transpose + pack: the operand form of grad_output^T in a linear layer's
+        # weight gradient; algorithmic bytes = input + codes + scales
+        from microxcaling_amd.fused import pack_mx_t
+        x = torch.randn(16384, 14336, generator=torch.Generator().manual_seed(12)).to(torch.bfloat16)
+        return dict(x=x, gpu=lambda t: pack_mx_t(t, "fp8_e4m3"),
+                    cpu=lambda t: O.quantize_mx(t, 8, "fp8_e4m3", axes=[-2], block_size=32).t().contiguous(),
+                    bytes=x.numel() * 3 + x.numel() // 32, dtype="bf16", sample_axis=1,
+                    desc="MXFP8 e4m3 transposing pack (blocks of 32 along axis -2), bf16 [16384,14336] -> "
+                         "codes [14336,16384] + scale bytes (CPU leg: fake quantization + transpose)")
+    if name == "mxfp8_fp32_8192_tiles":
+        # one exponent per 32 x 32 tile (two shared axes): the general-shape kernel
+        x = torch.randn(8192, 8192, generator=torch.Generator().manual_seed(0))
+        return dict(x=x, gpu=lambda t: _quantize_mx(t, 8, "fp8_e4m3", axes=[-2, -1], block_size=32),
+                    cpu=lambda t: O.quantize_mx(t, 8, "fp8_e4m3", axes=[-2, -1], block_size=32),
+                    bytes=x.numel() * 8, dtype="f32", sample_axis=0,
+                    desc="_quantize_mx fp8_e4m3, one exponent per 32 x 32 tile (axes -2 and -1), fp32 [8192,8192]")
     if name == "copy_fp32_8192":
         # a plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         x = torch.randn(8192, 8192, generator=torch.Generator().manual_seed(0))

@@ -55,6 +55,19 @@ struct LaunchStrided {
 template <int DT, int RMODE, bool ZE, bool LEAN>
 struct LaunchAxes {
     static void run(const void* in, void* out, MxqAxes a, int64_t n_tiles, MxParams p, hipStream_t s) {
+        // 32 x 32 tiles of the last two axes of an aligned tensor: the register-resident tile kernel,
+        // the lanes of a tile sharing their maxima
+        constexpr int VW8 = (DT == MXQ_F32) ? 2 : 4;
+        if (a.s[2] == 1 && a.o[1] == 1 && a.o[2] == 1 && a.o[3] == 1 && a.t[0] == 32 && a.t[1] == 32 &&
+            a.s[0] % 32 == 0 && a.s[1] % 32 == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 7) == 0) {
+            const int64_t pv = a.s[1] / VW8, tiles_r = a.s[0] / 32;
+            const int64_t items = a.o[0] * tiles_r * pv, blocks = ceil_div(items, kThreads);
+            if (blocks <= 0x7FFFFFFF) {
+                mx_strided_tile_kernel<DT, RMODE, ZE, LEAN, 32, true><<<(unsigned)blocks, kThreads, 0, s>>>(
+                    reinterpret_cast<const u32x2*>(in), reinterpret_cast<u32x2*>(out), items, tiles_r, pv, p);
+                return;
+            }
+        }
         const int64_t grid = n_tiles < 8 * kMaxBlocks ? n_tiles : 8 * kMaxBlocks;
         mx_axes_kernel<DT, RMODE, ZE, LEAN><<<(unsigned)grid, kThreads, 0, s>>>(in, out, a, n_tiles, p);
     }

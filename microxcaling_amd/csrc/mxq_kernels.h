@@ -185,7 +185,9 @@ template <int DT> struct Col8 {                      // the 8 bytes a lane owns 
     static constexpr int VW = (DT == MXQ_F32) ? 2 : 4;
 };
 
-template <int DT, int RMODE, bool ZONE_ELEM, bool LEAN, int ROWS>
+// SQUARE: the exponent is shared over ROWS x ROWS tiles of the last two axes (post = columns, a
+// multiple of ROWS): the ROWS / VW neighbouring lanes that hold a tile's columns combine their maxima.
+template <int DT, int RMODE, bool ZONE_ELEM, bool LEAN, int ROWS, bool SQUARE = false>
 __global__ __launch_bounds__(TPB) void mx_strided_tile_kernel(const u32x2* __restrict__ in,
                                                               u32x2* __restrict__ out,
                                                               int64_t items, int64_t n_tiles,
@@ -228,6 +230,14 @@ __global__ __launch_bounds__(TPB) void mx_strided_tile_kernel(const u32x2* __res
         for (int k = 0; k < 4; ++k)
             um[k % VW] = (DT == MXQ_BF16) ? (uint32_t)h[k] << 16
                                           : abs_bits((float)__builtin_bit_cast(_Float16, h[k]));
+    }
+    if constexpr (SQUARE) {
+        uint32_t m = um[0];
+#pragma unroll
+        for (int k = 1; k < VW; ++k) m = max(m, um[k]);
+        m = group_max<ROWS / VW>(m);                 // lanes of a group are all live or all idle
+#pragma unroll
+        for (int k = 0; k < VW; ++k) um[k] = m;
     }
     MxqScale sc[VW];
 #pragma unroll
@@ -355,7 +365,13 @@ __global__ __launch_bounds__(TPB) void mx_axes_kernel(const void* __restrict__ i
         int64_t base, len[3], st[3];
         mxq_axes_tile(a, tile, &base, len, st);
         const int64_t count = len[0] * len[1] * len[2], l12 = len[1] * len[2];
+        const bool narrow = count < ((int64_t)1 << 31);      // 32-bit index arithmetic: far cheaper
+        const uint32_t l12n = (uint32_t)l12, l2n = (uint32_t)len[2];
         auto offset = [&](int64_t e) {
+            if (narrow) {
+                const uint32_t en = (uint32_t)e, i0 = en / l12n, r = en - i0 * l12n, i1 = r / l2n;
+                return base + i0 * st[0] + i1 * st[1] + (r - i1 * l2n) * st[2];
+            }
             const int64_t i0 = e / l12, r = e % l12;
             return base + i0 * st[0] + (r / len[2]) * st[1] + (r % len[2]) * st[2];
         };

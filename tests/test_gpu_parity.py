@@ -214,7 +214,9 @@ def test_mx_shapes(dev, shape, axis, bs, dtype):
 @pytest.mark.parametrize("shape,axes,bs", [((70, 45), [-2, -1], 32), ((3, 40, 5, 33), [1, 3], 8),
                                            ((6, 10, 12), [0, 1, 2], 4), ((5, 64, 64), [1, 2], 0),
                                            ((4, 7, 9), [2, 0], 32), ((2, 3, 4, 5, 6), [1, 2, 4], 2),
-                                           ((256, 384), [0, 1], 32), ((3, 100, 300), [1, 2], 64)])
+                                           ((256, 384), [0, 1], 32), ((3, 100, 300), [1, 2], 64),
+                                           ((3, 64, 96), [1, 2], 32), ((2, 5, 32, 32), [-2, -1], 32),
+                                           ((64, 96, 2), [0, 1], 32)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_mx_several_axes(dev, shape, axes, bs, dtype):
     """One exponent per tile of bs x bs (x bs) elements over two or three axes (mx/mx_ops.py:95-154,
