@@ -607,6 +607,59 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     const bool inside = m0 + GEMM_BM <= g.M && n0 + GEMM_BN <= g.N && (g.N & 3) == 0 &&
                         ((uintptr_t)g.c & 15) == 0;
     const bool inside8 = inside && (g.N & 7) == 0 && ((uintptr_t)g.bias & 15) == 0;
+    if constexpr (PAIR) {
+        if (inside8) {                                       // uniform per workgroup
+            // A lane holds two 16-byte pieces of row frow of the wave's 64 columns: columns 8 fg .. and
+            // 32 + 8 fg ...  Lanes frow and frow ^ 8 trade one piece each (row_ror:8 inside the 16 lanes
+            // of a DPP row), after which eight lanes hold the eight pieces of one row: a store
+            // instruction then writes eight full 128-byte lines instead of sixteen half lines.
+            const bool low = frow < 8;
+            const int ncol = n0 + wx * 64 + (low ? 0 : 32) + fg * 8;
+            // bfloat16 quantization without a bias, plain range: while every value of the wave's 16 x 64
+            // piece is a normal number below the NaN threshold, the quantizer is "odd significand -> + 1"
+            // on both halves of a dword at once (three instructions per value with the range check,
+            // against a dozen: the epilogue, not the stores, bounded the one-step products)
+            const bool try_plain = OUT_DT == MXQ_BF16 && g.bias == nullptr && g.q_nan_from != 0u;
+            const unsigned short span = (unsigned short)((g.q_nan_from >> 16) - 0x0080u);
+#pragma unroll
+            for (int ti = 0; ti < 4; ++ti) {
+                u32x4 p0, p1;
+                bool plain = false;
+                if (try_plain) {
+                    uint32_t w[8];
+                    u16x2 worst = {0, 0};
+#pragma unroll
+                    for (int d = 0; d < 8; ++d) {
+                        const v4f& a = acc[ti][d >> 1];
+                        w[d] = Pack<MXQ_BF16>::put(a[(d & 1) * 2], a[(d & 1) * 2 + 1]);
+                        worst = __builtin_elementwise_max(
+                            worst, __builtin_bit_cast(u16x2, w[d] & 0x7FFF7FFFu) - u16x2{0x0080, 0x0080});
+                    }
+                    plain = __all(worst[0] < span && worst[1] < span);
+                    if (plain) {
+#pragma unroll
+                        for (int d = 0; d < 8; ++d) w[d] += w[d] & 0x00010001u;
+                        p0 = u32x4{w[0], w[1], w[2], w[3]};
+                        p1 = u32x4{w[4], w[5], w[6], w[7]};
+                    }
+                }
+                if (!plain) {
+                    p0 = epilogue_pack8<OUT_DT>(g.bias, g.q_nan_from, n0 + wx * 64 + fg * 8, acc[ti][0], acc[ti][1]);
+                    p1 = epilogue_pack8<OUT_DT>(g.bias, g.q_nan_from, n0 + wx * 64 + 32 + fg * 8, acc[ti][2], acc[ti][3]);
+                }
+                const u32x4 send = low ? p1 : p0;
+                u32x4 recv;
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    recv[d] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send[d], 0x128, 0xF, 0xF, false);
+                const int row = m0 + wy * 64 + ti * 16 + (frow & 7);
+                unsigned short* dst = reinterpret_cast<unsigned short*>(g.c) + cbase + (int64_t)row * g.N + ncol;
+                MXQ_C_STORE(reinterpret_cast<u32x4*>(dst), (low ? p0 : recv));
+                MXQ_C_STORE(reinterpret_cast<u32x4*>(dst + (int64_t)8 * g.N), (low ? recv : p1));
+            }
+            return;
+        }
+    }
 #pragma unroll
     for (int ti = 0; ti < 4; ++ti)
 #pragma unroll
@@ -615,7 +668,7 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
             if constexpr (PAIR) {
                 if (tj & 1)
                     store_c8<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, n0 + wx * 64 + (tj >> 1) * 32 + fg * 8,
-                                     g.M, g.N, inside8, acc[ti][tj - 1], acc[ti][tj]);
+                                     g.M, g.N, false, acc[ti][tj - 1], acc[ti][tj]);
             } else {
                 store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, m, n0 + wx * 64 + tj * 16 + fg * 4, g.M, g.N,
                                  inside, acc[ti][tj]);

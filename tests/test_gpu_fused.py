@@ -236,6 +236,46 @@ def test_fp4_gemm_on_nibbles_against_fp64(dev, M, N, K, batch):
         gemm_nt(pa, pack_mx(b.to(dev), "fp4_e2m1"), torch.float32)
 
 
+@pytest.mark.parametrize("fmt,K", [("fp8_e4m3", 128), ("fp4_e2m1", 256)])
+@pytest.mark.parametrize("M,N,batch", [(2048, 2048, 16), (2000, 1990, 17), (130, 4100, 130)])
+def test_one_step_products_with_thousands_of_tiles(dev, fmt, K, M, N, batch):
+    """K of a single 128-byte step and thousands of output tiles (attention scores), full and ragged
+    tiles: against the unpacked operands multiplied by torch, and bit for bit against the same product
+    taken one batch entry at a time."""
+    from microxcaling_amd.fused import pack_mx, gemm_nt, unpack_mx
+    g = torch.Generator().manual_seed(M + N + batch)
+    nib = fmt == "fp4_e2m1"
+    a = torch.randn(batch, M, K, generator=g).to(torch.bfloat16).to(dev)
+    b = torch.randn(batch, N, K, generator=g).to(torch.bfloat16).to(dev)
+    pa, pb = pack_mx(a, fmt, nibbles=nib), pack_mx(b, fmt, nibbles=nib)
+    got = gemm_nt(pa, pb, torch.float32)
+    qa, qb = unpack_mx(*pa, torch.float32), unpack_mx(*pb, torch.float32)
+    want = torch.bmm(qa.double(), qb.double().transpose(-1, -2))
+    assert rel_err(got, want) < 1e-3
+    den = torch.bmm(qa.abs(), qb.abs().transpose(-1, -2))
+    assert ((got.double() - want).abs() <= 2e-4 * den + 1e-30).all()
+    # bfloat16 quantization in the epilogue (plain-range form on whole pieces, general form where a
+    # piece holds a zero or a NaN): the separate steps on the fp32 product, bit for bit
+    from microxcaling_amd.elemwise_ops import _quantize_bfloat
+    a2 = a.clone()
+    a2[0, :40] = 0.0                                         # exact zeros in the product
+    a2[1, 7, 3] = float("nan")
+    pa2 = pack_mx(a2, fmt, nibbles=nib)
+    want_q = _quantize_bfloat(gemm_nt(pa2, pb, torch.float32).to(torch.bfloat16), 16, round="nearest")
+    got_q = gemm_nt(pa2, pb, torch.bfloat16, epilogue_quant=True)
+    assert torch.equal(torch.isnan(got_q), torch.isnan(want_q))
+    assert torch.equal(torch.nan_to_num(got_q).view(torch.int16), torch.nan_to_num(want_q).view(torch.int16))
+    del want_q, got_q, a2, pa2
+    bias = torch.randn(N, generator=g).to(dev).to(torch.bfloat16)
+    got16 = gemm_nt(pa, pb, torch.bfloat16, bias=bias, epilogue_quant=True)
+    for i in (0, batch // 2, batch - 1):
+        one_a = tuple(t[i].contiguous() if torch.is_tensor(t) else t for t in pa)
+        one_b = tuple(t[i].contiguous() if torch.is_tensor(t) else t for t in pb)
+        assert torch.equal(gemm_nt(one_a, one_b, torch.float32), got[i])
+        assert torch.equal(gemm_nt(one_a, one_b, torch.bfloat16, bias=bias, epilogue_quant=True).view(torch.int16),
+                           got16[i].view(torch.int16))
+
+
 def test_gemm_propagates_nan_blocks(dev):
     from microxcaling_amd.fused import pack_mx, gemm_nt
     a = torch.randn(128, 128)
