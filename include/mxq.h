@@ -43,6 +43,10 @@ extern "C" {
 #define MXQ_FLAG_EXACT_EXPONENT 1 /* bit-field exponents instead of torch's floor(log2(x)) */
 #define MXQ_FLAG_PACK_NIBBLES 4   /* mxq_pack_mx / _t, fp4 (e2m1) only: 4-bit codes, two per byte */
 #define MXQ_FLAG_PACK_SIXBIT 8    /* mxq_pack_mx / _t, fp6 (e2m3, e3m2) only: 6-bit codes, four in three bytes */
+#define MXQ_FLAG_PRE_BFLOAT16 32   /* mxq_pack_mx, bf16 tensors only: every element first goes through the
+                                     elementwise quantizer to bfloat16 with round-half-away (bits 9, exp_bits 8,
+                                     subnormals kept) -- what the layers apply to an operand before its MX
+                                     quantization (mx/bmm.py:27-32, mx/matmul.py:45-50) -- in the same pass */
 #define MXQ_FLAG_GENERAL_FORM 16  /* softmax / norm / activation kernels: no shortcut for values in the plain
                                    * range of the bfloat16 quantizer (same results, slower; for tests) */
 

@@ -2,7 +2,7 @@
 import torch
 
 from .elemwise_ops import quantize_elemwise_op
-from .gemm import mx_grad_contract, mx_matmul_contract
+from .gemm import inputs_can_skip_bfloat16_pass, mx_grad_contract, mx_matmul_contract
 from .mx_ops import quantize_mx_op
 from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
 
@@ -15,6 +15,18 @@ class BMMFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, in1, in2, mx_specs, name):
+        if inputs_can_skip_bfloat16_pass(ctx.needs_input_grad[:2], (in1, in2), mx_specs,
+                                         mx_specs["round_output"]):
+            # inference: nothing keeps the quantized operands, the pack kernels quantize them
+            out, finished = mx_matmul_contract(in1, in2, mx_specs["a_elem_format"],
+                                               mx_specs["a_elem_format"], mx_specs,
+                                               mx_specs["round_mx_output"], batched=True,
+                                               out_round=mx_specs["round_output"], pre_bfloat16=True)
+            if out is not None:
+                if not finished:
+                    out = quantize_elemwise_op(out, mx_specs=mx_specs, round=mx_specs["round_output"])
+                ctx.mx_specs = get_backwards_mx_specs(mx_specs)
+                return out
         bf_in1 = quantize_elemwise_op(in1, mx_specs=mx_specs, round=mx_specs["round_output"])
         bf_in2 = quantize_elemwise_op(in2, mx_specs=mx_specs, round=mx_specs["round_output"])
         if mx_specs["quantize_backprop"]:

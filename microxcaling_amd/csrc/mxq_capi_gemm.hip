@@ -203,6 +203,14 @@ int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t ro
     if (!in || !codes || !scales) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     if (!aligned16(in) || !aligned16(codes))
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    if (flags & MXQ_FLAG_PRE_BFLOAT16) {
+        if (dtype != MXQ_DTYPE_BF16)
+            return fail(MXQ_ERR_ARGUMENT, "%s: MXQ_FLAG_PRE_BFLOAT16 is for bf16 tensors", who);
+        ElemParams q;
+        rc = make_elem_params(dtype, 9, 8, 3.3895313892515355e38f, MXQ_ROUND_NEAREST, 0, 1, flags, &q, who);
+        if (rc) return rc;
+        p.pre_nan_from = q.fmt.nan_from;
+    }
     dispatch<LaunchPack>(dtype, rmode, ze, true, in, codes, scales, total / (16 / elem_size(dtype)), kind,
                          direct_max_code(kind, elem_ebits, elem_mbits, p), p, (hipStream_t)hip_stream);
     return check_launch(who);

@@ -81,6 +81,31 @@ __global__ __launch_bounds__(TPB) void mx_pack_kernel(const u32x4* __restrict__ 
             const int64_t i = base + j * TPB;
             v[j] = (i < n_vec) ? in[i] : u32x4{0, 0, 0, 0};
         }
+        if constexpr (DT == MXQ_BF16) {
+            if (p.pre_nan_from != 0u) {                    // uniform: the bfloat16 quantizer first
+                const unsigned short span = (unsigned short)((p.pre_nan_from >> 16) - 0x0080u);
+#pragma unroll
+                for (int j = 0; j < UNROLL; ++j) {
+                    // plain range (normal numbers below the NaN threshold) in the whole wave: "odd
+                    // significand -> + 1" on both halves of a dword at once; else element by element
+                    u16x2 worst = {0, 0};
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+                        worst = __builtin_elementwise_max(
+                            worst, __builtin_bit_cast(u16x2, v[j][d] & 0x7FFF7FFFu) - u16x2{0x0080, 0x0080});
+                    if (__all(worst[0] < span && worst[1] < span)) {
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) v[j][d] += v[j][d] & 0x00010001u;
+                    } else {
+#pragma unroll
+                        for (int d = 0; d < 4; ++d)
+                            v[j][d] = Pack<MXQ_BF16>::put(
+                                mxq_quant_bf16_to_bfloat16_nearest(Pack<MXQ_BF16>::get(v[j][d], 0), p.pre_nan_from),
+                                mxq_quant_bf16_to_bfloat16_nearest(Pack<MXQ_BF16>::get(v[j][d], 1), p.pre_nan_from));
+                    }
+                }
+            }
+        }
 #pragma unroll
         for (int j = 0; j < UNROLL; ++j) {
             const int64_t i = base + j * TPB;

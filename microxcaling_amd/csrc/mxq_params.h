@@ -20,6 +20,7 @@ struct MxParams {
     int flush;
     int zone_row;     // which round-up-zone table
     int zshift;       // 0 for fp32 significands, 16 for bf16
+    uint32_t pre_nan_from;   // mxq_pack_mx with MXQ_FLAG_PRE_BFLOAT16: NaN threshold of that quantizer, else 0
 };
 
 struct ElemParams {
@@ -154,6 +155,7 @@ inline int make_mx_params(int dtype, int scale_bits, int ebits, int mbits, float
     p->scale_emax = (1 << (scale_bits - 1)) - 1;
     p->flush = flush ? 1 : 0;
     zone_for(dtype, flags, &p->zone_row, &p->zshift);
+    p->pre_nan_from = 0u;
     *zone_elem = elem_zone_matters(dtype, flags, p->fmt, rmode);
     return MXQ_OK;
 }

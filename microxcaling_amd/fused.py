@@ -48,11 +48,17 @@ def _pack_flag(kind):
         _FLAG_PACK_SIXBIT if kind in (CODES_E2M3, CODES_E3M2) else 0
 
 
-def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=False, nibbles=False):
+_FLAG_PRE_BFLOAT16 = 32
+
+
+def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=False, nibbles=False,
+            pre_bfloat16=False):
     """MX-quantize A along its last axis (block 32) into (codes, scales, code_kind): codes uint8 of
     A's shape (one e4m3 / e5m2 byte per element) or, with nibbles=True, of half the last axis for
     fp4 (two e2m1 codes per byte, the lower index in the low nibble) and of 3/4 of it for fp6 (6-bit
-    codes as a little-endian bit stream); scales uint8 with the last axis divided by 32."""
+    codes as a little-endian bit stream); scales uint8 with the last axis divided by 32.
+    pre_bfloat16 (bf16 tensors): the elements first go through the elementwise bfloat16 quantizer
+    with round-half-away, in the same pass."""
     who = "pack_mx"
     fmt = _as_format(elem_format)
     if fmt not in _PACKABLE:
@@ -73,7 +79,8 @@ def pack_mx(A, elem_format, scale_bits=8, round="nearest", flush_fp32_subnorms=F
         rc = lib.mxq_pack_mx(A.data_ptr(), codes.data_ptr(), scales.data_ptr(), _DTYPE[A.dtype],
                              rows, K, scale_bits, ebits, mbits, max_norm,
                              int(bool(flush_fp32_subnorms)), int(RoundingMode[round]),
-                             _flags_value() | _pack_flag(kind), _stream(A))
+                             _flags_value() | _pack_flag(kind) | (_FLAG_PRE_BFLOAT16 if pre_bfloat16 else 0),
+                             _stream(A))
     _lib.check(rc, lib)
     return codes, scales, kind
 
@@ -176,11 +183,13 @@ def _use_nibbles(fa, fb, K):
     return fa == ElemFormat.fp4 and fb == ElemFormat.fp4 and K % (2 * GEMM_K_MULTIPLE) == 0
 
 
-def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_quant=False):
+def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_quant=False,
+               pre_bfloat16=False):
     """a (..., M, K) x b_kmajor (N, K) or (..., N, K), both MX-quantized along K: the fused
     equivalent of quantize_mx_op(a, axes=[-1]) @ quantize_mx_op(b, axes=[-1]).T (+ bias, see
-    gemm_nt).  Returns None when the operands do not qualify (the caller then takes the unfused
-    path)."""
+    gemm_nt).  pre_bfloat16: both operands are bf16 tensors that have not been through the layers'
+    elementwise bfloat16 / round-half-away quantization yet; the pack kernels apply it.  Returns None
+    when the operands do not qualify (the caller then takes the unfused path)."""
     fa, fb = _as_format(a_fmt), _as_format(b_fmt)
     if fa not in _PACKABLE or fb not in _PACKABLE:
         return None
@@ -213,9 +222,11 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
         return None
     if epilogue_quant and a.dtype != torch.bfloat16:
         return None
+    if pre_bfloat16 and (a.dtype != torch.bfloat16 or b_kmajor.dtype != torch.bfloat16):
+        return None
     nibbles = _use_nibbles(fa, fb, K)
-    pa = pack_mx(a2, fa, scale_bits, round, flush, nibbles)
-    pb = pack_mx(b2, fb, scale_bits, round, flush, nibbles)
+    pa = pack_mx(a2, fa, scale_bits, round, flush, nibbles, pre_bfloat16)
+    pb = pack_mx(b2, fb, scale_bits, round, flush, nibbles, pre_bfloat16)
     return gemm_nt(pa, pb, out_dtype=a.dtype, bias=bias, epilogue_quant=epilogue_quant).reshape(out_shape)
 
 

@@ -47,7 +47,7 @@ def _epilogue_mode(mx_specs, round, dtype):
     return None
 
 
-def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, out_round=None, bias=None):
+def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, out_round=None, bias=None, pre_bfloat16=False):
     """a: (..., M, K); b_kmajor: (..., N, K) -- both contiguous along K.  Returns (out, finished):
     out is None when the fused path does not apply; finished says whether the output quantization
     with rounding `out_round` and the bias add have been done in the epilogue."""
@@ -57,10 +57,10 @@ def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, out_round=None, bias=
     mode = _epilogue_mode(mx_specs, out_round, a.dtype) if out_round is not None else None
     if mode is not None and (bias is None or bias.dtype == a.dtype):
         out = fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=bias,
-                               epilogue_quant=mode == 1)
+                               epilogue_quant=mode == 1, pre_bfloat16=pre_bfloat16)
         if out is not None:
             return out, True
-    return fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round), False
+    return fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, pre_bfloat16=pre_bfloat16), False
 
 
 def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, out_round=None, bias=None):
@@ -79,16 +79,30 @@ def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, out_round=None, bias
     return f_linear(qx, qw), False
 
 
-def mx_matmul_contract(a, b, a_fmt, b_fmt, mx_specs, round, batched=False, out_round=None, bias=None):
+def inputs_can_skip_bfloat16_pass(needs_grad, tensors, mx_specs, round):
+    """May a layer leave its operands' elementwise quantization to the pack kernels of the fused GEMM?
+    Only when nothing keeps the quantized operands (no gradient is wanted), they are bf16 GPU tensors
+    and the quantizer is bfloat16 with round-half-away, the form those kernels know."""
+    return (_use_fused and not any(needs_grad)
+            and all(t.is_cuda and t.dtype == torch.bfloat16 for t in tensors)
+            and _epilogue_mode(mx_specs, round, torch.bfloat16) == 1)
+
+
+def mx_matmul_contract(a, b, a_fmt, b_fmt, mx_specs, round, batched=False, out_round=None, bias=None,
+                       pre_bfloat16=False):
     """a (..., M, K) times b (..., K, N): a shares exponents along -1, b along -2.  out_round / bias
-    and the return value: as for mx_linear_contract."""
+    and the return value: as for mx_linear_contract.  pre_bfloat16: a and b have not been through
+    the elementwise quantization yet (see inputs_can_skip_bfloat16_pass); only the fused path takes
+    them so, (None, False) means the caller has to quantize them and call again."""
     if b.dim() >= 2 and a.dim() >= 2:
         # the fused kernel wants both operands K-major; a transposed view of b often already is
         bt = b.transpose(-1, -2)
         if bt.is_contiguous() and a.is_contiguous():
-            out, finished = _try_fused(a, bt, a_fmt, b_fmt, mx_specs, round, out_round, bias)
+            out, finished = _try_fused(a, bt, a_fmt, b_fmt, mx_specs, round, out_round, bias, pre_bfloat16)
             if out is not None:
                 return out, finished
+    if pre_bfloat16:
+        return None, False
     qa = quantize_mx_op(a, mx_specs, elem_format=a_fmt, axes=[-1], round=round)
     qb = quantize_mx_op(b, mx_specs, elem_format=b_fmt, axes=[-2], round=round)
     return (torch_bmm(qa, qb) if batched else torch_matmul(qa, qb)), False

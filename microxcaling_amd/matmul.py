@@ -3,7 +3,7 @@ import numpy as np
 import torch
 
 from .elemwise_ops import quantize_elemwise_op
-from .gemm import mx_grad_contract, mx_matmul_contract
+from .gemm import inputs_can_skip_bfloat16_pass, mx_grad_contract, mx_matmul_contract
 from .mx_ops import quantize_mx_op
 from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
 
@@ -23,6 +23,19 @@ class MatMulFunction(torch.autograd.Function):
     def forward(ctx, in1, in2, bias, mx_specs, name, mode_config='aa'):
         assert mode_config in ["aa", "aw", "wa"]
         ctx.mode_config = mode_config
+        if bias is None and inputs_can_skip_bfloat16_pass(ctx.needs_input_grad[:2], (in1, in2), mx_specs,
+                                                          mx_specs["round_output"]):
+            # inference: nothing keeps the quantized operands, the pack kernels quantize them
+            out, finished = mx_matmul_contract(in1, in2, _fmt(mx_specs, mode_config[0]),
+                                               _fmt(mx_specs, mode_config[1]), mx_specs,
+                                               mx_specs["round_mx_output"],
+                                               out_round=mx_specs["round_output"], pre_bfloat16=True)
+            if out is not None:
+                if not finished:
+                    out = quantize_elemwise_op(out, mx_specs=mx_specs, round=mx_specs["round_output"])
+                ctx.bias_shape = None
+                ctx.mx_specs = get_backwards_mx_specs(mx_specs)
+                return out
         bf_in1 = quantize_elemwise_op(in1, mx_specs=mx_specs, round=mx_specs["round_output"])
         bf_in2 = quantize_elemwise_op(in2, mx_specs=mx_specs, round=mx_specs["round_output"])
         if bias is not None:

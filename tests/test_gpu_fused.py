@@ -276,6 +276,43 @@ def test_one_step_products_with_thousands_of_tiles(dev, fmt, K, M, N, batch):
                            got16[i].view(torch.int16))
 
 
+@pytest.mark.parametrize("fmt", ["fp8_e4m3", "fp6_e2m3", "fp4_e2m1"])
+def test_pack_with_the_bfloat16_quantizer_first(dev, fmt):
+    """pack_mx(pre_bfloat16=True) = the elementwise bfloat16 / round-half-away quantizer, then pack_mx:
+    bit for bit, on plain data and on rows with zeros, subnormals, Inf, NaN and the largest values."""
+    from microxcaling_amd.elemwise_ops import _quantize_bfloat
+    from microxcaling_amd.fused import pack_mx
+    g = torch.Generator().manual_seed(31)
+    x = (torch.randn(300, 256, generator=g) * torch.exp2(torch.randint(-8, 8, (300, 256), generator=g).float())).to(torch.bfloat16)
+    x[3, :9] = torch.tensor([0.0, -0.0, float("inf"), float("-inf"), float("nan"), 1e-39, -1e-40, 3.38e38, -3.3e38]).to(torch.bfloat16)
+    x[7] = 0.0
+    x[9, 40:80] *= 1e-38
+    xd = x.to(dev)
+    two_steps = pack_mx(_quantize_bfloat(xd, 16, round="nearest"), fmt)
+    one_step = pack_mx(xd, fmt, pre_bfloat16=True)
+    assert torch.equal(one_step[0], two_steps[0]) and torch.equal(one_step[1], two_steps[1])
+    with pytest.raises(RuntimeError, match="bf16"):
+        pack_mx(xd.float(), fmt, pre_bfloat16=True)
+
+
+@pytest.mark.parametrize("fn", ["bmm", "matmul"])
+def test_inference_skips_the_operand_quantization_pass(dev, fn):
+    """Without gradients mx.bmm / mx.matmul leave the bfloat16 quantization of their operands to the
+    pack kernels: same output, bit for bit, as with gradients wanted (separate passes)."""
+    from microxcaling_amd.bmm import bmm
+    from microxcaling_amd.matmul import matmul
+    specs = _specs(a_elem_format="fp6_e2m3", w_elem_format="fp6_e2m3", block_size=32, bfloat=16)
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(6, 200, 128, generator=g).to(torch.bfloat16).to(dev)
+    b = torch.randn(6, 264, 128, generator=g).to(torch.bfloat16).to(dev).transpose(-1, -2)
+    a[0, 0, :5] = 0.0
+    f = bmm if fn == "bmm" else matmul
+    plain = f(a, b, mx_specs=specs)
+    with_grad = f(a.clone().requires_grad_(True), b, mx_specs=specs)
+    assert with_grad.requires_grad and not plain.requires_grad
+    assert torch.equal(plain.view(torch.int16), with_grad.detach().view(torch.int16))
+
+
 def test_gemm_propagates_nan_blocks(dev):
     from microxcaling_amd.fused import pack_mx, gemm_nt
     a = torch.randn(128, 128)
