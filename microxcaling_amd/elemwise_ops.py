@@ -133,6 +133,8 @@ def fused_chain_args(x, mx_specs, round=None):
     if not (gemm.fused_enabled() and x.is_cuda):
         return None
     rnd = mx_specs['round'] if round is None else round
+    if rnd == "dither":                  # needs a noise tensor per step: the separate steps draw it
+        return None
     plan = elemwise_plan(mx_specs, rnd)
     if plan[0] == "to_bf16":
         x = x.to(torch.bfloat16)

@@ -218,3 +218,29 @@ def test_fused_norm_kernel_against_the_separate_steps(dev, dtype, layer, shape, 
             gemm.set_fused(True)
     for got, want, what in zip(res[0], res[1], ("forward", "grad_input", "grad_weight", "grad_bias")):
         _near(got, want, what)
+
+
+def test_layers_with_dither_rounding(dev):
+    """mx_specs['round'] = 'dither': the kernels that run a whole chain of steps decline (each step
+    needs its own noise), the layers run their separate steps with the dither kernels, forward and
+    backward; results stay within the formats' steps of the round-to-nearest ones."""
+    from microxcaling_amd.activations import gelu
+    from microxcaling_amd.layernorm import LayerNorm
+    from microxcaling_amd.linear import Linear
+    from microxcaling_amd.softmax import softmax
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(64, 256, generator=g).to(torch.bfloat16).to(dev)
+    out = {}
+    for rnd in ("nearest", "dither"):
+        specs = _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32, bfloat=16, round=rnd)
+        torch.manual_seed(1)
+        lin = Linear(256, 128, mx_specs=specs).to(torch.bfloat16).to(dev)
+        ln = LayerNorm(128, eps=1e-5, mx_specs=specs).to(torch.bfloat16).to(dev)
+        xi = x.clone().requires_grad_(True)
+        y = softmax(gelu(ln(lin(xi)), mx_specs=specs), dim=-1, mx_specs=specs)
+        (y * torch.arange(128, device=dev).to(torch.bfloat16)).sum().backward()
+        assert torch.isfinite(y).all() and torch.isfinite(xi.grad).all() and torch.isfinite(lin.weight.grad).all()
+        out[rnd] = (y.detach().float(), xi.grad.float())
+    assert (out["dither"][0] - out["nearest"][0]).abs().max().item() <= 0.05
+    assert (out["dither"][0].sum(-1) - 1).abs().max().item() <= 0.05
+    assert not torch.equal(out["dither"][0], out["nearest"][0])
