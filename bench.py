@@ -98,7 +98,7 @@ def make_workload(name):
                     launches=1 if dim == -1 else 2,
                     desc="reduce %s over axis %d, fp32 [16384,8192]" % (op, dim))
     if name in ("mx_linear", "mx_linear_unfused", "mx_linear_fp4", "mx_linear_fp4_unfused",
-                "mx_linear_fp6", "mx_linear_fp6_unfused"):
+                "mx_linear_fp6", "mx_linear_fp6_unfused", "mx_linear_bfloat16", "mx_linear_bfloat16_unfused"):
         # config 4: mx.Linear forward, MXFP8 e4m3 (or MXFP4 e2m1) both operands, block 32 along K, bias
         from microxcaling_amd import gemm
         from microxcaling_amd.linear import linear
@@ -109,7 +109,10 @@ def make_workload(name):
         w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
         b = torch.randn(N, generator=g).to(torch.bfloat16)
         ef = "fp4_e2m1" if "fp4" in name else "fp6_e2m3" if "fp6" in name else "fp8_e4m3"
-        specs = finalize_mx_specs({"w_elem_format": ef, "a_elem_format": ef, "block_size": 32})
+        spec_dict = {"w_elem_format": ef, "a_elem_format": ef, "block_size": 32}
+        if "bfloat16" in name:                   # the same layer with bfloat16 vector quantization as well:
+            spec_dict["bfloat"] = 16             # operands, product and bias sum go through it
+        specs = finalize_mx_specs(spec_dict)
         dev_extra = {}
         fused = not name.endswith("_unfused")
 
@@ -118,7 +121,8 @@ def make_workload(name):
                 dev_extra["w"], dev_extra["b"] = w.to(xd.device), b.to(xd.device)
             gemm.set_fused(fused)
             return linear(xd, dev_extra["w"], dev_extra["b"], mx_specs=specs)
-        return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, ef, ef),
+        bf = 16 if "bfloat16" in name else 0
+        return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, ef, ef, bfloat=bf),
                     flops=2.0 * M * N * K, bytes=0, dtype="%s x %s -> f32 acc" % (ef, ef), sample_axis=0,
                     cpu_rows=1024, launches=5, peak="fp4" if ef == "fp4_e2m1" else "fp8",   # fp6 runs on byte codes: fp8 rate
                     desc="mx.Linear forward: x bf16 [16384,4096], W bf16 [14336,4096] ~N(0,0.02), bias; %s "

@@ -474,8 +474,40 @@ __device__ __forceinline__ void store_c8(void* c, const void* bias, uint32_t q_n
 
 // Epilogue of eight consecutive columns n .. n + 7 of one row, packed to a 16-bit output type
 // (inside tiles only: n + 7 < N, bias 16-byte aligned at n).
+// With the bfloat16 quantization (q_nan_from != 0) the plain range is tried first: while every value
+// the wave handles in this call -- the rounded products and, with a bias, the rounded sums -- is a
+// normal number below the NaN threshold, the quantizer is "odd significand -> + 1" on both halves of a
+// dword at once (convert, range check with packed 16-bit subtract / max, add: three to four
+// instructions per value against a dozen per quantization, which bounded write-heavy products).
+// Must be called by all lanes of a wave together.
 template <int OUT_DT>
 __device__ __forceinline__ u32x4 epilogue_pack8(const void* bias, uint32_t q_nan_from, int n, v4f lo, v4f hi) {
+    if constexpr (OUT_DT == MXQ_BF16) {
+        if (q_nan_from != 0u) {                              // uniform
+            const unsigned short span = (unsigned short)((q_nan_from >> 16) - 0x0080u);
+            uint32_t w[4] = {Pack<MXQ_BF16>::put(lo[0], lo[1]), Pack<MXQ_BF16>::put(lo[2], lo[3]),
+                             Pack<MXQ_BF16>::put(hi[0], hi[1]), Pack<MXQ_BF16>::put(hi[2], hi[3])};
+            u16x2 worst = {0, 0};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                worst = __builtin_elementwise_max(
+                    worst, __builtin_bit_cast(u16x2, w[d] & 0x7FFF7FFFu) - u16x2{0x0080, 0x0080});
+                w[d] += w[d] & 0x00010001u;
+            }
+            if (bias != nullptr) {
+                const u32x4 bw = *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned short*>(bias) + n);
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    w[d] = Pack<MXQ_BF16>::put(Pack<MXQ_BF16>::get(w[d], 0) + Pack<MXQ_BF16>::get(bw[d], 0),
+                                               Pack<MXQ_BF16>::get(w[d], 1) + Pack<MXQ_BF16>::get(bw[d], 1));
+                    worst = __builtin_elementwise_max(
+                        worst, __builtin_bit_cast(u16x2, w[d] & 0x7FFF7FFFu) - u16x2{0x0080, 0x0080});
+                    w[d] += w[d] & 0x00010001u;
+                }
+            }
+            if (__all(worst[0] < span && worst[1] < span)) return u32x4{w[0], w[1], w[2], w[3]};
+        }
+    }
     float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     if (bias != nullptr) {
         const u32x4 bw = *reinterpret_cast<const u32x4*>(reinterpret_cast<const unsigned short*>(bias) + n);
@@ -640,38 +672,10 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
             // instruction then writes eight full 128-byte lines instead of sixteen half lines.
             const bool low = frow < 8;
             const int ncol = n0 + wx * 64 + (low ? 0 : 32) + fg * 8;
-            // bfloat16 quantization without a bias, plain range: while every value of the wave's 16 x 64
-            // piece is a normal number below the NaN threshold, the quantizer is "odd significand -> + 1"
-            // on both halves of a dword at once (three instructions per value with the range check,
-            // against a dozen: the epilogue, not the stores, bounded the one-step products)
-            const bool try_plain = OUT_DT == MXQ_BF16 && g.bias == nullptr && g.q_nan_from != 0u;
-            const unsigned short span = (unsigned short)((g.q_nan_from >> 16) - 0x0080u);
 #pragma unroll
             for (int ti = 0; ti < 4; ++ti) {
-                u32x4 p0, p1;
-                bool plain = false;
-                if (try_plain) {
-                    uint32_t w[8];
-                    u16x2 worst = {0, 0};
-#pragma unroll
-                    for (int d = 0; d < 8; ++d) {
-                        const v4f& a = acc[ti][d >> 1];
-                        w[d] = Pack<MXQ_BF16>::put(a[(d & 1) * 2], a[(d & 1) * 2 + 1]);
-                        worst = __builtin_elementwise_max(
-                            worst, __builtin_bit_cast(u16x2, w[d] & 0x7FFF7FFFu) - u16x2{0x0080, 0x0080});
-                    }
-                    plain = __all(worst[0] < span && worst[1] < span);
-                    if (plain) {
-#pragma unroll
-                        for (int d = 0; d < 8; ++d) w[d] += w[d] & 0x00010001u;
-                        p0 = u32x4{w[0], w[1], w[2], w[3]};
-                        p1 = u32x4{w[4], w[5], w[6], w[7]};
-                    }
-                }
-                if (!plain) {
-                    p0 = epilogue_pack8<OUT_DT>(g.bias, g.q_nan_from, n0 + wx * 64 + fg * 8, acc[ti][0], acc[ti][1]);
-                    p1 = epilogue_pack8<OUT_DT>(g.bias, g.q_nan_from, n0 + wx * 64 + 32 + fg * 8, acc[ti][2], acc[ti][3]);
-                }
+                const u32x4 p0 = epilogue_pack8<OUT_DT>(g.bias, g.q_nan_from, n0 + wx * 64 + fg * 8, acc[ti][0], acc[ti][1]);
+                const u32x4 p1 = epilogue_pack8<OUT_DT>(g.bias, g.q_nan_from, n0 + wx * 64 + 32 + fg * 8, acc[ti][2], acc[ti][3]);
                 const u32x4 send = low ? p1 : p0;
                 u32x4 recv;
 #pragma unroll

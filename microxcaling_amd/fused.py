@@ -187,8 +187,8 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
                pre_bfloat16=False):
     """a (..., M, K) x b_kmajor (N, K) or (..., N, K), both MX-quantized along K: the fused
     equivalent of quantize_mx_op(a, axes=[-1]) @ quantize_mx_op(b, axes=[-1]).T (+ bias, see
-    gemm_nt).  pre_bfloat16: both operands are bf16 tensors that have not been through the layers'
-    elementwise bfloat16 / round-half-away quantization yet; the pack kernels apply it.  Returns None
+    gemm_nt).  pre_bfloat16 (a bool, or one per operand): the operand is a bf16 tensor that has not been
+    through the layers' elementwise bfloat16 / round-half-away quantization yet; its pack kernel applies it.  Returns None
     when the operands do not qualify (the caller then takes the unfused path)."""
     fa, fb = _as_format(a_fmt), _as_format(b_fmt)
     if fa not in _PACKABLE or fb not in _PACKABLE:
@@ -222,11 +222,12 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
         return None
     if epilogue_quant and a.dtype != torch.bfloat16:
         return None
-    if pre_bfloat16 and (a.dtype != torch.bfloat16 or b_kmajor.dtype != torch.bfloat16):
+    pre_a, pre_b = pre_bfloat16 if isinstance(pre_bfloat16, tuple) else (pre_bfloat16, pre_bfloat16)
+    if (pre_a and a.dtype != torch.bfloat16) or (pre_b and b_kmajor.dtype != torch.bfloat16):
         return None
     nibbles = _use_nibbles(fa, fb, K)
-    pa = pack_mx(a2, fa, scale_bits, round, flush, nibbles, pre_bfloat16)
-    pb = pack_mx(b2, fb, scale_bits, round, flush, nibbles, pre_bfloat16)
+    pa = pack_mx(a2, fa, scale_bits, round, flush, nibbles, pre_a)
+    pb = pack_mx(b2, fb, scale_bits, round, flush, nibbles, pre_b)
     return gemm_nt(pa, pb, out_dtype=a.dtype, bias=bias, epilogue_quant=epilogue_quant).reshape(out_shape)
 
 

@@ -63,14 +63,17 @@ def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, out_round=None, bias=
     return fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, pre_bfloat16=pre_bfloat16), False
 
 
-def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, out_round=None, bias=None):
+def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, out_round=None, bias=None, pre_bfloat16=False):
     """x (..., K) times w (N, K) transposed: both operands share exponents along their last axis.
     out_round / bias: what the caller does next -- elementwise-quantize the product with that
     rounding, add the (already quantized) bias, quantize again.  Returns (out, finished); when
-    finished, those steps have been done in the GEMM's epilogue."""
-    out, finished = _try_fused(x, w, a_fmt, w_fmt, mx_specs, round, out_round, bias)
+    finished, those steps have been done in the GEMM's epilogue.  pre_bfloat16 (one flag per operand):
+    as for mx_matmul_contract."""
+    out, finished = _try_fused(x, w, a_fmt, w_fmt, mx_specs, round, out_round, bias, pre_bfloat16)
     if out is not None:
         return out, finished
+    if pre_bfloat16:
+        return None, False
     qx = quantize_mx_op(x, mx_specs, elem_format=a_fmt, axes=[-1], round=round)
     qw = quantize_mx_op(w, mx_specs, elem_format=w_fmt, axes=[-1], round=round)
     # prequantized bf16 weights meet inputs of another dtype (mx/linear.py:77-80)

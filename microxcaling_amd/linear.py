@@ -3,7 +3,7 @@ import torch
 import torch.nn.functional as F
 
 from .elemwise_ops import quantize_elemwise_op
-from .gemm import mx_grad_contract, mx_linear_contract
+from .gemm import inputs_can_skip_bfloat16_pass, mx_grad_contract, mx_linear_contract
 from .mx_ops import quantize_mx_op
 from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
 
@@ -20,6 +20,31 @@ class LinearFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, weight, bias=None, mx_specs=None, prequantized_weights=False,
                 name=None):
+        # inference: nothing keeps the quantized operands, so their bfloat16 quantization is left to the
+        # pack kernels of the fused GEMM (prequantized weights imply round-half-even, where that
+        # quantization is a cast and there is nothing to leave)
+        if not prequantized_weights and \
+                inputs_can_skip_bfloat16_pass(ctx.needs_input_grad[:2], (input, weight), mx_specs,
+                                              mx_specs["round_output"]) and \
+                inputs_can_skip_bfloat16_pass((), (), mx_specs, mx_specs["round_weight"]):
+            bf_bias = None if bias is None else quantize_elemwise_op(
+                bias, mx_specs=mx_specs, round=mx_specs["round_weight"])
+            output, finished = mx_linear_contract(input, weight, mx_specs["a_elem_format"],
+                                                  mx_specs["w_elem_format"], mx_specs,
+                                                  mx_specs["round_mx_output"],
+                                                  out_round=mx_specs["round_output"], bias=bf_bias,
+                                                  pre_bfloat16=True)
+            if output is not None:
+                if not finished:
+                    output = quantize_elemwise_op(output, mx_specs=mx_specs, round=mx_specs["round_output"])
+                    if bias is not None:
+                        output = quantize_elemwise_op(output + bf_bias, mx_specs=mx_specs,
+                                                      round=mx_specs["round_output"])
+                ctx.has_bias = bias is not None
+                ctx.mx_specs = get_backwards_mx_specs(mx_specs)
+                ctx.prequantized_weights = prequantized_weights
+                ctx.name = name
+                return output
         bf_in = quantize_elemwise_op(input, mx_specs=mx_specs, round=mx_specs["round_output"])
         if prequantized_weights:
             assert weight.dtype == torch.bfloat16

@@ -313,6 +313,35 @@ def test_inference_skips_the_operand_quantization_pass(dev, fn):
     assert torch.equal(plain.view(torch.int16), with_grad.detach().view(torch.int16))
 
 
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("shape", [(640, 512, 768), (1030, 520, 1152), (70, 136, 256)])
+def test_linear_inference_skips_the_operand_quantization_passes(dev, with_bias, shape):
+    """mx.Linear under bfloat=16 without gradients: operands quantized by the pack kernels, product
+    and bias sum by the GEMM's epilogue (plain-range form where it applies) -- bit for bit the output
+    of the same layer with gradients wanted (separate passes), large and small tiles."""
+    from microxcaling_amd.linear import Linear, linear
+    M, N, K = shape
+    specs = _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32, bfloat=16)
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(dev)
+    x[0, :40] = 0.0
+    w = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    w[3] = 0.0                                               # a column of exact zeros in the product
+    b = torch.randn(N, generator=g).to(torch.bfloat16).to(dev) if with_bias else None
+    plain = linear(x, w, b, mx_specs=specs)
+    with_grad = linear(x.clone().requires_grad_(True), w, b, mx_specs=specs)
+    assert with_grad.requires_grad and not plain.requires_grad
+    assert torch.equal(plain.view(torch.int16), with_grad.detach().view(torch.int16))
+    mod = Linear(K, N, bias=with_bias, mx_specs=specs).to(torch.bfloat16).to(dev)
+    with torch.no_grad():
+        mod.weight.copy_(w)
+        if with_bias:
+            mod.bias.copy_(b)
+    assert torch.equal(mod(x).detach().view(torch.int16), plain.view(torch.int16))      # parameters want gradients
+    with torch.no_grad():
+        assert torch.equal(mod(x).view(torch.int16), plain.view(torch.int16))
+
+
 def test_gemm_propagates_nan_blocks(dev):
     from microxcaling_amd.fused import pack_mx, gemm_nt
     a = torch.randn(128, 128)
