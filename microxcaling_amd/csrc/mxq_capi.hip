@@ -293,6 +293,14 @@ int mxq_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int b
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     if (!aligned16(in) || !aligned16(out))
         return fail(MXQ_ERR_ARGUMENT, "%s: pointers must be 16-byte aligned", who);
+    // bf16 tensor -> bfloat16, round-half-away, subnormals kept, overflow to Inf: the closed form
+    if (dtype == MXQ_DTYPE_BF16 && bits == 9 && exp_bits == 8 && rmode == MXQ_ROUND_NEAREST && allow_denorm &&
+        !saturate_normals && p.fmt.max_bits == 0x7F7F0000u &&
+        !(flags & (MXQ_FLAG_EXACT_EXPONENT | MXQ_FLAG_GENERAL_FORM))) {
+        const int grid = grid_for(ceil_div(ceil_div(n, 8), (int64_t)kThreads * kElemUnroll));
+        elemwise_bf16_closed_kernel<kElemUnroll><<<grid, kThreads, 0, (hipStream_t)hip_stream>>>(in, out, n, p.fmt.nan_from);
+        return check_launch(who);
+    }
     dispatch<LaunchElemwise>(dtype, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode), lean_ok(dtype, p.fmt, rmode, true), in, out, n, p, (hipStream_t)hip_stream);
     return check_launch(who);
 }

@@ -473,6 +473,58 @@ __global__ __launch_bounds__(TPB) void elemwise_kernel(const void* __restrict__ 
 }
 
 // ================================================================================================
+// Elementwise quantization of a bf16 tensor to bfloat16 with round-half-away (the vector format of
+// most MX configurations, applied to every operand, product and gradient): the closed form of
+// mxq_quant_bf16_to_bfloat16_nearest instead of the general rounding.  While all of a wave's values
+// are normal numbers below the NaN threshold it is "odd significand -> + 1" on both halves of a dword
+// at once; a wave that sees anything else goes element by element.
+// ================================================================================================
+template <int UNROLL>
+__global__ __launch_bounds__(TPB) void elemwise_bf16_closed_kernel(const void* __restrict__ in_,
+                                                                   void* __restrict__ out_, int64_t n,
+                                                                   uint32_t nan_from) {
+    const u32x4* in = reinterpret_cast<const u32x4*>(in_);
+    u32x4* out = reinterpret_cast<u32x4*>(out_);
+    const unsigned short span = (unsigned short)((nan_from >> 16) - 0x0080u);
+    const int64_t n_vec = n / 8;
+    const int64_t stride = (int64_t)gridDim.x * TPB * UNROLL;
+    for (int64_t base = (int64_t)blockIdx.x * TPB * UNROLL + threadIdx.x; base - threadIdx.x < n_vec;
+         base += stride) {
+        u32x4 v[UNROLL];
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            const int64_t i = base + (int64_t)j * TPB;
+            v[j] = (i < n_vec) ? in[i] : u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+        }
+#pragma unroll
+        for (int j = 0; j < UNROLL; ++j) {
+            const int64_t i = base + (int64_t)j * TPB;
+            u16x2 worst = {0, 0};
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                worst = __builtin_elementwise_max(
+                    worst, __builtin_bit_cast(u16x2, v[j][d] & 0x7FFF7FFFu) - u16x2{0x0080, 0x0080});
+            u32x4 o;
+            if (__all(worst[0] < span && worst[1] < span)) {
+#pragma unroll
+                for (int d = 0; d < 4; ++d) o[d] = v[j][d] + (v[j][d] & 0x00010001u);
+            } else {
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+                    o[d] = Pack<MXQ_BF16>::put(
+                        mxq_quant_bf16_to_bfloat16_nearest(Pack<MXQ_BF16>::get(v[j][d], 0), nan_from),
+                        mxq_quant_bf16_to_bfloat16_nearest(Pack<MXQ_BF16>::get(v[j][d], 1), nan_from));
+            }
+            if (i < n_vec) __builtin_nontemporal_store(o, &out[i]);
+        }
+    }
+    const int64_t t0 = n_vec * 8;
+    const int64_t gi = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (gi < n - t0)
+        store_scalar<MXQ_BF16>(out_, t0 + gi, mxq_quant_bf16_to_bfloat16_nearest(load_scalar<MXQ_BF16>(in_, t0 + gi), nan_from));
+}
+
+// ================================================================================================
 // round='dither' (mx/elemwise_ops.py:57-59): floor(scaled value + noise) with noise in [0, 1) drawn
 // by the caller in the tensor dtype, one per element.  A training-time option off the hot path:
 // one element per lane, op-by-op form of the rounding.

@@ -262,6 +262,24 @@ def test_dither_with_the_reference_noise(dev):
     assert torch.isfinite(got).all()
 
 
+def test_bf16_to_bfloat16_closed_form_every_code(dev):
+    """bf16 tensors quantized to bfloat16 with round-half-away take a kernel of their own (closed
+    form, packed pairs in the plain range): every bf16 code, in waves of plain values only and in
+    mixed order, with a ragged tail, against the oracle."""
+    codes = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    mags = codes.float().abs()
+    plain = codes[(mags >= 2.0 ** -126) & (mags < 2.0 ** 127)]
+    g = torch.Generator().manual_seed(21)
+    x = torch.cat([plain.repeat(4), codes[torch.randperm(65536, generator=g)], codes, plain[:4099]])
+    mn = 2 ** 127 * 255 / 128
+    want = O.quantize_elemwise_core(x, 9, 8, mn, round="nearest")
+    got = elem_gpu(x.to(dev), 9, 8, mn, round="nearest")
+    assert_bits_equal(got, want, "closed form")
+    # the neighbouring cases stay on the general kernel and agree with the oracle as before
+    for kw in (dict(round="floor"), dict(round="nearest", saturate_normals=True), dict(round="nearest", allow_denorm=False)):
+        assert_bits_equal(elem_gpu(x.to(dev), 9, 8, mn, **kw), O.quantize_elemwise_core(x, 9, 8, mn, **kw), str(kw))
+
+
 def test_mx_given_max_entry_point(dev):
     """quantize_mx_func_cuda: the caller reshapes to blocks and supplies the abs-max
     (mx/mx_ops.py:226-256)."""
