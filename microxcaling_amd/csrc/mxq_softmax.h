@@ -1312,11 +1312,44 @@ __global__ __launch_bounds__(TPB) void norm_param_grad_partial_kernel(const void
         for (int j = 0; j < UNROLL; ++j) {
             const int64_t rr = r + j * WAVES;
             const bool ok = live && rr < r1;
-            vg[j] = ok ? __builtin_nontemporal_load(&g[rr * nvec_row]) : u32x4{0, 0, 0, 0};
-            vz[j] = ok ? __builtin_nontemporal_load(&z[rr * nvec_row]) : u32x4{0, 0, 0, 0};
+            // rows past the chunk read as +0 (they add nothing); lanes past the row read as 1.0 so that
+            // they do not spoil the wave's vote below (their sums are never stored)
+            const u32x4 pad = live ? u32x4{0, 0, 0, 0} : u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+            vg[j] = ok ? __builtin_nontemporal_load(&g[rr * nvec_row]) : pad;
+            vz[j] = ok ? __builtin_nontemporal_load(&z[rr * nvec_row]) : pad;
         }
 #pragma unroll
         for (int j = 0; j < UNROLL; ++j) {
+            if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) {
+                // plain range: while every gradient of the wave's row piece and every rounded product is a
+                // normal number below the NaN threshold, both quantizations are "odd significand -> + 1"
+                // on the two halves of a dword at once; the sums take the same values in the same order
+                const unsigned short span = (unsigned short)((q.fmt.nan_from >> 16) - 0x0080u);
+                u16x2 worst = {0, 0};
+                uint32_t gq[4], pq[4];
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    worst = __builtin_elementwise_max(
+                        worst, __builtin_bit_cast(u16x2, vg[j][d] & 0x7FFF7FFFu) - u16x2{0x0080, 0x0080});
+                    gq[d] = vg[j][d] + (vg[j][d] & 0x00010001u);
+                    const uint32_t pw = Pack<MXQ_BF16>::put(
+                        Pack<MXQ_BF16>::get(gq[d], 0) * Pack<MXQ_BF16>::get(vz[j][d], 0),
+                        Pack<MXQ_BF16>::get(gq[d], 1) * Pack<MXQ_BF16>::get(vz[j][d], 1));
+                    worst = __builtin_elementwise_max(
+                        worst, __builtin_bit_cast(u16x2, pw & 0x7FFF7FFFu) - u16x2{0x0080, 0x0080});
+                    pq[d] = pw + (pw & 0x00010001u);
+                }
+                if (__all(!q.general_only && worst[0] < span && worst[1] < span)) {
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            acc_w[d * 2 + h] += Pack<MXQ_BF16>::get(pq[d], h);
+                            acc_b[d * 2 + h] += Pack<MXQ_BF16>::get(gq[d], h);
+                        }
+                    continue;
+                }
+            }
 #pragma unroll
             for (int d = 0; d < 4; ++d)                    // rows past the chunk were read as +0
 #pragma unroll

@@ -831,6 +831,17 @@ def test_fused_norm_param_grads(dev, dtype, spec, shape):
     z = (torch.randn(*shape, generator=gen) * 1.5).to(dtype).to(dev)
     fused = L._fused_param_grads(g, z, specs)
     assert fused is not None
+    # the packed plain-range form (bf16 tensors, bfloat16) and the general form add the same values in
+    # the same order: bit for bit, also with zeros, tiny and huge values in some rows
+    g2, z2 = g.clone(), z.clone()
+    g2.view(-1, shape[-1])[0, :4] = 0.0
+    z2.view(-1, shape[-1])[-1, :3] = torch.tensor([1e-30, 3e38, float("inf")]).to(dtype).to(dev)
+    for gg, zz in ((g, z), (g2, z2)):
+        a = L._fused_param_grads(gg, zz, specs)
+        with _general_form():
+            b = L._fused_param_grads(gg, zz, specs)
+        assert torch.equal(torch.nan_to_num(a[0].float()), torch.nan_to_num(b[0].float()))
+        assert torch.equal(torch.isnan(a[0]), torch.isnan(b[0])) and torch.equal(a[1], b[1])
     gemm.set_fused(False)
     try:
         assert L._fused_param_grads(g, z, specs) is None
