@@ -201,6 +201,7 @@ def make_workload(name):
         specs = finalize_mx_specs({"bfloat": 16})
         fused = not name.endswith("unfused")
         g = torch.Generator().manual_seed(6)
+        extra = {}
         if name.startswith("softmax"):
             x = (torch.randn(16384, 2048, generator=g) * 3).to(torch.bfloat16).repeat(16, 1)
             per_elem, what = 4, "softmax over the last axis, bf16 [262144,2048]"
@@ -222,7 +223,8 @@ def make_workload(name):
                     return ln["m"](xd)
             cpu_ln = LayerNorm(4096, eps=1e-5, mx_specs=specs).to(torch.bfloat16)
             cpu = lambda t: cpu_ln(t)
-        return dict(x=x, gpu=run, cpu=cpu, bytes=x.numel() * per_elem, dtype="bf16", sample_axis=0,
+            extra["cpu_what"] = "this package's LayerNorm on CPU tensors (host-library quantizers)"
+        return dict(x=x, gpu=run, cpu=cpu, bytes=x.numel() * per_elem, dtype="bf16", sample_axis=0, **extra,
                     launches=1 if fused else 12,
                     desc="%s, bfloat16 quantization after every step, %s" % (what, "one kernel" if fused else
                                                                              "separate tensor passes"))
@@ -249,6 +251,7 @@ def make_workload(name):
             return xi.grad
         cpu_ln = LayerNorm(4096, eps=1e-5, mx_specs=specs).to(torch.bfloat16)
         return dict(x=x, gpu=run, cpu=lambda t: cpu_ln(t), bytes=x.numel() * (6 + 6 + 4), dtype="bf16", sample_axis=0,
+                    cpu_what="this package's LayerNorm forward on CPU tensors (host-library quantizers)",
                     launches=8 if fused else 50,
                     desc="LayerNorm forward + backward, bf16 [32768,4096], bfloat16 quantization after every step, %s"
                          % ("two row kernels + column-sum kernels for the parameter gradients" if fused else "separate tensor passes"))
@@ -321,6 +324,7 @@ def make_workload(name):
         zc = (torch.randn(x.shape, generator=torch.Generator().manual_seed(10)) * 1.5).to(torch.bfloat16)
         return dict(x=x, gpu=run, cpu=lambda t: _param_grads(t, zc[:t.shape[0], :t.shape[1]].contiguous(), specs), bytes=x.numel() * 4,
                     dtype="bf16", sample_axis=0, launches=2,
+                    cpu_what="this package's separate steps on CPU tensors (host-library quantizers)",
                     desc="LayerNorm weight and bias gradients, bf16 [32768,4096], bfloat16 quantization: "
                          "two column-sum launches (CPU leg: this package's separate steps on CPU tensors)")
     if name == "pack_t_bf16":
@@ -373,9 +377,9 @@ def cpu_baseline(wl, budget_s=15.0):
     t = times[len(times) // 2]
     return {"value": round(wl["bytes"] / t / 1e9, 4), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": "the full workload tensor (%s), %d passes in %.1f s, median pass %.3f s; torch %s "
-                      "op-by-op oracle (oracle/mx_oracle.py), %d threads"
+                      "%s, %d threads"
                       % ("x".join(str(n) for n in x.shape), len(times), time.perf_counter() - t_all, t,
-                         torch.__version__, cores)}
+                         torch.__version__, wl.get("cpu_what", "op-by-op oracle (oracle/mx_oracle.py)"), cores)}
 
 
 # MI355X dense MFMA peaks, published: fp8 (e4m3 / e5m2 byte codes, which also carry fp6 elements) and

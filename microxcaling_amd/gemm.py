@@ -86,9 +86,14 @@ def inputs_can_skip_bfloat16_pass(needs_grad, tensors, mx_specs, round):
     """May a layer leave its operands' elementwise quantization to the pack kernels of the fused GEMM?
     Only when nothing keeps the quantized operands (no gradient is wanted), they are bf16 GPU tensors
     and the quantizer is bfloat16 with round-half-away, the form those kernels know."""
-    return (_use_fused and not any(needs_grad)
-            and all(t.is_cuda and t.dtype == torch.bfloat16 for t in tensors)
-            and _epilogue_mode(mx_specs, round, torch.bfloat16) == 1)
+    return (not any(needs_grad) and all(t.is_cuda and t.dtype == torch.bfloat16 for t in tensors)
+            and pack_can_quantize_first(mx_specs, round))
+
+
+def pack_can_quantize_first(mx_specs, round):
+    """Is quantize_elemwise_op(., mx_specs, round) on a bf16 tensor the bfloat16 / round-half-away
+    quantizer that the pack kernel can apply itself, and are the fused kernels in use?"""
+    return _use_fused and _epilogue_mode(mx_specs, round, torch.bfloat16) == 1
 
 
 def mx_matmul_contract(a, b, a_fmt, b_fmt, mx_specs, round, batched=False, out_round=None, bias=None,

@@ -3,7 +3,8 @@ import torch
 import torch.nn.functional as F
 
 from .elemwise_ops import quantize_elemwise_op
-from .gemm import inputs_can_skip_bfloat16_pass, mx_grad_contract, mx_linear_contract
+from .gemm import (inputs_can_skip_bfloat16_pass, mx_grad_contract, mx_linear_contract,
+                   pack_can_quantize_first)
 from .mx_ops import quantize_mx_op
 from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
 
@@ -26,7 +27,7 @@ class LinearFunction(torch.autograd.Function):
         if not prequantized_weights and \
                 inputs_can_skip_bfloat16_pass(ctx.needs_input_grad[:2], (input, weight), mx_specs,
                                               mx_specs["round_output"]) and \
-                inputs_can_skip_bfloat16_pass((), (), mx_specs, mx_specs["round_weight"]):
+                pack_can_quantize_first(mx_specs, mx_specs["round_weight"]):
             bf_bias = None if bias is None else quantize_elemwise_op(
                 bias, mx_specs=mx_specs, round=mx_specs["round_weight"])
             output, finished = mx_linear_contract(input, weight, mx_specs["a_elem_format"],
