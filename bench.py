@@ -9,13 +9,19 @@ baseline (the torch op-sequence oracle timed on this box's host cores on a bound
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
 
-Workloads (all sizes from BASELINE.json):
+Workloads (config N = the N-th benchmark configuration of this build's baseline file):
     mxfp8_fp32_8192      headline (default)
     mxfp8_fp32_4096      config 1 (fits in the 256 MB Infinity Cache -- not an HBM figure)
     mxfp6_e3m2_bf16_m1 / mxfp6_e2m3_bf16_m1 / mxfp4_bf16_m1      config 2, axis -1
     mxfp6_e3m2_bf16_m2 / mxfp6_e2m3_bf16_m2 / mxfp4_bf16_m2      config 2, axis -2
     elem_bf16_fp32 / elem_fp16_fp32                              config 3, elementwise
     reduce_sum_m1 / reduce_max_m1 / reduce_sum_0 / reduce_max_0  config 3, reductions
+    mx_linear / mx_linear_fp4 / mx_linear_fp6 / mx_linear_bfloat16  config 4: mx.Linear forward (TFLOP/s)
+    mx_linear_train                                              ... forward + backward
+    mx_bmm_softmax                                               config 5: mx.bmm + bfloat16 softmax
+    softmax_bf16 / layernorm_bf16 / gelu_bf16 / silu_bf16 (+ _train), norm_param_grads_bf16, pack_t_bf16,
+    mxfp8_fp32_8192_tiles                                        single kernels of the layers around the path
+    (suffix _unfused where it exists: the same step as separate tensor passes)
     copy_fp32_8192       torch copy_ of the headline tensor (calibrates the rocprof byte counters)
 """
 import argparse

@@ -359,7 +359,7 @@ def _specs(**kw):
 @pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear_forward_matches_reference_forward(dev, fused, dtype):
-    """mx.Linear forward (BASELINE config 4 at a reduced size): quantize-then-fp32-matmul oracle,
+    """mx.Linear forward (the benchmark's MXFP8 linear layer at a reduced size): quantize-then-fp32-matmul oracle,
     relative tolerance 1e-3 (max |diff| / RMS of the output)."""
     from microxcaling_amd import gemm
     from microxcaling_amd.linear import linear
