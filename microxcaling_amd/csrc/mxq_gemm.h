@@ -190,7 +190,8 @@ __global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict_
     constexpr int UPC = PACKT_TILES * UPT;               // ... per column of the workgroup
     constexpr int LDC = UPC + 1;                         // padded column pitch in LDS
     __shared__ unsigned char zone[ZONE_PAD];
-    __shared__ u32x2 stage[NCOL * LDC];
+    constexpr int HV = VW / 2;                           // columns of a lane per hand-over
+    __shared__ u32x2 stage[(NCOL / 2) * LDC];
     __shared__ uint32_t stage_scales[NCOL];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -218,45 +219,48 @@ __global__ __launch_bounds__(TPB) void mx_pack_t_kernel(const u32x2* __restrict_
             for (int h = 0; h < PD; ++h)
                 um[d * PD + h] = max(um[d * PD + h], abs_bits(Pack<DT>::get(raw[r][d], h)));
 
-    uint32_t scale_bytes[VW];
-#pragma unroll
-    for (int k = 0; k < VW; ++k) {
-        const MxqScale sc = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, ZS);
-        uint32_t out[8] = {};
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-            const uint32_t code = mx_code_of<RMODE, ADT, ZONE_ELEM, KIND, DIRECT>(
-                Pack<DT>::get(raw[r][k / PD], k % PD), sc, p, zone, ZS, max_code);
-            if (code_bits<KIND>() == 6) {
-                out[(6 * r) >> 5] |= code << ((6 * r) & 31);
-                if (((6 * r) & 31) > 26) out[((6 * r) >> 5) + 1] |= code >> (32 - ((6 * r) & 31));
-            } else if (KIND == 4) out[r / 8] |= code << (4 * (r % 8));
-            else out[r / 4] |= code << (8 * (r % 4));
-        }
-        u32x2* dst = stage + (lane * VW + k) * LDC + wave * UPT;
-#pragma unroll
-        for (int u = 0; u < UPT; ++u) dst[u] = u32x2{out[2 * u], out[2 * u + 1]};
-        scale_bytes[k] = mxq_encode_e8m0(sc.scale);
-    }
-#pragma unroll
-    for (int k = 0; k < VW; ++k)
-        reinterpret_cast<unsigned char*>(stage_scales)[(lane * VW + k) * PACKT_TILES + wave] =
-            (unsigned char)scale_bytes[k];
-    __syncthreads();
-
-    // hand-over: consecutive lanes write consecutive 8-byte units of a column
+    // hand-over in two halves (the lane's first VW / 2 columns, then the rest) so that the staging
+    // area is half the size and twice as many workgroups fit a CU: consecutive lanes write
+    // consecutive 8-byte units of a column
     const int64_t C = pv * VW;
     const int64_t col0 = cg * NCOL;
     const int64_t t0 = tg * PACKT_TILES;
     const int live_tiles = (n_tiles - t0 < PACKT_TILES) ? (int)(n_tiles - t0) : PACKT_TILES;
     const int live_units = live_tiles * UPT;
     const int64_t col_bytes = n_tiles * (UPT * 8);                  // bytes of codes per output column
-    for (int q = threadIdx.x; q < NCOL * UPC; q += TPB) {
-        const int cb = q / UPC, u = q % UPC;
-        if (u < live_units && col0 + cb < C) {
-            u32x2* dst = reinterpret_cast<u32x2*>(codes + (pre_i * C + col0 + cb) * col_bytes + t0 * (UPT * 8));
-            dst[u] = stage[cb * LDC + u];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+        for (int kk = 0; kk < HV; ++kk) {
+            const int k = half * HV + kk;
+            const MxqScale sc = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+            uint32_t out[8] = {};
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const uint32_t code = mx_code_of<RMODE, ADT, ZONE_ELEM, KIND, DIRECT>(
+                    Pack<DT>::get(raw[r][k / PD], k % PD), sc, p, zone, ZS, max_code);
+                if (code_bits<KIND>() == 6) {
+                    out[(6 * r) >> 5] |= code << ((6 * r) & 31);
+                    if (((6 * r) & 31) > 26) out[((6 * r) >> 5) + 1] |= code >> (32 - ((6 * r) & 31));
+                } else if (KIND == 4) out[r / 8] |= code << (4 * (r % 8));
+                else out[r / 4] |= code << (8 * (r % 4));
+            }
+            u32x2* dst = stage + (lane * HV + kk) * LDC + wave * UPT;
+#pragma unroll
+            for (int u = 0; u < UPT; ++u) dst[u] = u32x2{out[2 * u], out[2 * u + 1]};
+            reinterpret_cast<unsigned char*>(stage_scales)[(lane * VW + k) * PACKT_TILES + wave] =
+                (unsigned char)mxq_encode_e8m0(sc.scale);
         }
+        __syncthreads();
+        for (int q = threadIdx.x; q < (NCOL / 2) * UPC; q += TPB) {
+            const int cb = q / UPC, u = q % UPC;                    // cb = lane * HV + kk
+            const int64_t col = col0 + (cb / HV) * VW + half * HV + (cb % HV);
+            if (u < live_units && col < C) {
+                u32x2* dst = reinterpret_cast<u32x2*>(codes + (pre_i * C + col) * col_bytes + t0 * (UPT * 8));
+                dst[u] = stage[cb * LDC + u];
+            }
+        }
+        __syncthreads();                                            // the staging area is reused
     }
     for (int cb = threadIdx.x; cb < NCOL; cb += TPB) {
         if (col0 + cb < C) {
