@@ -64,6 +64,29 @@ def test_gpu_entry_points_reject_bad_arguments_without_a_gpu():
     assert rc == 1 and b"null" in lib.mxq_last_error()
     assert lib.mxq_quantize_mx_by_tile(None, None, 0, 0, 32, 1, 8, 4, 5, 448.0, 32, 0, 0, 0, None) == 0
     assert lib.mxq_reduce_outer_workspace_bytes(16384, 8192) > 0
+    # the entry points for several shared axes, dither, parameter gradients and the packing flags
+    import ctypes
+    ext = (ctypes.c_int64 * 5)(1, 64, 1, 64, 1)
+    rc = lib.mxq_quantize_mx_axes(None, None, 0, 4, ext, 8, 4, 5, 448.0, 32, 0, 0, 0, None)
+    assert rc == 1 and b"shared axes" in lib.mxq_last_error()
+    rc = lib.mxq_quantize_mx_axes(None, None, 0, 2, ext, 8, 4, 5, 448.0, 32, 0, 0, 0, None)
+    assert rc == 1 and b"null" in lib.mxq_last_error()
+    ext0 = (ctypes.c_int64 * 5)(1, 64, 0, 64, 1)
+    assert lib.mxq_quantize_mx_axes(None, None, 0, 2, ext0, 8, 4, 5, 448.0, 32, 0, 0, 0, None) == 0
+    rc = lib.mxq_quantize_elemwise_dither(None, None, None, 0, 16, 9, 8, 1.0, 0, 1, 0, None)
+    assert rc == 1 and b"null" in lib.mxq_last_error()
+    rc = lib.mxq_quantize_mx_dither_by_tile(None, None, None, 0, 1, 32, 1, 9, 4, 5, 448.0, 32, 0, 0, None)
+    assert rc == 1 and b"scale_bits" in lib.mxq_last_error()
+    need = lib.mxq_norm_param_grads_workspace_bytes(2, 32768, 4096)
+    assert need > 0 and need % (2 * 4096 * 4) == 0
+    assert lib.mxq_norm_param_grads_workspace_bytes(2, 32768, 4100) == 0          # not a multiple of 16 bytes
+    rc = lib.mxq_norm_param_grads(None, None, None, None, None, 0, 2, 8, 4100, 9, 8, 1.0, 0, 1, 0, None)
+    assert rc == 1 and b"multiple" in lib.mxq_last_error()
+    rc = lib.mxq_norm_param_grads(None, None, None, None, None, 0, 2, 8, 4096, 9, 8, 1.0, 0, 1, 0, None)
+    assert rc == 1 and b"null" in lib.mxq_last_error()
+    rc = lib.mxq_pack_mx(ctypes.c_void_p(16), ctypes.c_void_p(16), ctypes.c_void_p(16), 0, 4, 64, 8, 4, 5, 448.0,
+                         0, 0, 32, None)                                         # pre-bfloat16 flag on an fp32 tensor
+    assert rc == 1 and b"bf16" in lib.mxq_last_error()
 
 
 def test_host_functions_reject_gpu_only_misuse():
