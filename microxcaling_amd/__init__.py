@@ -9,7 +9,6 @@ from .specs import (MxSpecs, get_default_mx_specs, get_backwards_mx_specs, apply
 from .formats import ElemFormat, RoundingMode
 from .mx_ops import quantize_mx_op
 from .elemwise_ops import quantize_elemwise_op
-from .quantize import quantize_bfloat
 from .linear import Linear, linear
 from .matmul import matmul
 from .bmm import bmm
@@ -18,10 +17,3 @@ from .layernorm import LayerNorm, RMSNorm, layer_norm
 from .activations import (sigmoid, tanh, relu, relu6, leaky_relu, silu, gelu,
                           Sigmoid, Tanh, ReLU, ReLU6, LeakyReLU, SiLU, GELU)
 from .convolution import Conv1d, Conv2d, Conv3d, conv1d, conv2d, conv3d
-from .transpose_convolution import ConvTranspose2d
-from .rnn import LSTM
-from .adaptive_avg_pooling import adaptive_avg_pool2d, AdaptiveAvgPool2d
-from .batchnorm import BatchNorm1d, BatchNorm2d, BatchNorm3d
-from .groupnorm import GroupNorm
-from .simd_ops import (simd_add, simd_sub, simd_mul, simd_div, simd_split, simd_sqrt, simd_square,
-                       simd_exp, simd_log, simd_reduce_sum, simd_reduce_mean, simd_norm)

@@ -21,11 +21,12 @@ class LinearFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, weight, bias=None, mx_specs=None, prequantized_weights=False,
                 name=None):
-        # inference: nothing keeps the quantized operands, so their bfloat16 quantization is left to the
+        # inference (no gradient wanted for input, weight or bias, so backward never runs and nothing
+        # keeps the quantized operands): their bfloat16 quantization is left to the
         # pack kernels of the fused GEMM (prequantized weights imply round-half-even, where that
         # quantization is a cast and there is nothing to leave)
         if not prequantized_weights and \
-                inputs_can_skip_bfloat16_pass(ctx.needs_input_grad[:2], (input, weight), mx_specs,
+                inputs_can_skip_bfloat16_pass(ctx.needs_input_grad[:3], (input, weight), mx_specs,
                                               mx_specs["round_output"]) and \
                 pack_can_quantize_first(mx_specs, mx_specs["round_weight"]):
             bf_bias = None if bias is None else quantize_elemwise_op(
@@ -88,9 +89,11 @@ class LinearFunction(torch.autograd.Function):
                                            round=specs["round_grad_input"])
 
         # grad_weight = grad_output^T x input, contracted over the example axis; both operands share
-        # exponents along axis -2.  When that axis is a multiple of 32 the blocks do not straddle
-        # batch entries and the tensors can be flattened to 2-D first (one GEMM over all examples)
-        if input.dim() == 2 or input.shape[-2] % 32 == 0:
+        # exponents along axis -2 of the N-D tensors (mx/linear.py:124-143).  When that axis is a whole
+        # number of blocks, no block straddles two batch entries and the tensors can be flattened to
+        # 2-D first (one GEMM over all examples); block_size 0 means one block per batch entry
+        block = specs["block_size"]
+        if input.dim() == 2 or (block > 0 and input.shape[-2] % block == 0):
             grad_weight = mx_grad_contract(
                 grad_output.reshape(-1, out_dim), specs["a_elem_format_bp_ex"],
                 specs["round_mx_grad_output_grad_weight"], True,

@@ -1,6 +1,5 @@
 """Writes reference_layer_vectors.npz: forward outputs and gradients of the reference's MX layers
-(linear, bmm, softmax, LayerNorm, RMSNorm, the activations, convolutions, batch / group norm,
-adaptive pooling, the simd ops, LSTM) on the CPU (``custom_cuda=False``), on small seeded inputs.  Run once, in a
+(linear, bmm, softmax, LayerNorm, RMSNorm, the activations, convolutions) on the CPU (``custom_cuda=False``), on small seeded inputs.  Run once, in a
 container where the reference checkout exists:
 ``python tests/golden/gen_reference_layer_vectors.py /root/reference``.
 Only inputs and the reference's outputs are stored; none of the reference's code is.  The fixtures
@@ -119,15 +118,8 @@ def main(ref_root):
             store(d, "act/%s/%s/out" % (aname, dt_name), out)
             store(d, "act/%s/%s/gx" % (aname, dt_name), xi.grad)
 
-    # convolutions, batch / group norm, pooling, simd ops, LSTM (fp32 tensors)
+    # convolutions (fp32 tensors)
     from mx.convolution import Conv1d, Conv2d
-    from mx.transpose_convolution import ConvTranspose2d
-    from mx.batchnorm import BatchNorm2d
-    from mx.groupnorm import GroupNorm
-    from mx.adaptive_avg_pooling import adaptive_avg_pool2d
-    from mx import simd_ops as so
-    from mx.rnn import LSTM
-    from torch.nn.utils.rnn import pack_padded_sequence
     cspecs = finalize_mx_specs(dict(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32,
                                     bfloat=16, quantize_backprop=True, custom_cuda=False))
 
@@ -160,83 +152,24 @@ def main(ref_root):
     c1go = torch.randn(m(c1).shape, generator=g)
     store(d, "in/c1go", c1go)
     run_module("conv1d/", m, c1, c1go)
-    m = ConvTranspose2d(64, 32, 3, stride=2, padding=1, output_padding=1, mx_specs=cspecs)
-    tgo = torch.randn(m(cx).shape, generator=g)
-    store(d, "in/tgo", tgo)
-    run_module("convT2d/", m, cx, tgo)
 
-    m = BatchNorm2d(64, mx_specs=specs)
-    with torch.no_grad():
-        m.weight.copy_(torch.randn(64, generator=g)); m.bias.copy_(torch.randn(64, generator=g))
-    bgo = torch.randn(cx.shape, generator=g)
-    store(d, "in/bgo", bgo)
-    run_module("bn_train/", m, cx, bgo)
-    store(d, "bn_train/running_mean", m.running_mean)
-    store(d, "bn_train/running_var", m.running_var)
-    m.eval()
-    run_module("bn_eval/", m, cx, bgo, params=False)
-    m = GroupNorm(4, 64, mx_specs=specs)
-    with torch.no_grad():
-        m.weight.copy_(torch.randn(64, generator=g)); m.bias.copy_(torch.randn(64, generator=g))
-    run_module("gn/", m, cx, bgo)
-
-    xi = cx.clone().requires_grad_(True)
-    out = adaptive_avg_pool2d(xi, (2, 3), mx_specs=specs)
-    pgo = torch.randn(out.shape, generator=g)
-    store(d, "in/pgo", pgo)
-    out.backward(pgo)
-    store(d, "pool/out", out)
-    store(d, "pool/gx", xi.grad)
-
-    sa = torch.randn(4, 8, 16, generator=g)
-    sb = torch.randn(8, 1, generator=g) + 2.5
-    sgo = torch.randn(4, 8, 16, generator=g)
-    for name, t in (("sa", sa), ("sb", sb), ("ssgo", sgo)):
-        store(d, "in/" + name, t)
-    binary = {"add": so.simd_add, "sub": so.simd_sub, "mul": so.simd_mul, "div": so.simd_div}
-    for name, fn in binary.items():
-        a, b = sa.clone().requires_grad_(True), sb.clone().requires_grad_(True)
-        out = fn(a, b, mx_specs=specs)
-        out.backward(sgo)
-        store(d, "simd/%s/out" % name, out); store(d, "simd/%s/g1" % name, a.grad); store(d, "simd/%s/g2" % name, b.grad)
-        a = sa.clone().requires_grad_(True)
-        out = fn(a, 1.7, mx_specs=specs)
-        out.backward(sgo)
-        store(d, "simd/%s_const/out" % name, out); store(d, "simd/%s_const/g1" % name, a.grad)
-    unary = {"square": so.simd_square, "sqrt": so.simd_sqrt, "exp": so.simd_exp, "log": so.simd_log}
-    for name, fn in unary.items():
-        a = (sa.abs() + 0.1).clone().requires_grad_(True)
-        out = fn(a, mx_specs=specs)
-        out.backward(sgo)
-        store(d, "simd/%s/out" % name, out); store(d, "simd/%s/g1" % name, a.grad)
-    a = sa.clone().requires_grad_(True)
-    out = so.simd_reduce_sum(a, [0, 2], mx_specs=specs)
-    out.backward(torch.ones_like(out) * 0.37)
-    store(d, "simd/reduce_sum/out", out); store(d, "simd/reduce_sum/g1", a.grad)
-    a = sa.clone().requires_grad_(True)
-    out = so.simd_reduce_mean(a, -1, keepdim=True, mx_specs=specs)
-    out.backward(torch.ones_like(out) * 0.37)
-    store(d, "simd/reduce_mean/out", out); store(d, "simd/reduce_mean/g1", a.grad)
-    a = sa.clone().requires_grad_(True)
-    out = so.simd_norm(a, mx_specs=specs)
-    out.backward()
-    store(d, "simd/norm/out", out); store(d, "simd/norm/g1", a.grad)
-
-    torch.manual_seed(12)
-    lstm = LSTM(32, 64, num_layers=2, bidirectional=True, mx_specs=cspecs)
-    lx = torch.randn(5, 3, 32, generator=g)
-    lgo = torch.randn(5, 3, 128, generator=g)
-    store(d, "in/lx", lx); store(d, "in/lgo", lgo)
-    xi = lx.clone().requires_grad_(True)
-    out, (hn, cn) = lstm(xi)
-    (out * lgo).sum().backward()
-    store(d, "lstm/out", out); store(d, "lstm/hn", hn); store(d, "lstm/cn", cn); store(d, "lstm/gx", xi.grad)
-    for n, p in lstm.named_parameters():
-        store(d, "lstm/p_" + n, p)
-        store(d, "lstm/g_" + n, p.grad)
-    packed = pack_padded_sequence(lx, [5, 3, 2])
-    outp, (hn, cn) = lstm(packed)
-    store(d, "lstm_packed/out", outp.data); store(d, "lstm_packed/hn", hn); store(d, "lstm_packed/cn", cn)
+    # linear layers whose blocks do not divide the example axis of a 3-D input (block sizes 64 and
+    # "whole axis"): the weight gradient shares exponents per batch entry (mx/linear.py:124-143)
+    x3 = torch.randn(3, 96, 64, generator=g)
+    go3 = torch.randn(3, 96, 48, generator=g)
+    store(d, "in/x3", x3)
+    store(d, "in/go3", go3)
+    for block in (64, 0):
+        bspecs = finalize_mx_specs(dict(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=block,
+                                        bfloat=16, quantize_backprop=True, custom_cuda=False))
+        xi, wi, bi = (t.clone().requires_grad_(True) for t in (x3, w, b))
+        out = linear(xi, wi, bi, mx_specs=bspecs)
+        out.backward(go3)
+        key = "linear_block%d/" % block
+        store(d, key + "out", out)
+        store(d, key + "gx", xi.grad)
+        store(d, key + "gw", wi.grad)
+        store(d, key + "gb", bi.grad)
 
     np.savez_compressed(os.path.join(HERE, "reference_layer_vectors.npz"), **d)
     print("wrote %d arrays, torch %s" % (len(d), torch.__version__))

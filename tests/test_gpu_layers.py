@@ -110,76 +110,12 @@ def _near_loose(got, want, what):
 
 def test_convolutions(dev):
     from microxcaling_amd.convolution import Conv2d
-    from microxcaling_amd.transpose_convolution import ConvTranspose2d
     s = _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32, bfloat=16,
                quantize_backprop=True)
     g = torch.Generator().manual_seed(8)
     x = torch.randn(4, 64, 12, 12, generator=g)
     _run_both(dev, lambda: Conv2d(64, 96, 3, stride=2, padding=1, mx_specs=s), x,
               torch.randn(4, 96, 6, 6, generator=g), loose=True)
-    _run_both(dev, lambda: ConvTranspose2d(64, 32, 3, stride=2, padding=1, output_padding=1, mx_specs=s), x,
-              torch.randn(4, 32, 24, 24, generator=g), loose=True)
-
-
-def test_batch_group_norm_and_pooling(dev):
-    from microxcaling_amd.adaptive_avg_pooling import AdaptiveAvgPool2d
-    from microxcaling_amd.batchnorm import BatchNorm2d
-    from microxcaling_amd.groupnorm import GroupNorm
-    s = _specs(bfloat=16, quantize_backprop=True)
-    g = torch.Generator().manual_seed(9)
-    x = torch.randn(8, 32, 10, 10, generator=g) * 2 + 0.5
-    go = torch.randn(8, 32, 10, 10, generator=g)
-    _run_both(dev, lambda: BatchNorm2d(32, mx_specs=s), x, go)
-    _run_both(dev, lambda: GroupNorm(4, 32, mx_specs=s), x, go)
-    _run_both(dev, lambda: AdaptiveAvgPool2d((3, 2), mx_specs=s), x, torch.randn(8, 32, 3, 2, generator=g))
-
-
-def test_simd_ops(dev):
-    from microxcaling_amd import simd_ops as so
-    s = _specs(bfloat=16, quantize_backprop=True)
-    g = torch.Generator().manual_seed(10)
-    a = torch.randn(16, 8, 64, generator=g)
-    b = torch.randn(8, 1, generator=g) + 2.5
-    go = torch.randn(16, 8, 64, generator=g)
-    for fn in (so.simd_add, so.simd_sub, so.simd_mul, so.simd_div):
-        ac, bc = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
-        ag, bg = a.to(dev).requires_grad_(True), b.to(dev).requires_grad_(True)
-        oc, og = fn(ac, bc, mx_specs=s), fn(ag, bg, mx_specs=s)
-        oc.backward(go)
-        og.backward(go.to(dev))
-        _near(og, oc, fn.__name__)
-        _near(ag.grad, ac.grad, "g1")
-        _near(bg.grad, bc.grad, "g2")
-    for fn in (so.simd_exp, so.simd_log, so.simd_sqrt, so.simd_square):
-        ac = (a.abs() + 0.1).clone().requires_grad_(True)
-        ag = (a.abs() + 0.1).to(dev).requires_grad_(True)
-        oc, og = fn(ac, mx_specs=s), fn(ag, mx_specs=s)
-        oc.backward(go)
-        og.backward(go.to(dev))
-        _near(og, oc, "unary")
-        _near(ag.grad, ac.grad, "unary grad")
-    _near(so.simd_norm(a.to(dev), mx_specs=s), so.simd_norm(a, mx_specs=s), "norm")
-    _near(so.simd_reduce_mean(a.to(dev), [0, 2], mx_specs=s), so.simd_reduce_mean(a, [0, 2], mx_specs=s), "mean")
-
-
-def test_lstm(dev):
-    """Recurrent: every step feeds on the previous one's quantized state, so single-step
-    differences compound; compared loosely, and the final states as well."""
-    from microxcaling_amd.rnn import LSTM
-    s = _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32, bfloat=16,
-               quantize_backprop=True)
-    g = torch.Generator().manual_seed(11)
-    x = torch.randn(6, 4, 64, generator=g)
-    torch.manual_seed(1)
-    ref = LSTM(64, 128, num_layers=2, bidirectional=True, mx_specs=s)
-    gpu = LSTM(64, 128, num_layers=2, bidirectional=True, mx_specs=s)
-    gpu.load_state_dict(ref.state_dict())
-    gpu.to(dev)
-    oc, (hc, cc) = ref(x)
-    og, (hg, cg) = gpu(x.to(dev))
-    for got, want in ((og, oc), (hg, hc), (cg, cc)):
-        diff = (got.detach().cpu() - want.detach()).abs()
-        assert diff.max().item() <= 0.05 and diff.mean().item() <= 2e-3, (diff.max().item(), diff.mean().item())
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
