@@ -11,7 +11,9 @@
  *     default stream, mx/cpp/mx.cu:57);
  *   - failures return a non-zero status and leave a message for mxq_last_error(); the reference
  *     prints and calls exit() (mx/cpp/common.cuh:247-255).
- * Entry points never allocate, never synchronise and keep no state between calls.
+ * Entry points never allocate and never synchronise.  Results never depend on earlier calls; the only
+ * state the library keeps is set-up done once per device under a lock (the dynamic-LDS limit of the
+ * large-tile GEMM kernel with that device's CU count), so calls may come from several host threads.
  *
  * Numerics: results are bit-identical to the reference's pure-PyTorch CPU path
  * (custom_cuda=False) for fp32 and bf16 tensors, including its floor(log2(x)) rounding just
@@ -133,6 +135,7 @@ int mxq_reduce_sum_outer(const float* in, float* out, void* workspace, int64_t o
                          int64_t inner, void* hip_stream);
 int mxq_reduce_max_outer(const float* in, float* out, void* workspace, int64_t outer,
                          int64_t inner, void* hip_stream);
+
 
 /* SoftmaxFunction.forward (mx/softmax.py:20-54) over the last axis of a contiguous (rows, n) fp32
  * or bf16 tensor, as one kernel: quantize, row maximum, subtract, exponential, row sum, divide, with
@@ -272,12 +275,15 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const 
                    void* workspace, int64_t workspace_bytes, void* hip_stream);
 /* 0 when the product would not be split. */
 int64_t mxq_gemm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int a_kind);
-
-/* Measurement aid (no counterpart in the reference): launches `workgroups` x 256 lanes, each wave
- * issuing iters x 16 scaled 16x16x128 MFMAs on register-resident operands of kind MXQ_CODES_E4M3 or
- * MXQ_CODES_E2M1 (workgroups * 4 * iters * 16 * 65536 flop in total).  `sink` is any 4 writable
- * device bytes. */
-int mxq_probe_mfma_rate(int64_t workgroups, int iters, int code_kind, void* sink, void* hip_stream);
+/* Which kernel mxq_gemm_mx_nt launches for a shape (no counterpart in the reference; for tests and
+ * benchmarks that must know what they measured), or -1 for a shape it refuses:
+ * persistent workgroups on 256 x 256 tiles; 128 x 128 tiles; the same with K split over several
+ * workgroups per tile (needs the workspace, else unsplit); 128 x 128 tiles whose K is a single step. */
+#define MXQ_GEMM_PLAN_SMALL_TILES 0
+#define MXQ_GEMM_PLAN_SPLIT_K 1
+#define MXQ_GEMM_PLAN_LARGE_TILES 2
+#define MXQ_GEMM_PLAN_ONE_STEP 3
+int mxq_gemm_plan(int64_t batch, int64_t M, int64_t N, int64_t K, int a_kind);
 
 /* ---- libmxq_host.so: the same arithmetic compiled for the host ----------------------------------
  * quantize_mx_func_cpp (mx/cpp/funcs.cpp:23-98) and quantize_elemwise_func_cpp

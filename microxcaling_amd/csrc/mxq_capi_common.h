@@ -19,6 +19,7 @@ int check_launch(const char* what) {
 
 constexpr int kThreads = 256;
 constexpr int64_t kMaxBlocks = 256 * 8;      // 256 CUs x 8 resident blocks of 256 lanes
+constexpr int kMaxDevices = 64;               // per-device state is kept in tables of this size
 
 int grid_for(int64_t work_items_per_block_iter_total) {
     int64_t g = work_items_per_block_iter_total;

@@ -1,4 +1,6 @@
 // C ABI of libmxq_gfx950.so, continued: packed MX tensors and the scaled-MFMA GEMM.
+#include <mutex>
+
 #include "mxq_capi_common.h"
 #include "mxq_gemm.h"
 
@@ -107,21 +109,29 @@ int launch_gemm_dt(int64_t batch, const GemmArgs& g, void* workspace, int64_t wo
     const int64_t tiles_m = ceil_div(g.M, G2_BM), tiles_n = ceil_div(g.N, G2_BN);
     const int64_t total = tiles_m * tiles_n * batch;
     if (large_tiles(batch, g.M, g.N, g.K) && (int64_t)256 * g.kbytes < ((int64_t)1 << 31)) {
-        static bool configured = false;               // raising the dynamic-LDS limit is per kernel
-        static int cus = 0;
-        if (!configured) {
-            hipError_t e = hipFuncSetAttribute(
-                reinterpret_cast<const void*>(&mx_gemm_nt_kernel_256p<CB, BL, ODT>),
-                hipFuncAttributeMaxDynamicSharedMemorySize, G3_LDS_BYTES);
-            int dev = 0;
-            if (e == hipSuccess) e = hipGetDevice(&dev);
-            if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-            if (e != hipSuccess || cus <= 0)
-                return fail(MXQ_ERR_LAUNCH, "mxq_gemm_mx_nt: cannot configure the tile kernel (%d bytes of LDS): %s",
-                            G3_LDS_BYTES, hipGetErrorString(e));
-            cus -= cus % 8;                           // a workgroup must stay on its XCD from tile to tile
-            if (cus < 8) cus = 8;
-            configured = true;
+        // raising the dynamic-LDS limit is per kernel and per device: done once for each (this template
+        // instance, device), under a lock, and remembered with that device's CU count
+        static std::mutex config_mutex;
+        static int cus_of_device[kMaxDevices] = {};
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+            return fail(MXQ_ERR_LAUNCH, "mxq_gemm_mx_nt: no usable current device (%s)", hipGetErrorString(e));
+        int cus;
+        {
+            std::lock_guard<std::mutex> lock(config_mutex);
+            if (cus_of_device[dev] == 0) {
+                int n = 0;
+                e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mx_gemm_nt_kernel_256p<CB, BL, ODT>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, G3_LDS_BYTES);
+                if (e == hipSuccess) e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+                if (e != hipSuccess || n <= 0)
+                    return fail(MXQ_ERR_LAUNCH, "mxq_gemm_mx_nt: cannot configure the tile kernel (%d bytes of LDS): %s",
+                                G3_LDS_BYTES, hipGetErrorString(e));
+                n -= n % 8;                           // a workgroup must stay on its XCD from tile to tile
+                cus_of_device[dev] = n < 8 ? 8 : n;
+            }
+            cus = cus_of_device[dev];
         }
         const unsigned grid = (unsigned)(total < cus ? total : cus);
         mx_gemm_nt_kernel_256p<CB, BL, ODT><<<grid, 512, G3_LDS_BYTES, s>>>(g, (int)tiles_m, (int)tiles_n, (int)total);
@@ -341,18 +351,14 @@ int64_t mxq_gemm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K,
     return splits == 1 ? 0 : (int64_t)splits * batch * M * N * (int64_t)sizeof(float);
 }
 
-int mxq_probe_mfma_rate(int64_t workgroups, int iters, int code_kind, void* sink, void* hip_stream) {
-    const char* who = "mxq_probe_mfma_rate";
-    if (workgroups <= 0 || workgroups > 0x7FFFFFFF || iters <= 0 || !sink ||
-        (code_kind != MXQ_CODES_E4M3 && code_kind != MXQ_CODES_E2M1))
-        return fail(MXQ_ERR_ARGUMENT, "%s: bad argument", who);
-    if (code_kind == MXQ_CODES_E2M1)
-        mfma_rate_probe_kernel<4><<<(unsigned)workgroups, kThreads, 0, (hipStream_t)hip_stream>>>(
-            iters, reinterpret_cast<float*>(sink));
-    else
-        mfma_rate_probe_kernel<0><<<(unsigned)workgroups, kThreads, 0, (hipStream_t)hip_stream>>>(
-            iters, reinterpret_cast<float*>(sink));
-    return check_launch(who);
+int mxq_gemm_plan(int64_t batch, int64_t M, int64_t N, int64_t K, int a_kind) {
+    if (batch <= 0 || M <= 0 || N <= 0 || K <= 0) return -1;
+    const bool nib = a_kind == MXQ_CODES_E2M1;
+    if (K % (nib ? 2 * GEMM_BK : GEMM_BK) != 0) return -1;
+    const int64_t kbytes = nib ? K / 2 : K;
+    if (large_tiles(batch, M, N, K) && (int64_t)256 * kbytes < ((int64_t)1 << 31)) return MXQ_GEMM_PLAN_LARGE_TILES;
+    if (gemm_k_splits(batch, M, N, K, nib) > 1) return MXQ_GEMM_PLAN_SPLIT_K;
+    return kbytes == GEMM_BK ? MXQ_GEMM_PLAN_ONE_STEP : MXQ_GEMM_PLAN_SMALL_TILES;
 }
 
 }  // extern "C"

@@ -1051,25 +1051,4 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     }
 }
 
-// Register-resident MFMA loop: every wave issues `iters` x 16 independent scaled MFMAs on operands
-// it never reloads.  Its rate is the practical ceiling of the matrix pipes under this instruction
-// (datasheet: 5 PFLOP/s dense fp8, 10.1 PFLOP/s fp4).  FMT: 0 e4m3 bytes, 4 e2m1 nibbles.
-// `sink` only keeps the compiler from deleting the loop.
-template <int FMT>
-__global__ __launch_bounds__(TPB) void mfma_rate_probe_kernel(int iters, float* sink) {
-    v8i a = {(int)threadIdx.x, 1, 2, 3, 4, 5, 6, 7}, b = {7, 6, 5, 4, 3, 2, 1, (int)blockIdx.x};
-    v4f acc[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = v4f{0.f, 0.f, 0.f, 0.f};
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-            acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[i], FMT, FMT, 0, 127, 0, 127);
-    }
-    float t = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) t += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
-    if (t == 12345.678f) sink[0] = t;
-}
-
 }  // namespace

@@ -134,8 +134,9 @@ def _reduce_inner(A, sym, who):
     if A.dim() < 1:
         raise RuntimeError("%s: needs at least one dimension" % who)
     inner = A.shape[-1]
-    out = torch.zeros(A.shape[:-1], dtype=A.dtype, device=A.device,
-                      requires_grad=A.requires_grad)          # mx/cpp/reduce.cu:24-28
+    # the reference returns zeros(sizes[:-1]) carrying the input's requires_grad (mx/cpp/reduce.cu:24-28);
+    # the kernel writes every element, so the fill launch is left out
+    out = torch.empty(A.shape[:-1], dtype=A.dtype, device=A.device, requires_grad=A.requires_grad)
     rows = out.numel()
     lib = _lib.gpu()
     with torch.cuda.device(A.device):

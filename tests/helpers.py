@@ -96,3 +96,32 @@ def dither_cases():
             yield "mx", name, dtype, n, 1000 + n, case, x, from_bits(z["mx_%s_%d" % (name, n)], dtype)
         for n, case in enumerate(mod.ELEM_CASES):
             yield "elem", name, dtype, n, 2000 + n, case, x, from_bits(z["elem_%s_%d" % (name, n)], dtype)
+
+
+class PackageImpl:
+    """This package's own entry points behind the call signature of the oracles, so that one test
+    body can run against an oracle, against the host library (CPU tensors -> libmxq_host.so) and
+    against the HIP kernels (tensors moved to the GPU and back)."""
+
+    def __init__(self, device):
+        self.device = device
+
+    def _to(self, A):
+        if self.device == "cuda":
+            assert torch.cuda.is_available(), "this case needs a GPU"
+        return A.to(self.device)
+
+    def quantize_mx(self, A, scale_bits, elem_format, axes, block_size=0, round="nearest",
+                    flush_fp32_subnorms=False):
+        from microxcaling_amd.mx_ops import _quantize_mx
+        y = _quantize_mx(self._to(A), scale_bits, elem_format, axes=axes, block_size=block_size, round=round,
+                         flush_fp32_subnorms=flush_fp32_subnorms, custom_cuda=self.device == "cuda")
+        return y.cpu()
+
+    def quantize_elemwise_core(self, A, bits, exp_bits, max_norm, round="nearest", saturate_normals=False,
+                               allow_denorm=True):
+        from microxcaling_amd.elemwise_ops import _quantize_elemwise_core
+        y = _quantize_elemwise_core(self._to(A), bits, exp_bits, max_norm, round=round,
+                                    saturate_normals=saturate_normals, allow_denorm=allow_denorm,
+                                    custom_cuda=self.device == "cuda")
+        return y.cpu()

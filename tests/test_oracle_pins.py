@@ -1,7 +1,8 @@
 """Pins the CPU oracle (oracle/mx_oracle.py and the C restatement) to facts it did not produce
 itself: the literal known-answer vectors of the reference's own tests, library special cases
 (torch's bf16 / fp16 / fp8 casts), closed-form format constants, an exact-rational brute force,
-and the golden vectors written from the reference's pure path (tests/golden/)."""
+and the golden vectors written from the reference's pure path (tests/golden/).  The same bodies run
+against the product: the host library on CPU tensors, and (marked gpu) the HIP kernels."""
 import hashlib
 import math
 from fractions import Fraction
@@ -10,14 +11,19 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import assert_bits_equal, canon_bits, dither_cases, from_bits, golden, golden_inputs_module
+from helpers import (PackageImpl, assert_bits_equal, canon_bits, dither_cases, from_bits, golden,
+                     golden_inputs_module)
 from oracle import c_oracle as C
 from oracle import mx_oracle as O
 
 inf, nan = float("inf"), float("nan")
 ROUNDS = ["nearest", "floor", "even"]
 MX_FORMATS = ["fp8_e4m3", "fp8_e5m2", "fp6_e3m2", "fp6_e2m3", "fp4_e2m1", "int8", "int4"]
-ORACLES = [pytest.param(O, id="torch"), pytest.param(C, id="c")]
+# the two oracles, and -- same test bodies, same literal vectors -- the product itself: the host
+# library on CPU tensors and the HIP kernels on the GPU (through the C ABI)
+ORACLES = [pytest.param(O, id="torch"), pytest.param(C, id="c"),
+           pytest.param(PackageImpl("cpu"), id="host_library"),
+           pytest.param(PackageImpl("cuda"), id="hip", marks=pytest.mark.gpu)]
 
 
 def same_values(got, want):
