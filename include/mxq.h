@@ -13,7 +13,8 @@
  *     prints and calls exit() (mx/cpp/common.cuh:247-255).
  * Entry points never allocate and never synchronise.  Results never depend on earlier calls; the only
  * state the library keeps is set-up done once per device under a lock (the dynamic-LDS limit of the
- * large-tile GEMM kernel with that device's CU count), so calls may come from several host threads.
+ * large-tile GEMM kernel with that device's CU count, and the address of the scratch array of
+ * mxq_reduce_outer_static), so calls may come from several host threads.
  *
  * Numerics: results are bit-identical to the reference's pure-PyTorch CPU path
  * (custom_cuda=False) for fp32 and bf16 tensors, including its floor(log2(x)) rounding just
@@ -136,6 +137,19 @@ int mxq_reduce_sum_outer(const float* in, float* out, void* workspace, int64_t o
 int mxq_reduce_max_outer(const float* in, float* out, void* workspace, int64_t outer,
                          int64_t inner, void* hip_stream);
 
+/* The outer-axis reduction for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same kernels, same launch geometry and therefore the same bits as mxq_reduce_sum_outer (op 0) /
+ * mxq_reduce_max_outer (op 1), but the partial results live in a 16 MiB device array that is part of
+ * the library (every GPU the library runs on holds it until the process ends) instead of a
+ * caller-provided workspace.  Shapes for which mxq_reduce_outer_workspace_bytes(outer, inner) exceeds
+ * MXQ_REDUCE_OUTER_STATIC_BYTES are refused with MXQ_ERR_ARGUMENT ([16384, 8192] needs exactly that
+ * much).  Calls on one GPU share the array: two that overlap in time (different streams or host
+ * threads) race; calls on one stream are ordered and safe.  Nothing needs clearing between calls
+ * (every partial that is read has been written by the same call). */
+#define MXQ_REDUCE_OUTER_STATIC_BYTES (16 << 20)
+int mxq_reduce_outer_static(const float* in, float* out, int op, int64_t outer, int64_t inner,
+                            void* hip_stream);
 
 /* SoftmaxFunction.forward (mx/softmax.py:20-54) over the last axis of a contiguous (rows, n) fp32
  * or bf16 tensor, as one kernel: quantize, row maximum, subtract, exponential, row sum, divide, with

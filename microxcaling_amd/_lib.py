@@ -64,6 +64,7 @@ GPU_SYMBOLS = {
     "mxq_reduce_outer_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),
     "mxq_reduce_sum_outer": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),
     "mxq_reduce_max_outer": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),
+    "mxq_reduce_outer_static": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_ptr]),
 }
 HOST_SYMBOLS = {
     "mxq_host_last_error": (ctypes.c_char_p, []),

@@ -2,6 +2,8 @@
 // Declarations and the reference functions each entry point replaces are in include/mxq.h.
 // This file: MX and elementwise quantization, reductions.  mxq_capi_gemm.hip: packed MX tensors and
 // the GEMM.  mxq_capi_chain.hip: softmax, normalization and activation kernels.
+#include <mutex>
+
 #include "mxq_capi_common.h"
 
 namespace {
@@ -151,7 +153,31 @@ int reduce_outer(const float* in, float* out, void* workspace, int64_t outer, in
     return check_launch(who);
 }
 
-// shared by the chain kernels: format parameters, and which kernel instance serves them
+// Partial results of mxq_reduce_outer_static.  In host code the array's name is only a handle: the
+// address kernels can use comes from hipGetSymbolAddress, differs from GPU to GPU, and is looked up
+// once per device (with that device current) on the entry point's first call there.
+__attribute__((used)) static __device__ __align__(256) unsigned char scratch[MXQ_REDUCE_OUTER_STATIC_BYTES];
+std::mutex scratch_mutex;
+void* scratch_of_device[kMaxDevices] = {};
+
+int scratch_on_current_device(void** ptr, const char* who) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return fail(MXQ_ERR_LAUNCH, "%s: no usable current device (%s)", who, hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_of_device[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr)
+            return fail(MXQ_ERR_LAUNCH, "%s: cannot locate the scratch array on device %d (%s)", who, dev,
+                        hipGetErrorString(e));
+        scratch_of_device[dev] = p;
+    }
+    *ptr = scratch_of_device[dev];
+    return MXQ_OK;
+}
+
 }  // namespace
 
 #pragma GCC visibility push(default)
@@ -324,6 +350,25 @@ int mxq_reduce_sum_outer(const float* in, float* out, void* workspace, int64_t o
 int mxq_reduce_max_outer(const float* in, float* out, void* workspace, int64_t outer, int64_t inner,
                          void* hip_stream) {
     return reduce_outer<MaxOp>(in, out, workspace, outer, inner, hip_stream, "mxq_reduce_max_outer");
+}
+
+int mxq_reduce_outer_static(const float* in, float* out, int op, int64_t outer, int64_t inner,
+                            void* hip_stream) {
+    const char* who = "mxq_reduce_outer_static";
+    if (op != 0 && op != 1) return fail(MXQ_ERR_ARGUMENT, "%s: op must be 0 (sum) or 1 (max)", who);
+    if (outer < 0 || inner < 0) return fail(MXQ_ERR_ARGUMENT, "%s: negative size", who);
+    const int64_t need = mxq_reduce_outer_workspace_bytes(outer, inner);
+    if (need > (int64_t)MXQ_REDUCE_OUTER_STATIC_BYTES)
+        return fail(MXQ_ERR_ARGUMENT, "%s: (%lld, %lld) needs %lld bytes of partial results, the built-in "
+                    "scratch array holds %d; use mxq_reduce_%s_outer with a workspace", who, (long long)outer,
+                    (long long)inner, (long long)need, (int)MXQ_REDUCE_OUTER_STATIC_BYTES, op ? "max" : "sum");
+    void* ws = nullptr;
+    if (need > 0) {
+        const int rc = scratch_on_current_device(&ws, who);
+        if (rc) return rc;
+    }
+    return op ? reduce_outer<MaxOp>(in, out, ws, outer, inner, hip_stream, who)
+              : reduce_outer<SumOp>(in, out, ws, outer, inner, hip_stream, who);
 }
 
 }  // extern "C"
