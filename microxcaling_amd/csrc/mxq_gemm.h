@@ -22,6 +22,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "mxq_gemm_addr.h"
 #include "mxq_kernels.h"
 
 namespace {
@@ -308,6 +309,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int GEMM_BM = 128, GEMM_BN = 128, GEMM_BK = 128, GEMM_PITCH = GEMM_BK + 16;
+static_assert(GEMM_BK == mxq_addr::BK, "the address helpers assume 128-byte K steps");
 
 struct GemmArgs {
     const unsigned char* a;
@@ -326,24 +328,8 @@ struct GemmArgs {
     int64_t batch_a, batch_sa, batch_b, batch_sb, batch_c;   // strides between batches (bytes / elements of C)
 };
 
-// Which output tile a workgroup computes.  Workgroups are dealt round-robin to the 8 XCDs, each
-// with its own L2, so workgroup w runs on XCD w % 8.  Give every XCD a contiguous range of
-// "logical" tile numbers, and walk the tile grid in bands of 8 tile-rows: the ~32 tiles an XCD
-// works on at any time then form an 8 x 4 patch that shares 8 A tiles and 4 B tiles per K step
-// through that XCD's L2 instead of streaming 64 tiles from the fabric.
-__device__ __forceinline__ void tile_of_workgroup(int wg, int total, int tiles_m, int tiles_n,
-                                                  int* tm, int* tn) {
-    constexpr int XCDS = 8, BAND = 8;
-    const int q = total / XCDS, r = total % XCDS;
-    const int xcd = wg % XCDS, local = wg / XCDS;
-    const int logical = xcd * q + min(xcd, r) + local;
-    const int per_band = BAND * tiles_n;
-    const int band = logical / per_band, in_band = logical % per_band;
-    const int first_m = band * BAND;
-    const int rows = min(tiles_m - first_m, BAND);
-    *tm = first_m + in_band % rows;
-    *tn = in_band / rows;
-}
+// which output tile a workgroup computes (XCD-aware order), and the address arithmetic of the tile copies
+using mxq_addr::tile_of_workgroup;
 
 // a lane's MFMA operand: 16 codes at p (K = 16g ..) and 16 codes at p + 64 (K = 64 + 16g ..)
 __device__ __forceinline__ v8i load_frag(const unsigned char* p) {
@@ -575,18 +561,15 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     int64_t ga[4], gb[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int c = tid + j * TPB;
-        ld_row[j] = c >> 3;
-        ld_col[j] = (c & 7) * 16;
-        const int gm = min(m0 + ld_row[j], g.M - 1);         // rows past the edge are never stored
-        const int gn = min(n0 + ld_row[j], g.N - 1);
-        ga[j] = (int64_t)gm * g.kbytes + ld_col[j];
-        gb[j] = (int64_t)gn * g.kbytes + ld_col[j];
+        ld_row[j] = mxq_addr::small_piece_row(tid, j);
+        ld_col[j] = mxq_addr::small_piece_col(tid, j);
+        ga[j] = mxq_addr::small_code_offset(m0, g.M, g.kbytes, tid, j);   // rows past the edge are clamped:
+        gb[j] = mxq_addr::small_code_offset(n0, g.N, g.kbytes, tid, j);   // their outputs are never stored
     }
     const int srow = tid & 127;
     const bool s_is_a = tid < 128;
-    const int64_t gs = s_is_a ? (int64_t)min(m0 + srow, g.M - 1) * KB
-                              : (int64_t)min(n0 + srow, g.N - 1) * KB;
+    const int64_t gs = s_is_a ? mxq_addr::small_scale_offset(m0, g.M, KB, tid)
+                              : mxq_addr::small_scale_offset(n0, g.N, KB, tid);
 
     const int frow = lane & 15, fg = lane >> 4;
     u32x4 va[4], vb[4];
@@ -599,7 +582,7 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
         }
 #pragma unroll
         for (int e = 0; e < EPB; ++e)
-            sv[e] = *reinterpret_cast<const uint32_t*>((s_is_a ? SA : SB) + gs + ((k0 * EPB) >> 5) + 4 * e);
+            sv[e] = *reinterpret_cast<const uint32_t*>((s_is_a ? SA : SB) + gs + mxq_addr::scale_byte_of(k0, EPB) + 4 * e);
     };
     auto stash = [&]() {
 #pragma unroll
@@ -618,7 +601,7 @@ __global__ __launch_bounds__(TPB) void mx_gemm_nt_kernel(GemmArgs g) {
     const int kbeg = (int)blockIdx.z * per_split;
     const int nk = min(per_split, nk_all - kbeg);
     const int kstart = (int)((blockIdx.x * 5u + blockIdx.y) % (unsigned)nk);
-    auto kof = [&](int step) { return (kbeg + (kstart + step) % nk) * GEMM_BK; };
+    auto kof = [&](int step) { return mxq_addr::small_k_byte(kbeg, kstart, step, nk); };
     fetch(kof(0));
     stash();
     __syncthreads();
@@ -817,7 +800,7 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     // position of 16-byte column c of row r inside its LDS row: c ^ key(r); the key takes 8
     // different values over the even rows of any 16 consecutive rows (and again over the odd ones),
     // which is what a 16-byte read by 16 lanes needs to touch every bank once
-    auto key_a = [](int r) { return (r >> 1) & 7; };
+    auto key_a = [](int r) { return mxq_addr::large_key(r); };
     auto key_b = key_a;
 
     // ---- fetch side: which tile the tile copy is working on --------------------------------------
@@ -828,7 +811,6 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     uint32_t offa[4], offb[4], offs;
     int f_kstart;
     const bool s_is_b = wave >= 4;
-    const int s_row = (wave & 3) * 64 + lane;
     auto fetch_tile = [&](int logical) {
         const int bz = logical / per_batch;
         int tm, tn;
@@ -839,25 +821,17 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
         fS = s_is_b ? g.sb + bz * g.batch_sb + (int64_t)n0 * KB : g.sa + bz * g.batch_sa + (int64_t)m0 * KB;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int r = wave * 32 + i * 8 + (lane >> 3);
-            offa[i] = (uint32_t)min(r, g.M - 1 - m0) * (uint32_t)g.kbytes + ((lane & 7) ^ key_a(r)) * 16;
-            offb[i] = (uint32_t)min(r, g.N - 1 - n0) * (uint32_t)g.kbytes + ((lane & 7) ^ key_b(r)) * 16;
+            offa[i] = mxq_addr::large_code_offset(wave, lane, i, g.M - 1 - m0, g.kbytes);
+            offb[i] = mxq_addr::large_code_offset(wave, lane, i, g.N - 1 - n0, g.kbytes);
         }
-        offs = (uint32_t)min(s_row, (s_is_b ? g.N - n0 : g.M - m0) - 1) * (uint32_t)KB;
-        // The tiles of an XCD walk K in step, so that the A and B panels they share are fetched
-        // into that XCD's L2 once (a start staggered per tile cost up to 30 % on long-K shapes, whose
-        // panels do not stay in L2 that long).  The eight XCDs start at eight different places of a
-        // cyclic walk, which spreads the slices in flight over the memory channels -- unless the
-        // last scale group of a row is a partial one: then everybody starts at K = 0.
-        f_kstart = nfull != nk ? 0 : (int)(((unsigned)(logical % 8) * (unsigned)(nk / GS)) / 8u) * GS;
+        offs = mxq_addr::large_scale_offset(wave, lane, s_is_b ? g.N - n0 : g.M - m0, KB);
+        f_kstart = mxq_addr::large_kstart(logical, nk, nfull, GS);   // the XCD's place in the cyclic K walk
     };
     int f_groups = 0;                                        // scale groups fetched so far
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;     // LDS byte address of the array (normally 0)
     // load i (0..7 codes, 8 scales) of flat step t, which is K step fs of the fetch-side tile
     auto fetch_part = [&](int t, int fs, int i) {
-        int kidx = f_kstart + fs;
-        kidx = kidx >= nk ? kidx - nk : kidx;
-        const int k0 = kidx * GEMM_BK;
+        const int k0 = mxq_addr::large_kidx(f_kstart, fs, nk) * GEMM_BK;
         const uint32_t st = lds0 + (t & 1) * G3_STAGE_BYTES;
         if (i < 4) {
             dma16(st + (wave * 32 + i * 8) * 128, offa[i], fA + k0);
@@ -866,14 +840,14 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
         } else if (fs < nfull) {
             if (fs % GS == 0) {                              // a new group of GS K steps
                 dma16(lds0 + G3_SCALE_OFF + (f_groups & 1) * G3_SCALE_GROUP + wave * 1024, offs,
-                      fS + ((k0 * EPB) >> 5));
+                      fS + mxq_addr::scale_byte_of(k0, EPB));
                 ++f_groups;
             }
         } else {                                             // past the last whole group: this step only
 #pragma unroll
             for (int e = 0; e < EPB; ++e)
                 dma4(lds0 + G3_TAIL_OFF + (fs & 1) * G3_TAIL_SLOT + e * G3_TAIL_PLANE + wave * 256, offs,
-                     fS + ((k0 * EPB) >> 5) + 4 * e);
+                     fS + mxq_addr::scale_byte_of(k0, EPB) + 4 * e);
         }
     };
 

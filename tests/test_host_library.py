@@ -382,6 +382,27 @@ def test_direct_pack_codes_equal_the_encoded_rounded_values(tmp_path):
     assert out.count("zone variant") == 10
 
 
+def test_gemm_tile_copies_stay_inside_their_operands(tmp_path):
+    """tests/cpp/gemm_addr_check.cpp walks every (workgroup, tile, K step, load, wave, lane) of both
+    GEMM kernels through the address functions the kernels are compiled from
+    (microxcaling_amd/csrc/mxq_gemm_addr.h) and checks every 16- and 4-byte range against the size of
+    the operand it reads: the benchmark shapes, ragged M / N, K % 512 != 0, nibbles, batches, K
+    splits.  Exits non-zero at the first range outside."""
+    import shutil
+    import subprocess
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        pytest.skip("no host C++ compiler")
+    exe = str(tmp_path / "gemm_addr_check")
+    subprocess.run([cxx, "-O2", "-std=c++17", "-I", os.path.join(ROOT_DIR, "include"),
+                    "-I", os.path.join(ROOT_DIR, "microxcaling_amd", "csrc"), "-o", exe,
+                    os.path.join(ROOT_DIR, "tests", "cpp", "gemm_addr_check.cpp")], check=True)
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0 and "OUT OF BOUNDS" not in res.stdout, res.stdout[-2000:]
+    assert "byte ranges inside their operands" in res.stdout
+    assert res.stdout.count("256 x 256 tiles") == 11 and res.stdout.count("128 x 128 tiles") == 20
+
+
 def test_dither_reproduces_the_reference_under_the_same_seed():
     """round='dither' on CPU tensors: the package draws its noise like the reference
     (torch.rand_like under torch's generator) and the host library rounds floor(s + noise): the
