@@ -4,8 +4,11 @@
 One "step" = one `_quantize_mx` pass (MXFP8 e4m3, block 32 along the last axis, scale_bits 8,
 round 'nearest') over a seeded fp32 [8192, 8192] tensor that is already resident in HBM.
 Prints ONE JSON line: whole-job throughput in GB/s of algorithmic bytes (8 B per element: fp32 in,
-fp32 out), the roofline position of the kernel from HIP events around every launch, and the CPU
-baseline (the torch op-sequence oracle timed on this box's host cores on a bounded row sample).
+fp32 out), the roofline position of the kernel from HIP events around the timed launches, and the CPU
+baseline (the torch op-sequence oracle timed on this box's host cores).  The metric has a second half,
+the fused MX linear layer in TFLOP/s: without --workload the same line carries it as "secondary"
+(workload mx_linear timed for the same steps: whole-step TFLOP/s, the GEMM kernel's own launch time
+against the dense fp8 MFMA peak, its CPU baseline).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
 
@@ -18,6 +21,7 @@ Workloads (config N = the N-th benchmark configuration of this build's baseline 
     reduce_sum_m1 / reduce_max_m1 / reduce_sum_0 / reduce_max_0  config 3, reductions
     mx_linear / mx_linear_fp4 / mx_linear_fp6 / mx_linear_bfloat16  config 4: mx.Linear forward (TFLOP/s)
     mx_linear_train                                              ... forward + backward
+    mx_linear_prequantized                                       ... as an inference layer that keeps its weight's MX codes
     mx_bmm_softmax                                               config 5: mx.bmm + bfloat16 softmax
     softmax_bf16 / layernorm_bf16 / gelu_bf16 / silu_bf16 (+ _train), norm_param_grads_bf16, pack_t_bf16,
     mxfp8_fp32_8192_tiles                                        single kernels of the layers around the path
@@ -128,13 +132,58 @@ def make_workload(name):
             gemm.set_fused(fused)
             return linear(xd, dev_extra["w"], dev_extra["b"], mx_specs=specs)
         bf = 16 if "bfloat16" in name else 0
-        return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, ef, ef, bfloat=bf),
+
+        def gemm_only(xd):
+            # the GEMM kernel on its own: both operands packed once, as the layer packs them
+            from microxcaling_amd import fused
+            nib = ef == "fp4_e2m1"
+            pre = bool(bf)
+            pa = fused.pack_mx(xd, ef, 8, "nearest", False, nib, pre)
+            pb = fused.pack_mx(w.to(xd.device), ef, 8, "nearest", False, nib, pre)
+            bd = b.to(xd.device)
+            return lambda: fused.gemm_nt(pa, pb, out_dtype=torch.bfloat16, bias=bd, epilogue_quant=bool(bf))
+        extra = dict(gemm_only=gemm_only, gemm_flops=2.0 * M * N * K,
+                     gemm_kernel="mx_gemm_nt_kernel_256p") if fused else {}
+        return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, ef, ef, bfloat=bf), **extra,
+                    tolerance="vs the oracle's quantize-then-fp32-matmul on sampled rows (tests/test_gpu_baseline_shapes.py): "
+                              "fp32 tensors max|diff| / RMS < 1e-3; bf16 tensors (this run) |diff| <= 2^-6 (|out| + |bias|) "
+                              "+ 2e-3 RMS, i.e. one bf16 rounding step of the product and of the bias sum on top",
                     flops=2.0 * M * N * K, bytes=0, dtype="%s x %s -> f32 acc" % (ef, ef), sample_axis=0,
                     cpu_rows=1024, launches=5, peak="fp4" if ef == "fp4_e2m1" else "fp8",   # fp6 runs on byte codes: fp8 rate
                     desc="mx.Linear forward: x bf16 [16384,4096], W bf16 [14336,4096] ~N(0,0.02), bias; %s "
                          "block 32 along K, %s" % ({"fp4_e2m1": "MXFP4 e2m1", "fp6_e2m3": "MXFP6 e2m3"}.get(ef, "MXFP8 e4m3"),
                                                    ("packed codes + scaled-MFMA GEMM" if fused else
                                                     "fake-quantize kernels + torch (hipBLASLt) bf16 GEMM")))
+    if name == "mx_linear_prequantized":
+        # config 4 as an inference layer: mx.Linear.prequantize_weights() keeps the weight's MX codes, a
+        # forward pass packs the activations only
+        from microxcaling_amd.linear import Linear
+        from microxcaling_amd.specs import finalize_mx_specs
+        g = torch.Generator().manual_seed(4)
+        M, N, K = 16384, 14336, 4096
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+        b = torch.randn(N, generator=g).to(torch.bfloat16)
+        specs = finalize_mx_specs({"w_elem_format": "fp8_e4m3", "a_elem_format": "fp8_e4m3", "block_size": 32,
+                                   "bfloat": 16, "round": "even"})
+        st = {}
+
+        def run(xd):
+            if "m" not in st:
+                m = Linear(K, N, mx_specs=specs)
+                with torch.no_grad():
+                    m.weight.copy_(w)
+                    m.bias.copy_(b)
+                m.to(xd.device).eval()
+                m.prequantize_weights(keep_dense=False)
+                st["m"] = m
+            with torch.no_grad():
+                return st["m"](xd)
+        return dict(x=x, gpu=run, cpu=lambda t: O.mx_linear_forward(t, w, b, "fp8_e4m3", "fp8_e4m3", bfloat=16, round="even"),
+                    flops=2.0 * M * N * K, bytes=0, dtype="fp8_e4m3 x fp8_e4m3 -> f32 acc", sample_axis=0,
+                    cpu_rows=1024, launches=2,
+                    desc="mx.Linear forward with prequantized weights (MX codes + scales kept, 1 + 1/32 B per weight): "
+                         "x bf16 [16384,4096] packed per step, W [14336,4096] packed once; MXFP8 e4m3, bias")
     if name in ("mx_linear_train", "mx_linear_train_unfused"):
         # forward + backward of the same layer (three GEMMs: output, grad_input, grad_weight), every
         # operand MX-quantized along its contraction axis (mx/linear.py:20-198)
@@ -403,24 +452,68 @@ def measured_traffic(workload):
         return json.load(f).get(workload)
 
 
-def report_flops(args, wl, ms_per_step, step_gpu_ms):
-    """GEMM-shaped workloads: whole-step TFLOP/s (quantize + GEMM + epilogue ops all inside the
-    step) against the dense fp8 MFMA peak."""
-    value = wl["flops"] / (ms_per_step * 1e-3) / 1e12
-    achieved = wl["flops"] / (step_gpu_ms * 1e-3) / 1e12
+METRIC = "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s"
+
+
+def time_steps(fn, xd, steps, warmup):
+    """W untimed steps, then exactly K steps bracketed by a synchronize on both sides (wall clock) and
+    by one pair of HIP events recorded on the stream the kernels are launched on, torch's current
+    stream (GPU time of the K back-to-back steps).  Events between the launches would each cost a
+    ~10 us bubble on the queue, so there are none.  -> (wall ms per step, GPU ms per step)"""
+    for _ in range(warmup):
+        fn(xd)
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        y = fn(xd)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    del y
+    return wall * 1e3 / steps, ev0.elapsed_time(ev1) / steps
+
+
+def gemm_kernel_ms(wl, xd, steps, warmup):
+    """Average duration of the GEMM kernel alone at the workload's shape: the operands are packed once,
+    then K back-to-back launches of mxq_gemm_mx_nt are timed with one pair of HIP events."""
+    g = wl["gemm_only"](xd)
+    return time_steps(lambda _: g(), xd, steps, warmup)[1]
+
+
+def flops_report(name, wl, steps, warmup, ms_per_step, step_gpu_ms, kernel_ms, cpu):
+    """GEMM-shaped workloads.  value: whole-step TFLOP/s (quantize + pack of both operands, GEMM, bias
+    and epilogue all inside the step).  roofline: the dominant kernel, the scaled-MFMA GEMM --
+    2 M N K flop per launch over its average launch duration -- against the dense MFMA peak of its
+    operand format."""
     peak = MFMA_PEAK_TFLOPS[wl.get("peak", "fp8")]
-    out = {
-        "metric": "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s",
-        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"], "data": "synthetic",
-        "config": {"workload": args.workload, "detail": wl["desc"], "flop_per_step": wl["flops"]},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak,
-                     "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
-                     "traffic": measured_traffic(args.workload), "step_gpu_ms_avg": round(step_gpu_ms, 5),
-                     "note": "whole forward step (all launches) over the dense %s MFMA peak" % wl.get("peak", "fp8")},
-    }
-    if not args.no_cpu_baseline:
+    value = wl["flops"] / (ms_per_step * 1e-3) / 1e12
+    if kernel_ms is not None:
+        achieved = wl["gemm_flops"] / (kernel_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4), "traffic": measured_traffic(name),
+                "kernel": wl["gemm_kernel"], "launch_ms_avg": round(kernel_ms, 5),
+                "step_gpu_ms_avg": round(step_gpu_ms, 5),
+                "note": "GEMM kernel alone (operands packed beforehand) over the dense %s MFMA peak; the whole "
+                        "step runs at %.1f TFLOP/s = %.4f of it" % (wl.get("peak", "fp8"),
+                                                                    wl["flops"] / (step_gpu_ms * 1e-3) / 1e12,
+                                                                    wl["flops"] / (step_gpu_ms * 1e-3) / 1e12 / peak)}
+    else:
+        achieved = wl["flops"] / (step_gpu_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(achieved / peak, 4), "traffic": measured_traffic(name),
+                "step_gpu_ms_avg": round(step_gpu_ms, 5),
+                "note": "whole step (all launches) over the dense %s MFMA peak" % wl.get("peak", "fp8")}
+    out = {"metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps,
+           "warmup": warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"], "data": "synthetic",
+           "config": {"workload": name, "detail": wl["desc"], "flop_per_step": wl["flops"],
+                      "tolerance": wl.get("tolerance")},
+           "roofline": roof}
+    if cpu:
         x = wl["x"]
         cores = min(os.cpu_count() or 1, 16)
         torch.set_num_threads(cores)
@@ -433,7 +526,44 @@ def report_flops(args, wl, ms_per_step, step_gpu_ms):
                                "cores": cores, "kind": "port",
                                "sample": "first %d of %d rows/batches of the first operand, one pass, %.1f s; "
                                          "torch op-by-op oracle" % (rows, x.shape[0], t)}
-    print(json.dumps(out, ensure_ascii=False), flush=True)
+    return out
+
+
+def bytes_report(name, wl, steps, warmup, ms_per_step, kern_avg_ms, cpu):
+    value = wl["bytes"] / (ms_per_step * 1e-3) / 1e9
+    achieved = wl["bytes"] / (kern_avg_ms * 1e-3) / 1e9
+    out = {
+        "metric": METRIC,
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"], "data": "synthetic",
+        "config": {"workload": name, "detail": wl["desc"],
+                   "algorithmic_bytes_per_step": wl["bytes"],
+                   "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(name),
+                     "launch_ms_avg": round(kern_avg_ms, 5),
+                     "launches_per_step": wl.get("launches", 1)},
+    }
+    if cpu:
+        out["cpu_baseline"] = cpu_baseline(wl)
+    return out
+
+
+def run_workload(name, steps, warmup, cpu):
+    """One workload, inputs resident in HBM before the timed region -> its report (a dict)."""
+    wl = make_workload(name)
+    dev = torch.device("cuda:0")
+    xd = wl["x"].to(dev)
+    torch.cuda.synchronize()
+    ms_per_step, gpu_ms = time_steps(wl["gpu"], xd, steps, warmup)
+    if "flops" in wl:
+        kernel_ms = gemm_kernel_ms(wl, xd, steps, warmup) if "gemm_only" in wl else None
+        return flops_report(name, wl, steps, warmup, ms_per_step, gpu_ms, kernel_ms, cpu)
+    return bytes_report(name, wl, steps, warmup, ms_per_step, gpu_ms, cpu)
+
+
+HEADLINE, SECONDARY = "mxfp8_fp32_8192", "mx_linear"
 
 
 def main():
@@ -441,7 +571,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)     # the clocks need a few ms to ramp up
-    ap.add_argument("--workload", default="mxfp8_fp32_8192")
+    ap.add_argument("--workload", default=None,
+                    help="one workload only; default: the headline quantization, then the fused MX linear "
+                         "layer of the same metric as \"secondary\" in the same JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -450,55 +582,17 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU (torch.cuda.is_available() is False)")
 
-    wl = make_workload(args.workload)
-    dev = torch.device("cuda:0")
-    xd = wl["x"].to(dev)
-    torch.cuda.synchronize()
-
-    for _ in range(args.warmup):
-        wl["gpu"](xd)
-    torch.cuda.synchronize()
-
-    # Timed region: exactly K steps, bracketed by a synchronize on both sides (wall clock -> value)
-    # and by one pair of HIP events recorded on the stream the kernels are launched on (GPU time of
-    # the K back-to-back launches -> average launch duration).  Events between the launches would
-    # each cost a ~10 us bubble on the queue, so there are none.
-    ev0 = torch.cuda.Event(enable_timing=True)
-    ev1 = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ev0.record()
-    for i in range(args.steps):
-        y = wl["gpu"](xd)
-    ev1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    del y
-
-    ms_per_step = wall * 1e3 / args.steps
-    kern_avg_ms = ev0.elapsed_time(ev1) / args.steps
-    if "flops" in wl:
-        return report_flops(args, wl, ms_per_step, kern_avg_ms)
-    value = wl["bytes"] / (ms_per_step * 1e-3) / 1e9
-    achieved = wl["bytes"] / (kern_avg_ms * 1e-3) / 1e9
-
-    traffic = measured_traffic(args.workload)
-
-    out = {
-        "metric": "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"], "data": "synthetic",
-        "config": {"workload": args.workload, "detail": wl["desc"],
-                   "algorithmic_bytes_per_step": wl["bytes"],
-                   "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2)},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "launch_ms_avg": round(kern_avg_ms, 5),
-                     "launches_per_step": wl.get("launches", 1)},
-    }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(wl)
+    cpu = not args.no_cpu_baseline
+    if args.workload is not None:
+        out = run_workload(args.workload, args.steps, args.warmup, cpu)
+    else:
+        # both halves of the metric: the headline fields are the quantization throughput; the fused MX
+        # linear layer (config 4), timed for the same number of steps, rides along as "secondary"
+        out = run_workload(HEADLINE, args.steps, args.warmup, cpu)
+        sec = run_workload(SECONDARY, args.steps, args.warmup, cpu)
+        out["secondary"] = {k: sec[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "dtype",
+                                                "config", "roofline", "cpu_baseline") if k in sec}
+        out["secondary"]["metric"] = "fused MX-linear TFLOP/s"
     print(json.dumps(out, ensure_ascii=False), flush=True)
 
 

@@ -183,13 +183,34 @@ def _use_nibbles(fa, fb, K):
     return fa == ElemFormat.fp4 and fb == ElemFormat.fp4 and K % (2 * GEMM_K_MULTIPLE) == 0
 
 
+def pack_weight(w, a_fmt, w_fmt, mx_specs, round):
+    """The packed form mx_gemm_nt would build for a (N, K) weight on every call, built once: (codes,
+    scales, code kind) -- 1 byte per element (1/2 when both operand formats are fp4) plus 1/32 for
+    the scales, against 2 for a bf16 weight -- or None when the fused GEMM would not take it."""
+    fa, fb = _as_format(a_fmt), _as_format(w_fmt)
+    if fa not in _PACKABLE or fb not in _PACKABLE:
+        return None
+    if mx_specs["block_size"] != 32 or mx_specs["shared_exp_method"] != "max":
+        return None
+    if round not in RoundingMode.string_enums() or not w.is_cuda or w.dtype not in _DTYPE or w.dim() != 2:
+        return None
+    K = w.shape[-1]
+    if K == 0 or K % GEMM_K_MULTIPLE != 0 or w.numel() == 0:
+        return None
+    scale_bits = mx_specs["scale_bits"] if mx_specs["scale_bits"] != 0 else 8
+    return pack_mx(w.contiguous(), fb, scale_bits, round, mx_specs["mx_flush_fp32_subnorms"],
+                   _use_nibbles(fa, fb, K), False)
+
+
 def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_quant=False,
-               pre_bfloat16=False):
+               pre_bfloat16=False, packed_b=None):
     """a (..., M, K) x b_kmajor (N, K) or (..., N, K), both MX-quantized along K: the fused
     equivalent of quantize_mx_op(a, axes=[-1]) @ quantize_mx_op(b, axes=[-1]).T (+ bias, see
     gemm_nt).  pre_bfloat16 (a bool, or one per operand): the operand is a bf16 tensor that has not been
     through the layers' elementwise bfloat16 / round-half-away quantization yet; its pack kernel applies it.  Returns None
-    when the operands do not qualify (the caller then takes the unfused path)."""
+    when the operands do not qualify (the caller then takes the unfused path).  packed_b: what
+    pack_weight returned for b_kmajor (a 2-D weight) under the same formats, specs and rounding; the
+    pack of b is then skipped and b_kmajor is not looked at."""
     fa, fb = _as_format(a_fmt), _as_format(b_fmt)
     if fa not in _PACKABLE or fb not in _PACKABLE:
         return None
@@ -197,25 +218,36 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
         return None
     if round not in RoundingMode.string_enums():
         return None
-    if not (a.is_cuda and b_kmajor.is_cuda) or a.dtype not in _DTYPE or b_kmajor.dtype not in _DTYPE:
-        return None
-    if a.dim() < 2 or b_kmajor.dim() < 2 or a.shape[-1] != b_kmajor.shape[-1]:
+    if not a.is_cuda or a.dtype not in _DTYPE or a.dim() < 2:
         return None
     K = a.shape[-1]
-    if K == 0 or K % GEMM_K_MULTIPLE != 0 or a.numel() == 0 or b_kmajor.numel() == 0:
+    if K == 0 or K % GEMM_K_MULTIPLE != 0 or a.numel() == 0:
         return None
-    if b_kmajor.dim() == 2:
-        a2 = a.contiguous().reshape(-1, K)              # fold every leading axis into M
-        b2 = b_kmajor.contiguous()
-        out_shape = a.shape[:-1] + (b2.shape[0],)
-    elif b_kmajor.shape[:-2] == a.shape[:-2]:
-        a2 = a.contiguous().reshape(-1, a.shape[-2], K)
-        b2 = b_kmajor.contiguous().reshape(-1, b_kmajor.shape[-2], K)
-        out_shape = a.shape[:-1] + (b_kmajor.shape[-2],)
-        if a2.shape[0] > 65535:
-            return None
+    nibbles = _use_nibbles(fa, fb, K)
+    if packed_b is not None:
+        # a weight packed ahead of time: its codes and scales say what it is, b_kmajor is not read
+        if packed_b[1].dim() != 2 or packed_b[1].shape[1] * 32 != K or \
+                int(packed_b[2]) != _code_kind(fb, nibbles, "mx_gemm_nt"):
+            raise RuntimeError("mx_gemm_nt: packed_b does not belong to these formats or this K")
+        _packed_k(packed_b[0], packed_b[1], packed_b[2], "mx_gemm_nt")
+        a2, b2 = a.contiguous().reshape(-1, K), None
+        out_shape = a.shape[:-1] + (packed_b[1].shape[0],)
     else:
-        return None                                      # broadcast batch axes
+        if not b_kmajor.is_cuda or b_kmajor.dtype not in _DTYPE or b_kmajor.dim() < 2 or \
+                b_kmajor.shape[-1] != K or b_kmajor.numel() == 0:
+            return None
+        if b_kmajor.dim() == 2:
+            a2 = a.contiguous().reshape(-1, K)              # fold every leading axis into M
+            b2 = b_kmajor.contiguous()
+            out_shape = a.shape[:-1] + (b2.shape[0],)
+        elif b_kmajor.shape[:-2] == a.shape[:-2]:
+            a2 = a.contiguous().reshape(-1, a.shape[-2], K)
+            b2 = b_kmajor.contiguous().reshape(-1, b_kmajor.shape[-2], K)
+            out_shape = a.shape[:-1] + (b_kmajor.shape[-2],)
+            if a2.shape[0] > 65535:
+                return None
+        else:
+            return None                                      # broadcast batch axes
     scale_bits = mx_specs["scale_bits"] if mx_specs["scale_bits"] != 0 else 8
     flush = mx_specs["mx_flush_fp32_subnorms"]
     if bias is not None and (bias.dtype != a.dtype or bias.dim() != 1):
@@ -223,11 +255,10 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
     if epilogue_quant and a.dtype != torch.bfloat16:
         return None
     pre_a, pre_b = pre_bfloat16 if isinstance(pre_bfloat16, tuple) else (pre_bfloat16, pre_bfloat16)
-    if (pre_a and a.dtype != torch.bfloat16) or (pre_b and b_kmajor.dtype != torch.bfloat16):
+    if (pre_a and a.dtype != torch.bfloat16) or (pre_b and b2 is not None and b2.dtype != torch.bfloat16):
         return None
-    nibbles = _use_nibbles(fa, fb, K)
     pa = pack_mx(a2, fa, scale_bits, round, flush, nibbles, pre_a)
-    pb = pack_mx(b2, fb, scale_bits, round, flush, nibbles, pre_b)
+    pb = packed_b if packed_b is not None else pack_mx(b2, fb, scale_bits, round, flush, nibbles, pre_b)
     return gemm_nt(pa, pb, out_dtype=a.dtype, bias=bias, epilogue_quant=epilogue_quant).reshape(out_shape)
 
 

@@ -39,15 +39,16 @@ def _epilogue_mode(mx_specs, round, dtype):
     from .elemwise_ops import elemwise_plan
     from .formats import _get_max_norm
     plan = elemwise_plan(mx_specs, round)
-    if plan[0] == "identity":
-        return 0
+    if plan[0] == "identity" or (plan[0] == "to_bf16" and dtype == torch.bfloat16):
+        return 0                 # (a cast to bf16 of a bf16 tensor: the case of prequantized weights)
     if plan == ("quantize", 9, 8, _get_max_norm(8, 9), True) and round == "nearest" \
             and dtype == torch.bfloat16:
         return 1
     return None
 
 
-def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, out_round=None, bias=None, pre_bfloat16=False):
+def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, out_round=None, bias=None, pre_bfloat16=False,
+               packed_b=None):
     """a: (..., M, K); b_kmajor: (..., N, K) -- both contiguous along K.  Returns (out, finished):
     out is None when the fused path does not apply; finished says whether the output quantization
     with rounding `out_round` and the bias add have been done in the epilogue."""
@@ -57,21 +58,27 @@ def _try_fused(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, out_round=None, bias=
     mode = _epilogue_mode(mx_specs, out_round, a.dtype) if out_round is not None else None
     if mode is not None and (bias is None or bias.dtype == a.dtype):
         out = fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=bias,
-                               epilogue_quant=mode == 1, pre_bfloat16=pre_bfloat16)
+                               epilogue_quant=mode == 1, pre_bfloat16=pre_bfloat16, packed_b=packed_b)
         if out is not None:
             return out, True
-    return fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, pre_bfloat16=pre_bfloat16), False
+    return fused.mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, pre_bfloat16=pre_bfloat16,
+                            packed_b=packed_b), False
 
 
-def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, out_round=None, bias=None, pre_bfloat16=False):
+def mx_linear_contract(x, w, a_fmt, w_fmt, mx_specs, round, out_round=None, bias=None, pre_bfloat16=False,
+                       packed_w=None):
     """x (..., K) times w (N, K) transposed: both operands share exponents along their last axis.
     out_round / bias: what the caller does next -- elementwise-quantize the product with that
     rounding, add the (already quantized) bias, quantize again.  Returns (out, finished); when
     finished, those steps have been done in the GEMM's epilogue.  pre_bfloat16 (one flag per operand):
-    as for mx_matmul_contract."""
-    out, finished = _try_fused(x, w, a_fmt, w_fmt, mx_specs, round, out_round, bias, pre_bfloat16)
+    as for mx_matmul_contract.  packed_w: the weight's packed form kept by a layer with prequantized
+    weights (fused.pack_weight); w itself may then be an empty placeholder of the right dtype."""
+    out, finished = _try_fused(x, w, a_fmt, w_fmt, mx_specs, round, out_round, bias, pre_bfloat16, packed_w)
     if out is not None:
         return out, finished
+    if packed_w is not None and w.numel() == 0:
+        raise RuntimeError("this layer keeps its weight as packed MX codes only, which only the fused GEMM "
+                           "reads: the input must be a GPU tensor of the weight's dtype with the fused path on")
     if pre_bfloat16:
         return None, False
     qx = quantize_mx_op(x, mx_specs, elem_format=a_fmt, axes=[-1], round=round)

@@ -20,7 +20,7 @@ class LinearFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, input, weight, bias=None, mx_specs=None, prequantized_weights=False,
-                name=None):
+                name=None, packed_weight=None):
         # inference (no gradient wanted for input, weight or bias, so backward never runs and nothing
         # keeps the quantized operands): their bfloat16 quantization is left to the
         # pack kernels of the fused GEMM (prequantized weights imply round-half-even, where that
@@ -68,7 +68,8 @@ class LinearFunction(torch.autograd.Function):
         output, finished = mx_linear_contract(bf_in, bf_weight, mx_specs["a_elem_format"],
                                               mx_specs["w_elem_format"], mx_specs,
                                               mx_specs["round_mx_output"],
-                                              out_round=mx_specs["round_output"], bias=bf_bias)
+                                              out_round=mx_specs["round_output"], bias=bf_bias,
+                                              packed_w=packed_weight)
         if not finished:
             output = quantize_elemwise_op(output, mx_specs=mx_specs, round=mx_specs["round_output"])
             if bias is not None:
@@ -119,15 +120,18 @@ class LinearFunction(torch.autograd.Function):
         if ctx.has_bias:
             grad_bias = quantize_elemwise_op(grad_output.reshape(-1, out_dim).sum(0),
                                              mx_specs=specs, round=specs["round_grad_weight"])
-        return (grad_input, grad_weight, grad_bias, None, None, None)
+        return (grad_input, grad_weight, grad_bias, None, None, None, None)
 
 
-def linear(input, weight, bias=None, mx_specs=None, prequantized_weights=False, name=None):
+def linear(input, weight, bias=None, mx_specs=None, prequantized_weights=False, name=None,
+           packed_weight=None):
+    """mx/linear.py:203-213.  packed_weight (not in the reference): the weight's MX codes and scales as
+    Linear.prequantize_weights keeps them; the forward pass then skips the weight's quantization."""
     mx_assert_test(mx_specs)
     if mx_specs is None:
         return f_linear(input, weight, bias=bias)
     mx_specs = apply_mx_specs(mx_specs)
-    return LinearFunction.apply(input, weight, bias, mx_specs, prequantized_weights, name)
+    return LinearFunction.apply(input, weight, bias, mx_specs, prequantized_weights, name, packed_weight)
 
 
 class Linear(torch.nn.Linear):
@@ -136,6 +140,8 @@ class Linear(torch.nn.Linear):
         self.mx_none = mx_specs is None
         self.name = name
         self.prequantized_weights = False
+        self._packed_weight = None
+        self._keep_dense = True
         self.mx_specs = apply_mx_specs(mx_specs)
         super().__init__(in_features, out_features, bias)
 
@@ -147,8 +153,17 @@ class Linear(torch.nn.Linear):
     def append_name(self, postfix):
         self.name += postfix
 
-    def prequantize_weights(self):
-        """Store weight and bias as bfloat16 once, for inference (mx/linear.py:246-274)."""
+    def prequantize_weights(self, keep_dense=True):
+        """Store weight and bias as bfloat16 once, for inference (mx/linear.py:246-274).  On a GPU the
+        weight's MX form -- element codes + one E8M0 scale byte per block of 32, what the forward
+        pass would otherwise rebuild from the bf16 weight on every call -- is built once as well, at
+        the first forward pass (the layer may still move between devices until then), and the fused
+        GEMM reads it directly: 1 + 1/32 bytes per weight (1/2 + 1/32 when both formats are fp4)
+        against 2.  keep_dense=False also drops the bf16 weight once its codes exist (weight.data
+        becomes an empty tensor): the layer then holds a half to a quarter of the bytes and serves
+        GPU inputs through the fused GEMM only."""
+        self._keep_dense = keep_dense
+        self._packed_weight = None
         if self.mx_none:
             return
         assert self.mx_specs["round"] == 'even', \
@@ -167,10 +182,42 @@ class Linear(torch.nn.Linear):
                     round=self.mx_specs["round_weight"]).to(torch.bfloat16)
         self.prequantized_weights = True
 
+    def _packed(self, inputs):
+        """The cached MX form of the prequantized weight for this input, or None."""
+        from . import fused
+        from .gemm import fused_enabled
+        if not (self.prequantized_weights and fused_enabled() and inputs.is_cuda
+                and inputs.dtype == torch.bfloat16):
+            return None
+        w = self.weight
+        key = (w.data_ptr(), w._version, w.device, tuple(w.shape))
+        if self._packed_weight is None or (w.numel() and self._packed_weight[0] != key):
+            if not w.is_cuda or w.numel() == 0:
+                return None
+            packed = fused.pack_weight(w.data, self.mx_specs["a_elem_format"], self.mx_specs["w_elem_format"],
+                                       self.mx_specs, self.mx_specs["round_mx_output"])
+            if packed is None:
+                return None
+            if not self._keep_dense:
+                with torch.no_grad():
+                    self.weight.data = torch.empty(0, dtype=w.dtype, device=w.device)
+                key = None
+            self._packed_weight = (key, packed)
+        return self._packed_weight[1]
+
+    def packed_weight_bytes(self):
+        """Bytes of the cached MX form (codes + scales), 0 before the first GPU forward pass."""
+        if getattr(self, "_packed_weight", None) is None:
+            return 0
+        codes, scales, _ = self._packed_weight[1]
+        return codes.numel() + scales.numel()
+
     def forward(self, inputs):
         if self.mx_none:
             return super().forward(inputs)
+        packed = None
         if self.prequantized_weights:
             assert self.training == False, "Cannot use prequantized weights when training!"
+            packed = self._packed(inputs)
         return linear(input=inputs, weight=self.weight, bias=self.bias, mx_specs=self.mx_specs,
-                      prequantized_weights=self.prequantized_weights, name=self.name)
+                      prequantized_weights=self.prequantized_weights, name=self.name, packed_weight=packed)

@@ -342,6 +342,45 @@ def test_linear_inference_skips_the_operand_quantization_passes(dev, with_bias, 
         assert torch.equal(mod(x).view(torch.int16), plain.view(torch.int16))
 
 
+@pytest.mark.parametrize("fmt", ["fp8_e4m3", "fp6_e2m3", "fp4_e2m1"])
+@pytest.mark.parametrize("keep_dense", [True, False])
+def test_prequantized_linear_keeps_the_packed_weight(dev, fmt, keep_dense):
+    """Linear.prequantize_weights (mx/linear.py:246-274) on the fused path: the weight's MX codes and
+    scales are built at the first forward pass and reused; outputs are bit for bit those of the same
+    layer packing its bf16 weight on every call; keep_dense=False leaves only codes + scales."""
+    from microxcaling_amd.linear import Linear, linear
+    M, N, K = 640, 768, 512
+    specs = _specs(w_elem_format=fmt, a_elem_format=fmt, block_size=32, bfloat=16, round="even")
+    torch.manual_seed(11)
+    lin = Linear(K, N, mx_specs=specs).to(dev).eval()
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(3, M, K, generator=g).to(torch.bfloat16).to(dev)
+    lin.prequantize_weights(keep_dense=keep_dense)
+    assert lin.weight.dtype == torch.bfloat16 and lin.packed_weight_bytes() == 0
+    w, b = lin.weight.data.clone(), lin.bias.data.clone()
+    with torch.no_grad():
+        want = linear(x, w, b, mx_specs=specs, prequantized_weights=True)     # packs w on every call
+        got1 = lin(x)
+        got2 = lin(x[:, :100])                                                # reuses the codes
+    assert torch.equal(got1.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(got2.view(torch.int16), want[:, :100].contiguous().view(torch.int16))
+    per_weight = 0.5 if fmt == "fp4_e2m1" else 1.0
+    assert lin.packed_weight_bytes() == int(N * K * per_weight) + N * K // 32
+    assert lin.weight.numel() == (N * K if keep_dense else 0)
+    # against the oracle (round-half-even everywhere), the tolerance of bf16 tensors
+    ref = O.mx_linear_forward(x.cpu(), w.cpu(), b.cpu(), fmt, fmt, bfloat=16, round="even").float()
+    diff = (got1.float().cpu() - ref).abs()
+    assert bool((diff <= 2 ** -6 * (ref.abs() + b.float().cpu().abs()) + 2e-3 * ref.pow(2).mean().sqrt()).all())
+    if keep_dense:
+        # a changed weight is packed again
+        with torch.no_grad():
+            lin.weight.mul_(2.0)
+            again = lin(x)
+            assert torch.equal(again.view(torch.int16),
+                               linear(x, lin.weight.data, b, mx_specs=specs, prequantized_weights=True).view(torch.int16))
+        assert not torch.equal(again, got1)
+
+
 def test_gemm_propagates_nan_blocks(dev):
     from microxcaling_amd.fused import pack_mx, gemm_nt
     a = torch.randn(128, 128)
