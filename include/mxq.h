@@ -19,9 +19,10 @@
  * Numerics: results are bit-identical to the reference's pure-PyTorch CPU path
  * (custom_cuda=False) for fp32 and bf16 tensors, including its floor(log2(x)) rounding just
  * below powers of two; MXQ_FLAG_EXACT_EXPONENT switches to bit-field exponents, which is what the
- * reference's own CUDA kernels compute (mx/cpp/common.cuh:146-154).  fp16 tensors are widened to
- * fp32, quantized, and rounded back to fp16 like the reference's CUDA kernels do
- * (mx/cpp/mx.cuh:72,88).
+ * reference's own CUDA kernels compute (mx/cpp/common.cuh:146-154).  fp16 tensors are accepted
+ * under that flag only: they are widened to fp32, quantized and rounded back to fp16 like the
+ * reference's CUDA kernels do (mx/cpp/mx.cuh:72,88), which is not what its pure-PyTorch path gives
+ * (every op evaluated in fp16); without the flag MXQ_DTYPE_F16 is refused with MXQ_ERR_ARGUMENT.
  */
 #ifndef MXQ_H
 #define MXQ_H

@@ -141,13 +141,29 @@ inline bool elem_zone_matters(int dtype, int flags, const MxqFmt& f, int rmode) 
     return !(f.ebits <= 5 && f.t <= 3);
 }
 
+// fp16 tensors: the reference's pure-PyTorch path evaluates every op in fp16 (2**exponent overflows
+// from 2^16, log2 rounds to 11 bits, ...: mx/mx_ops.py:265-292, mx/elemwise_ops.py:127-163), which
+// these kernels do not reproduce.  What they compute for fp16 -- widen to fp32, bit-field exponents,
+// round back -- is what the reference's CUDA kernels compute (mx/cpp/mx.cuh:72,88), so it is only
+// offered under the flag that asks for those semantics; without it the call is refused rather than
+// answered with values that differ from the pure path in places.
+inline int fp16_only_with_exact_exponents(int dtype, int flags, const char* who) {
+    if (dtype == MXQ_DTYPE_F16 && !(flags & MXQ_FLAG_EXACT_EXPONENT))
+        return fail(MXQ_ERR_ARGUMENT, "%s: fp16 tensors are served with MXQ_FLAG_EXACT_EXPONENT only (fp32 arithmetic "
+                    "and bit-field exponents, the reference's CUDA semantics); the reference's pure-PyTorch path on "
+                    "fp16 tensors is not reproduced -- cast to float32 or bfloat16, or switch to exact exponents", who);
+    return MXQ_OK;
+}
+
 inline int make_mx_params(int dtype, int scale_bits, int ebits, int mbits, float max_norm, int flush,
                           int rmode, int flags, MxParams* p, bool* zone_elem, const char* who) {
     if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
     if (rmode < 0 || rmode > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown rounding mode %d", who, rmode);
     if (scale_bits < 1 || scale_bits > 8)
         return fail(MXQ_ERR_ARGUMENT, "%s: scale_bits %d outside [1, 8]", who, scale_bits);
-    int rc = make_fmt(dtype, ebits, mbits, max_norm, &p->fmt, who);
+    int rc = fp16_only_with_exact_exponents(dtype, flags, who);
+    if (rc) return rc;
+    rc = make_fmt(dtype, ebits, mbits, max_norm, &p->fmt, who);
     if (rc) return rc;
     // exponent of max_norm, the way the reference's kernels derive it (mx/cpp/shared_exp.cuh:33)
     int be = (int)((mxq_bits(max_norm) >> 23) & 0xFF);
@@ -164,7 +180,9 @@ inline int make_elem_params(int dtype, int bits, int exp_bits, float max_norm, i
                             int saturate, int allow_denorm, int flags, ElemParams* p, const char* who) {
     if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
     if (rmode < 0 || rmode > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown rounding mode %d", who, rmode);
-    int rc = make_fmt(dtype, exp_bits, bits, max_norm, &p->fmt, who);
+    int rc = fp16_only_with_exact_exponents(dtype, flags, who);
+    if (rc) return rc;
+    rc = make_fmt(dtype, exp_bits, bits, max_norm, &p->fmt, who);
     if (rc) return rc;
     p->saturate = saturate ? 1 : 0;
     p->allow_denorm = allow_denorm ? 1 : 0;

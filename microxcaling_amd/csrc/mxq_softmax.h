@@ -155,6 +155,7 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
         };
         auto low_of = [](uint32_t w) { return mxq_float(w << 16); };
         auto high_of = [](uint32_t w) { return mxq_float(w & 0xFFFF0000u); };
+        auto fast_exp2 = [](float v) { return __builtin_amdgcn_exp2f(v); };
         bool close = false;
         if constexpr (QMODE == SMQ_BF16 && DT == MXQ_BF16) close = __all(plain && lowest - m >= -85.0f);
         if (close) {
@@ -163,8 +164,11 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
                 for (int e = 0; e < EPL; e += 2) {
                     uint32_t dw = packed(x[e] - m, x[e + 1] - m);
                     if (p.exp_mode == 2) dw = packed(1.4453125f * low_of(dw), 1.4453125f * high_of(dw));
-                    const uint32_t ew = p.exp_mode == 0 ? packed(expf(low_of(dw)), expf(high_of(dw)))
-                                                        : packed(exp2f(low_of(dw)), exp2f(high_of(dw)));
+                    // arguments in [-85, 0] (2^x: [-123, 0]): the results are normal numbers, which the
+                    // hardware exponential (v_exp_f32, 1 ulp, flushes subnormal results only) returns
+                    // without the range handling of expf / exp2f
+                    const uint32_t ew = p.exp_mode == 0 ? packed(fast_exp2(1.44269504f * low_of(dw)), fast_exp2(1.44269504f * high_of(dw)))
+                                                        : packed(fast_exp2(low_of(dw)), fast_exp2(high_of(dw)));
                     x[e] = low_of(ew);
                     x[e + 1] = high_of(ew);
                     sum += x[e];

@@ -21,13 +21,16 @@ _flags = 0
 
 def set_exponent_mode(mode):
     """'torch' (default): exponents follow floor(log2(x)) as torch's CPU kernels evaluate it, so
-    results are bit-identical to the reference's pure-PyTorch path.  'exact': bit-field exponents,
-    which is what the reference's CUDA kernels compute."""
+    results are bit-identical to the reference's pure-PyTorch path (float32 and bfloat16 tensors;
+    float16 tensors are refused in this mode: that path evaluates every op in fp16, which the
+    kernels do not reproduce).  'exact': bit-field exponents, which is what the reference's CUDA
+    kernels compute; float16 tensors are widened to fp32 and rounded back, as those kernels do
+    (mx/cpp/mx.cuh:72,88)."""
     global _flags
     if mode == "torch":
-        _flags = 0
+        _flags = _flags & ~_lib.FLAG_EXACT_EXPONENT
     elif mode == "exact":
-        _flags = _lib.FLAG_EXACT_EXPONENT
+        _flags = _flags | _lib.FLAG_EXACT_EXPONENT
     else:
         raise ValueError("exponent mode must be 'torch' or 'exact'")
 

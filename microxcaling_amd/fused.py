@@ -9,6 +9,10 @@ import torch
 
 from . import _lib
 from .custom_extensions import _DTYPE, _check_gpu_input, _flags_value, _stream
+
+# tensor dtypes whose layers take the fused path (fp16 tensors are quantized in exact-exponent mode only
+# and stay on the separate steps)
+_FUSED_DTYPES = (torch.float32, torch.bfloat16)
 from .formats import ElemFormat, RoundingMode, _get_format_params
 
 _PACKABLE = (ElemFormat.fp8_e4m3, ElemFormat.fp8_e5m2, ElemFormat.fp6_e3m2, ElemFormat.fp6_e2m3,
@@ -192,7 +196,7 @@ def pack_weight(w, a_fmt, w_fmt, mx_specs, round):
         return None
     if mx_specs["block_size"] != 32 or mx_specs["shared_exp_method"] != "max":
         return None
-    if round not in RoundingMode.string_enums() or not w.is_cuda or w.dtype not in _DTYPE or w.dim() != 2:
+    if round not in RoundingMode.string_enums() or not w.is_cuda or w.dtype not in _FUSED_DTYPES or w.dim() != 2:
         return None
     K = w.shape[-1]
     if K == 0 or K % GEMM_K_MULTIPLE != 0 or w.numel() == 0:
@@ -218,7 +222,7 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
         return None
     if round not in RoundingMode.string_enums():
         return None
-    if not a.is_cuda or a.dtype not in _DTYPE or a.dim() < 2:
+    if not a.is_cuda or a.dtype not in _FUSED_DTYPES or a.dim() < 2:
         return None
     K = a.shape[-1]
     if K == 0 or K % GEMM_K_MULTIPLE != 0 or a.numel() == 0:
@@ -233,7 +237,7 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
         a2, b2 = a.contiguous().reshape(-1, K), None
         out_shape = a.shape[:-1] + (packed_b[1].shape[0],)
     else:
-        if not b_kmajor.is_cuda or b_kmajor.dtype not in _DTYPE or b_kmajor.dim() < 2 or \
+        if not b_kmajor.is_cuda or b_kmajor.dtype not in _FUSED_DTYPES or b_kmajor.dim() < 2 or \
                 b_kmajor.shape[-1] != K or b_kmajor.numel() == 0:
             return None
         if b_kmajor.dim() == 2:
@@ -275,7 +279,7 @@ def mx_gemm_operands(operands, mx_specs, out_dtype):
         f = _as_format(fmt)
         if f not in _PACKABLE or rnd not in RoundingMode.string_enums():
             return None
-        if not t.is_cuda or t.dtype not in _DTYPE or t.dim() < 2 or t.numel() == 0:
+        if not t.is_cuda or t.dtype not in _FUSED_DTYPES or t.dim() < 2 or t.numel() == 0:
             return None
         K = t.shape[-2] if transposed else t.shape[-1]
         if K % GEMM_K_MULTIPLE != 0 or (transposed and t.shape[-1] % (8 // t.element_size()) != 0):

@@ -85,3 +85,31 @@ def test_sparse_coo_values_are_quantized():
     y = _quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128, round="even")
     assert y.is_sparse
     assert_bits_equal(y.to_dense(), x.to_dense().to(torch.bfloat16).float())
+
+
+def test_fp16_tensors_are_refused_unless_exact_exponents_are_asked_for():
+    """The reference's pure path runs every op in fp16 on fp16 tensors (mx/mx_ops.py:265-292), which
+    the kernels do not reproduce: by default such tensors raise instead of coming back with values
+    that differ in places.  In 'exact' mode they get the semantics of the reference's CUDA kernels
+    (mx/cpp/mx.cuh:72,88): widen to fp32, quantize, round back."""
+    from microxcaling_amd import custom_extensions as ce
+    from microxcaling_amd.elemwise_ops import _quantize_elemwise_core
+    from microxcaling_amd.mx_ops import _quantize_mx
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(8, 64, generator=g) * 3).half()
+    with pytest.raises(RuntimeError, match="fp16 tensors"):
+        _quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=32)
+    with pytest.raises(RuntimeError, match="fp16 tensors"):
+        _quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128)
+    ce.set_exponent_mode("exact")
+    try:
+        for rnd in ("nearest", "floor", "even"):
+            y = _quantize_mx(x, 8, "fp6_e2m3", axes=[-1], block_size=32, round=rnd)
+            wide = _quantize_mx(x.float(), 8, "fp6_e2m3", axes=[-1], block_size=32, round=rnd)
+            assert y.dtype == torch.float16
+            assert_bits_equal(y, wide.half(), "mx " + rnd)
+            y = _quantize_elemwise_core(x, 5, 4, 448.0, round=rnd, saturate_normals=True)
+            wide = _quantize_elemwise_core(x.float(), 5, 4, 448.0, round=rnd, saturate_normals=True)
+            assert_bits_equal(y, wide.half(), "elementwise " + rnd)
+    finally:
+        ce.set_exponent_mode("torch")
