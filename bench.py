@@ -22,7 +22,7 @@ Workloads (config N = the N-th benchmark configuration of this build's baseline 
     mx_linear / mx_linear_fp4 / mx_linear_fp6 / mx_linear_bfloat16  config 4: mx.Linear forward (TFLOP/s)
     mx_linear_train                                              ... forward + backward
     mx_linear_prequantized                                       ... as an inference layer that keeps its weight's MX codes
-    mx_bmm_softmax                                               config 5: mx.bmm + bfloat16 softmax
+    mx_bmm_softmax (_two_kernels: product and softmax separately) config 5: mx.bmm + bfloat16 softmax
     softmax_bf16 / layernorm_bf16 / gelu_bf16 / silu_bf16 (+ _train), norm_param_grads_bf16, pack_t_bf16,
     mxfp8_fp32_8192_tiles                                        single kernels of the layers around the path
     (suffix _unfused where it exists: the same step as separate tensor passes)
@@ -218,10 +218,10 @@ def make_workload(name):
                     desc="mx.Linear forward + backward: x bf16 [16384,4096], W bf16 [14336,4096], bias; MXFP8 "
                          "e4m3 block 32 along every contraction axis, %s" %
                          ("packed codes + scaled-MFMA GEMMs" if fused else "fake-quantize kernels + torch GEMMs"))
-    if name in ("mx_bmm_softmax", "mx_bmm_softmax_unfused"):
+    if name in ("mx_bmm_softmax", "mx_bmm_softmax_two_kernels", "mx_bmm_softmax_unfused"):
         # config 5: mx.bmm Q.K^T, MXFP6 e2m3 along head_dim, then the bfloat16 softmax chain
         from microxcaling_amd import gemm
-        from microxcaling_amd.bmm import bmm
+        from microxcaling_amd.bmm import bmm, bmm_softmax
         from microxcaling_amd.softmax import softmax
         from microxcaling_amd.specs import finalize_mx_specs
         g = torch.Generator().manual_seed(5)
@@ -230,12 +230,14 @@ def make_workload(name):
         k = torch.randn(B, S, D, generator=g).to(torch.bfloat16)
         specs = finalize_mx_specs({"a_elem_format": "fp6_e2m3", "block_size": 32, "bfloat": 16})
         dev_extra = {}
-        fused = name == "mx_bmm_softmax"
+        fused = name != "mx_bmm_softmax_unfused"
 
         def run(qd):
             if "k" not in dev_extra:
                 dev_extra["k"] = k.to(qd.device)
             gemm.set_fused(fused)
+            if name == "mx_bmm_softmax":         # one launch for the product and the softmax (+ two packs)
+                return bmm_softmax(qd, dev_extra["k"].transpose(-1, -2), mx_specs=specs)
             logits = bmm(qd, dev_extra["k"].transpose(-1, -2), mx_specs=specs)
             return softmax(logits, dim=-1, mx_specs=specs)
 
@@ -245,7 +247,8 @@ def make_workload(name):
         return dict(x=q, gpu=run, cpu=cpu, flops=2.0 * B * S * S * D, bytes=0,
                     dtype="fp6_e2m3 x fp6_e2m3 -> f32 acc", sample_axis=0, cpu_rows=8, launches=20,
                     desc="mx.bmm Q.K^T bf16 [128,2048,128] MXFP6 e2m3 along head_dim + bfloat16 softmax, %s"
-                         % ("packed codes + scaled-MFMA GEMM" if fused else "fake-quantize + torch.bmm"))
+                         % ("packed codes, product and softmax in one kernel (logits in registers)" if name == "mx_bmm_softmax"
+                            else "packed codes + scaled-MFMA GEMM, softmax kernel" if fused else "fake-quantize + torch.bmm"))
     if name in ("softmax_bf16", "softmax_bf16_unfused", "layernorm_bf16", "layernorm_bf16_unfused"):
         # the fused row kernels on their own: bfloat16 softmax over [128*2048, 2048] (the logits of
         # config 5) and bfloat16 LayerNorm over [32768, 4096]

@@ -288,6 +288,19 @@ int mxq_gemm_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const 
                    const void* b_scales, int b_kind, const void* bias, void* c, int c_dtype,
                    int64_t batch, int64_t M, int64_t N, int64_t K, int epilogue_quant,
                    void* workspace, int64_t workspace_bytes, void* hip_stream);
+/* Attention scores in one launch (no counterpart in the reference, which runs mx.bmm and mx.softmax
+ * as separate tensor passes: mx/bmm.py:40-59, mx/softmax.py:26-48):
+ *   out[b] = softmax over the last axis of Q(A[b] x B[b]^T),  bf16 (batch, M, N)
+ * for packed operands with 8-bit codes (MXQ_CODES_E4M3 / _E5M2) and K = 128 (head_dim 128), N a multiple
+ * of 32 up to 2048, with the elementwise quantizer of mx_specs['bfloat'] = 16 and round-half-away
+ * after the product and after every softmax step (exp2 = 1: 2^x as with softmax_exp2).  The logits
+ * stay in registers.  Results agree with mxq_gemm_mx_nt(epilogue_quant = 1) + mxq_softmax_lastdim
+ * within those kernels' own tolerance against the CPU chain (exp within 1 ulp, order of the row sum).
+ * flags: MXQ_FLAG_GENERAL_FORM. */
+int mxq_bmm_softmax_mx_nt(const void* a_codes, const void* a_scales, int a_kind, const void* b_codes,
+                          const void* b_scales, int b_kind, void* out, int64_t batch, int64_t M, int64_t N,
+                          int64_t K, int exp2, int flags, void* hip_stream);
+
 /* 0 when the product would not be split. */
 int64_t mxq_gemm_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int a_kind);
 /* Which kernel mxq_gemm_mx_nt launches for a shape (no counterpart in the reference; for tests and

@@ -11,7 +11,7 @@ from .mx_ops import quantize_mx_op
 from .elemwise_ops import quantize_elemwise_op
 from .linear import Linear, linear
 from .matmul import matmul
-from .bmm import bmm
+from .bmm import bmm, bmm_softmax
 from .softmax import Softmax, softmax
 from .layernorm import LayerNorm, RMSNorm, layer_norm
 from .activations import (sigmoid, tanh, relu, relu6, leaky_relu, silu, gelu,

@@ -59,6 +59,8 @@ GPU_SYMBOLS = {
                                 _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr, _c_i64, _c_ptr]),
     "mxq_gemm_workspace_bytes": (_c_i64, [_c_i64, _c_i64, _c_i64, _c_i64, _c_int]),
     "mxq_gemm_plan": (_c_int, [_c_i64, _c_i64, _c_i64, _c_i64, _c_int]),
+    "mxq_bmm_softmax_mx_nt": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_i64, _c_i64,
+                                       _c_i64, _c_i64, _c_int, _c_int, _c_ptr]),
     "mxq_reduce_sum_inner": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),
     "mxq_reduce_max_inner": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr]),
     "mxq_reduce_outer_workspace_bytes": (_c_i64, [_c_i64, _c_i64]),

@@ -64,3 +64,33 @@ def bmm(in1, in2, mx_specs=None, name=None):
         return torch_bmm(in1, in2)
     mx_specs = apply_mx_specs(mx_specs)
     return BMMFunction.apply(in1, in2, mx_specs, name)
+
+
+def bmm_softmax(in1, in2, mx_specs=None, name=None):
+    """softmax(bmm(in1, in2), dim=-1): attention scores.  Same result as calling mx.bmm and then
+    mx.softmax (mx/bmm.py:132-138, mx/softmax.py:91-97), which is also what runs whenever the one-launch
+    form does not apply.  That form -- the logits stay in registers between the product and the
+    softmax -- takes bf16 GPU operands when no gradient is wanted, in1 (..., M, 128), in2 a transposed
+    view of a contiguous (..., N, 128) tensor with N a multiple of 32 up to 2048, an 8-bit-code MX
+    format with block size 32, and mx_specs['bfloat'] = 16 with round-half-away (the quantizer applied
+    after the product and after every softmax step).  It agrees with the two separate kernels
+    within their own tolerance against the CPU chain (exp within 1 ulp, order of the row sum)."""
+    from .softmax import softmax
+    mx_assert_test(mx_specs)
+    if mx_specs is None:
+        return torch.softmax(torch_bmm(in1, in2), dim=-1)
+    specs = apply_mx_specs(mx_specs)
+    from .gemm import pack_can_quantize_first
+    wants_grad = torch.is_grad_enabled() and (in1.requires_grad or in2.requires_grad)
+    if (not wants_grad and in1.dim() >= 2 and in2.dim() >= 2
+            and inputs_can_skip_bfloat16_pass((False, False), (in1, in2), specs, specs["round_output"])
+            and pack_can_quantize_first(specs, specs["round"])
+            and not specs["vec_use_exp2"] and not specs["vec_use_recip"]):
+        bt = in2.transpose(-1, -2)
+        if bt.is_contiguous() and in1.is_contiguous():
+            from . import fused
+            out = fused.mx_bmm_softmax(in1, bt, specs["a_elem_format"], specs, specs["round_mx_output"],
+                                       exp2=bool(specs.get("softmax_exp2", False)))
+            if out is not None:
+                return out
+    return softmax(bmm(in1, in2, mx_specs=mx_specs, name=name), dim=-1, mx_specs=mx_specs)

@@ -37,7 +37,8 @@ def _run(cmd, verbose):
         print(out, flush=True)
 
 
-GPU_SOURCES = ["mxq_capi.hip", "mxq_capi_gemm.hip", "mxq_capi_chain.hip", "mxq_capi_norm.hip"]
+GPU_SOURCES = ["mxq_capi.hip", "mxq_capi_gemm.hip", "mxq_capi_chain.hip", "mxq_capi_norm.hip",
+               "mxq_capi_scores.hip"]
 
 
 def build_gpu(verbose=True):

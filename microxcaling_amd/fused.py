@@ -266,6 +266,45 @@ def mx_gemm_nt(a, b_kmajor, a_fmt, b_fmt, mx_specs, round, bias=None, epilogue_q
     return gemm_nt(pa, pb, out_dtype=a.dtype, bias=bias, epilogue_quant=epilogue_quant).reshape(out_shape)
 
 
+SCORES_K, SCORES_MAX_N = 128, 2048
+
+
+def mx_bmm_softmax(a, b_kmajor, fmt, mx_specs, round, exp2=False):
+    """softmax(Q(a x b_kmajor^T), dim = -1) in one launch (include/mxq.h: mxq_bmm_softmax_mx_nt) for
+    bf16 GPU operands a (..., M, 128), b_kmajor (..., N, 128) that have not been through the layers'
+    elementwise bfloat16 quantization yet (the pack kernels apply it), N a multiple of 32 up to 2048,
+    under the bfloat16 / round-half-away quantizer.  Returns None when the operands do not qualify."""
+    f = _as_format(fmt)
+    if f not in _PACKABLE or mx_specs["block_size"] != 32 or mx_specs["shared_exp_method"] != "max":
+        return None
+    if round not in RoundingMode.string_enums():
+        return None
+    if not (a.is_cuda and b_kmajor.is_cuda) or a.dtype != torch.bfloat16 or b_kmajor.dtype != torch.bfloat16:
+        return None
+    if a.dim() < 2 or a.dim() != b_kmajor.dim() or a.shape[:-2] != b_kmajor.shape[:-2]:
+        return None
+    K, M, N = a.shape[-1], a.shape[-2], b_kmajor.shape[-2]
+    if K != SCORES_K or b_kmajor.shape[-1] != K or N == 0 or N % 32 != 0 or N > SCORES_MAX_N or M == 0:
+        return None
+    a3 = a.contiguous().reshape(-1, M, K)
+    b3 = b_kmajor.contiguous().reshape(-1, N, K)
+    batch = a3.shape[0]
+    if batch == 0 or batch > 65535:
+        return None
+    scale_bits = mx_specs["scale_bits"] if mx_specs["scale_bits"] != 0 else 8
+    flush = mx_specs["mx_flush_fp32_subnorms"]
+    ac, asc, ak = pack_mx(a3, f, scale_bits, round, flush, False, True)
+    bc, bsc, bk = pack_mx(b3, f, scale_bits, round, flush, False, True)
+    out = torch.empty(a.shape[:-1] + (N,), dtype=torch.bfloat16, device=a.device)
+    lib = _lib.gpu()
+    with torch.cuda.device(a.device):
+        rc = lib.mxq_bmm_softmax_mx_nt(ac.data_ptr(), asc.data_ptr(), int(ak), bc.data_ptr(), bsc.data_ptr(),
+                                       int(bk), out.data_ptr(), batch, M, N, K, int(bool(exp2)),
+                                       _flags_value(), _stream(a))
+    _lib.check(rc, lib)
+    return out
+
+
 def mx_gemm_operands(operands, mx_specs, out_dtype):
     """General form of mx_gemm_nt for the gradient GEMMs: `operands` = two (tensor, format, round,
     transposed) entries.  transposed=False: the tensor is (..., rows, K), quantized along its last

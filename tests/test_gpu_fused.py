@@ -450,6 +450,101 @@ def test_bmm_and_softmax_forward(dev, fused):
     assert (sm - sm_want).abs().max() <= 2 ** -8 * 4
 
 
+def _grid_step_apart(got, want, share=0.02):
+    """Probabilities after the bfloat16 quantizer with round-half-away lie on a grid of even bf16
+    significands: neighbours are 2^-6 of their value apart at most (2^-7 just below 1.0).  One such
+    step (two on at most one element in 10 000), and at most `share` of the elements different at all
+    (far below 2^-126 the step is that of bf16's subnormals)."""
+    d = (got - want).abs()
+    steps = d / (2 ** -6 * want.abs() + 2.0 ** -133)
+    assert steps.max().item() <= 2.0, steps.max().item()            # a step in the row sum and one in the value
+    assert (steps > 1.0).float().mean().item() <= 1e-4, (steps > 1.0).float().mean().item()
+    assert (d > 0).float().mean().item() <= share, (d > 0).float().mean().item()
+
+
+@pytest.mark.parametrize("shape", [(4, 256, 2048), (1, 70, 64), (3, 33, 544), (2, 2048, 1024), (130, 32, 32)])
+@pytest.mark.parametrize("fmt,exp2", [("fp6_e2m3", False), ("fp8_e4m3", True), ("fp8_e5m2", False), ("fp4_e2m1", False)])
+def test_bmm_softmax_in_one_launch(dev, shape, fmt, exp2):
+    """mx.bmm_softmax (attention scores, logits kept in registers) against (1) mx.softmax(mx.bmm(...)),
+    the two separate kernels, and (2) the oracle's softmax chain on the logits those kernels produced:
+    absolute 2^-8 (one bf16 step at 1.0), at most 2 % of the elements different at all -- the
+    tolerance the separate softmax kernel has against the CPU chain (exp, order of the row sum)."""
+    from microxcaling_amd.bmm import bmm, bmm_softmax
+    from microxcaling_amd.softmax import softmax
+    B, M, N = shape
+    specs = _specs(a_elem_format=fmt, block_size=32, bfloat=16, softmax_exp2=exp2)
+    g = torch.Generator().manual_seed(B * 7 + M + N)
+    q = torch.randn(B, M, 128, generator=g).to(torch.bfloat16).to(dev)
+    k = (torch.randn(B, N, 128, generator=g) * (0.3 if fmt == "fp8_e5m2" else 1.0)).to(torch.bfloat16).to(dev)
+    q[0, 0] = 0.0                                            # a row of zero logits: uniform probabilities
+    k[0, 5, :32] = 0.0
+    got = bmm_softmax(q, k.transpose(-1, -2), mx_specs=specs)
+    logits = bmm(q, k.transpose(-1, -2), mx_specs=specs)
+    two = softmax(logits, dim=-1, mx_specs=specs)
+    torch.cuda.synchronize()
+    assert got.shape == two.shape and got.dtype == torch.bfloat16
+    _grid_step_apart(got.float(), two.float())
+    want = O.softmax_forward(logits.cpu(), -1, bfloat=16, use_exp2=exp2).float()
+    _grid_step_apart(got.float().cpu(), want)
+    assert torch.equal(got[0, 0].float().cpu(), want[0, 0])  # zero logits: exp(0) = 1 exactly, sum = N exactly
+
+
+def test_bmm_softmax_special_values_and_general_form(dev):
+    """Workgroups that leave the plain range (an Inf / NaN block, huge or tiny logits) take the
+    element-by-element form: NaN rows where the chain gives NaN rows, same tolerance elsewhere; and
+    that form, forced for every workgroup, agrees with the packed one on ordinary data."""
+    from microxcaling_amd import custom_extensions as ce
+    from microxcaling_amd.bmm import bmm, bmm_softmax
+    from microxcaling_amd.softmax import softmax
+    specs = _specs(a_elem_format="fp8_e4m3", block_size=32, bfloat=16)
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(3, 96, 128, generator=g).to(torch.bfloat16)
+    k = torch.randn(3, 160, 128, generator=g).to(torch.bfloat16)
+    q[0, 3, 7] = float("inf")                                # NaN block -> row 3 of batch 0 is NaN
+    k[1, 9, 100] = float("nan")                              # -> column 9 of batch 1 is NaN -> every row NaN
+    q[2, :32] *= 2.0 ** 60                                   # logits around 2^120: outside the plain range
+    k[2, :80] *= 2.0 ** 60
+    q[2, 64:] *= 2.0 ** -70                                  # and around 2^-140 ... 2^-10
+    qd, kd = q.to(dev), k.to(dev)
+    got = bmm_softmax(qd, kd.transpose(-1, -2), mx_specs=specs)
+    two = softmax(bmm(qd, kd.transpose(-1, -2), mx_specs=specs), dim=-1, mx_specs=specs)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.isnan(got), torch.isnan(two))
+    assert bool(torch.isnan(got[0, 3]).all()) and bool(torch.isnan(got[1]).all()) and not bool(torch.isnan(got[0, 4]).any())
+    fin = ~torch.isnan(two)
+    _grid_step_apart(got.float()[fin], two.float()[fin])
+    q2 = torch.randn(2, 64, 128, generator=g).to(torch.bfloat16).to(dev)
+    k2 = torch.randn(2, 2048, 128, generator=g).to(torch.bfloat16).to(dev)
+    packed = bmm_softmax(q2, k2.transpose(-1, -2), mx_specs=specs)
+    ce.set_general_form(True)
+    try:
+        general = bmm_softmax(q2, k2.transpose(-1, -2), mx_specs=specs)
+    finally:
+        ce.set_general_form(False)
+    _grid_step_apart(packed.float(), general.float(), share=0.01)
+
+
+def test_bmm_softmax_declines_what_it_does_not_cover(dev):
+    """Other head dims, row lengths, gradients, fp32 tensors: the two separate ops run, same values
+    as calling them directly."""
+    from microxcaling_amd.bmm import bmm, bmm_softmax
+    from microxcaling_amd.softmax import softmax
+    specs = _specs(a_elem_format="fp6_e2m3", block_size=32, bfloat=16)
+    g = torch.Generator().manual_seed(22)
+    for shape_q, shape_k, dt in (((2, 40, 64), (2, 96, 64), torch.bfloat16), ((2, 40, 128), (2, 100, 128), torch.bfloat16),
+                                 ((2, 40, 128), (2, 96, 128), torch.float32)):
+        q = torch.randn(*shape_q, generator=g).to(dt).to(dev)
+        k = torch.randn(*shape_k, generator=g).to(dt).to(dev)
+        a = bmm_softmax(q, k.transpose(-1, -2), mx_specs=specs)
+        b = softmax(bmm(q, k.transpose(-1, -2), mx_specs=specs), dim=-1, mx_specs=specs)
+        assert torch.equal(a, b)
+    q = torch.randn(2, 40, 128, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
+    k = torch.randn(2, 96, 128, generator=g).to(torch.bfloat16).to(dev)
+    out = bmm_softmax(q, k.transpose(-1, -2), mx_specs=specs)
+    out.sum().backward()
+    assert q.grad is not None and torch.isfinite(q.grad).all()
+
+
 def test_linear_backward_runs(dev):
     from microxcaling_amd.linear import Linear
     specs = _specs(w_elem_format="fp6_e3m2", a_elem_format="fp6_e3m2", block_size=32, bfloat=16)
