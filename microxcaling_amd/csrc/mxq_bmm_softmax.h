@@ -94,8 +94,11 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
         const int r = i * 8 + (lane >> 3);
         boff[i] = (uint32_t)(r * 128 + (((lane & 7) ^ mxq_addr::large_key(r)) * 16));
     }
-    auto fetch_b = [&](int i) {                               // tile number i of this wave into slot i % BS_RING
-        const int t = i * 4 + wave;
+    // tile number i of this wave: the waves take pairs of neighbouring tiles (64 columns = one 128-byte
+    // line of output per row) in turn
+    auto tile_of = [&](int i) { return 8 * (i >> 1) + 2 * wave + (i & 1); };
+    auto fetch_b = [&](int i) {                               // ... into slot i % BS_RING
+        const int t = tile_of(i);
         if (t < ntiles) {                                     // uniform per wave
             const unsigned char* src = Bt + (int64_t)t * BS_TILE_BYTES;
 #pragma unroll
@@ -109,13 +112,17 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
 #pragma unroll
     for (int q = 0; q < 4; ++q) b_addr[q] = b_lane * 128 + (((2 * q + fg) ^ mxq_addr::large_key(b_lane)) * 16);
     const unsigned char* my_ring = ring + wave * (BS_RING * BS_TILE_BYTES);
+    // this wave's tiles are numbers 0 .. my_tiles - 1 of its sequence (tile_of grows with i)
+    int my_tiles = 0;
+#pragma unroll
+    for (int i = 0; i < BS_TILES; ++i) my_tiles += tile_of(i) < ntiles ? 1 : 0;
     // the scale bytes of this lane's B rows, all tiles, shifted so that block fg comes first
     int sbw[BS_TILES];
     {
         const unsigned char* SB = g.sb + bz * g.batch_sb + (int64_t)b_lane * 4;
 #pragma unroll
         for (int i = 0; i < BS_TILES; ++i) {
-            const int t = i * 4 + wave;
+            const int t = tile_of(i);
             sbw[i] = t < ntiles ? (int)(*reinterpret_cast<const uint32_t*>(SB + (int64_t)t * (32 * 4)) >> (8 * fg)) : 0;
         }
     }
@@ -140,17 +147,18 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
     // counter of loads in flight below counts tile copies only
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int i = 0; i < BS_RING - 1; ++i) fetch_b(i);
+    for (int i = 0; i < BS_RING; ++i) fetch_b(i);
+    // the MFMAs of tile i + 1 are issued before the conversion of tile i, so that the matrix pipe works
+    // in the shadow of the vector instructions
+    auto multiply = [&](int i) {
+        v16f acc;
 #pragma unroll
-    for (int i = 0; i < BS_TILES; ++i) {
-        const int t = i * 4 + wave;
-        if (i + BS_RING - 1 < BS_TILES) fetch_b(i + BS_RING - 1);   // slot of tile i - 1, whose reads are done
-        if (t < ntiles) {                                     // uniform per wave
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+        if (tile_of(i) < ntiles) {                            // uniform per wave
             // loads complete in order: at most the copies of the tiles fetched after tile i may still
             // be in flight (4 instructions each)
-            const int later = min(BS_RING - 1, BS_TILES - 1 - i);
-            if (later == 3) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-            else if (later == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            const int later = min(BS_RING - 1, my_tiles - 1 - i);
+            if (later >= 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
             else if (later == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             Frag bf;
@@ -159,11 +167,19 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
             for (int q = 0; q < 4; ++q) bf.r[q] = *reinterpret_cast<const u32x4*>(slot + b_addr[q]);
             Scales sb;
             sb.w[0] = sbw[i];
-            v16f acc;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[v] = 0.f;
             acc = mx_mfma32<CBSZ, BLGP>(bf, af, acc, sb, sa, 0);
             acc = mx_mfma32<CBSZ, BLGP>(bf, af, acc, sb, sa, 1);
+        }
+        return acc;
+    };
+    v16f acc = multiply(0);
+#pragma unroll
+    for (int i = 0; i < BS_TILES; ++i) {
+        v16f next = acc;
+        // the fragment of tile i has been read (its MFMAs have been issued): its slot takes tile i + BS_RING
+        if (i + BS_RING < BS_TILES) fetch_b(i + BS_RING);
+        if (i + 1 < BS_TILES) next = multiply(i + 1);
+        if (tile_of(i) < ntiles) {                            // uniform per wave
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const uint32_t w = Pack<MXQ_BF16>::put(acc[2 * j], acc[2 * j + 1]);
@@ -174,6 +190,7 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
                 mx = fmaxf(mx, fmaxf(low_of(w), high_of(w)));
             }
         }
+        acc = next;
     }
     // all logits of the workgroup finite, below 2^100, and zero or at least 2^-100?
     const unsigned short top = hi[0] > hi[1] ? hi[0] : hi[1], bottom = lo[0] < lo[1] ? lo[0] : lo[1];
@@ -191,7 +208,7 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
         const float c = g.exp2 ? 0.5f : 0.72134752f;          // half of 1, or of log2(e)
 #pragma unroll
         for (int i = 0; i < BS_TILES; ++i) {
-            if (i * 4 + wave < ntiles) {
+            if (tile_of(i) < ntiles) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t x = qpair(lg[i][j]);
@@ -211,7 +228,7 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
         float mg = -__builtin_inff();
 #pragma unroll
         for (int i = 0; i < BS_TILES; ++i) {
-            if (i * 4 + wave < ntiles) {
+            if (tile_of(i) < ntiles) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const float x0 = Qd(low_of(lg[i][j])), x1 = Qd(high_of(lg[i][j]));
@@ -226,7 +243,7 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
         m = MaxOp::apply(MaxOp::apply(red[1][0][fi], red[1][1][fi]), MaxOp::apply(red[1][2][fi], red[1][3][fi]));
 #pragma unroll
         for (int i = 0; i < BS_TILES; ++i) {
-            if (i * 4 + wave < ntiles) {
+            if (tile_of(i) < ntiles) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const float d0 = Q(low_of(lg[i][j]) - m), d1 = Q(high_of(lg[i][j]) - m);
@@ -245,30 +262,46 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
     const float s = Qp(((red[1][0][fi] + red[1][1][fi]) + red[1][2][fi]) + red[1][3][fi]);
 
     // ---- phase 3: the quotients ---------------------------------------------------------------------
-    const bool row_ok = m0 + fi < g.M;
-    unsigned short* out = reinterpret_cast<unsigned short*>(g.out) + bz * g.batch_c + (int64_t)(m0 + fi) * g.N + 8 * fg;
     // one refined reciprocal per row; e * r is within two units in the last place of e / s, which
     // the rounding to bf16 hides except within that distance of a rounding boundary
     const float r0 = __builtin_amdgcn_rcpf(s);
     const float r1 = fmaf(fmaf(-s, r0, 1.0f), r0, r0);
+    // A lane holds, of a pair of tiles, four 16-byte pieces of its row's 128-byte line: pieces fg and
+    // 2 + fg of either tile.  They go through the wave's (now idle) part of the ring so that the store
+    // instructions write whole lines: piece p of row r sits at position p ^ (r & 7) of the row's 128
+    // bytes (conflict-free both ways); lane L then picks up piece L % 8 of the rows 8 k + L / 8.
+    unsigned char* stage = const_cast<unsigned char*>(my_ring);
+    const int srow = lane >> 3, spiece = lane & 7;
+    unsigned short* out = reinterpret_cast<unsigned short*>(g.out) + bz * g.batch_c + (int64_t)(m0 + srow) * g.N + 8 * spiece;
 #pragma unroll
-    for (int i = 0; i < BS_TILES; ++i) {
-        const int t = i * 4 + wave;
-        if (t < ntiles) {
-            uint32_t o[8];
+    for (int k = 0; k < BS_TILES / 2; ++k) {
+        const int t0 = tile_of(2 * k);
+        if (t0 < ntiles) {                                    // uniform per wave
+            unsigned char* buf = stage + (k & 1) * BS_TILE_BYTES;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float e0 = low_of(lg[i][j]), e1 = high_of(lg[i][j]);
-                if (plain) {
-                    o[j] = qpair_nonneg(Pack<MXQ_BF16>::put(e0 * r1, e1 * r1));
-                } else {
-                    const float q0 = Qp(e0 / s), q1 = Qp(e1 / s);
-                    o[j] = (mxq_bits(q0) >> 16) | (mxq_bits(q1) & 0xFFFF0000u);
+            for (int p = 0; p < 2; ++p) {
+                const int i = 2 * k + p;
+                uint32_t o[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float e0 = low_of(lg[i][j]), e1 = high_of(lg[i][j]);
+                    if (plain) {
+                        o[j] = qpair_nonneg(Pack<MXQ_BF16>::put(e0 * r1, e1 * r1));
+                    } else {
+                        const float q0 = Qp(e0 / s), q1 = Qp(e1 / s);
+                        o[j] = (mxq_bits(q0) >> 16) | (mxq_bits(q1) & 0xFFFF0000u);
+                    }
                 }
+                *reinterpret_cast<u32x4*>(buf + fi * 128 + (((4 * p + fg) ^ (fi & 7)) * 16)) = u32x4{o[0], o[1], o[2], o[3]};
+                *reinterpret_cast<u32x4*>(buf + fi * 128 + (((4 * p + 2 + fg) ^ (fi & 7)) * 16)) = u32x4{o[4], o[5], o[6], o[7]};
             }
-            if (row_ok) {
-                __builtin_nontemporal_store(u32x4{o[0], o[1], o[2], o[3]}, reinterpret_cast<u32x4*>(out + t * 32));
-                __builtin_nontemporal_store(u32x4{o[4], o[5], o[6], o[7]}, reinterpret_cast<u32x4*>(out + t * 32 + 16));
+            const bool second = t0 + 1 < ntiles;              // an odd number of tiles: the last line is half a line
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = 8 * r + srow;
+                const u32x4 v = *reinterpret_cast<const u32x4*>(buf + row * 128 + ((spiece ^ (row & 7)) * 16));
+                if (m0 + row < g.M && (second || spiece < 4))
+                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out + (int64_t)(8 * r) * g.N + t0 * 32));
             }
         }
     }
