@@ -352,30 +352,32 @@ __device__ __forceinline__ v4f mx_mfma(const v8i& b, const v8i& a, v4f c, int sb
     }
 }
 
-// One 32 x 32 x 64 MFMA of the large-tile kernel: operand registers and scale byte of MFMA h of a
-// K step out of the four 16-byte reads r[0..3] of a lane (see the kernel).  `sb`, `sa` hold the
-// row's scale bytes shifted so that this lane's block comes first; op_sel picks byte 0 or 2.
-template <int CBSZ, int BLGP, class Frag, class Scales>
-__device__ __forceinline__ v16f mx_mfma32(const Frag& b, const Frag& a, v16f c, const Scales& sb,
-                                          const Scales& sa, int h) {
+// One 32 x 32 x 64 MFMA of the large-tile kernel, MFMA h of a K step, from the part of either
+// fragment that it reads: two 16-byte pieces of a lane's row (8-bit codes) or one (nibbles), so that
+// the kernel holds half fragments only.  `sb`, `sa` hold the row's scale bytes shifted so that this
+// lane's block comes first; op_sel picks byte 0 or 2.
+template <class Half> struct QOF { static constexpr int Q = sizeof(Half) / 16; };
+template <int CBSZ, int BLGP, class Half, class Scales>
+__device__ __forceinline__ v16f mx_mfma32_half(const Half& b, const Half& a, v16f c, const Scales& sb,
+                                               const Scales& sa, int h) {
     if constexpr (CBSZ == 4) {
-#define MXQ_MMA4(H)                                                                                       \
+#define MXQ_MMA4H(H)                                                                                      \
     __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                                                      \
-        v8i{(int)b.r[H][0], (int)b.r[H][1], (int)b.r[H][2], (int)b.r[H][3], 0, 0, 0, 0},                  \
-        v8i{(int)a.r[H][0], (int)a.r[H][1], (int)a.r[H][2], (int)a.r[H][3], 0, 0, 0, 0}, c, 4, 4,          \
+        v8i{(int)b.r[0][0], (int)b.r[0][1], (int)b.r[0][2], (int)b.r[0][3], 0, 0, 0, 0},                  \
+        v8i{(int)a.r[0][0], (int)a.r[0][1], (int)a.r[0][2], (int)a.r[0][3], 0, 0, 0, 0}, c, 4, 4,          \
         ((H) & 1) * 2, sb.w[(H) >> 1], ((H) & 1) * 2, sa.w[(H) >> 1])
-        return h == 0 ? MXQ_MMA4(0) : h == 1 ? MXQ_MMA4(1) : h == 2 ? MXQ_MMA4(2) : MXQ_MMA4(3);
-#undef MXQ_MMA4
+        return h == 0 ? MXQ_MMA4H(0) : h == 1 ? MXQ_MMA4H(1) : h == 2 ? MXQ_MMA4H(2) : MXQ_MMA4H(3);
+#undef MXQ_MMA4H
     } else {
-#define MXQ_MMA8(H)                                                                                       \
+#define MXQ_MMA8H(H)                                                                                      \
     __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                                                      \
-        v8i{(int)b.r[2 * H][0], (int)b.r[2 * H][1], (int)b.r[2 * H][2], (int)b.r[2 * H][3],               \
-            (int)b.r[2 * H + 1][0], (int)b.r[2 * H + 1][1], (int)b.r[2 * H + 1][2], (int)b.r[2 * H + 1][3]}, \
-        v8i{(int)a.r[2 * H][0], (int)a.r[2 * H][1], (int)a.r[2 * H][2], (int)a.r[2 * H][3],               \
-            (int)a.r[2 * H + 1][0], (int)a.r[2 * H + 1][1], (int)a.r[2 * H + 1][2], (int)a.r[2 * H + 1][3]}, \
+        v8i{(int)b.r[0][0], (int)b.r[0][1], (int)b.r[0][2], (int)b.r[0][3],                               \
+            (int)b.r[QOF<Half>::Q - 1][0], (int)b.r[QOF<Half>::Q - 1][1], (int)b.r[QOF<Half>::Q - 1][2], (int)b.r[QOF<Half>::Q - 1][3]}, \
+        v8i{(int)a.r[0][0], (int)a.r[0][1], (int)a.r[0][2], (int)a.r[0][3],                               \
+            (int)a.r[QOF<Half>::Q - 1][0], (int)a.r[QOF<Half>::Q - 1][1], (int)a.r[QOF<Half>::Q - 1][2], (int)a.r[QOF<Half>::Q - 1][3]}, \
         c, BLGP, CBSZ, (H) * 2, sb.w[0], (H) * 2, sa.w[0])
-        return h == 0 ? MXQ_MMA8(0) : MXQ_MMA8(1);
-#undef MXQ_MMA8
+        return h == 0 ? MXQ_MMA8H(0) : MXQ_MMA8H(1);
+#undef MXQ_MMA8H
     }
 }
 
@@ -870,69 +872,141 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     const int sa_off = G3_SCALE_OFF + a_lane * 16, sa_tail = G3_TAIL_OFF + a_lane * 4;
     const int sb_off = G3_SCALE_OFF + 4096 + b_lane * 16, sb_tail = G3_TAIL_OFF + (256 + b_lane) * 4;
     const int sshift = fg * 8;
-    struct Frag { u32x4 r[4]; };
-    auto frag = [&](const unsigned char* stage, const int* addr, int tile) {
-        Frag f;
+    constexpr int QH = 4 / NH;                               // 16-byte reads of a fragment per MFMA
+    struct Half { u32x4 r[QH]; };
+    auto half = [&](const unsigned char* stage, const int* addr, int tile, int h) {
+        Half f;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) f.r[q] = *reinterpret_cast<const u32x4*>(stage + addr[q] + tile * 32 * 128);
+        for (int q = 0; q < QH; ++q)
+            f.r[q] = *reinterpret_cast<const u32x4*>(stage + addr[h * QH + q] + tile * 32 * 128);
         return f;
     };
     struct Scales { int w[EPB]; };
     int c_groups = 0, c_slot = 0;                            // scale groups started, the one in use
-    // flat step t, K step cs of the tile: multiply the stage t & 1 while the tile copy fills the
-    // other one with K step fs of the fetch-side tile
-    auto step = [&](int t, int cs, int fs) {
-        const unsigned char* cur = lds + (t & 1) * G3_STAGE_BYTES;
-        const bool tail = cs >= nfull;
+    // ---- the flat sequence of K steps ---------------------------------------------------------------
+    // Step t multiplies stage t & 1.  A K step is walked MFMA number by MFMA number (h = 0: the first
+    // 64 bytes of K for every tile, then h = 1, ...), in NG groups of two MFMAs (one B half, both A
+    // halves): a wave holds only the parts of the fragments that the current MFMAs read.  The step's one
+    // barrier stands before its last two groups: by then the wave has read everything it needs from
+    // this stage (the B halves of those two groups included) and the copy of the next stage has
+    // landed, so right behind the barrier it reads the operands of the next step's first group, and
+    // the burst of LDS reads that all eight waves make at that point runs under the MFMAs of the last
+    // two groups instead of under nothing.  The same barrier frees this stage: the copy of step t + 2
+    // starts behind it (six of its nine loads in the last two groups, the rest in the first two
+    // groups of step t + 1), which gives it more than a step to land.
+    constexpr int NG = NH * 4;
+    constexpr int BP = NG - 3;                               // the group behind whose MFMAs the barrier stands
+    // fetch side: the K step that the copy instructions issued now belong to
+    int f_logical = blockIdx.x, f_fs = 0;
+    auto fetch_advance = [&]() {
+        if (++f_fs == nk) {
+            f_fs = 0;
+            if (f_logical + G < total) {
+                f_logical += G;
+                fetch_tile(f_logical);
+            }                                                // else: this tile's first step once more; nobody reads it
+        }
+    };
+    // compute side: where the scale bytes of a K step sit (inside a group of 16 bytes per row, or in
+    // the planes of a single step of 4 bytes per row each)
+    bool tail = false;
+    const unsigned char* sc = lds;
+    auto scale_place = [&](int cs) {                         // once per step, in step order
+        tail = cs >= nfull;
         if (!tail && cs % GS == 0) c_slot = c_groups++ & 1;
-        // the scale bytes of this step: inside the current group (16 bytes per row), or the planes
-        // of a single step (4 bytes per row each)
-        const unsigned char* sc = tail ? lds + (cs & 1) * G3_TAIL_SLOT
-                                       : lds + c_slot * G3_SCALE_GROUP + (cs % GS) * SBY;
-        auto scales = [&](int in_group, int in_tail) {       // the row's scale bytes, this lane's block first
-            Scales r;
+        sc = tail ? lds + (cs & 1) * G3_TAIL_SLOT : lds + c_slot * G3_SCALE_GROUP + (cs % GS) * SBY;
+    };
+    auto scales = [&](int in_group, int in_tail) {           // the row's scale bytes, this lane's block first
+        Scales r;
 #pragma unroll
-            for (int e = 0; e < EPB; ++e) {
-                const unsigned char* p = tail ? sc + in_tail + e * G3_TAIL_PLANE : sc + in_group + 4 * e;
-                r.w[e] = (int)(*reinterpret_cast<const uint32_t*>(p) >> sshift);
-            }
-            return r;
-        };
-        Frag af[2];
-        Scales sa[2];
+        for (int e = 0; e < EPB; ++e) {
+            const unsigned char* p = tail ? sc + in_tail + e * G3_TAIL_PLANE : sc + in_group + 4 * e;
+            r.w[e] = (int)(*reinterpret_cast<const uint32_t*>(p) >> sshift);
+        }
+        return r;
+    };
+    // operands of the first group of the step about to run (read behind the previous step's barrier)
+    Scales sa[2], sb0;
+    Half afh[2], bfh;
+    auto first_operands = [&](const unsigned char* stage) {
+        bfh = half(stage, b_addr, 0, 0);
+        sb0 = scales(sb_off, sb_tail);
 #pragma unroll
         for (int ti = 0; ti < 2; ++ti) {
-            af[ti] = frag(cur, a_addr, ti);
+            afh[ti] = half(stage, a_addr, ti, 0);
             sa[ti] = scales(sa_off + ti * 512, sa_tail + ti * 128);
         }
-        Frag bf = frag(cur, b_addr, 0);
-        Scales sb = scales(sb_off, sb_tail);
+    };
+    // t: flat step number; next_cs: the K step (of its tile) that follows this one
+    auto step = [&](int t, int next_cs) {
+        const unsigned char* cur = lds + (t & 1) * G3_STAGE_BYTES;
+        const unsigned char* nxt = lds + ((t + 1) & 1) * G3_STAGE_BYTES;
+        Scales sbv[4], sa_n[2], sb0_n;
+        sbv[0] = sb0;
+        Half late[2], afh_n[2], bfh_n;                       // B halves of the two groups behind the barrier; the next step's
 #pragma unroll
-        for (int tj = 0; tj < 4; ++tj) {
-            Frag bf_next = bf;                               // the next B fragment is read in the
-            Scales sb_next = sb;                             // shadow of this fragment's MFMAs
-            if (tj + 1 < 4) {
-                bf_next = frag(cur, b_addr, tj + 1);
-                sb_next = scales(sb_off + (tj + 1) * 512, sb_tail + (tj + 1) * 128);
+        for (int gi = 0; gi < NG; ++gi) {
+            const int h = gi / 4, tj = gi % 4;
+            Half bfh_next = bfh, afh_next[2] = {afh[0], afh[1]};    // the next group's operands are read
+            if (gi < BP) {                                            // in the shadow of this group's MFMAs
+                const int h2 = (gi + 1) / 4, tj2 = (gi + 1) % 4;
+                bfh_next = half(cur, b_addr, tj2, h2);
+                if (h2 == 0) sbv[tj2] = scales(sb_off + tj2 * 512, sb_tail + tj2 * 128);
+                if (tj2 == 0) {
+#pragma unroll
+                    for (int ti = 0; ti < 2; ++ti) afh_next[ti] = half(cur, a_addr, ti, h2);
+                }
+            } else if (gi == BP) {                           // ... here those of both groups behind the barrier
+                late[0] = half(cur, b_addr, 2, NH - 1);
+                late[1] = half(cur, b_addr, 3, NH - 1);
+                bfh_next = late[0];
+            } else if (gi == BP + 1) {
+                bfh_next = late[1];
             }
+            // Fences for the instruction scheduler: left alone it sinks every LDS read to just above the MFMA
+            // that uses it (read, wait, multiply: the read's latency in the open, group after group), and
+            // it hoists the copy instructions above the MFMAs, so that every wave of the workgroup sits in
+            // the memory pipe's queue at the same time with the matrix pipes idle.
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int h = 0; h < NH; ++h)
-#pragma unroll
-                for (int ti = 0; ti < 2; ++ti)
-                    acc[ti][tj] = mx_mfma32<CBSZ, BLGP>(bf, af[ti], acc[ti][tj], sb, sa[ti], h);
-            // The tile copy of the next step goes out behind this group's MFMAs, three loads per
-            // group.  The empty asm pins the MFMAs above it: the compiler would otherwise issue
-            // all loads first, and every wave of the workgroup would sit in the memory pipe's
-            // queue at the same time with the matrix pipes idle.
+            for (int ti = 0; ti < 2; ++ti)
+                acc[ti][tj] = mx_mfma32_half<CBSZ, BLGP>(bfh, afh[ti], acc[ti][tj], sbv[tj], sa[ti], h);
             asm volatile("" : "+v"(acc[0][tj]), "+v"(acc[1][tj]));
+            __builtin_amdgcn_sched_barrier(0);
+            if (gi == 0) {                                   // copy of the next step, loads 6 .. 8
+                fetch_part(t + 1, f_fs, 6);
+                fetch_part(t + 1, f_fs, 7);
+            } else if (gi == 1) {
+                fetch_part(t + 1, f_fs, 8);
+            } else if (gi == BP) {
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // this wave's share of the next stage is in,
+                __syncthreads();                                              // everybody's is; and this stage is free
+                fetch_advance();
+                scale_place(next_cs);
+                bfh_n = half(nxt, b_addr, 0, 0);
+                sb0_n = scales(sb_off, sb_tail);
 #pragma unroll
-            for (int i = 0; i < 9; ++i)
-                if (i / 3 == tj) fetch_part(t + 1, fs, i);
-            bf = bf_next;
-            sb = sb_next;
+                for (int ti = 0; ti < 2; ++ti) {
+                    afh_n[ti] = half(nxt, a_addr, ti, 0);
+                    sa_n[ti] = scales(sa_off + ti * 512, sa_tail + ti * 128);
+                }
+            }
+            if (gi > BP) {                                   // copy of the step after next, loads 0 .. 5
+#pragma unroll
+                for (int i = 0; i < 3; ++i) fetch_part(t, f_fs, (gi - BP - 1) * 3 + i);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            bfh = bfh_next;
+            afh[0] = afh_next[0];
+            afh[1] = afh_next[1];
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // this wave's share of the next stage is in
-        __syncthreads();                                     // ... everybody's is, and this stage is free
+        bfh = bfh_n;
+        sb0 = sb0_n;
+#pragma unroll
+        for (int ti = 0; ti < 2; ++ti) {
+            afh[ti] = afh_n[ti];
+            sa[ti] = sa_n[ti];
+        }
     };
 
     int logical = blockIdx.x;                                // tile being multiplied
@@ -941,16 +1015,16 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     for (int i = 0; i < 9; ++i) fetch_part(0, 0, i);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    fetch_advance();
+    scale_place(0);
+    first_operands(lds);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) fetch_part(1, f_fs, i);
 
     int t = 0;
     while (true) {
-        for (int cs = 0; cs + 1 < nk; ++cs, ++t) step(t, cs, cs + 1);
-        // last K step of this tile: the tile copy moves on to the next tile (or, when there is none,
-        // fetches this tile's first step once more; nobody reads it)
+        for (int cs = 0; cs < nk; ++cs, ++t) step(t, cs + 1 < nk ? cs + 1 : 0);
         const int next = logical + G;
-        if (next < total) fetch_tile(next);
-        step(t, nk - 1, 0);
-        ++t;
 
         const int bz = logical / per_batch;
         int tm, tn;
@@ -1023,6 +1097,7 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
         if (next >= total) break;
         logical = next;
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // the copy ran ahead: nothing may still be landing in LDS
 }
 
 }  // namespace
