@@ -352,10 +352,36 @@ __device__ __forceinline__ v4f mx_mfma(const v8i& b, const v8i& a, v4f c, int sb
     }
 }
 
-// One 32 x 32 x 64 MFMA of the large-tile kernel, MFMA h of a K step, from the part of either
-// fragment that it reads: two 16-byte pieces of a lane's row (8-bit codes) or one (nibbles), so that
-// the kernel holds half fragments only.  `sb`, `sa` hold the row's scale bytes shifted so that this
-// lane's block comes first; op_sel picks byte 0 or 2.
+// One 32 x 32 x 64 MFMA: operand registers and scale byte of MFMA h of a K step out of the four
+// 16-byte reads r[0..3] of a lane (lane (i, g) reads the 16-byte columns 2 q + g, q = 0..3, of its
+// row).  `sb`, `sa` hold the row's scale bytes shifted so that this lane's block comes first; op_sel
+// picks byte 0 or 2.  Used by the attention-score kernel, whose K is a single step.
+template <int CBSZ, int BLGP, class Frag, class Scales>
+__device__ __forceinline__ v16f mx_mfma32(const Frag& b, const Frag& a, v16f c, const Scales& sb,
+                                          const Scales& sa, int h) {
+    if constexpr (CBSZ == 4) {
+#define MXQ_MMA4(H)                                                                                       \
+    __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                                                      \
+        v8i{(int)b.r[H][0], (int)b.r[H][1], (int)b.r[H][2], (int)b.r[H][3], 0, 0, 0, 0},                  \
+        v8i{(int)a.r[H][0], (int)a.r[H][1], (int)a.r[H][2], (int)a.r[H][3], 0, 0, 0, 0}, c, 4, 4,          \
+        ((H) & 1) * 2, sb.w[(H) >> 1], ((H) & 1) * 2, sa.w[(H) >> 1])
+        return h == 0 ? MXQ_MMA4(0) : h == 1 ? MXQ_MMA4(1) : h == 2 ? MXQ_MMA4(2) : MXQ_MMA4(3);
+#undef MXQ_MMA4
+    } else {
+#define MXQ_MMA8(H)                                                                                       \
+    __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(                                                      \
+        v8i{(int)b.r[2 * H][0], (int)b.r[2 * H][1], (int)b.r[2 * H][2], (int)b.r[2 * H][3],               \
+            (int)b.r[2 * H + 1][0], (int)b.r[2 * H + 1][1], (int)b.r[2 * H + 1][2], (int)b.r[2 * H + 1][3]}, \
+        v8i{(int)a.r[2 * H][0], (int)a.r[2 * H][1], (int)a.r[2 * H][2], (int)a.r[2 * H][3],               \
+            (int)a.r[2 * H + 1][0], (int)a.r[2 * H + 1][1], (int)a.r[2 * H + 1][2], (int)a.r[2 * H + 1][3]}, \
+        c, BLGP, CBSZ, (H) * 2, sb.w[0], (H) * 2, sa.w[0])
+        return h == 0 ? MXQ_MMA8(0) : MXQ_MMA8(1);
+#undef MXQ_MMA8
+    }
+}
+
+// The same MFMA from the part of either fragment that it reads: two 16-byte pieces of a lane's row
+// (8-bit codes) or one (nibbles), so that the large-tile kernel holds half fragments only.
 template <class Half> struct QOF { static constexpr int Q = sizeof(Half) / 16; };
 template <int CBSZ, int BLGP, class Half, class Scales>
 __device__ __forceinline__ v16f mx_mfma32_half(const Half& b, const Half& a, v16f c, const Scales& sb,
