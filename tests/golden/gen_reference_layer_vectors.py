@@ -171,6 +171,36 @@ def main(ref_root):
         store(d, key + "gw", wi.grad)
         store(d, key + "gb", bi.grad)
 
+    # a layer with prequantized weights (mx/linear.py:246-274): weight and bias stored as bf16 once,
+    # inference on bf16 and on fp32 inputs (the bf16 weight then meets an input of another dtype, 77-80)
+    from mx.linear import Linear
+    pspecs = finalize_mx_specs(dict(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32,
+                                    bfloat=16, round="even", custom_cuda=False))
+    m = Linear(64, 48, bias=True, mx_specs=pspecs)
+    with torch.no_grad():
+        m.weight.copy_(w)
+        m.bias.copy_(b)
+    m.prequantize_weights()
+    m.eval()
+    store(d, "linear_prequantized/p_weight", m.weight.data)
+    store(d, "linear_prequantized/p_bias", m.bias.data)
+    with torch.no_grad():
+        store(d, "linear_prequantized/out_bf16", m(x.to(torch.bfloat16)))
+        store(d, "linear_prequantized/out_f32", m(x))
+
+    # attention scores: softmax over the last axis of a batched product (mx/bmm.py:132-138 followed by
+    # mx/softmax.py:91-97), forward and the gradients of both operands
+    aspecs = finalize_mx_specs(dict(a_elem_format="fp6_e2m3", block_size=32, bfloat=16, quantize_backprop=True,
+                                    custom_cuda=False))
+    for dt_name, dt in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+        ai, bi2 = x.to(dt).clone().requires_grad_(True), a2.to(dt).clone().requires_grad_(True)
+        out = softmax(bmm(ai, bi2, mx_specs=aspecs), dim=-1, mx_specs=aspecs)
+        out.backward(go2.to(dt))
+        key = "bmm_softmax/%s/" % dt_name
+        store(d, key + "out", out)
+        store(d, key + "g1", ai.grad)
+        store(d, key + "g2", bi2.grad)
+
     np.savez_compressed(os.path.join(HERE, "reference_layer_vectors.npz"), **d)
     print("wrote %d arrays, torch %s" % (len(d), torch.__version__))
 

@@ -60,6 +60,38 @@ def test_linear_oracle_and_cpu_layer(dt, bfloat):
     assert_bits_equal(bi.grad, fx(key + "gb"), "layer grad_bias")
 
 
+def test_linear_with_prequantized_weights():
+    """mx/linear.py:246-274: weight and bias stored as bf16 once (round-half-even), inference on bf16
+    inputs and on fp32 inputs (mx/linear.py:77-80).  On CPU tensors no packed form is built."""
+    from microxcaling_amd.linear import Linear
+    x, w, b = fx("in/x"), fx("in/w"), fx("in/b")
+    specs = _specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32, bfloat=16, round="even")
+    m = Linear(64, 48, bias=True, mx_specs=specs)
+    with torch.no_grad():
+        m.weight.copy_(w)
+        m.bias.copy_(b)
+    m.prequantize_weights()
+    m.eval()
+    assert m.weight.dtype == torch.bfloat16 and m.bias.dtype == torch.bfloat16
+    assert_bits_equal(m.weight.data, fx("linear_prequantized/p_weight"), "stored weight")
+    assert_bits_equal(m.bias.data, fx("linear_prequantized/p_bias"), "stored bias")
+    with torch.no_grad():
+        assert_bits_equal(m(x.to(torch.bfloat16)), fx("linear_prequantized/out_bf16"), "bf16 input")
+        assert_bits_equal(m(x), fx("linear_prequantized/out_f32"), "fp32 input")
+    assert m.packed_weight_bytes() == 0
+    m.train()
+    with pytest.raises(AssertionError, match="prequantized weights when training"):
+        m(x)
+    # a layer without MX specs has nothing to prequantize
+    plain = Linear(64, 48, mx_specs=None)
+    plain.prequantize_weights()
+    assert plain.weight.dtype == torch.float32 and not plain.prequantized_weights
+    # the reference's preconditions
+    with pytest.raises(AssertionError, match="'even'"):
+        Linear(64, 48, mx_specs=_specs(w_elem_format="fp8_e4m3", a_elem_format="fp8_e4m3", block_size=32,
+                                       bfloat=16, round="nearest")).prequantize_weights()
+
+
 @pytest.mark.parametrize("block", [64, 0])
 def test_linear_blocks_that_do_not_divide_the_example_axis(block):
     """3-D input (3, 96, 64) with block size 64 or "whole axis": the weight gradient's exponents
@@ -103,6 +135,29 @@ def test_bmm_oracle_and_cpu_layer(dt):
     assert_bits_equal(o.detach(), fx(key + "out"), "layer forward")
     assert_bits_equal(ai.grad, fx(key + "g1"), "layer grad_in1")
     assert_bits_equal(bi.grad, fx(key + "g2"), "layer grad_in2")
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_attention_scores_oracle_and_cpu_layer(dt):
+    """softmax(bmm(a, b)) over the last axis (mx/bmm.py:132-138, mx/softmax.py:91-97): the oracle's chain and
+    mx.bmm_softmax, which on CPU tensors -- and whenever a gradient is wanted -- is the two layers in a row."""
+    a, b, go = (fx("in/" + n).to(DT[dt]) for n in ("x", "a2", "go2"))
+    key = "bmm_softmax/%s/" % dt
+    logits = O.mx_bmm_forward(a, b, "fp6_e2m3", bfloat=16)
+    assert_bits_equal(O.softmax_forward(logits, -1, bfloat=16), fx(key + "out"), "oracle forward")
+
+    from microxcaling_amd.bmm import bmm_softmax
+    specs = _specs(a_elem_format="fp6_e2m3", block_size=32, bfloat=16, quantize_backprop=True)
+    ai, bi = a.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    o = bmm_softmax(ai, bi, mx_specs=specs)
+    o.backward(go)
+    assert_bits_equal(o.detach(), fx(key + "out"), "layer forward")
+    assert_bits_equal(ai.grad, fx(key + "g1"), "layer grad_in1")
+    assert_bits_equal(bi.grad, fx(key + "g2"), "layer grad_in2")
+    with torch.no_grad():
+        assert_bits_equal(bmm_softmax(a, b, mx_specs=specs), fx(key + "out"), "layer forward, no gradient")
+        plain = bmm_softmax(a, b, mx_specs=None)
+    assert torch.equal(plain, torch.softmax(torch.bmm(a, b), dim=-1))
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
