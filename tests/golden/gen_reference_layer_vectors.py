@@ -201,6 +201,53 @@ def main(ref_root):
         store(d, key + "g1", ai.grad)
         store(d, key + "g2", bi2.grad)
 
+    # mx.matmul (mx/matmul.py): 2-D x 2-D with a bias and the second operand in the weight format,
+    # batched x batched, and a batched first operand against a 2-D second one (broadcast)
+    from mx.matmul import matmul
+    mspecs = finalize_mx_specs(dict(w_elem_format="fp4_e2m1", a_elem_format="fp8_e4m3", block_size=32, bfloat=16,
+                                    quantize_backprop=True, custom_cuda=False))
+    wt = w.t().contiguous()
+    mcases = {"2d_aw_bias": (x[0], wt, b, "aw", go[0]), "3d_aa": (x, a2, None, "aa", go2),
+              "bcast_aw": (x, wt, None, "aw", go), "2d_wa": (w, x[1].t().contiguous(), None, "wa", go[1].t().contiguous())}
+    for cname, (m1, m2, mb, mode, mgo) in mcases.items():
+        for dt_name, dt in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+            i1, i2 = m1.to(dt).clone().requires_grad_(True), m2.to(dt).clone().requires_grad_(True)
+            ib = None if mb is None else mb.to(dt).clone().requires_grad_(True)
+            out = matmul(i1, i2, bias=ib, mx_specs=mspecs, mode_config=mode)
+            out.backward(mgo.to(dt))
+            key = "matmul/%s/%s/" % (cname, dt_name)
+            store(d, key + "out", out)
+            store(d, key + "g1", i1.grad)
+            store(d, key + "g2", i2.grad)
+            if ib is not None:
+                store(d, key + "gb", ib.grad)
+
+    # the vector ops (mx/vector_ops.py:38-128) on their own: bfloat16, fp16 format, the exp2 / reciprocal
+    # variants, and no format at all; fp32 and bf16 tensors
+    from mx import vector_ops as V
+    va = nx[0]
+    vb = ngo[0] + 0.25
+    vspecs = {"bfloat16": dict(bfloat=16), "fp16": dict(fp=16), "exp2_recip": dict(bfloat=16, vec_use_exp2=True,
+              vec_use_recip=True), "floor": dict(bfloat=16, round="floor"), "none": dict()}
+    for vname, kw in vspecs.items():
+        sp = finalize_mx_specs(dict(custom_cuda=False, **kw), early_exit=False)
+        for dt_name, dt in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+            a_, b_ = va.to(dt), vb.to(dt)
+            key = "vec/%s/%s/" % (vname, dt_name)
+            store(d, key + "quantize", V.vec_quantize(a_, mx_specs=sp))
+            store(d, key + "add", V.vec_add(a_, b_, mx_specs=sp))
+            store(d, key + "sub", V.vec_sub(a_, b_, mx_specs=sp))
+            store(d, key + "mul", V.vec_mul(a_, b_, mx_specs=sp))
+            store(d, key + "div", V.vec_div(a_, b_, mx_specs=sp))
+            store(d, key + "exp", V.vec_exp(a_, mx_specs=sp))
+            store(d, key + "exp2", V.vec_exp2(a_, mx_specs=sp))
+            store(d, key + "recip", V.vec_recip(b_, mx_specs=sp))
+            store(d, key + "sqrt", V.vec_sqrt(a_.abs(), mx_specs=sp))
+            store(d, key + "tanh", V.vec_tanh(a_, mx_specs=sp))
+            store(d, key + "reduce_sum", V.vec_reduce_sum(a_, 1, keepdim=True, mx_specs=sp))
+            if not kw.get("vec_use_recip"):       # the reference hands a numpy scalar to the quantizer there
+                store(d, key + "reduce_mean", V.vec_reduce_mean(a_, [0, 1], mx_specs=sp))
+
     np.savez_compressed(os.path.join(HERE, "reference_layer_vectors.npz"), **d)
     print("wrote %d arrays, torch %s" % (len(d), torch.__version__))
 

@@ -113,3 +113,56 @@ def test_fp16_tensors_are_refused_unless_exact_exponents_are_asked_for():
             assert_bits_equal(y, wide.half(), "elementwise " + rnd)
     finally:
         ce.set_exponent_mode("torch")
+
+
+def test_specs_module_against_the_reference_fixture():
+    """Defaults, finalize_mx_specs (dependent entries, early exit), get_backwards_mx_specs, apply_mx_specs and
+    add_mx_args + get_mx_specs return what the reference's mx/specs.py returned for the same dictionaries and
+    command lines (tests/golden/gen_reference_specs.py wrote them down)."""
+    import argparse
+    import json
+    import os
+    from helpers import ROOT_DIR
+    from microxcaling_amd import specs as S
+    ref = json.load(open(os.path.join(ROOT_DIR, "tests", "golden", "reference_specs.json")))
+    plain = lambda d: None if d is None else {k: d[k] for k in sorted(d.keys())}
+    assert plain(S.get_default_mx_specs()) == ref["defaults"]
+    for case in ref["finalize"]:
+        assert plain(S.finalize_mx_specs(dict(case["in"]))) == case["out"], case["in"]
+    for case, back, app in zip(ref["finalize_no_early_exit"], ref["backwards"], ref["apply"]):
+        f = S.finalize_mx_specs(dict(case["in"]), early_exit=False)
+        assert plain(f) == case["out"], case["in"]
+        assert plain(S.get_backwards_mx_specs(f)) == back["out"], case["in"]
+        assert plain(S.apply_mx_specs(dict(app["in"]))) == app["out"], app["in"]
+    parser = S.add_mx_args(argparse.ArgumentParser())
+    assert {k: v for k, v in sorted(vars(parser.parse_args([])).items())} == ref["argparse_defaults"]
+    for case in ref["command_lines"]:
+        args = S.add_mx_args(argparse.ArgumentParser()).parse_args(case["in"])
+        assert plain(S.get_mx_specs(args)) == case["out"], case["in"]
+    with pytest.raises(KeyError, match="Unknown key"):
+        S.apply_mx_specs({"no_such_spec": 1})
+
+
+def test_formats_module_against_the_reference_fixture():
+    """mx/formats.py: _get_format_params for every member of ElemFormat (by name and through the enum), the
+    enums' members and values, _get_min_norm / _get_max_norm."""
+    import json
+    import os
+    from helpers import ROOT_DIR
+    from microxcaling_amd import formats as F
+    ref = json.load(open(os.path.join(ROOT_DIR, "tests", "golden", "reference_specs.json")))
+    assert sorted(F.ElemFormat.__members__) == sorted(ref["formats"])
+    for n, want in ref["formats"].items():
+        assert list(F._get_format_params(n)) == want, n
+        assert list(F._get_format_params(F.ElemFormat[n])) == ref["formats_by_enum"][n], n
+        assert F.ElemFormat[n].value == ref["elem_format_values"][n]
+        assert F.ElemFormat.from_str(n.upper()) is F.ElemFormat[n]
+    assert {n: int(F.RoundingMode[n]) for n in F.RoundingMode.__members__} == ref["rounding_modes"]
+    assert list(F.RoundingMode.string_enums()) == ref["rounding_mode_strings"]
+    for e, want in ref["min_norm"].items():
+        assert F._get_min_norm(int(e)) == want
+    for em, want in ref["max_norm"].items():
+        e, m = (int(v) for v in em.split(","))
+        assert F._get_max_norm(e, m) == want
+    with pytest.raises(Exception, match="Undefined elem format"):
+        F.ElemFormat.from_str("fp7")

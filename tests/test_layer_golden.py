@@ -138,6 +138,59 @@ def test_bmm_oracle_and_cpu_layer(dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("case", ["2d_aw_bias", "3d_aa", "bcast_aw", "2d_wa"])
+def test_matmul_cpu_layer(case, dt):
+    """mx.matmul (mx/matmul.py:32-200): 2-D x 2-D with a bias and the second operand in the weight format,
+    batched x batched, a batched first operand against a 2-D second one, and weight x activation."""
+    from microxcaling_amd.matmul import matmul
+    x, w, b, a2, go, go2 = (fx("in/" + n) for n in ("x", "w", "b", "a2", "go", "go2"))
+    wt = w.t().contiguous()
+    m1, m2, mb, mode, mgo = {"2d_aw_bias": (x[0], wt, b, "aw", go[0]), "3d_aa": (x, a2, None, "aa", go2),
+                             "bcast_aw": (x, wt, None, "aw", go),
+                             "2d_wa": (w, x[1].t().contiguous(), None, "wa", go[1].t().contiguous())}[case]
+    specs = _specs(w_elem_format="fp4_e2m1", a_elem_format="fp8_e4m3", block_size=32, bfloat=16,
+                   quantize_backprop=True)
+    i1, i2 = m1.to(DT[dt]).clone().requires_grad_(True), m2.to(DT[dt]).clone().requires_grad_(True)
+    ib = None if mb is None else mb.to(DT[dt]).clone().requires_grad_(True)
+    out = matmul(i1, i2, bias=ib, mx_specs=specs, mode_config=mode)
+    out.backward(mgo.to(DT[dt]))
+    key = "matmul/%s/%s/" % (case, dt)
+    assert_bits_equal(out.detach(), fx(key + "out"), "forward")
+    assert_bits_equal(i1.grad, fx(key + "g1"), "grad_in1")
+    assert_bits_equal(i2.grad, fx(key + "g2"), "grad_in2")
+    if ib is not None:
+        assert_bits_equal(ib.grad, fx(key + "gb"), "grad_bias")
+
+
+VEC_SPECS = {"bfloat16": dict(bfloat=16), "fp16": dict(fp=16),
+             "exp2_recip": dict(bfloat=16, vec_use_exp2=True, vec_use_recip=True),
+             "floor": dict(bfloat=16, round="floor"), "none": dict()}
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("variant", list(VEC_SPECS))
+def test_vector_ops_on_cpu_tensors(variant, dt):
+    """The vec_* ops on their own (mx/vector_ops.py:38-128): a tensor op followed by the elementwise
+    quantizer, in its bfloat16 / fp16 / round-down forms, with the 2^x and reciprocal variants, and
+    with no format at all."""
+    from microxcaling_amd import vector_ops as V
+    from microxcaling_amd.specs import finalize_mx_specs
+    sp = finalize_mx_specs(dict(VEC_SPECS[variant]), early_exit=False)
+    a, b = fx("in/nx")[0].to(DT[dt]), (fx("in/ngo")[0] + 0.25).to(DT[dt])
+    key = "vec/%s/%s/" % (variant, dt)
+    got = {"quantize": V.vec_quantize(a, mx_specs=sp), "add": V.vec_add(a, b, mx_specs=sp),
+           "sub": V.vec_sub(a, b, mx_specs=sp), "mul": V.vec_mul(a, b, mx_specs=sp),
+           "div": V.vec_div(a, b, mx_specs=sp), "exp": V.vec_exp(a, mx_specs=sp),
+           "exp2": V.vec_exp2(a, mx_specs=sp), "recip": V.vec_recip(b, mx_specs=sp),
+           "sqrt": V.vec_sqrt(a.abs(), mx_specs=sp), "tanh": V.vec_tanh(a, mx_specs=sp),
+           "reduce_sum": V.vec_reduce_sum(a, 1, keepdim=True, mx_specs=sp)}
+    if not VEC_SPECS[variant].get("vec_use_recip"):
+        got["reduce_mean"] = V.vec_reduce_mean(a, [0, 1], mx_specs=sp)
+    for name, t in got.items():
+        assert_bits_equal(t, fx(key + name), "vec_" + name)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
 def test_attention_scores_oracle_and_cpu_layer(dt):
     """softmax(bmm(a, b)) over the last axis (mx/bmm.py:132-138, mx/softmax.py:91-97): the oracle's chain and
     mx.bmm_softmax, which on CPU tensors -- and whenever a gradient is wanted -- is the two layers in a row."""
