@@ -248,6 +248,20 @@ def main(ref_root):
             if not kw.get("vec_use_recip"):       # the reference hands a numpy scalar to the quantizer there
                 store(d, key + "reduce_mean", V.vec_reduce_mean(a_, [0, 1], mx_specs=sp))
 
+    # quantize_mx_op with shared_exp_method="none" (an exponent per element, mx/mx_ops.py:49-92 with
+    # method "none"), along the last and along the first axis, with and without blocks
+    from mx.mx_ops import quantize_mx_op
+    qa = nx[0] * torch.exp2(torch.randint(-6, 7, nx[0].shape, generator=g).float())
+    store(d, "in/qa", qa)
+    for fmt in ("fp8_e4m3", "fp6_e2m3", "fp4_e2m1", "int8"):
+        for block in (32, 0):
+            nspecs = finalize_mx_specs(dict(a_elem_format=fmt, w_elem_format=fmt, block_size=block,
+                                            shared_exp_method="none", custom_cuda=False))
+            for dt_name, dt in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+                for ax in (-1, 0):
+                    store(d, "mx_none/%s/block%d/%s/axis%d" % (fmt, block, dt_name, ax),
+                          quantize_mx_op(qa.to(dt), nspecs, elem_format=fmt, axes=[ax], round="nearest"))
+
     np.savez_compressed(os.path.join(HERE, "reference_layer_vectors.npz"), **d)
     print("wrote %d arrays, torch %s" % (len(d), torch.__version__))
 

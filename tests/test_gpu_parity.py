@@ -211,6 +211,29 @@ def test_mx_shapes(dev, shape, axis, bs, dtype):
         assert_bits_equal(got, want, "%s %s %s" % (shape, fmt, rnd))
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("fmt", ["fp8_e4m3", "fp6_e2m3", "fp4_e2m1", "int8"])
+def test_an_exponent_per_element_on_the_gpu(dev, fmt, dt):
+    """shared_exp_method="none" (mx/mx_ops.py:49-92 with method "none") = blocks of one element, against
+    what the reference returned (tests/golden/gen_reference_layer_vectors.py)."""
+    import numpy as np
+    import os
+    from helpers import ROOT_DIR
+    from microxcaling_amd.mx_ops import quantize_mx_op
+    from microxcaling_amd.specs import finalize_mx_specs
+    fix = np.load(os.path.join(ROOT_DIR, "tests", "golden", "reference_layer_vectors.npz"))
+    qa = torch.from_numpy(fix["in/qa:f32"].copy()).view(torch.float32)
+    tdt = torch.float32 if dt == "f32" else torch.bfloat16
+    for block in (32, 0):
+        specs = finalize_mx_specs(dict(a_elem_format=fmt, w_elem_format=fmt, block_size=block,
+                                       shared_exp_method="none"))
+        for ax in (-1, 0):
+            key = "mx_none/%s/block%d/%s/axis%d:%s" % (fmt, block, dt, ax, dt)
+            want = torch.from_numpy(fix[key].copy()).view(tdt)
+            got = quantize_mx_op(qa.to(tdt).to(dev), specs, elem_format=fmt, axes=[ax], round="nearest")
+            assert_bits_equal(got.cpu(), want, key)
+
+
 @pytest.mark.parametrize("shape,axes,bs", [((70, 45), [-2, -1], 32), ((3, 40, 5, 33), [1, 3], 8),
                                            ((6, 10, 12), [0, 1, 2], 4), ((5, 64, 64), [1, 2], 0),
                                            ((4, 7, 9), [2, 0], 32), ((2, 3, 4, 5, 6), [1, 2, 4], 2),

@@ -315,3 +315,17 @@ def test_convolutions_on_cpu():
     _check_module("conv2d_groups/", Conv2d(64, 64, 3, padding=1, groups=2, bias=False, mx_specs=s), cx,
                   fx("in/cgo2"))
     _check_module("conv1d/", Conv1d(32, 40, 5, padding=2, mx_specs=s), fx("in/c1"), fx("in/c1go"))
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("block", [32, 0])
+@pytest.mark.parametrize("fmt", ["fp8_e4m3", "fp6_e2m3", "fp4_e2m1", "int8"])
+def test_an_exponent_per_element(fmt, block, dt):
+    """quantize_mx_op with shared_exp_method="none" (mx/mx_ops.py:49-92 with method "none"): every element
+    takes its own exponent, whatever the block size and the axis."""
+    from microxcaling_amd.mx_ops import quantize_mx_op
+    specs = _specs(a_elem_format=fmt, w_elem_format=fmt, block_size=block, shared_exp_method="none")
+    qa = fx("in/qa").to(DT[dt])
+    for ax in (-1, 0):
+        got = quantize_mx_op(qa, specs, elem_format=fmt, axes=[ax], round="nearest")
+        assert_bits_equal(got, fx("mx_none/%s/block%d/%s/axis%d" % (fmt, block, dt, ax)), "axis %d" % ax)
