@@ -166,3 +166,67 @@ def test_formats_module_against_the_reference_fixture():
         assert F._get_max_norm(e, m) == want
     with pytest.raises(Exception, match="Undefined elem format"):
         F.ElemFormat.from_str("fp7")
+
+
+def _none_cases():
+    import torch.nn as nn
+    import torch.nn.functional as F
+    import microxcaling_amd as mx
+    return [
+        ("sigmoid", torch.sigmoid, mx.sigmoid, {}), ("tanh", torch.tanh, mx.tanh, {}), ("relu", F.relu, mx.relu, {}),
+        ("relu6", F.relu6, mx.relu6, {}), ("leaky_relu", F.leaky_relu, mx.leaky_relu, {"negative_slope": 0.4}),
+        ("silu", F.silu, mx.silu, {}), ("softmax", F.softmax, mx.softmax, {"dim": -1}),
+        ("Sigmoid", nn.Sigmoid, mx.Sigmoid, {}), ("Tanh", nn.Tanh, mx.Tanh, {}), ("ReLU", nn.ReLU, mx.ReLU, {}),
+        ("ReLU6", nn.ReLU6, mx.ReLU6, {}), ("SiLU", nn.SiLU, mx.SiLU, {}), ("Softmax", nn.Softmax, mx.Softmax, {"dim": -1}),
+    ]
+
+
+@pytest.mark.parametrize("case", range(13))
+def test_without_specs_every_layer_is_the_torch_layer(case):
+    """mx_specs=None: outputs and input gradients equal torch's own, bit for bit (the reference's
+    mx/tests/test_mxfp_none.py:30-141, for the functions and modules this package carries)."""
+    import torch.nn as nn
+    name, f1, f2, kwargs = _none_cases()[case]
+    g = torch.Generator().manual_seed(0xBEEF + case)
+    x = torch.randn(4, 16, generator=g)
+    x1, x2 = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    if isinstance(f1, type) and issubclass(f1, nn.Module):
+        q1, q2 = f1(**kwargs)(x1), f2(mx_specs=None, **kwargs)(x2)
+    else:
+        q1, q2 = f1(x1, **kwargs), f2(x2, mx_specs=None, **kwargs)
+    (q1 ** 2).mean().sqrt().backward()
+    (q2 ** 2).mean().sqrt().backward()
+    assert torch.equal(q1, q2), name
+    assert torch.equal(x1.grad, x2.grad), name
+
+
+def test_without_specs_the_matmul_layers_are_torch_layers():
+    """The same for linear / Linear, matmul (with and without bias), bmm, layer_norm / LayerNorm and the
+    convolutions."""
+    import torch.nn as nn
+    import torch.nn.functional as F
+    import microxcaling_amd as mx
+    g = torch.Generator().manual_seed(0xABCD)
+    x, w, b = torch.randn(3, 8, 16, generator=g), torch.randn(12, 16, generator=g), torch.randn(12, generator=g)
+    assert torch.equal(mx.linear(x, w, b, mx_specs=None), F.linear(x, w, b))
+    assert torch.equal(mx.matmul(x, w.t(), mx_specs=None), torch.matmul(x, w.t()))
+    assert torch.equal(mx.matmul(x[0], w.t(), bias=b, mx_specs=None), torch.addmm(b, x[0], w.t()))
+    y = torch.randn(3, 16, 5, generator=g)
+    assert torch.equal(mx.bmm(x, y, mx_specs=None), torch.bmm(x, y))
+    torch.manual_seed(3)
+    l1 = nn.Linear(16, 12)
+    torch.manual_seed(3)
+    l2 = mx.Linear(16, 12, mx_specs=None)
+    assert torch.equal(l1(x), l2(x))
+    lw, lb = torch.randn(16, generator=g), torch.randn(16, generator=g)
+    assert torch.equal(mx.layer_norm(x, (16,), lw, lb, 1e-5, mx_specs=None), F.layer_norm(x, (16,), lw, lb, 1e-5))
+    n1, n2 = nn.LayerNorm(16, eps=1e-12), mx.LayerNorm(16, mx_specs=None)    # the reference's default eps
+    assert n2.eps == 1e-12
+    assert torch.equal(n1(x), n2(x))
+    cx, cw = torch.randn(2, 4, 9, 9, generator=g), torch.randn(6, 4, 3, 3, generator=g)
+    assert torch.equal(mx.conv2d(cx, cw, None, 1, 1, 1, 1, mx_specs=None), F.conv2d(cx, cw, None, 1, 1, 1, 1))
+    torch.manual_seed(5)
+    c1 = nn.Conv2d(4, 6, 3, padding=1)
+    torch.manual_seed(5)
+    c2 = mx.Conv2d(4, 6, 3, padding=1, mx_specs=None)
+    assert torch.equal(c1(cx), c2(cx))
