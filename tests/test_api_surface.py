@@ -230,3 +230,20 @@ def test_without_specs_the_matmul_layers_are_torch_layers():
     torch.manual_seed(5)
     c2 = mx.Conv2d(4, 6, 3, padding=1, mx_specs=None)
     assert torch.equal(c1(cx), c2(cx))
+
+
+def test_bench_refuses_more_than_one_gpu_and_needs_one():
+    """bench.py measures one GPU: --gpus above 1 exits with a message that says so; without a GPU the default
+    run fails loudly instead of timing anything on the CPU."""
+    import os
+    import subprocess
+    import sys
+    from helpers import ROOT_DIR
+    bench = os.path.join(ROOT_DIR, "bench.py")
+    res = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0 and "one GPU" in (res.stdout + res.stderr)
+    if not torch.cuda.is_available():
+        res = subprocess.run([sys.executable, bench, "--steps", "1", "--warmup", "0", "--no-cpu-baseline"],
+                             capture_output=True, text=True, timeout=300)
+        assert res.returncode != 0
+        assert '"metric"' not in res.stdout
