@@ -17,12 +17,15 @@
  * mxq_reduce_outer_static), so calls may come from several host threads.
  *
  * Numerics: results are bit-identical to the reference's pure-PyTorch CPU path
- * (custom_cuda=False) for fp32 and bf16 tensors, including its floor(log2(x)) rounding just
- * below powers of two; MXQ_FLAG_EXACT_EXPONENT switches to bit-field exponents, which is what the
- * reference's own CUDA kernels compute (mx/cpp/common.cuh:146-154).  fp16 tensors are accepted
- * under that flag only: they are widened to fp32, quantized and rounded back to fp16 like the
- * reference's CUDA kernels do (mx/cpp/mx.cuh:72,88), which is not what its pure-PyTorch path gives
- * (every op evaluated in fp16); without the flag MXQ_DTYPE_F16 is refused with MXQ_ERR_ARGUMENT.
+ * (custom_cuda=False) for fp32, bf16 and fp16 tensors, including its floor(log2(x)) rounding just
+ * below powers of two and, for the 16-bit dtypes, the rounding to the tensor dtype after every op
+ * (fp16: 2**shared_exp overflows from 2^16 and underflows below 2^-24, which turns such blocks --
+ * all-zero blocks at scale_bits 8 among them -- into NaN, as it does there; a clamp bound beyond the
+ * fp16 range is MXQ_ERR_ARGUMENT, where the reference's torch.clamp raises).
+ * MXQ_FLAG_EXACT_EXPONENT switches to bit-field exponents, which is what the reference's own CUDA
+ * kernels compute (mx/cpp/common.cuh:146-154); fp16 tensors are then widened to fp32, quantized and
+ * rounded back to fp16 once, as those kernels do (mx/cpp/mx.cuh:72,88).  The packing entry points
+ * take fp16 tensors under that flag only.
  */
 #ifndef MXQ_H
 #define MXQ_H

@@ -210,11 +210,11 @@ int mxq_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre, i
     if (post == 1 && ptr_ok && axis_size % tile == 0 && tile % vec_elems == 0) {
         const int64_t lpt = tile / vec_elems;
         if (lpt == 1 || lpt == 2 || lpt == 4 || lpt == 8 || lpt == 16) {
-            dispatch<LaunchLastAxis>(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, total / vec_elems, (int)lpt, p, s);
+            dispatch_any<LaunchLastAxis>(dtype, flags, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, total / vec_elems, (int)lpt, p, s);
             return check_launch(who);
         }
     }
-    dispatch<LaunchStrided>(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, pre, axis_size, post, tile, ptr_ok, p, s);
+    dispatch_any<LaunchStrided>(dtype, flags, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, pre, axis_size, post, tile, ptr_ok, p, s);
     return check_launch(who);
 }
 
@@ -234,7 +234,7 @@ int mxq_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, const
     if (rc) return rc;
     if (total == 0) return MXQ_OK;
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
-    dispatch<LaunchAxes>(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, a, mxq_axes_tiles(a), p,
+    dispatch_any<LaunchAxes>(dtype, flags, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, a, mxq_axes_tiles(a), p,
                          (hipStream_t)hip_stream);
     return check_launch(who);
 }
@@ -262,6 +262,8 @@ int mxq_quantize_mx_dither_by_tile(const void* in, const void* noise, void* out,
         mx_dither_kernel<MXQ_F32><<<grid, kThreads, 0, s>>>(in, noise, out, pre, axis_size, post, tile, num_tiles, p);
     else if (dtype == MXQ_DTYPE_BF16)
         mx_dither_kernel<MXQ_BF16><<<grid, kThreads, 0, s>>>(in, noise, out, pre, axis_size, post, tile, num_tiles, p);
+    else if (f16_ops(dtype, flags))
+        mx_dither_kernel<MXQ_F16OPS><<<grid, kThreads, 0, s>>>(in, noise, out, pre, axis_size, post, tile, num_tiles, p);
     else
         mx_dither_kernel<MXQ_F16><<<grid, kThreads, 0, s>>>(in, noise, out, pre, axis_size, post, tile, num_tiles, p);
     return check_launch(who);
@@ -282,6 +284,7 @@ int mxq_quantize_elemwise_dither(const void* in, const void* noise, void* out, i
     const int grid = grid_for(ceil_div(n, kThreads));
     if (dtype == MXQ_DTYPE_F32) elemwise_dither_kernel<MXQ_F32><<<grid, kThreads, 0, s>>>(in, noise, out, n, p);
     else if (dtype == MXQ_DTYPE_BF16) elemwise_dither_kernel<MXQ_BF16><<<grid, kThreads, 0, s>>>(in, noise, out, n, p);
+    else if (f16_ops(dtype, flags)) elemwise_dither_kernel<MXQ_F16OPS><<<grid, kThreads, 0, s>>>(in, noise, out, n, p);
     else elemwise_dither_kernel<MXQ_F16><<<grid, kThreads, 0, s>>>(in, noise, out, n, p);
     return check_launch(who);
 }
@@ -301,7 +304,7 @@ int mxq_quantize_mx_given_max(const void* in, void* out, const void* max_values,
     if (mul_overflows(pre, axis_size, post, &total)) return fail(MXQ_ERR_ARGUMENT, "%s: size overflows int64", who);
     if (total == 0) return MXQ_OK;
     if (!in || !out || !max_values) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
-    dispatch<LaunchGivenMax>(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, max_values, total, axis_size, post, p,
+    dispatch_any<LaunchGivenMax>(dtype, flags, rmode, ze, lean_ok(dtype, p.fmt, rmode, false), in, out, max_values, total, axis_size, post, p,
                              (hipStream_t)hip_stream);
     return check_launch(who);
 }
@@ -327,7 +330,7 @@ int mxq_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, int b
         elemwise_bf16_closed_kernel<kElemUnroll><<<grid, kThreads, 0, (hipStream_t)hip_stream>>>(in, out, n, p.fmt.nan_from);
         return check_launch(who);
     }
-    dispatch<LaunchElemwise>(dtype, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode), lean_ok(dtype, p.fmt, rmode, true), in, out, n, p, (hipStream_t)hip_stream);
+    dispatch_any<LaunchElemwise>(dtype, flags, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode), lean_ok(dtype, p.fmt, rmode, true), in, out, n, p, (hipStream_t)hip_stream);
     return check_launch(who);
 }
 

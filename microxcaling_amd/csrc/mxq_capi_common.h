@@ -61,6 +61,19 @@ void dispatch(int dtype, int rmode, bool zone_elem, bool lean, A... a) {
     else dispatch_round<F, MXQ_F16>(rmode, zone_elem, lean, a...);
 }
 
+// The same, for the entry points that also serve fp16 tensors op by op in fp16 (f16_ops): that
+// arithmetic exists in the op-by-op form only.
+template <template <int, int, bool, bool> class F, typename... A>
+void dispatch_any(int dtype, int flags, int rmode, bool zone_elem, bool lean, A... a) {
+    if (f16_ops(dtype, flags)) {
+        if (rmode == MXQ_ROUND_FLOOR) F<MXQ_F16OPS, MXQ_FLOOR, true, false>::run(a...);
+        else if (rmode == MXQ_ROUND_NEAREST) F<MXQ_F16OPS, MXQ_NEAREST, true, false>::run(a...);
+        else F<MXQ_F16OPS, MXQ_EVEN, true, false>::run(a...);
+        return;
+    }
+    dispatch<F>(dtype, rmode, zone_elem, lean, a...);
+}
+
 constexpr int kLastAxisUnroll = 4;
 
 

@@ -200,6 +200,9 @@ int mxq_pack_mx(const void* in, void* codes, void* scales, int dtype, int64_t ro
     const char* who = "mxq_pack_mx";
     MxParams p;
     bool ze;
+    if (f16_ops(dtype, flags))
+        return fail(MXQ_ERR_ARGUMENT, "%s: fp16 tensors have a packed form under MXQ_FLAG_EXACT_EXPONENT only "
+                    "(the op-by-op fp16 arithmetic of the default mode has no packing kernel)", who);
     int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
                             flush_fp32_subnorms, rmode, flags, &p, &ze, who);
     if (rc) return rc;
@@ -232,6 +235,9 @@ int mxq_pack_mx_t(const void* in, void* codes, void* scales, int dtype, int64_t 
     const char* who = "mxq_pack_mx_t";
     MxParams p;
     bool ze;
+    if (f16_ops(dtype, flags))
+        return fail(MXQ_ERR_ARGUMENT, "%s: fp16 tensors have a packed form under MXQ_FLAG_EXACT_EXPONENT only "
+                    "(the op-by-op fp16 arithmetic of the default mode has no packing kernel)", who);
     int rc = make_mx_params(dtype, scale_bits, elem_ebits, elem_mbits, elem_max_norm,
                             flush_fp32_subnorms, rmode, flags, &p, &ze, who);
     if (rc) return rc;

@@ -21,6 +21,10 @@
 #endif
 
 enum MxqDtype { MXQ_F32 = 0, MXQ_F16 = 1, MXQ_BF16 = 2 };
+// Not a tensor dtype of the C ABI: an fp16 tensor whose every op is rounded to fp16, the way torch's
+// CPU kernels evaluate the reference's pure path on such a tensor (compute in fp32, round to fp16).
+// MXQ_F16 as a template argument means "fp16 tensor, fp32 arithmetic" (the reference's CUDA kernels).
+#define MXQ_F16OPS 3
 enum MxqRound { MXQ_NEAREST = 0, MXQ_FLOOR = 1, MXQ_EVEN = 2 };   // mx/formats.py:12-19
 // round='dither' (mx/elemwise_ops.py:57-59) is not in that enum: floor(s + u) with u in [0, 1) drawn
 // by the caller, one per element.  Only the op-by-op form of the rounding knows it.
@@ -47,11 +51,49 @@ MXQ_HD float mxq_round_bf16(float f) {
 #endif
 }
 
+// fp32 -> fp16 bits, round to nearest even, subnormals kept, overflow to Inf (v_cvt_f16_f32 on
+// gfx950; the kernels run with fp16 denormals enabled), and back.
+#if defined(__clang__)
+// On the device the value passes through an empty asm statement first: left alone, the compiler
+// fuses a preceding multiplication into v_fma_mixlo_f16 a, b, +0, and (-0) + (+0) = +0 loses the
+// sign of a zero product.
+MXQ_HD unsigned short mxq_f16_bits(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm("" : "+v"(f));
+#endif
+    return __builtin_bit_cast(unsigned short, (_Float16)f);
+}
+MXQ_HD float mxq_f16_value(unsigned short h) { return (float)__builtin_bit_cast(_Float16, h); }
+#else
+// a host compiler without _Float16 (g++ 11 on x86): the same conversions in integer arithmetic
+MXQ_HD unsigned short mxq_f16_bits(float f) {
+    const uint32_t u = mxq_bits(f), sign = (u >> 16) & 0x8000u;
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > MXQ_INF_BITS) return (unsigned short)(sign | 0x7E00u);
+    if (a >= 0x477FF000u) return (unsigned short)(sign | 0x7C00u);       // 65520 and up round to Inf
+    if (a < 0x38800000u)                                                 // below 2^-14: units of 2^-24,
+        return (unsigned short)(sign | (mxq_bits(mxq_float(a) + 0.5f) - 0x3F000000u));   // the ulp of [0.5, 1)
+    a += 0xFFFu + ((a >> 13) & 1u);
+    return (unsigned short)(sign | ((a - 0x38000000u) >> 13));
+}
+MXQ_HD float mxq_f16_value(unsigned short h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 31u, m = h & 1023u;
+    if (e == 0u) return mxq_float(sign | mxq_bits(ldexpf((float)m, -24)));
+    if (e == 31u) return mxq_float(sign | MXQ_INF_BITS | (m << 13));
+    return mxq_float(sign | ((e + 112u) << 23) | (m << 13));
+}
+#endif
+MXQ_HD float mxq_round_f16(float f) { return mxq_f16_value(mxq_f16_bits(f)); }
+
 template <int DT>
 MXQ_HD float mxq_round_dt(float f) {
     if (DT == MXQ_BF16) return mxq_round_bf16(f);
+    if (DT == MXQ_F16OPS) return mxq_round_f16(f);
     return f;
 }
+
+// Shift of the round-up-zone counts for the arithmetic dtype (units of the 24-bit significand).
+template <int DT> struct MxqZoneShift { static constexpr int value = DT == MXQ_BF16 ? 16 : DT == MXQ_F16OPS ? 13 : 0; };
 
 // ---- exponent shared over the blocks of several axes ----------------------------------------------
 // A contiguous tensor seen as (o[0], s[0], o[1], s[1], o[2], s[2], o[3]): up to three shared axes s
@@ -145,6 +187,37 @@ MXQ_HD MxqScale mxq_block_scale(uint32_t um, int emax, int scale_emax, bool flus
     return r;
 }
 
+// The same for an fp16 tensor evaluated op by op in fp16.  What differs from the wide dtypes:
+//  * FP32_MIN_NORMAL * (max == 0) is 0 in fp16, so an all-zero block has log2(0) = -inf and its scale
+//    exponent is the lower clamp -scale_emax;
+//  * 2**se is an fp16 number: Inf from se = 16 and 0 up to se = -25 (2^-25 ties to even).  Either
+//    turns the whole block into NaN (x / Inf = 0 and 0 * Inf = NaN; x / 0 = Inf or NaN, the element
+//    rounding returns Inf for Inf, and Inf * 0 = NaN);
+//  * a nonzero fp16 maximum is at least 2^-24, so flush_fp32_subnorms only meets all-zero blocks,
+//    whose elements are zeros before and after.
+// um: max |x| widened to fp32 (never an fp32 subnormal).
+MXQ_HD MxqScale mxq_block_scale_f16ops(uint32_t um, int emax, int scale_emax, const unsigned char* zone) {
+    const uint32_t eb = um >> 23;
+    const uint32_t gap = 0x800000u - (um & 0x7FFFFFu);
+    const int E = (um == 0u) ? -100000 : (int)eb - 127 + (gap <= ((uint32_t)zone[eb + 22] << 13) ? 1 : 0);
+    int se = E - emax;
+    bool nan = um >= MXQ_INF_BITS || se > scale_emax;
+    se = se < -scale_emax ? -scale_emax : se;
+    nan = nan || se >= 16 || se <= -25;
+    se = se < -25 ? -25 : (se > 16 ? 16 : se);
+    MxqScale r;
+    r.scale = nan ? mxq_float(MXQ_QNAN_BITS) : ldexpf(1.0f, se);
+    r.inv_scale = ldexpf(1.0f, -se);
+    return r;
+}
+
+template <int DT>
+MXQ_HD MxqScale mxq_block_scale_dt(uint32_t um, int emax, int scale_emax, bool flush_subnorms,
+                                   const unsigned char* zone) {
+    if (DT == MXQ_F16OPS) return mxq_block_scale_f16ops(um, emax, scale_emax, zone);
+    return mxq_block_scale(um, emax, scale_emax, flush_subnorms, zone, MxqZoneShift<DT>::value);
+}
+
 // ---- element rounding, lean form ----------------------------------------------------------------
 // a: input in the tensor dtype, already divided by the block scale.  Valid for fp32 tensors with
 // any t <= 22 and for bf16 tensors with t <= 6: there the only place where the dtype rounding of
@@ -216,7 +289,8 @@ MXQ_HD float mxq_round_every_op(float a, const MxqFmt& f, bool saturate, const u
             k += (gap <= ((uint32_t)zone[k + 149] << zshift)) ? 1 : 0;
         }
         e = k > f.min_exp ? k : f.min_exp;
-        if (e >= 128) return mxq_float(MXQ_QNAN_BITS);    // 2**128 = inf -> 0 * inf
+        // 2**e = inf (fp16: from 2^16) -> x / inf = 0 and 0 * inf
+        if (e >= (DT == MXQ_F16OPS ? 16 : 128)) return mxq_float(MXQ_QNAN_BITS);
     }
     float s = mxq_round_dt<DT>(ldexpf(mxq_float(ua), -e));  // out / 2**e
     s = mxq_round_dt<DT>(ldexpf(s, f.t));                   // * 2**(bits-2)

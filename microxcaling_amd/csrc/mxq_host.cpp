@@ -15,7 +15,7 @@ namespace {
 
 using namespace mxq_detail;
 
-const unsigned char kZone[3][MXQ_ZONE_PAD] = {{MXQ_ZONE_ROW_F32}, {MXQ_ZONE_ROW_BF16}, {0}};
+const unsigned char kZone[4][MXQ_ZONE_PAD] = {{MXQ_ZONE_ROW_F32}, {MXQ_ZONE_ROW_BF16}, {0}, {MXQ_ZONE_ROW_F16}};
 
 float load_as_float(const void* p, int dtype, int64_t i) {
     if (dtype == MXQ_DTYPE_F32) return reinterpret_cast<const float*>(p)[i];
@@ -46,7 +46,8 @@ MxElemFn pick_mx(int rmode, bool ze) {
     return ze ? mxq_quant_mx_elem<MXQ_EVEN, DT, true, LEAN> : mxq_quant_mx_elem<MXQ_EVEN, DT, false, LEAN>;
 }
 // lean = false selects the op-by-op form, which always consults the zone table
-MxElemFn pick_mx(int dtype, int rmode, bool ze, bool lean) {
+MxElemFn pick_mx(int dtype, int flags, int rmode, bool ze, bool lean) {
+    if (f16_ops(dtype, flags)) return pick_mx<MXQ_F16OPS, false>(rmode, true);
     if (dtype == MXQ_DTYPE_BF16) return lean ? pick_mx<MXQ_BF16, true>(rmode, ze) : pick_mx<MXQ_BF16, false>(rmode, true);
     return lean ? pick_mx<MXQ_F32, true>(rmode, ze) : pick_mx<MXQ_F32, false>(rmode, true);
 }
@@ -56,9 +57,15 @@ ElemFn pick_elem(int rmode, bool ze) {
     if (rmode == MXQ_ROUND_NEAREST) return ze ? mxq_quant_elemwise<MXQ_NEAREST, DT, true, LEAN> : mxq_quant_elemwise<MXQ_NEAREST, DT, false, LEAN>;
     return ze ? mxq_quant_elemwise<MXQ_EVEN, DT, true, LEAN> : mxq_quant_elemwise<MXQ_EVEN, DT, false, LEAN>;
 }
-ElemFn pick_elem(int dtype, int rmode, bool ze, bool lean) {
+ElemFn pick_elem(int dtype, int flags, int rmode, bool ze, bool lean) {
+    if (f16_ops(dtype, flags)) return pick_elem<MXQ_F16OPS, false>(rmode, true);
     if (dtype == MXQ_DTYPE_BF16) return lean ? pick_elem<MXQ_BF16, true>(rmode, ze) : pick_elem<MXQ_BF16, false>(rmode, true);
     return lean ? pick_elem<MXQ_F32, true>(rmode, ze) : pick_elem<MXQ_F32, false>(rmode, true);
+}
+
+MxqScale block_scale(int dtype, int flags, uint32_t um, const MxParams& p, const unsigned char* zone) {
+    if (f16_ops(dtype, flags)) return mxq_block_scale_f16ops(um, p.emax, p.scale_emax, zone);
+    return mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
 }
 
 }  // namespace
@@ -85,7 +92,7 @@ int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t p
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const int64_t tile = (tile_size <= 0 || tile_size > axis_size) ? axis_size : tile_size;
     const unsigned char* zone = kZone[p.zone_row];
-    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
+    MxElemFn fn = pick_mx(dtype, flags, rmode, ze, lean_ok(dtype, p.fmt, rmode, false) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < pre; ++i)
         for (int64_t k0 = 0; k0 < axis_size; k0 += tile)
             for (int64_t j = 0; j < post; ++j) {
@@ -93,7 +100,7 @@ int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t p
                 uint32_t um = 0;
                 for (int64_t k = k0; k < k1; ++k)
                     um = std::max(um, mxq_bits(load_as_float(in, dtype, (i * axis_size + k) * post + j)) & 0x7FFFFFFFu);
-                MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+                MxqScale sc = block_scale(dtype, flags, um, p, zone);
                 for (int64_t k = k0; k < k1; ++k) {
                     const int64_t idx = (i * axis_size + k) * post + j;
                     store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift, 0.0f));
@@ -118,7 +125,7 @@ int mxq_host_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, 
     if (total == 0) return MXQ_OK;
     if (!in || !out) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const unsigned char* zone = kZone[p.zone_row];
-    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
+    MxElemFn fn = pick_mx(dtype, flags, rmode, ze, lean_ok(dtype, p.fmt, rmode, false) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     const int64_t n_tiles = mxq_axes_tiles(a);
     for (int64_t tile = 0; tile < n_tiles; ++tile) {
         int64_t base, len[3], st[3];
@@ -128,7 +135,7 @@ int mxq_host_quantize_mx_axes(const void* in, void* out, int dtype, int n_axes, 
             for (int64_t j = 0; j < len[1]; ++j)
                 for (int64_t k = 0; k < len[2]; ++k)
                     um = std::max(um, mxq_bits(load_as_float(in, dtype, base + i * st[0] + j * st[1] + k * st[2])) & 0x7FFFFFFFu);
-        MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+        MxqScale sc = block_scale(dtype, flags, um, p, zone);
         for (int64_t i = 0; i < len[0]; ++i)
             for (int64_t j = 0; j < len[1]; ++j)
                 for (int64_t k = 0; k < len[2]; ++k) {
@@ -158,8 +165,9 @@ int mxq_host_quantize_mx_dither_by_tile(const void* in, const void* noise, void*
     if (!in || !out || !noise) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const int64_t tile = (tile_size <= 0 || tile_size > axis_size) ? axis_size : tile_size;
     const unsigned char* zone = kZone[p.zone_row];
-    MxElemFn fn = dtype == MXQ_DTYPE_BF16 ? mxq_quant_mx_elem<MXQ_DITHER, MXQ_BF16, true, false>
-                                          : mxq_quant_mx_elem<MXQ_DITHER, MXQ_F32, true, false>;
+    MxElemFn fn = f16_ops(dtype, flags)     ? mxq_quant_mx_elem<MXQ_DITHER, MXQ_F16OPS, true, false>
+                  : dtype == MXQ_DTYPE_BF16 ? mxq_quant_mx_elem<MXQ_DITHER, MXQ_BF16, true, false>
+                                            : mxq_quant_mx_elem<MXQ_DITHER, MXQ_F32, true, false>;
     for (int64_t i = 0; i < pre; ++i)
         for (int64_t k0 = 0; k0 < axis_size; k0 += tile)
             for (int64_t j = 0; j < post; ++j) {
@@ -167,7 +175,7 @@ int mxq_host_quantize_mx_dither_by_tile(const void* in, const void* noise, void*
                 uint32_t um = 0;
                 for (int64_t k = k0; k < k1; ++k)
                     um = std::max(um, mxq_bits(load_as_float(in, dtype, (i * axis_size + k) * post + j)) & 0x7FFFFFFFu);
-                MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+                MxqScale sc = block_scale(dtype, flags, um, p, zone);
                 for (int64_t k = k0; k < k1; ++k) {
                     const int64_t idx = (i * axis_size + k) * post + j;
                     store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift,
@@ -189,8 +197,9 @@ int mxq_host_quantize_elemwise_dither(const void* in, const void* noise, void* o
     if (n == 0) return MXQ_OK;
     if (!in || !out || !noise) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const unsigned char* zone = kZone[p.zone_row];
-    ElemFn fn = dtype == MXQ_DTYPE_BF16 ? mxq_quant_elemwise<MXQ_DITHER, MXQ_BF16, true, false>
-                                        : mxq_quant_elemwise<MXQ_DITHER, MXQ_F32, true, false>;
+    ElemFn fn = f16_ops(dtype, flags)     ? mxq_quant_elemwise<MXQ_DITHER, MXQ_F16OPS, true, false>
+                : dtype == MXQ_DTYPE_BF16 ? mxq_quant_elemwise<MXQ_DITHER, MXQ_BF16, true, false>
+                                          : mxq_quant_elemwise<MXQ_DITHER, MXQ_F32, true, false>;
     for (int64_t i = 0; i < n; ++i)
         store_from_float(out, dtype, i, fn(load_as_float(in, dtype, i), p.fmt, p.saturate != 0, p.allow_denorm != 0,
                                            zone, p.zshift, load_as_float(noise, dtype, i)));
@@ -213,11 +222,11 @@ int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_va
     if (total == 0) return MXQ_OK;
     if (!in || !out || !max_values) return fail(MXQ_ERR_ARGUMENT, "%s: null pointer", who);
     const unsigned char* zone = kZone[p.zone_row];
-    MxElemFn fn = pick_mx(dtype, rmode, ze, lean_ok(dtype, p.fmt, rmode, false) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
+    MxElemFn fn = pick_mx(dtype, flags, rmode, ze, lean_ok(dtype, p.fmt, rmode, false) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < pre; ++i)
         for (int64_t j = 0; j < post; ++j) {
             const uint32_t um = mxq_bits(load_as_float(max_values, dtype, i * post + j)) & 0x7FFFFFFFu;
-            MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, p.zshift);
+            MxqScale sc = block_scale(dtype, flags, um, p, zone);
             for (int64_t k = 0; k < axis_size; ++k) {
                 const int64_t idx = (i * axis_size + k) * post + j;
                 store_from_float(out, dtype, idx, fn(load_as_float(in, dtype, idx), sc, p.fmt, zone, p.zshift, 0.0f));
@@ -250,7 +259,7 @@ int mxq_host_quantize_elemwise(const void* in, void* out, int dtype, int64_t n, 
         return MXQ_OK;
     }
     const unsigned char* zone = kZone[p.zone_row];
-    ElemFn fn = pick_elem(dtype, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode),
+    ElemFn fn = pick_elem(dtype, flags, rmode, elem_zone_matters(dtype, flags, p.fmt, rmode),
                            lean_ok(dtype, p.fmt, rmode, true) && !(flags & MXQ_HOST_FLAG_ROUND_EVERY_OP));
     for (int64_t i = 0; i < n; ++i)
         store_from_float(out, dtype, i,

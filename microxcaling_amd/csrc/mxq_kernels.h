@@ -13,10 +13,11 @@
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// round-up zone tables in device memory: [0] fp32, [1] bf16, [2] all zero (bit-field exponents)
+// round-up zone tables in device memory: [0] fp32, [1] bf16, [2] all zero (bit-field exponents),
+// [3] fp16
 #define ZONE_PAD MXQ_ZONE_PAD
-__device__ const unsigned char g_zone_tables[3][ZONE_PAD] = {
-    {MXQ_ZONE_ROW_F32}, {MXQ_ZONE_ROW_BF16}, {0}};
+__device__ const unsigned char g_zone_tables[4][ZONE_PAD] = {
+    {MXQ_ZONE_ROW_F32}, {MXQ_ZONE_ROW_BF16}, {0}, {MXQ_ZONE_ROW_F16}};
 
 namespace {
 
@@ -54,14 +55,17 @@ template <> struct Pack<MXQ_F16> {
         return (float)__builtin_bit_cast(_Float16, h);
     }
     static __device__ __forceinline__ uint32_t put(float lo, float hi) {   // RNE, like torch
-        unsigned short l = __builtin_bit_cast(unsigned short, (_Float16)lo);
-        unsigned short h = __builtin_bit_cast(unsigned short, (_Float16)hi);
-        return (uint32_t)l | ((uint32_t)h << 16);
+        return (uint32_t)mxq_f16_bits(lo) | ((uint32_t)mxq_f16_bits(hi) << 16);
     }
 };
 
-// dtype whose op-by-op rounding the arithmetic follows (fp16 tensors are computed as fp32)
-template <int DT> struct Arith { static constexpr int DT_ = (DT == MXQ_BF16) ? MXQ_BF16 : MXQ_F32; };
+template <> struct Pack<MXQ_F16OPS> : Pack<MXQ_F16> {};
+
+// dtype whose op-by-op rounding the arithmetic follows.  MXQ_F16: an fp16 tensor computed as fp32 and
+// rounded once (bit-field exponents); MXQ_F16OPS: an fp16 tensor with every op rounded to fp16.
+template <int DT> struct Arith {
+    static constexpr int DT_ = (DT == MXQ_BF16) ? MXQ_BF16 : (DT == MXQ_F16OPS) ? MXQ_F16OPS : MXQ_F32;
+};
 
 template <int DT>
 __device__ __forceinline__ float load_scalar(const void* p, int64_t i) {
@@ -77,7 +81,7 @@ __device__ __forceinline__ void store_scalar(void* p, int64_t i, float v) {
     } else if (DT == MXQ_BF16) {
         reinterpret_cast<unsigned short*>(p)[i] = (unsigned short)(mxq_bits(v) >> 16);
     } else {
-        reinterpret_cast<unsigned short*>(p)[i] = __builtin_bit_cast(unsigned short, (_Float16)v);
+        reinterpret_cast<unsigned short*>(p)[i] = mxq_f16_bits(v);
     }
 }
 
@@ -126,7 +130,7 @@ __global__ __launch_bounds__(TPB) void mx_lastaxis_kernel(const u32x4* __restric
                                                           u32x4* __restrict__ out, int64_t n_vec,
                                                           MxParams p) {
     constexpr int ADT = Arith<DT>::DT_;
-    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
+    constexpr int ZS = MxqZoneShift<ADT>::value;        // significand units of the zone table
     constexpr int PD = Pack<DT>::PER_DWORD;
     constexpr int64_t CHUNK = (int64_t)TPB * UNROLL;      // vectors per block and iteration
     __shared__ unsigned char zone[ZONE_PAD];
@@ -148,7 +152,7 @@ __global__ __launch_bounds__(TPB) void mx_lastaxis_kernel(const u32x4* __restric
         for (int j = 0; j < UNROLL; ++j) {
             const int64_t i = base + j * TPB;
             const uint32_t um = group_max<LPT>(vec_abs_max<DT>(v[j]));
-            const MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+            const MxqScale sc = mxq_block_scale_dt<ADT>(um, p.emax, p.scale_emax, p.flush != 0, zone);
             u32x4 o;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
@@ -193,7 +197,7 @@ __global__ __launch_bounds__(TPB) void mx_strided_tile_kernel(const u32x2* __res
                                                               int64_t items, int64_t n_tiles,
                                                               int64_t pv, MxParams p) {
     constexpr int ADT = Arith<DT>::DT_;
-    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
+    constexpr int ZS = MxqZoneShift<ADT>::value;        // significand units of the zone table
     constexpr int VW = Col8<DT>::VW;
     constexpr int PD = Pack<DT>::PER_DWORD;
     __shared__ unsigned char zone[ZONE_PAD];
@@ -242,7 +246,7 @@ __global__ __launch_bounds__(TPB) void mx_strided_tile_kernel(const u32x2* __res
     MxqScale sc[VW];
 #pragma unroll
     for (int k = 0; k < VW; ++k)
-        sc[k] = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+        sc[k] = mxq_block_scale_dt<ADT>(um[k], p.emax, p.scale_emax, p.flush != 0, zone);
 
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
@@ -268,6 +272,8 @@ template <> struct ColVec<MXQ_BF16, 1> { typedef unsigned short T; static conste
 template <> struct ColVec<MXQ_BF16, 8> { typedef u32x4 T; static constexpr int DW = 4; };
 template <> struct ColVec<MXQ_F16, 1> { typedef unsigned short T; static constexpr int DW = 1; };
 template <> struct ColVec<MXQ_F16, 8> { typedef u32x4 T; static constexpr int DW = 4; };
+template <> struct ColVec<MXQ_F16OPS, 1> : ColVec<MXQ_F16, 1> {};
+template <> struct ColVec<MXQ_F16OPS, 8> : ColVec<MXQ_F16, 8> {};
 
 template <int DT, int VW>
 __device__ __forceinline__ void unpack_cols(const typename ColVec<DT, VW>::T& raw, float* x) {
@@ -289,7 +295,7 @@ __device__ __forceinline__ typename ColVec<DT, VW>::T pack_cols(const float* q) 
     if constexpr (VW == 1) {
         if (DT == MXQ_F32) r = mxq_bits(q[0]);
         else if (DT == MXQ_BF16) r = (unsigned short)(mxq_bits(q[0]) >> 16);
-        else r = __builtin_bit_cast(unsigned short, (_Float16)q[0]);
+        else r = mxq_f16_bits(q[0]);
     } else {
         constexpr int PD = Pack<DT>::PER_DWORD;
 #pragma unroll
@@ -305,7 +311,7 @@ __global__ __launch_bounds__(TPB) void mx_strided_kernel(const void* __restrict_
                                                          int64_t tile, int64_t num_tiles,
                                                          MxParams p) {
     constexpr int ADT = Arith<DT>::DT_;
-    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
+    constexpr int ZS = MxqZoneShift<ADT>::value;        // significand units of the zone table
     typedef typename ColVec<DT, VW>::T V;
     __shared__ unsigned char zone[ZONE_PAD];
     load_zone(zone, g_zone_tables[p.zone_row]);
@@ -335,7 +341,7 @@ __global__ __launch_bounds__(TPB) void mx_strided_kernel(const void* __restrict_
         MxqScale sc[VW];
 #pragma unroll
         for (int k = 0; k < VW; ++k)
-            sc[k] = mxq_block_scale(um[k], p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+            sc[k] = mxq_block_scale_dt<ADT>(um[k], p.emax, p.scale_emax, p.flush != 0, zone);
         for (int64_t r = 0; r < rows; ++r) {
             float x[VW], q[VW];
             unpack_cols<DT, VW>(in[off0 + r * pv], x);
@@ -357,7 +363,7 @@ template <int DT, int RMODE, bool ZONE_ELEM, bool LEAN>
 __global__ __launch_bounds__(TPB) void mx_axes_kernel(const void* __restrict__ in, void* __restrict__ out,
                                                       MxqAxes a, int64_t n_tiles, MxParams p) {
     constexpr int ADT = Arith<DT>::DT_;
-    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int ZS = MxqZoneShift<ADT>::value;
     __shared__ unsigned char zone[ZONE_PAD];
     __shared__ uint32_t wave_max[TPB / 64];
     load_zone(zone, g_zone_tables[p.zone_row]);
@@ -382,7 +388,7 @@ __global__ __launch_bounds__(TPB) void mx_axes_kernel(const void* __restrict__ i
         __syncthreads();
 #pragma unroll
         for (int w = 0; w < TPB / 64; ++w) um = max(um, wave_max[w]);
-        const MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+        const MxqScale sc = mxq_block_scale_dt<ADT>(um, p.emax, p.scale_emax, p.flush != 0, zone);
         for (int64_t e = threadIdx.x; e < count; e += TPB) {
             const int64_t off = offset(e);
             store_scalar<DT>(out, off, mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, LEAN>(load_scalar<DT>(in, off), sc,
@@ -403,7 +409,7 @@ __global__ __launch_bounds__(TPB) void mx_given_max_kernel(const void* __restric
                                                            int64_t total, int64_t axis_size,
                                                            int64_t post, MxParams p) {
     constexpr int ADT = Arith<DT>::DT_;
-    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
+    constexpr int ZS = MxqZoneShift<ADT>::value;        // significand units of the zone table
     __shared__ unsigned char zone[ZONE_PAD];
     load_zone(zone, g_zone_tables[p.zone_row]);
     for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < total;
@@ -411,7 +417,7 @@ __global__ __launch_bounds__(TPB) void mx_given_max_kernel(const void* __restric
         const int64_t j = i % post;
         const int64_t pi = i / (post * axis_size);
         const uint32_t um = abs_bits(load_scalar<DT>(maxv, pi * post + j));
-        MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+        MxqScale sc = mxq_block_scale_dt<ADT>(um, p.emax, p.scale_emax, p.flush != 0, zone);
         float q = mxq_quant_mx_elem<RMODE, ADT, ZONE_ELEM, LEAN>(load_scalar<DT>(in, i), sc, p.fmt,
                                                                  zone, ZS);
         store_scalar<DT>(out, i, q);
@@ -426,7 +432,7 @@ __global__ __launch_bounds__(TPB) void elemwise_kernel(const void* __restrict__ 
                                                        void* __restrict__ out_, int64_t n,
                                                        ElemParams p) {
     constexpr int ADT = Arith<DT>::DT_;
-    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;      // significand units of the zone table
+    constexpr int ZS = MxqZoneShift<ADT>::value;        // significand units of the zone table
     constexpr int PD = Pack<DT>::PER_DWORD;
     constexpr int EPV = 4 * PD;
     __shared__ unsigned char zone[ZONE_PAD];
@@ -534,7 +540,7 @@ __global__ __launch_bounds__(TPB) void elemwise_dither_kernel(const void* __rest
                                                               const void* __restrict__ noise,
                                                               void* __restrict__ out, int64_t n, ElemParams p) {
     constexpr int ADT = Arith<DT>::DT_;
-    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int ZS = MxqZoneShift<ADT>::value;
     __shared__ unsigned char zone[ZONE_PAD];
     load_zone(zone, g_zone_tables[p.zone_row]);
     for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (int64_t)gridDim.x * TPB)
@@ -552,7 +558,7 @@ __global__ __launch_bounds__(TPB) void mx_dither_kernel(const void* __restrict__
                                                         int64_t post, int64_t tile, int64_t num_tiles,
                                                         MxParams p) {
     constexpr int ADT = Arith<DT>::DT_;
-    constexpr int ZS = (ADT == MXQ_BF16) ? 16 : 0;
+    constexpr int ZS = MxqZoneShift<ADT>::value;
     __shared__ unsigned char zone[ZONE_PAD];
     load_zone(zone, g_zone_tables[p.zone_row]);
     const int64_t total = pre * num_tiles * post;
@@ -565,7 +571,7 @@ __global__ __launch_bounds__(TPB) void mx_dither_kernel(const void* __restrict__
         const int64_t off0 = (pi * axis_size + row0) * post + c;
         uint32_t um = 0;
         for (int64_t r = 0; r < rows; ++r) um = max(um, abs_bits(load_scalar<DT>(in, off0 + r * post)));
-        const MxqScale sc = mxq_block_scale(um, p.emax, p.scale_emax, p.flush != 0, zone, ZS);
+        const MxqScale sc = mxq_block_scale_dt<ADT>(um, p.emax, p.scale_emax, p.flush != 0, zone);
         for (int64_t r = 0; r < rows; ++r) {
             const int64_t i = off0 + r * post;
             store_scalar<DT>(out, i, mxq_quant_mx_elem<MXQ_DITHER, ADT, true, false>(

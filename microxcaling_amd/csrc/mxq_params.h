@@ -11,7 +11,7 @@
 #include "mxq_core.h"
 #include "mxq_log2_tables.h"
 
-enum { ZONE_ROW_F32 = 0, ZONE_ROW_BF16 = 1, ZONE_ROW_NONE = 2 };
+enum { ZONE_ROW_F32 = 0, ZONE_ROW_BF16 = 1, ZONE_ROW_NONE = 2, ZONE_ROW_F16 = 3 };
 
 struct MxParams {
     MxqFmt fmt;
@@ -19,7 +19,7 @@ struct MxParams {
     int scale_emax;   // 2^(scale_bits-1) - 1
     int flush;
     int zone_row;     // which round-up-zone table
-    int zshift;       // 0 for fp32 significands, 16 for bf16
+    int zshift;       // 0 for fp32 significands, 16 for bf16, 13 for fp16
     uint32_t pre_nan_from;   // mxq_pack_mx with MXQ_FLAG_PRE_BFLOAT16: NaN threshold of that quantizer, else 0
 };
 
@@ -35,7 +35,12 @@ struct ElemParams {
 namespace mxq_detail {
 
 // host copy of the round-up-zone tables (the kernels read theirs from device memory)
-static const unsigned char zone_rows[2][MXQ_ZONE_PAD] = {{MXQ_ZONE_ROW_F32}, {MXQ_ZONE_ROW_BF16}};
+static const unsigned char zone_rows[4][MXQ_ZONE_PAD] = {{MXQ_ZONE_ROW_F32}, {MXQ_ZONE_ROW_BF16}, {0}, {MXQ_ZONE_ROW_F16}};
+
+// fp16 tensors: every op rounded to fp16 (the reference's pure-PyTorch path on such a tensor), unless
+// the caller asks for bit-field exponents -- then they are widened to fp32, quantized and rounded
+// back once, which is what the reference's CUDA kernels do (mx/cpp/mx.cuh:72,88).
+inline bool f16_ops(int dtype, int flags) { return dtype == MXQ_DTYPE_F16 && !(flags & MXQ_FLAG_EXACT_EXPONENT); }
 
 inline std::string& last_error() {
     static thread_local std::string s;
@@ -86,7 +91,8 @@ inline int make_mx_axes(int n_axes, const int64_t* extents, int64_t tile_size, M
     return MXQ_OK;
 }
 
-inline int make_fmt(int dtype, int ebits, int mbits, float max_norm, MxqFmt* fmt, const char* who) {
+inline int make_fmt(int dtype, int flags, int ebits, int mbits, float max_norm, bool clamps, MxqFmt* fmt,
+                    const char* who) {
     if (ebits < 0 || ebits > 8) return fail(MXQ_ERR_ARGUMENT, "%s: exponent bits %d outside [0, 8]", who, ebits);
     if (mbits < 2 || mbits > 24)
         return fail(MXQ_ERR_ARGUMENT, "%s: bits %d outside [2, 24] (sign + implicit one + fraction)", who, mbits);
@@ -97,6 +103,14 @@ inline int make_fmt(int dtype, int ebits, int mbits, float max_norm, MxqFmt* fmt
     fmt->min_exp = ebits ? 2 - (1 << (ebits - 1)) : 0;
     // torch casts the clamp bound to the tensor dtype (65504 becomes 65536 for a bf16 tensor)
     fmt->max_bits = mxq_bits(dtype == MXQ_DTYPE_BF16 ? mxq_round_bf16(max_norm) : max_norm);
+    if (f16_ops(dtype, flags)) {
+        // a bound beyond the fp16 range: torch.clamp refuses to convert it (mx/elemwise_ops.py:154
+        // raises), the comparison of the non-saturating branch (156) sees it as Inf
+        fmt->max_bits = mxq_bits(mxq_round_f16(max_norm));
+        if (clamps && max_norm > 65504.0f)
+            return fail(MXQ_ERR_ARGUMENT, "%s: max_norm %g cannot be converted to float16 without overflow "
+                        "(the clamp of a float16 tensor needs its bound in float16)", who, (double)max_norm);
+    }
     fmt->min_eb = ebits ? (uint32_t)(fmt->min_exp + 127) : 127u;
     fmt->t127 = fmt->t + 127;
     // "s + 0.5" is rounded to the tensor dtype before the floor: in bf16 that turns 1 - 2^-9 into
@@ -110,8 +124,11 @@ inline int make_fmt(int dtype, int ebits, int mbits, float max_norm, MxqFmt* fmt
 
 inline void zone_for(int dtype, int flags, int* row, int* zshift) {
     *zshift = 0;
-    if ((flags & MXQ_FLAG_EXACT_EXPONENT) || dtype == MXQ_DTYPE_F16) {
+    if (flags & MXQ_FLAG_EXACT_EXPONENT) {
         *row = ZONE_ROW_NONE;
+    } else if (dtype == MXQ_DTYPE_F16) {
+        *row = ZONE_ROW_F16;
+        *zshift = 13;
     } else if (dtype == MXQ_DTYPE_BF16) {
         *row = ZONE_ROW_BF16;
         *zshift = 16;
@@ -124,6 +141,7 @@ inline void zone_for(int dtype, int flags, int* row, int* zshift) {
 // fraction bits: the elementwise quantizer handles the one extra case of nearest mode (BUMP), floor
 // mode has none, torch's emulation of even mode has too many (op-by-op form).  MX element formats
 // never have more than 6 fraction bits.
+// fp16 tensors evaluated op by op (f16_ops) always take the op-by-op form; callers test that first.
 inline bool lean_ok(int dtype, const MxqFmt& f, int rmode, bool elementwise) {
     return dtype != MXQ_DTYPE_BF16 || f.t <= 6 || (elementwise && rmode != MXQ_ROUND_EVEN);
 }
@@ -141,29 +159,13 @@ inline bool elem_zone_matters(int dtype, int flags, const MxqFmt& f, int rmode) 
     return !(f.ebits <= 5 && f.t <= 3);
 }
 
-// fp16 tensors: the reference's pure-PyTorch path evaluates every op in fp16 (2**exponent overflows
-// from 2^16, log2 rounds to 11 bits, ...: mx/mx_ops.py:265-292, mx/elemwise_ops.py:127-163), which
-// these kernels do not reproduce.  What they compute for fp16 -- widen to fp32, bit-field exponents,
-// round back -- is what the reference's CUDA kernels compute (mx/cpp/mx.cuh:72,88), so it is only
-// offered under the flag that asks for those semantics; without it the call is refused rather than
-// answered with values that differ from the pure path in places.
-inline int fp16_only_with_exact_exponents(int dtype, int flags, const char* who) {
-    if (dtype == MXQ_DTYPE_F16 && !(flags & MXQ_FLAG_EXACT_EXPONENT))
-        return fail(MXQ_ERR_ARGUMENT, "%s: fp16 tensors are served with MXQ_FLAG_EXACT_EXPONENT only (fp32 arithmetic "
-                    "and bit-field exponents, the reference's CUDA semantics); the reference's pure-PyTorch path on "
-                    "fp16 tensors is not reproduced -- cast to float32 or bfloat16, or switch to exact exponents", who);
-    return MXQ_OK;
-}
-
 inline int make_mx_params(int dtype, int scale_bits, int ebits, int mbits, float max_norm, int flush,
                           int rmode, int flags, MxParams* p, bool* zone_elem, const char* who) {
     if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
     if (rmode < 0 || rmode > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown rounding mode %d", who, rmode);
     if (scale_bits < 1 || scale_bits > 8)
         return fail(MXQ_ERR_ARGUMENT, "%s: scale_bits %d outside [1, 8]", who, scale_bits);
-    int rc = fp16_only_with_exact_exponents(dtype, flags, who);
-    if (rc) return rc;
-    rc = make_fmt(dtype, ebits, mbits, max_norm, &p->fmt, who);
+    int rc = make_fmt(dtype, flags, ebits, mbits, max_norm, true, &p->fmt, who);
     if (rc) return rc;
     // exponent of max_norm, the way the reference's kernels derive it (mx/cpp/shared_exp.cuh:33)
     int be = (int)((mxq_bits(max_norm) >> 23) & 0xFF);
@@ -180,18 +182,17 @@ inline int make_elem_params(int dtype, int bits, int exp_bits, float max_norm, i
                             int saturate, int allow_denorm, int flags, ElemParams* p, const char* who) {
     if (dtype < 0 || dtype > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown dtype code %d", who, dtype);
     if (rmode < 0 || rmode > 2) return fail(MXQ_ERR_ARGUMENT, "%s: unknown rounding mode %d", who, rmode);
-    int rc = fp16_only_with_exact_exponents(dtype, flags, who);
-    if (rc) return rc;
-    rc = make_fmt(dtype, exp_bits, bits, max_norm, &p->fmt, who);
+    int rc = make_fmt(dtype, flags, exp_bits, bits, max_norm, saturate || exp_bits == 0, &p->fmt, who);
     if (rc) return rc;
     p->saturate = saturate ? 1 : 0;
     p->allow_denorm = allow_denorm ? 1 : 0;
     p->general_only = (flags & MXQ_FLAG_GENERAL_FORM) ? 1 : 0;
     zone_for(dtype, flags, &p->zone_row, &p->zshift);
-    // the top binade's round-up zone: floor(log2|x|) = 128 there
-    static const unsigned char top_count[3] = {zone_rows[0][276], zone_rows[1][276], 0};
-    p->fmt.nan_from = exp_bits ? MXQ_INF_BITS - ((uint32_t)top_count[p->zone_row] << p->zshift)
-                               : MXQ_INF_BITS;
+    // the top binade's round-up zone: floor(log2|x|) = 128 there (16 for an fp16 tensor, whose top
+    // binade is k = 15), and 2**that is Inf
+    const uint32_t top_bits = p->zone_row == ZONE_ROW_F16 ? 0x47800000u : MXQ_INF_BITS;
+    const uint32_t top_count = zone_rows[p->zone_row][p->zone_row == ZONE_ROW_F16 ? 15 + 149 : 276];
+    p->fmt.nan_from = exp_bits ? top_bits - (top_count << p->zshift) : MXQ_INF_BITS;
     return MXQ_OK;
 }
 

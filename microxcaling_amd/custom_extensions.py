@@ -21,11 +21,10 @@ _flags = 0
 
 def set_exponent_mode(mode):
     """'torch' (default): exponents follow floor(log2(x)) as torch's CPU kernels evaluate it, so
-    results are bit-identical to the reference's pure-PyTorch path (float32 and bfloat16 tensors;
-    float16 tensors are refused in this mode: that path evaluates every op in fp16, which the
-    kernels do not reproduce).  'exact': bit-field exponents, which is what the reference's CUDA
-    kernels compute; float16 tensors are widened to fp32 and rounded back, as those kernels do
-    (mx/cpp/mx.cuh:72,88)."""
+    results are bit-identical to the reference's pure-PyTorch path (float32, bfloat16 and float16
+    tensors; on 16-bit tensors every op is rounded to the tensor dtype, as that path does).
+    'exact': bit-field exponents, which is what the reference's CUDA kernels compute; float16 tensors
+    are widened to fp32 and rounded back once, as those kernels do (mx/cpp/mx.cuh:72,88)."""
     global _flags
     if mode == "torch":
         _flags = _flags & ~_lib.FLAG_EXACT_EXPONENT

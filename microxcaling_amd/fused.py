@@ -10,8 +10,8 @@ import torch
 from . import _lib
 from .custom_extensions import _DTYPE, _check_gpu_input, _flags_value, _stream
 
-# tensor dtypes whose layers take the fused path (fp16 tensors are quantized in exact-exponent mode only
-# and stay on the separate steps)
+# tensor dtypes whose layers take the fused path (fp16 tensors have no packed form in the default
+# exponent mode, where every op is rounded to fp16, and stay on the separate steps)
 _FUSED_DTYPES = (torch.float32, torch.bfloat16)
 from .formats import ElemFormat, RoundingMode, _get_format_params
 

@@ -8,7 +8,7 @@ from . import build_oracle
 from .mx_oracle import format_params
 
 _lib = None
-_DT = {torch.float32: 0, torch.bfloat16: 2}
+_DT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 
 def lib():
@@ -31,6 +31,10 @@ _RMODE = {"nearest": 0, "floor": 1, "even": 2}
 def quantize_elemwise_core(A, bits, exp_bits, max_norm, round="nearest", saturate_normals=False,
                            allow_denorm=True):
     A = A.contiguous()
+    if A.dtype == torch.float16 and (saturate_normals or exp_bits == 0) and max_norm > 65504.0:
+        # torch.clamp converts its bounds to the tensor dtype and refuses one that overflows it
+        # (mx/elemwise_ops.py:154 on an fp16 tensor)
+        raise RuntimeError("value cannot be converted to type at::Half without overflow")
     out = torch.empty_like(A)
     lib().oracle_quantize_elemwise(A.data_ptr(), out.data_ptr(), _DT[A.dtype], A.numel(), bits,
                                    exp_bits, max_norm, _RMODE[round], int(saturate_normals),

@@ -1,9 +1,9 @@
 /* Scalar C restatement of the reference's pure-PyTorch quantization path.  TEST INFRASTRUCTURE
  * ONLY: it checks the HIP kernels and the torch oracle (mx_oracle.py); no product code links it.
  *
- * Every torch tensor op of the reference becomes one IEEE fp32 operation followed, for bf16
- * tensors, by a round-to-nearest-even to bf16 -- which is how torch's CPU kernels evaluate bf16
- * ops.  log2 is taken in double and rounded to fp32 (then to the tensor dtype), i.e. a correctly
+ * Every torch tensor op of the reference becomes one IEEE fp32 operation followed, for bf16 and
+ * fp16 tensors, by a round-to-nearest-even to that dtype -- which is how torch's CPU kernels
+ * evaluate ops on 16-bit tensors.  log2 is taken in double and rounded to fp32 (then to the tensor dtype), i.e. a correctly
  * rounded log2; torch's CPU log2 agrees with that on every input the tests sweep.  Nothing here
  * shares code with the kernels: exponents come from log2(), not from bit fields or tables.
  *
@@ -14,14 +14,39 @@
 #include <stdint.h>
 #include <string.h>
 
-enum { DT_F32 = 0, DT_BF16 = 2 };
+enum { DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2 };
 enum { RD_NEAREST = 0, RD_FLOOR = 1, RD_EVEN = 2 };     /* mx/formats.py:12-19 */
 
 static uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
 static float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
 
+/* fp32 -> fp16 bits, round to nearest even: subnormals down to 2^-24, Inf from 65520 */
+static uint16_t f2h(float v) {
+    uint32_t u = f2u(v), sign = (u >> 16) & 0x8000u, a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u);
+    if (a >= 0x47800000u) return (uint16_t)(sign | 0x7C00u);          /* >= 2^16 (or Inf) */
+    double d = fabs((double)v);
+    /* units of the result: 2^(e-10) for a normal of exponent e >= -14, 2^-24 below */
+    int e;
+    frexp(d, &e);                                                     /* d = m * 2^e, 0.5 <= m < 1 */
+    e -= 1;
+    if (d == 0.0) return (uint16_t)sign;
+    if (e < -14) e = -14;
+    double q = ldexp(d, 10 - e);                                      /* exact: in [0, 2048) */
+    double n = nearbyint(q);                                          /* ties to even (default mode) */
+    uint32_t mant = (uint32_t)n;                                      /* may be 2048: carries */
+    uint32_t h = (uint32_t)(e + 14) * 1024u + mant;                   /* subnormal: field 0 + mant */
+    return (uint16_t)(sign | h);                                      /* 65520 and up gives 0x7C00 */
+}
+static float h2f(uint16_t h) {
+    uint32_t e = (h >> 10) & 31u, m = h & 1023u;
+    float v = e == 31u ? (m ? NAN : INFINITY) : e ? ldexpf((float)(1024u + m), (int)e - 25) : ldexpf((float)m, -24);
+    return (h & 0x8000u) ? -v : v;
+}
+
 /* result of a torch op on a tensor of dtype dt */
 static float R(float v, int dt) {
+    if (dt == DT_F16) return h2f(f2h(v));
     if (dt != DT_BF16) return v;
     uint32_t u = f2u(v);
     if ((u & 0x7FFFFFFFu) > 0x7F800000u) return u2f(0x7FC00000u);
@@ -85,10 +110,12 @@ static float elem_core(float a, int bits, int exp_bits, float max_norm, int rmod
 
 static float load(const void* p, int dt, int64_t i) {
     if (dt == DT_F32) return ((const float*)p)[i];
+    if (dt == DT_F16) return h2f(((const uint16_t*)p)[i]);
     return u2f((uint32_t)((const uint16_t*)p)[i] << 16);
 }
 static void store(void* p, int dt, int64_t i, float v) {
     if (dt == DT_F32) ((float*)p)[i] = v;
+    else if (dt == DT_F16) ((uint16_t*)p)[i] = f2h(v);
     else ((uint16_t*)p)[i] = (uint16_t)(f2u(R(v, DT_BF16)) >> 16);
 }
 

@@ -24,7 +24,8 @@ ELEM_CASES = [(9, 8, 2 ** 127 * 255 / 128, False), (12, 5, 65504.0, False), (12,
 
 def inputs(dtype):
     g = torch.Generator().manual_seed(4242)
-    x = torch.randn(64, 96, generator=g) * torch.exp2(torch.randint(-24, 24, (64, 96), generator=g).float())
+    span = 12 if dtype == torch.float16 else 24         # fp16 holds 2**-24 .. 2**16
+    x = torch.randn(64, 96, generator=g) * torch.exp2(torch.randint(-span, span, (64, 96), generator=g).float())
     x = x.to(dtype)
     x[0, :8] = torch.tensor([0.0, -0.0, float("inf"), float("-inf"), float("nan"), 1e-39, 3e38, -1e-41]).to(dtype)
     x[1] = 0.0                                   # a block of zeros
@@ -41,7 +42,7 @@ def main(ref_root):
     from mx.mx_ops import _quantize_mx                      # noqa: E402
     from mx.elemwise_ops import _quantize_elemwise_core     # noqa: E402
     out = {}
-    for name, dtype in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+    for name, dtype in (("f32", torch.float32), ("bf16", torch.bfloat16), ("f16", torch.float16)):
         x = inputs(dtype)
         out["x_" + name] = raw(x)
         for n, (fmt, axis, bs) in enumerate(MX_CASES):

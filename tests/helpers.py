@@ -90,7 +90,7 @@ def dither_cases():
     """(kind, dtype name, torch dtype, case number, seed, parameters, input tensor, expected output) for
     every stored case."""
     z, mod = dither_golden()
-    for name, dtype in (("f32", torch.float32), ("bf16", torch.bfloat16)):
+    for name, dtype in (("f32", torch.float32), ("bf16", torch.bfloat16), ("f16", torch.float16)):
         x = from_bits(z["x_" + name], dtype)
         for n, case in enumerate(mod.MX_CASES):
             yield "mx", name, dtype, n, 1000 + n, case, x, from_bits(z["mx_%s_%d" % (name, n)], dtype)

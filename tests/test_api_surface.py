@@ -87,20 +87,25 @@ def test_sparse_coo_values_are_quantized():
     assert_bits_equal(y.to_dense(), x.to_dense().to(torch.bfloat16).float())
 
 
-def test_fp16_tensors_are_refused_unless_exact_exponents_are_asked_for():
-    """The reference's pure path runs every op in fp16 on fp16 tensors (mx/mx_ops.py:265-292), which
-    the kernels do not reproduce: by default such tensors raise instead of coming back with values
-    that differ in places.  In 'exact' mode they get the semantics of the reference's CUDA kernels
-    (mx/cpp/mx.cuh:72,88): widen to fp32, quantize, round back."""
+def test_fp16_tensors_in_both_exponent_modes():
+    """fp16 tensors.  Default ('torch') mode: every op rounded to fp16, like the reference's pure path
+    (mx/mx_ops.py:265-292, mx/elemwise_ops.py:127-163) -- compared with the oracle here and with the
+    reference's own outputs in test_oracle_pins.py.  'exact' mode: the semantics of the reference's CUDA
+    kernels (mx/cpp/mx.cuh:72,88): widen to fp32, quantize with bit-field exponents, round back."""
     from microxcaling_amd import custom_extensions as ce
     from microxcaling_amd.elemwise_ops import _quantize_elemwise_core
     from microxcaling_amd.mx_ops import _quantize_mx
+    from oracle import mx_oracle as O
     g = torch.Generator().manual_seed(1)
     x = (torch.randn(8, 64, generator=g) * 3).half()
-    with pytest.raises(RuntimeError, match="fp16 tensors"):
-        _quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=32)
-    with pytest.raises(RuntimeError, match="fp16 tensors"):
-        _quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128)
+    for rnd in ("nearest", "floor", "even"):
+        assert_bits_equal(_quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=32, round=rnd),
+                          O.quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=32, round=rnd), "mx " + rnd)
+        assert_bits_equal(_quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128, round=rnd),
+                          O.quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128, round=rnd), "elementwise " + rnd)
+    # the clamp of the saturating branch needs its bound in fp16: the reference raises, and so does this
+    with pytest.raises(RuntimeError, match="float16"):
+        _quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128, saturate_normals=True)
     ce.set_exponent_mode("exact")
     try:
         for rnd in ("nearest", "floor", "even"):

@@ -359,25 +359,30 @@ def test_headline_size_properties(dev):
 
 
 def test_fp16_tensors_on_the_gpu(dev):
-    """Refused by default (the pure path's all-fp16 arithmetic is not reproduced); with exact
-    exponents: the widened fp32 computation rounded back, as on CPU tensors."""
+    """Default mode: the all-fp16 arithmetic of the pure path (bit for bit against the oracle; the
+    reference's own outputs are compared in test_oracle_pins.py).  Exact exponents: the widened fp32
+    computation rounded back, as on CPU tensors -- bit for bit, the sign of a zero included."""
     from microxcaling_amd import custom_extensions as ce
     g = torch.Generator().manual_seed(2)
     x = (torch.randn(64, 256, generator=g) * 3).half()
-    with pytest.raises(RuntimeError, match="fp16 tensors"):
-        mx_gpu(x.to(dev), 8, "fp8_e4m3", axes=[-1], block_size=32)
-    with pytest.raises(RuntimeError, match="fp16 tensors"):
-        elem_gpu(x.to(dev), 9, 8, 2 ** 127 * 255 / 128)
+    for axis in (-1, 0):
+        for rnd in ("nearest", "floor", "even"):
+            got = mx_gpu(x.to(dev), 8, "fp8_e4m3", axes=[axis], block_size=32, round=rnd)
+            assert_bits_equal(got, O.quantize_mx(x, 8, "fp8_e4m3", axes=[axis], block_size=32, round=rnd),
+                              "mx axis %d %s" % (axis, rnd))
+    assert_bits_equal(elem_gpu(x.to(dev), 9, 8, 2 ** 127 * 255 / 128),
+                      O.quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128), "elementwise")
+    with pytest.raises(RuntimeError, match="float16"):
+        elem_gpu(x.to(dev), 9, 8, 2 ** 127 * 255 / 128, saturate_normals=True)
     ce.set_exponent_mode("exact")
     try:
-        # values, not bit patterns: the sign of a zero is not part of these semantics (the reference's
-        # CUDA kernels return +0 for a negative value that rounds to zero, mx/cpp/quantize.cuh:99)
         for axis in (-1, 0):
             got = mx_gpu(x.to(dev), 8, "fp4_e2m1", axes=[axis], block_size=32)
             want = mx_gpu(x.float().to(dev), 8, "fp4_e2m1", axes=[axis], block_size=32).half()
-            assert got.dtype == torch.float16 and torch.equal(got.float(), want.float()), "mx axis %d" % axis
+            assert got.dtype == torch.float16
+            assert_bits_equal(got, want, "mx axis %d" % axis)
         got = elem_gpu(x.to(dev), 5, 4, 448.0, round="even", saturate_normals=True)
         want = elem_gpu(x.float().to(dev), 5, 4, 448.0, round="even", saturate_normals=True).half()
-        assert torch.equal(got.float(), want.float()), "elementwise"
+        assert_bits_equal(got, want, "elementwise")
     finally:
         ce.set_exponent_mode("torch")

@@ -125,6 +125,20 @@ def test_zone_tables_match_torch_log2_bf16():
     assert torch.equal(got[inrange], want[inrange])
 
 
+def test_zone_tables_match_torch_log2_fp16():
+    """Every positive finite fp16 code: the exponent the host library derives (bit field + zone table)
+    is torch's floor(log2(x)) evaluated in fp16.  Read back as above; where the exponent comes out as
+    16 the block scale 2**16 is Inf in fp16 and the block is NaN."""
+    codes = torch.arange(1, 0x7C00, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    want = torch.floor(torch.log2(codes)).float()
+    y = _quantize_mx(codes.view(-1, 1), 8, "int2", axes=[1], block_size=1, round="floor").float().view(-1)
+    true_k = torch.floor(torch.log2(codes.double())).float()
+    got = torch.where((y == 0) | y.isnan(), true_k + 1, true_k)
+    assert (got != true_k).sum() > 50                           # the zones are there
+    assert torch.equal(got, want)
+    assert torch.equal(y.isnan(), want == 16)
+
+
 def test_zone_tables_match_torch_log2_fp32():
     parts = []
     for be in range(1, 255):
@@ -380,6 +394,38 @@ def test_direct_pack_codes_equal_the_encoded_rounded_values(tmp_path):
     assert out.count("inputs agree") == 30 and "MISMATCH" not in out
     # nearest and even are served by the shortcut (floor takes the round-up-zone variant)
     assert out.count("zone variant") == 10
+
+
+@pytest.mark.parametrize("compiler", ["g++", "/opt/rocm/lib/llvm/bin/clang++"])
+def test_fp16_conversions_of_the_scalar_core(tmp_path, compiler):
+    """mxq_f16_bits / mxq_f16_value (the rounding after every op of an fp16 tensor) against torch's
+    conversions: every fp16 code, both neighbours of every rounding boundary between two codes, the
+    boundaries themselves, and a sweep of fp32 patterns.  g++ compiles the integer form, clang the
+    _Float16 form."""
+    import shutil
+    import subprocess
+    cxx = shutil.which(compiler)
+    if cxx is None:
+        pytest.skip("no " + compiler)
+    codes = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(torch.float16)
+    pos = codes[:0x7C00].float()
+    mid = (pos[:-1].double() + pos[1:].double()) / 2                 # exact in fp32: one more bit
+    mid = torch.cat([mid, torch.tensor([65520.0], dtype=torch.float64)]).float()
+    mb = mid.view(torch.int32)
+    sweep = torch.arange(0, 2 ** 32, 40961, dtype=torch.int64).to(torch.int32).view(torch.float32)
+    x = torch.cat([codes.float(), mid, (mb - 1).view(torch.float32), (mb + 1).view(torch.float32), sweep])
+    x = torch.cat([x, -x])
+    src, hb, fb = (str(tmp_path / n) for n in ("x.bin", "h.bin", "f.bin"))
+    x.numpy().tofile(src)
+    exe = str(tmp_path / "f16_round_check")
+    subprocess.run([cxx, "-O2", "-std=c++17", "-ffp-contract=off", "-I", os.path.join(ROOT_DIR, "include"),
+                    "-I", os.path.join(ROOT_DIR, "microxcaling_amd", "csrc"), "-o", exe,
+                    os.path.join(ROOT_DIR, "tests", "cpp", "f16_round_check.cpp")], check=True)
+    subprocess.run([exe, src, hb, fb], check=True, capture_output=True, timeout=120)
+    got_h = torch.from_numpy(np.fromfile(hb, dtype=np.int16)).view(torch.float16)
+    got_f = torch.from_numpy(np.fromfile(fb, dtype=np.float32))
+    assert_bits_equal(got_h, x.half(), "fp32 -> fp16")
+    assert_bits_equal(got_f, x.half().float(), "fp16 -> fp32")
 
 
 def test_gemm_tile_copies_stay_inside_their_operands(tmp_path):
