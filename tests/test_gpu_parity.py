@@ -261,6 +261,8 @@ def test_dither_with_the_reference_noise(dev):
     from microxcaling_amd.custom_extensions import funcs
     from microxcaling_amd.formats import _get_format_params
     for kind, name, dtype, case_no, seed, case, x, want in dither_cases():
+        if dtype == torch.float16:
+            continue                                  # tests/test_zx_fp16_tensors.py
         torch.manual_seed(seed)
         noise = torch.rand_like(x).to(dev)
         if kind == "mx":
@@ -356,33 +358,3 @@ def test_headline_size_properties(dev):
     rows = torch.randperm(8192, generator=g)[:128]
     want = O.quantize_mx(x[rows], 8, "fp8_e4m3", axes=[-1], block_size=32)
     assert_bits_equal(y[rows.to(dev)], want, "sampled rows")
-
-
-def test_fp16_tensors_on_the_gpu(dev):
-    """Default mode: the all-fp16 arithmetic of the pure path (bit for bit against the oracle; the
-    reference's own outputs are compared in test_oracle_pins.py).  Exact exponents: the widened fp32
-    computation rounded back, as on CPU tensors -- bit for bit, the sign of a zero included."""
-    from microxcaling_amd import custom_extensions as ce
-    g = torch.Generator().manual_seed(2)
-    x = (torch.randn(64, 256, generator=g) * 3).half()
-    for axis in (-1, 0):
-        for rnd in ("nearest", "floor", "even"):
-            got = mx_gpu(x.to(dev), 8, "fp8_e4m3", axes=[axis], block_size=32, round=rnd)
-            assert_bits_equal(got, O.quantize_mx(x, 8, "fp8_e4m3", axes=[axis], block_size=32, round=rnd),
-                              "mx axis %d %s" % (axis, rnd))
-    assert_bits_equal(elem_gpu(x.to(dev), 9, 8, 2 ** 127 * 255 / 128),
-                      O.quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128), "elementwise")
-    with pytest.raises(RuntimeError, match="float16"):
-        elem_gpu(x.to(dev), 9, 8, 2 ** 127 * 255 / 128, saturate_normals=True)
-    ce.set_exponent_mode("exact")
-    try:
-        for axis in (-1, 0):
-            got = mx_gpu(x.to(dev), 8, "fp4_e2m1", axes=[axis], block_size=32)
-            want = mx_gpu(x.float().to(dev), 8, "fp4_e2m1", axes=[axis], block_size=32).half()
-            assert got.dtype == torch.float16
-            assert_bits_equal(got, want, "mx axis %d" % axis)
-        got = elem_gpu(x.to(dev), 5, 4, 448.0, round="even", saturate_normals=True)
-        want = elem_gpu(x.float().to(dev), 5, 4, 448.0, round="even", saturate_normals=True).half()
-        assert_bits_equal(got, want, "elementwise")
-    finally:
-        ce.set_exponent_mode("torch")

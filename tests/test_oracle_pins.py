@@ -386,96 +386,6 @@ def test_golden_exhaustive_bf16_digests():
                 assert _digest(y) == meta["bf16_exhaustive_digests"]["%d.%s.%s" % (Mexp, fmt, rnd)]
 
 
-# ---- fp16 tensors: every op evaluated in fp16 (tests/golden/gen_reference_fp16_vectors.py) ---------
-_fp16_golden = None
-
-
-def fp16_golden():
-    global _fp16_golden
-    if _fp16_golden is None:
-        import importlib.util
-        import json
-        import os
-        from helpers import GOLDEN
-        spec = importlib.util.spec_from_file_location("gen_reference_fp16_vectors",
-                                                      os.path.join(GOLDEN, "gen_reference_fp16_vectors.py"))
-        mod = importlib.util.module_from_spec(spec)
-        spec.loader.exec_module(mod)
-        with open(os.path.join(GOLDEN, "reference_fp16_vectors.json")) as f:
-            meta = json.load(f)
-        _fp16_golden = (np.load(os.path.join(GOLDEN, "reference_fp16_vectors.npz")), meta, mod)
-    return _fp16_golden
-
-
-@pytest.mark.parametrize("orc", ORACLES)
-def test_golden_fp16_mx_blocks(orc):
-    """Blocks with maxima at every fp16 exponent, inside and beside the round-up zones of log2, with
-    scales that overflow and underflow in fp16, zeros, Inf and NaN: the reference's outputs, stored."""
-    z, _, _ = fp16_golden()
-    x = from_bits(z["mx_x"], torch.float16)
-    for fmt in MX_FORMATS:
-        for rnd in ROUNDS:
-            y = orc.quantize_mx(x.clone(), 8, fmt, axes=[-1], block_size=32, round=rnd)
-            assert_bits_equal(y, from_bits(z["mx_y.%s.%s" % (fmt, rnd)], torch.float16), fmt + rnd)
-    y = orc.quantize_mx(x.t().contiguous(), 5, "fp8_e4m3", axes=[0], block_size=32, round="even",
-                        flush_fp32_subnorms=True)
-    assert_bits_equal(y, from_bits(z["mx_y.t.fp8_e4m3.even.sb5.flush"], torch.float16), "transposed")
-    y = orc.quantize_mx(x.clone(), 8, "fp6_e2m3", axes=[-1], block_size=32, round="nearest", flush_fp32_subnorms=True)
-    assert_bits_equal(y, from_bits(z["mx_y.fp6_e2m3.nearest.flush"], torch.float16), "flush")
-    y = orc.quantize_mx(x.clone(), 4, "int8", axes=[-1], block_size=8, round="floor")
-    assert_bits_equal(y, from_bits(z["mx_y.int8.floor.sb4.bs8"], torch.float16), "scale_bits 4, blocks of 8")
-    y = orc.quantize_mx(x[:, :24].contiguous(), 8, "fp4_e2m1", axes=[-1], block_size=16, round="even")
-    assert_bits_equal(y, from_bits(z["mx_y.fp4_e2m1.even.ragged24.bs16"], torch.float16), "ragged last block")
-
-
-@pytest.mark.parametrize("orc", ORACLES)
-def test_golden_fp16_mx_every_code(orc):
-    """Every finite fp16 code as an element under 14 block maxima x 7 formats x 3 roundings x scale_bits
-    8 and 5: digests of the reference's outputs, two cases stored in full."""
-    z, meta, gen = fp16_golden()
-    n = 0
-    for (exp, frac) in gen.EXHAUSTIVE_MAXIMA:
-        blk = gen.exhaustive_block(exp, frac)
-        for fmt in MX_FORMATS:
-            for rnd in ROUNDS:
-                for sb in (8, 5):
-                    y = orc.quantize_mx(blk.clone(), sb, fmt, axes=[-1], block_size=32, round=rnd)
-                    key = "%d.%d.%s.%s.%d" % (exp, frac, fmt, rnd, sb)
-                    stored = "mx_exh_y." + key
-                    if stored in z.files:
-                        assert_bits_equal(y, from_bits(z[stored], torch.float16), key)
-                    assert _digest(y) == meta["mx_digests"][key], key
-                    n += 1
-    assert n == len(meta["mx_digests"]) == 588
-
-
-@pytest.mark.parametrize("orc", ORACLES)
-def test_golden_fp16_elementwise_every_code(orc):
-    """The elementwise quantizer on all 65 536 fp16 codes: 7 formats (bfloat16, fp16, two fp8, a 20-bit
-    format whose scaled values overflow fp16, one with 6 exponent bits, int8) x 3 roundings x saturate x
-    denorm.  Where the clamp bound does not fit fp16 the reference raises; so must every implementation."""
-    z, meta, gen = fp16_golden()
-    codes = gen.all_fp16_codes()
-    n = 0
-    for name, (bits, ebits, mx) in gen.ELEM_CFG.items():
-        for rnd in ROUNDS:
-            for sat in (False, True):
-                for den in (True, False):
-                    key = "%s.%s.%d.%d" % (name, rnd, sat, den)
-                    if key in meta["elem_raises"]:
-                        with pytest.raises(RuntimeError):
-                            orc.quantize_elemwise_core(codes.clone(), bits, ebits, mx, round=rnd,
-                                                       saturate_normals=sat, allow_denorm=den)
-                        continue
-                    y = orc.quantize_elemwise_core(codes.clone(), bits, ebits, mx, round=rnd,
-                                                   saturate_normals=sat, allow_denorm=den)
-                    if "elem_y." + key in z.files:
-                        assert_bits_equal(y, from_bits(z["elem_y." + key], torch.float16), key)
-                    assert _digest(y) == meta["elem_digests"][key], key
-                    n += 1
-    assert n == len(meta["elem_digests"]) == 78 and len(meta["elem_raises"]) == 6
-
-
 def test_golden_dither():
     """round='dither' (mx/elemwise_ops.py:57-59): under the same torch seed the torch oracle draws
     the noise the reference drew and reproduces its outputs bit for bit (no test of the reference
