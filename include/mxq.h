@@ -75,6 +75,12 @@ const char* mxq_last_error(void);
 /* Library version (major * 100 + minor). */
 int mxq_version(void);
 
+/* Hex sha256 of the source files this library was compiled from (include/mxq.h and every .h, .hip
+ * and .cpp under microxcaling_amd/csrc, as microxcaling_amd/build_ext.py computes it), or "unknown"
+ * for a build made another way.  No counterpart in the reference: it lets a caller, and the tests,
+ * tell a stale library from the one that belongs to the sources at hand. */
+const char* mxq_build_digest(void);
+
 /* quantize_mx_by_tile_func_cuda (mx/cpp/funcs.cpp:177-197, mx/cpp/mx.cu:116-287).
  * MX-quantize `in`, shape (pre, axis_size, post) contiguous, sharing one exponent per
  * `tile_size` consecutive elements of the middle axis (a shorter last tile is allowed;
@@ -329,6 +335,7 @@ int mxq_gemm_plan(int64_t batch, int64_t M, int64_t N, int64_t K, int a_kind);
                                               +Inf and NaN (other inputs: unspecified) */
 
 const char* mxq_host_last_error(void);
+const char* mxq_host_build_digest(void); /* as mxq_build_digest, for libmxq_host.so */
 int mxq_host_quantize_mx_given_max(const void* in, void* out, const void* max_values, int dtype,
                                    int64_t pre, int64_t axis_size, int64_t post, int scale_bits,
                                    int elem_ebits, int elem_mbits, float elem_max_norm,

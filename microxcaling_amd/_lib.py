@@ -19,6 +19,7 @@ _c_int, _c_i64, _c_f32, _c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, c
 GPU_SYMBOLS = {
     "mxq_last_error": (ctypes.c_char_p, []),
     "mxq_version": (_c_int, []),
+    "mxq_build_digest": (ctypes.c_char_p, []),
     "mxq_quantize_mx_by_tile": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_int,
                                          _c_int, _c_int, _c_f32, _c_i64, _c_int, _c_int, _c_int,
                                          _c_ptr]),
@@ -70,6 +71,7 @@ GPU_SYMBOLS = {
 }
 HOST_SYMBOLS = {
     "mxq_host_last_error": (ctypes.c_char_p, []),
+    "mxq_host_build_digest": (ctypes.c_char_p, []),
     "mxq_host_quantize_mx_given_max": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_i64, _c_i64,
                                                 _c_i64, _c_int, _c_int, _c_int, _c_f32, _c_int,
                                                 _c_int, _c_int]),

@@ -7,6 +7,7 @@ Usage:  python -m microxcaling_amd.build_ext
 hipcc cross-compiles, so no GPU is needed to build.
 """
 import concurrent.futures
+import hashlib
 import os
 import subprocess
 import tempfile
@@ -22,6 +23,25 @@ HOST_LIB = os.path.join(PKG, "libmxq_host.so")
 
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-fvisibility=hidden",
           "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+
+
+def source_digest():
+    """sha256 over every file the two libraries are compiled from (names and contents).  Both builds
+    compile it in (mxq_build_digest / mxq_host_build_digest), so a library can be told apart from
+    one built from other sources -- the tests compare it with the tree they run in."""
+    h = hashlib.sha256()
+    files = [os.path.join(ROOT, "include", "mxq.h")]
+    files += sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".hip", ".cpp")))
+    for path in files:
+        h.update(os.path.basename(path).encode() + b"\0")
+        with open(path, "rb") as f:
+            h.update(f.read())
+        h.update(b"\0")
+    return h.hexdigest()
+
+
+def _digest_flag():
+    return '-DMXQ_BUILD_DIGEST="%s"' % source_digest()
 
 
 def _run(cmd, verbose):
@@ -47,7 +67,7 @@ def build_gpu(verbose=True):
     flags = ["--offload-arch=gfx950",
              # keep fp32 math scalar: packed fp32 instructions are not used by these kernels
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-             *[f for f in COMMON if f != "-shared"]]
+             *[f for f in COMMON if f != "-shared"], _digest_flag()]
     with tempfile.TemporaryDirectory(prefix="mxq_build_") as tmp:
         objects = [os.path.join(tmp, os.path.splitext(src)[0] + ".o") for src in GPU_SOURCES]
         with concurrent.futures.ThreadPoolExecutor(max_workers=len(GPU_SOURCES)) as pool:
@@ -60,10 +80,25 @@ def build_gpu(verbose=True):
 
 
 def build_host(verbose=True):
-    cmd = [os.path.join(ROCM, "lib", "llvm", "bin", "clang++"), *COMMON, "-o", HOST_LIB,
+    cmd = [os.path.join(ROCM, "lib", "llvm", "bin", "clang++"), *COMMON, _digest_flag(), "-o", HOST_LIB,
            os.path.join(CSRC, "mxq_host.cpp")]
     _run(cmd, verbose)
     return HOST_LIB
+
+
+def check_sources(verbose=False):
+    """Front-end pass (-fsyntax-only, host and gfx950) over every translation unit: seconds instead of
+    minutes, and enough to catch a source tree that does not compile (an identifier removed from one
+    header and still used by another file)."""
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    flags = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             *[f for f in COMMON if f != "-shared"], "-fsyntax-only"]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=len(GPU_SOURCES)) as pool:
+        jobs = [pool.submit(_run, [hipcc, *flags, os.path.join(CSRC, src)], verbose) for src in GPU_SOURCES]
+        for job in jobs:
+            job.result()
+    _run([os.path.join(ROCM, "lib", "llvm", "bin", "clang++"), *[f for f in COMMON if f != "-shared"], "-fsyntax-only",
+          os.path.join(CSRC, "mxq_host.cpp")], verbose)
 
 
 def build_all(verbose=True):

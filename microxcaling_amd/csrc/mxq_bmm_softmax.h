@@ -46,14 +46,14 @@ struct BmmSoftmaxArgs {
 namespace {
 
 constexpr int BS_ROWS = 32;                  // rows per workgroup
-constexpr int BS_TILES = 16;                 // 32-column tiles per wave: 4 x 16 x 32 = 2048 columns
+constexpr int BS_TILES = mxq_addr::S_TILES;  // 32-column tiles per wave: 4 x 16 x 32 = 2048 columns
 constexpr int BS_MAX_N = 4 * BS_TILES * 32;
-constexpr int BS_TILE_BYTES = 32 * 128;      // codes of a B tile
-constexpr int BS_RING = 3;                   // B tiles per wave in LDS: the one being multiplied and two on their way
+constexpr int BS_TILE_BYTES = mxq_addr::S_TILE_BYTES;   // codes of a B tile
+constexpr int BS_RING = mxq_addr::S_RING;    // B tiles per wave in LDS: the one being multiplied and two on their way
 
 template <int CBSZ, int BLGP>
 __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g) {
-    __shared__ __attribute__((aligned(16))) unsigned char ring[4 * BS_RING * BS_TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) unsigned char ring[mxq_addr::S_LDS_BYTES];
     __shared__ float red[2][4][BS_ROWS];
     __shared__ int votes[4];
 
@@ -86,31 +86,28 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
     // at position c ^ key(r), which makes the fragment reads below conflict free; the lanes pick
     // their global column accordingly.  A wave only reads what it fetched itself: s_waitcnt orders
     // the two, no barrier.
-    const uint32_t ring0 = (uint32_t)(uintptr_t)ring + (uint32_t)wave * (BS_RING * BS_TILE_BYTES);
+    const uint32_t ring0 = (uint32_t)(uintptr_t)ring;
     const unsigned char* Bt = g.b + bz * g.batch_b;
     uint32_t boff[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = i * 8 + (lane >> 3);
-        boff[i] = (uint32_t)(r * 128 + (((lane & 7) ^ mxq_addr::large_key(r)) * 16));
-    }
+    for (int i = 0; i < 4; ++i) boff[i] = mxq_addr::scores_code_offset(lane, i);
     // tile number i of this wave: the waves take pairs of neighbouring tiles (64 columns = one 128-byte
     // line of output per row) in turn
-    auto tile_of = [&](int i) { return 8 * (i >> 1) + 2 * wave + (i & 1); };
+    auto tile_of = [&](int i) { return mxq_addr::scores_tile_of(wave, i); };
     auto fetch_b = [&](int i) {                               // ... into slot i % BS_RING
         const int t = tile_of(i);
         if (t < ntiles) {                                     // uniform per wave
             const unsigned char* src = Bt + (int64_t)t * BS_TILE_BYTES;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) dma16(ring0 + (uint32_t)((i % BS_RING) * BS_TILE_BYTES + k * 1024), boff[k], src);
+            for (int k = 0; k < 4; ++k) dma16(ring0 + mxq_addr::scores_lds_dst(wave, i, k), boff[k], src);
         }
     };
     // fragment row fi is B row (permuted fi) of the tile, see the 256 x 256 kernel: accumulator
     // registers 0-7 of a lane are columns 8 fg .. 8 fg + 7 of the tile, 8-15 columns 16 + 8 fg .. + 7
-    const int b_lane = (fi & 16) + ((fi & 4) << 1) + ((fi & 8) >> 1) + (fi & 3);
+    const int b_lane = mxq_addr::large_frag_row_b(fi, true);
     int b_addr[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) b_addr[q] = b_lane * 128 + (((2 * q + fg) ^ mxq_addr::large_key(b_lane)) * 16);
+    for (int q = 0; q < 4; ++q) b_addr[q] = mxq_addr::scores_lds_addr(b_lane, 2 * q + fg);
     const unsigned char* my_ring = ring + wave * (BS_RING * BS_TILE_BYTES);
     // this wave's tiles are numbers 0 .. my_tiles - 1 of its sequence (tile_of grows with i)
     int my_tiles = 0;
@@ -176,8 +173,13 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
 #pragma unroll
     for (int i = 0; i < BS_TILES; ++i) {
         v16f next = acc;
-        // the fragment of tile i has been read (its MFMAs have been issued): its slot takes tile i + BS_RING
-        if (i + BS_RING < BS_TILES) fetch_b(i + BS_RING);
+        // the slot of tile i takes tile i + BS_RING once the reads of its fragment have returned their data:
+        // the copy is issued by inline assembly, which the compiler may move ahead of the MFMAs and of the
+        // wait it puts in front of them, and bytes written into LDS must not overtake a read still on its way
+        if (i + BS_RING < BS_TILES) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            fetch_b(i + BS_RING);
+        }
         if (i + 1 < BS_TILES) next = multiply(i + 1);
         if (tile_of(i) < ntiles) {                            // uniform per wave
 #pragma unroll
@@ -292,14 +294,14 @@ __global__ __launch_bounds__(TPB, 2) void mx_bmm_softmax_kernel(BmmSoftmaxArgs g
                         o[j] = (mxq_bits(q0) >> 16) | (mxq_bits(q1) & 0xFFFF0000u);
                     }
                 }
-                *reinterpret_cast<u32x4*>(buf + fi * 128 + (((4 * p + fg) ^ (fi & 7)) * 16)) = u32x4{o[0], o[1], o[2], o[3]};
-                *reinterpret_cast<u32x4*>(buf + fi * 128 + (((4 * p + 2 + fg) ^ (fi & 7)) * 16)) = u32x4{o[4], o[5], o[6], o[7]};
+                *reinterpret_cast<u32x4*>(buf + mxq_addr::scores_stage_addr(fi, 4 * p + fg)) = u32x4{o[0], o[1], o[2], o[3]};
+                *reinterpret_cast<u32x4*>(buf + mxq_addr::scores_stage_addr(fi, 4 * p + 2 + fg)) = u32x4{o[4], o[5], o[6], o[7]};
             }
             const bool second = t0 + 1 < ntiles;              // an odd number of tiles: the last line is half a line
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = 8 * r + srow;
-                const u32x4 v = *reinterpret_cast<const u32x4*>(buf + row * 128 + ((spiece ^ (row & 7)) * 16));
+                const u32x4 v = *reinterpret_cast<const u32x4*>(buf + mxq_addr::scores_stage_addr(row, spiece));
                 if (m0 + row < g.M && (second || spiece < 4))
                     __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out + (int64_t)(8 * r) * g.N + t0 * 32));
             }

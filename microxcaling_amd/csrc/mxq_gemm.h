@@ -774,14 +774,12 @@ __global__ __launch_bounds__(TPB) void gemm_split_reduce_kernel(const float* __r
 // fetches the first step of the next one, and the stores of a finished tile drain while the next
 // tile computes.
 // ================================================================================================
-constexpr int G3_TILE_BYTES = 256 * 128;
-constexpr int G3_STAGE_BYTES = 2 * G3_TILE_BYTES;            // codes of A and B for one K step
-constexpr int G3_SCALE_OFF = 2 * G3_STAGE_BYTES;
-constexpr int G3_SCALE_GROUP = 512 * 16;                     // 512 rows x 4 K steps x 4 bytes
-constexpr int G3_TAIL_OFF = G3_SCALE_OFF + 2 * G3_SCALE_GROUP;
-constexpr int G3_TAIL_PLANE = 512 * 4;                       // 512 rows x 4 scale bytes
-constexpr int G3_TAIL_SLOT = 2 * G3_TAIL_PLANE;              // one K step: one plane (8-bit) or two (nibbles)
-constexpr int G3_LDS_BYTES = G3_TAIL_OFF + 2 * G3_TAIL_SLOT;
+// the LDS image (mxq_gemm_addr.h)
+constexpr int G3_STAGE_BYTES = mxq_addr::L_STAGE_BYTES;      // codes of A and B for one K step
+constexpr int G3_SCALE_GROUP = mxq_addr::L_SCALE_GROUP;      // 512 rows x 4 K steps x 4 bytes
+constexpr int G3_TAIL_PLANE = mxq_addr::L_TAIL_PLANE;        // 512 rows x 4 scale bytes
+constexpr int G3_TAIL_SLOT = mxq_addr::L_TAIL_SLOT;          // one K step: one plane (8-bit) or two (nibbles)
+constexpr int G3_LDS_BYTES = mxq_addr::L_LDS_BYTES;
 
 __device__ __forceinline__ void dma16(uint32_t lds_base, uint32_t voff, const unsigned char* sbase) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -828,8 +826,6 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     // position of 16-byte column c of row r inside its LDS row: c ^ key(r); the key takes 8
     // different values over the even rows of any 16 consecutive rows (and again over the odd ones),
     // which is what a 16-byte read by 16 lanes needs to touch every bank once
-    auto key_a = [](int r) { return mxq_addr::large_key(r); };
-    auto key_b = key_a;
 
     // ---- fetch side: which tile the tile copy is working on --------------------------------------
     // Wave w brings in rows 32 w .. 32 w + 31 of A and of B, 8 rows per instruction; lane L lands at
@@ -860,21 +856,20 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     // load i (0..7 codes, 8 scales) of flat step t, which is K step fs of the fetch-side tile
     auto fetch_part = [&](int t, int fs, int i) {
         const int k0 = mxq_addr::large_kidx(f_kstart, fs, nk) * GEMM_BK;
-        const uint32_t st = lds0 + (t & 1) * G3_STAGE_BYTES;
         if (i < 4) {
-            dma16(st + (wave * 32 + i * 8) * 128, offa[i], fA + k0);
+            dma16(lds0 + mxq_addr::large_lds_code_dst(t, wave, i), offa[i], fA + k0);
         } else if (i < 8) {
-            dma16(st + G3_TILE_BYTES + (wave * 32 + (i - 4) * 8) * 128, offb[i - 4], fB + k0);
+            dma16(lds0 + mxq_addr::large_lds_code_dst(t, wave, i), offb[i - 4], fB + k0);
         } else if (fs < nfull) {
             if (fs % GS == 0) {                              // a new group of GS K steps
-                dma16(lds0 + G3_SCALE_OFF + (f_groups & 1) * G3_SCALE_GROUP + wave * 1024, offs,
+                dma16(lds0 + mxq_addr::large_lds_scale_group_dst(f_groups, wave), offs,
                       fS + mxq_addr::scale_byte_of(k0, EPB));
                 ++f_groups;
             }
         } else {                                             // past the last whole group: this step only
 #pragma unroll
             for (int e = 0; e < EPB; ++e)
-                dma4(lds0 + G3_TAIL_OFF + (fs & 1) * G3_TAIL_SLOT + e * G3_TAIL_PLANE + wave * 256, offs,
+                dma4(lds0 + mxq_addr::large_lds_scale_tail_dst(fs, e, wave), offs,
                      fS + mxq_addr::scale_byte_of(k0, EPB) + 4 * e);
         }
     };
@@ -888,15 +883,15 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     constexpr int NH = 2 * EPB;                              // MFMAs per fragment pair and K step
     const int fi = lane & 31, fg = lane >> 5;
     const int a_lane = wy * 64 + fi;                                          // row of A fragment 0
-    const int b_lane = wx * 128 + (PAIR ? (fi & 16) + ((fi & 4) << 1) + ((fi & 8) >> 1) + (fi & 3) : fi);
+    const int b_lane = wx * 128 + mxq_addr::large_frag_row_b(fi, PAIR);
     int a_addr[4], b_addr[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        a_addr[q] = a_lane * 128 + ((fg ^ key_a(a_lane) ^ (2 * q)) * 16);
-        b_addr[q] = G3_TILE_BYTES + b_lane * 128 + ((fg ^ key_b(b_lane) ^ (2 * q)) * 16);
+        a_addr[q] = mxq_addr::large_lds_code_addr(0, a_lane, 2 * q + fg);
+        b_addr[q] = mxq_addr::large_lds_code_addr(1, b_lane, 2 * q + fg);
     }
-    const int sa_off = G3_SCALE_OFF + a_lane * 16, sa_tail = G3_TAIL_OFF + a_lane * 4;
-    const int sb_off = G3_SCALE_OFF + 4096 + b_lane * 16, sb_tail = G3_TAIL_OFF + (256 + b_lane) * 4;
+    const int sa_off = mxq_addr::large_lds_scale_group_addr(0, a_lane), sa_tail = mxq_addr::large_lds_scale_tail_addr(0, a_lane);
+    const int sb_off = mxq_addr::large_lds_scale_group_addr(1, b_lane), sb_tail = mxq_addr::large_lds_scale_tail_addr(1, b_lane);
     const int sshift = fg * 8;
     constexpr int QH = 4 / NH;                               // 16-byte reads of a fragment per MFMA
     struct Half { u32x4 r[QH]; };
@@ -921,7 +916,7 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     // starts behind it (six of its nine loads in the last two groups, the rest in the first two
     // groups of step t + 1), which gives it more than a step to land.
     constexpr int NG = NH * 4;
-    constexpr int BP = NG - 3;                               // the group behind whose MFMAs the barrier stands
+    constexpr int BP = mxq_addr::large_barrier_group(NG);    // the group behind whose MFMAs the barrier stands
     // fetch side: the K step that the copy instructions issued now belong to
     int f_logical = blockIdx.x, f_fs = 0;
     auto fetch_advance = [&]() {
@@ -999,12 +994,7 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
                 acc[ti][tj] = mx_mfma32_half<CBSZ, BLGP>(bfh, afh[ti], acc[ti][tj], sbv[tj], sa[ti], h);
             asm volatile("" : "+v"(acc[0][tj]), "+v"(acc[1][tj]));
             __builtin_amdgcn_sched_barrier(0);
-            if (gi == 0) {                                   // copy of the next step, loads 6 .. 8
-                fetch_part(t + 1, f_fs, 6);
-                fetch_part(t + 1, f_fs, 7);
-            } else if (gi == 1) {
-                fetch_part(t + 1, f_fs, 8);
-            } else if (gi == BP) {
+            if (gi == BP) {
                 asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // this wave's share of the next stage is in,
                 __syncthreads();                                              // everybody's is; and this stage is free
                 fetch_advance();
@@ -1017,10 +1007,11 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
                     sa_n[ti] = scales(sa_off + ti * 512, sa_tail + ti * 128);
                 }
             }
-            if (gi > BP) {                                   // copy of the step after next, loads 0 .. 5
+            // this group's share of the tile copy: loads 0 .. 5 of the step after next in the two groups
+            // behind the barrier, loads 6 .. 8 of what is then the next step in the first two groups
 #pragma unroll
-                for (int i = 0; i < 3; ++i) fetch_part(t, f_fs, (gi - BP - 1) * 3 + i);
-            }
+            for (int i = 0; i < mxq_addr::large_copy_count(gi, NG); ++i)
+                fetch_part(t + mxq_addr::large_copy_ahead(gi, NG), f_fs, mxq_addr::large_copy_first(gi, NG) + i);
             __builtin_amdgcn_sched_barrier(0);
             bfh = bfh_next;
             afh[0] = afh_next[0];
@@ -1063,7 +1054,6 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
         // Inside tiles: a lane holds the 16-byte pieces fg, 2 + fg (, 4 + fg, 6 + fg) of its row of
         // a fragment; after the exchange with lane L +- 16 it holds piece 2 * (L / 16 % 2) + fg of
         // row L % 16 and the same piece of row 16 + L % 16 (see swap_with_lane16).
-        const int half = (lane >> 4) & 1, m16 = lane & 15;
 #pragma unroll
         for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
@@ -1076,18 +1066,20 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
                         u32x4 p[2];
 #pragma unroll
                         for (int h = 0; h < 2; ++h)
-                            p[h] = epilogue_pack8<OUT_DT>(g.bias, g.q_nan_from, nt + 16 * h + 8 * fg,
+                            p[h] = epilogue_pack8<OUT_DT>(g.bias, g.q_nan_from, nt + mxq_addr::large_own_col(lane, h, 8),
                                                           v4f{c[8 * h], c[8 * h + 1], c[8 * h + 2], c[8 * h + 3]},
                                                           v4f{c[8 * h + 4], c[8 * h + 5], c[8 * h + 6], c[8 * h + 7]});
                         swap_with_lane16(p[0], p[1]);
-                        unsigned short* out = reinterpret_cast<unsigned short*>(g.c) + cbase +
-                                              (int64_t)(mt + m16) * g.N + nt + 8 * (2 * half + fg);
-                        MXQ_C_STORE(reinterpret_cast<u32x4*>(out), p[0]);
-                        MXQ_C_STORE(reinterpret_cast<u32x4*>(out + (int64_t)16 * g.N), p[1]);
+                        unsigned short* out = reinterpret_cast<unsigned short*>(g.c) + cbase + nt +
+                                              mxq_addr::large_swapped_col(lane, 8);
+#pragma unroll
+                        for (int w = 0; w < 2; ++w)
+                            MXQ_C_STORE(reinterpret_cast<u32x4*>(out + (int64_t)(mt + mxq_addr::large_swapped_row(lane, w)) * g.N), p[w]);
                     } else {
 #pragma unroll
                         for (int h = 0; h < 2; ++h)
-                            store_c8<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, mt + fi, nt + 16 * h + 8 * fg, g.M, g.N,
+                            store_c8<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, mt + mxq_addr::large_own_row(lane),
+                                             nt + mxq_addr::large_own_col(lane, h, 8), g.M, g.N,
                                              false, v4f{c[8 * h], c[8 * h + 1], c[8 * h + 2], c[8 * h + 3]},
                                              v4f{c[8 * h + 4], c[8 * h + 5], c[8 * h + 6], c[8 * h + 7]});
                     }
@@ -1101,15 +1093,17 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
 #pragma unroll
                                 for (int r = 0; r < 4; ++r) p[e][r] = __float_as_uint(c[4 * (q + e) + r]);
                             swap_with_lane16(p[0], p[1]);
-                            float* out = reinterpret_cast<float*>(g.c) + cbase + (int64_t)(mt + m16) * g.N + nt +
-                                         8 * q + 4 * (2 * half + fg);
-                            MXQ_C_STORE(reinterpret_cast<u32x4*>(out), p[0]);
-                            MXQ_C_STORE(reinterpret_cast<u32x4*>(out + (int64_t)16 * g.N), p[1]);
+                            float* out = reinterpret_cast<float*>(g.c) + cbase + nt + 8 * q +
+                                         mxq_addr::large_swapped_col(lane, 4);
+#pragma unroll
+                            for (int w = 0; w < 2; ++w)
+                                MXQ_C_STORE(reinterpret_cast<u32x4*>(out + (int64_t)(mt + mxq_addr::large_swapped_row(lane, w)) * g.N), p[w]);
                         }
                     } else {
 #pragma unroll
                         for (int q = 0; q < 4; ++q)
-                            store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, mt + fi, nt + 8 * q + 4 * fg, g.M, g.N,
+                            store_c4<OUT_DT>(g.c, g.bias, g.q_nan_from, cbase, mt + mxq_addr::large_own_row(lane),
+                                             nt + mxq_addr::large_own_col(lane, q, 4), g.M, g.N,
                                              inside, v4f{c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]});
                     }
                 }

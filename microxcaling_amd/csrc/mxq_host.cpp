@@ -75,6 +75,11 @@ extern "C" {
 
 const char* mxq_host_last_error(void) { return last_error().c_str(); }
 
+#ifndef MXQ_BUILD_DIGEST
+#define MXQ_BUILD_DIGEST "unknown"
+#endif
+const char* mxq_host_build_digest(void) { return MXQ_BUILD_DIGEST; }
+
 int mxq_host_quantize_mx_by_tile(const void* in, void* out, int dtype, int64_t pre, int64_t axis_size,
                                  int64_t post, int scale_bits, int elem_ebits, int elem_mbits,
                                  float elem_max_norm, int64_t tile_size, int flush_fp32_subnorms,

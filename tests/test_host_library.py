@@ -48,6 +48,22 @@ def test_libraries_export_every_declared_symbol():
     assert set(_lib.GPU_SYMBOLS) | set(_lib.HOST_SYMBOLS) == set(declared_symbols())
 
 
+def test_every_translation_unit_compiles():
+    """A front-end pass over every source of both libraries (seconds): a tree in which one file uses what
+    another no longer defines does not get past this."""
+    from microxcaling_amd import build_ext
+    build_ext.check_sources()
+
+
+def test_the_libraries_in_the_tree_are_built_from_the_sources_in_the_tree():
+    """Both libraries carry the digest of the sources they were compiled from; it must be the digest of
+    the source files next to them (otherwise: python -m microxcaling_amd.build_ext)."""
+    from microxcaling_amd import build_ext
+    want = build_ext.source_digest().encode()
+    assert _lib.gpu().mxq_build_digest() == want, "libmxq_gfx950.so is stale: rebuild it"
+    assert _lib.host().mxq_host_build_digest() == want, "libmxq_host.so is stale: rebuild it"
+
+
 def test_gpu_entry_points_reject_bad_arguments_without_a_gpu():
     lib = _lib.gpu()
     assert lib.mxq_version() >= 100
@@ -428,12 +444,7 @@ def test_fp16_conversions_of_the_scalar_core(tmp_path, compiler):
     assert_bits_equal(got_f, x.half().float(), "fp16 -> fp32")
 
 
-def test_gemm_tile_copies_stay_inside_their_operands(tmp_path):
-    """tests/cpp/gemm_addr_check.cpp walks every (workgroup, tile, K step, load, wave, lane) of both
-    GEMM kernels through the address functions the kernels are compiled from
-    (microxcaling_amd/csrc/mxq_gemm_addr.h) and checks every 16- and 4-byte range against the size of
-    the operand it reads: the benchmark shapes, ragged M / N, K % 512 != 0, nibbles, batches, K
-    splits.  Exits non-zero at the first range outside."""
+def _build_gemm_addr_check(tmp_path, include_dir=None):
     import shutil
     import subprocess
     cxx = shutil.which("g++") or shutil.which("c++")
@@ -441,12 +452,67 @@ def test_gemm_tile_copies_stay_inside_their_operands(tmp_path):
         pytest.skip("no host C++ compiler")
     exe = str(tmp_path / "gemm_addr_check")
     subprocess.run([cxx, "-O2", "-std=c++17", "-I", os.path.join(ROOT_DIR, "include"),
-                    "-I", os.path.join(ROOT_DIR, "microxcaling_amd", "csrc"), "-o", exe,
+                    "-I", include_dir or os.path.join(ROOT_DIR, "microxcaling_amd", "csrc"), "-o", exe,
                     os.path.join(ROOT_DIR, "tests", "cpp", "gemm_addr_check.cpp")], check=True)
-    res = subprocess.run([exe], capture_output=True, text=True, timeout=600)
-    assert res.returncode == 0 and "OUT OF BOUNDS" not in res.stdout, res.stdout[-2000:]
-    assert "byte ranges inside their operands" in res.stdout
-    assert res.stdout.count("256 x 256 tiles") == 11 and res.stdout.count("128 x 128 tiles") == 20
+    return exe
+
+
+def test_gemm_copies_lds_image_schedule_and_stores_on_the_host(tmp_path):
+    """tests/cpp/gemm_addr_check.cpp, through the address functions the kernels are compiled from
+    (microxcaling_amd/csrc/mxq_gemm_addr.h): every 16- and 4-byte range of the tile copies of both GEMM
+    kernels inside its operand (benchmark shapes, ragged M / N, K % 512 != 0, nibbles, batches, K
+    splits); the 256 x 256 kernel's LDS replayed K step by K step (landing ranges, the bytes every
+    fragment and scale read returns, copies against the barriers, registers against the MFMA groups);
+    its output stores (every element once, by the lane that holds it, inside and aligned); the
+    attention-score kernel's ring, waits, staging and stores.  Exits non-zero at the first violation."""
+    import subprocess
+    exe = _build_gemm_addr_check(tmp_path)
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=900)
+    out = res.stdout
+    assert res.returncode == 0, out[-2000:]
+    for word in ("OUT OF BOUNDS", "LDS MODEL:", "STORES:", "SCORES:"):
+        assert word not in out, out[-2000:]
+    assert "byte ranges inside their operands" in out
+    assert out.count("256 x 256 tiles") == 11 and out.count("128 x 128 tiles") == 20
+    assert out.count("all as the MFMAs want them") == 11
+    assert out.count("each once and in place") == 33 and out.count("scores kernel") == 6
+
+
+@pytest.mark.parametrize("what, old, new, says", [
+    ("the step's barrier one group later",
+     "constexpr int large_barrier_group(int ng) { return ng - 3; }",
+     "constexpr int large_barrier_group(int ng) { return ng - 2; }", "LDS MODEL:"),
+    ("copies behind the barrier aimed at the stage still being read",
+     "return gi > large_barrier_group(ng) ? 2 : 1; }", "return 1; }", "LDS MODEL: copy issued into bytes that are read"),
+    ("a copy instruction short per step",
+     "gi > large_barrier_group(ng) ? 3 : 0;", "gi > large_barrier_group(ng) ? 2 : 0;", "LDS MODEL: a fragment read returns the wrong bytes"),
+    ("code rows landing one row down",
+     "(wave * 32 + (i & 3) * 8) * 128);", "(wave * 32 + (i & 3) * 8 + 1) * 128);", "LDS MODEL: copy lands outside its LDS region"),
+    ("the exchanged pieces stored at the wrong columns",
+     "return elems * (2 * ((lane >> 4) & 1) + (lane >> 5)); }", "return elems * (((lane >> 4) & 1) + 2 * (lane >> 5)); }",
+     "STORES: a value is stored at another element's place"),
+    ("another permutation of the B fragment rows",
+     "(fi & 16) + ((fi & 4) << 1) + ((fi & 8) >> 1) + (fi & 3)", "(fi & 16) + (fi & 8) + (fi & 4) + (fi & 3)",
+     "STORES: a lane's own columns are not where its registers belong"),
+    ("score tiles dealt to the waves one by one",
+     "return 8 * (i >> 1) + 2 * wave + (i & 1); }", "return 4 * i + wave; }", "SCORES:"),
+    ("score copies fetching a neighbouring column",
+     "(((lane & 7) ^ large_key(r)) * 16));\n}\n// where column col16 of tile row", "(((lane & 7) ^ large_key(r + 2)) * 16));\n}\n// where column col16 of tile row",
+     "SCORES: a fragment read returns the wrong bytes"),
+])
+def test_the_host_check_notices_a_wrong_address_function(tmp_path, what, old, new, says):
+    """The check above must be able to fail: the same program compiled against a copy of the address
+    header with one function changed stops at the violation that change causes."""
+    import subprocess
+    src = open(os.path.join(ROOT_DIR, "microxcaling_amd", "csrc", "mxq_gemm_addr.h")).read()
+    old, new = old.replace("\\n", "\n"), new.replace("\\n", "\n")
+    assert src.count(old) == 1, what
+    inc = tmp_path / "inc"
+    inc.mkdir()
+    (inc / "mxq_gemm_addr.h").write_text(src.replace(old, new))
+    exe = _build_gemm_addr_check(tmp_path, str(inc))
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=900)
+    assert res.returncode == 1 and says in res.stdout, (what, res.stdout[-1500:])
 
 
 def test_dither_reproduces_the_reference_under_the_same_seed():
