@@ -2,10 +2,10 @@
 import torch
 import torch.nn.functional as F
 
-from .norm_utils import _norm_backward_LN, _norm_forward
+from .norm_utils import (layer_norm_rows, layer_norm_rows_grad_input, rms_norm_rows,
+                         rms_norm_rows_grad_input)
 from .specs import apply_mx_specs, get_backwards_mx_specs, mx_assert_test
-from .vector_ops import (vec_add, vec_mul, vec_quantize, vec_recip, vec_reduce_mean, vec_reduce_sum,
-                         vec_sqrt, vec_sub)
+from .vector_ops import vec_mul, vec_quantize, vec_reduce_sum
 
 torch_layer_norm = F.layer_norm
 
@@ -156,8 +156,8 @@ class LayerNormFunction(torch.autograd.Function):
         if fused is not None:
             output, x_norm, x_vare = fused
         else:
-            x = vec_quantize(x, mx_specs=mx_specs)
-            output, _, x_norm, _, _, x_vare = _norm_forward(x, -1, bf_weight, bf_bias, eps, mx_specs)
+            output, x_norm, x_vare = layer_norm_rows(vec_quantize(x, mx_specs=mx_specs), bf_weight, bf_bias, eps,
+                                                     mx_specs)
         ctx.save_for_backward(x_norm, x_vare, bf_weight if mx_specs['quantize_backprop'] else weight)
         ctx.mx_specs = get_backwards_mx_specs(mx_specs)
         return output
@@ -173,7 +173,7 @@ class LayerNormFunction(torch.autograd.Function):
         grad_weight, grad_bias = _param_grads(grad_output, x_norm, s)
         grad_input = _fused_grad_input(grad_output, weight, x_norm, x_vare, s, rms=False)
         if grad_input is None:
-            grad_input = _norm_backward_LN(grad_output, -1, weight, x_norm, x_vare, s)
+            grad_input = layer_norm_rows_grad_input(grad_output, weight, x_norm, x_vare, s)
         return (grad_input, grad_weight, grad_bias, None, None, None)
 
 
@@ -190,11 +190,7 @@ class RMSNormFunction(torch.autograd.Function):
         if fused is not None:
             output, x_norm, rms_inv = fused
         else:
-            x = vec_quantize(x, mx_specs=s)
-            ms = vec_reduce_mean(vec_mul(x, x, mx_specs=s), -1, keepdim=True, mx_specs=s)
-            rms_inv = vec_recip(vec_sqrt(vec_add(ms, eps, mx_specs=s), mx_specs=s), mx_specs=s)
-            x_norm = vec_mul(x, rms_inv, mx_specs=s)
-            output = vec_add(vec_mul(bf_weight, x_norm, mx_specs=s), bf_bias, mx_specs=s)
+            output, x_norm, rms_inv = rms_norm_rows(vec_quantize(x, mx_specs=s), bf_weight, bf_bias, eps, s)
         ctx.save_for_backward(x_norm, rms_inv, bf_weight if s['quantize_backprop'] else weight)
         ctx.mx_specs = get_backwards_mx_specs(s)
         return output
@@ -211,10 +207,7 @@ class RMSNormFunction(torch.autograd.Function):
         fused = _fused_grad_input(grad_output, weight, x_norm, rms_inv, s, rms=True)
         if fused is not None:
             return (fused, grad_weight, grad_bias, None, None, None)
-        dx1 = vec_mul(vec_mul(grad_output, weight, mx_specs=s), rms_inv, mx_specs=s)
-        proj = vec_reduce_mean(vec_mul(dx1, x_norm, mx_specs=s), -1, keepdim=True, mx_specs=s)
-        # the last subtraction carries no mx_specs in the reference (mx/layernorm.py:166): unquantized
-        grad_input = vec_sub(dx1, vec_mul(x_norm, proj, mx_specs=s))
+        grad_input = rms_norm_rows_grad_input(grad_output, weight, x_norm, rms_inv, s)
         return (grad_input, grad_weight, grad_bias, None, None, None)
 
 
