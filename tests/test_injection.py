@@ -70,3 +70,56 @@ def test_injected_ffn_on_cpu():
 @pytest.mark.gpu
 def test_injected_ffn_on_gpu():
     _run("cuda")
+
+
+UNPORTED_SCRIPT = r'''
+import sys, warnings
+sys.path.insert(0, %(root)r)
+import torch
+import torch.nn.functional as F
+from microxcaling_amd import finalize_mx_specs, mx_mapping
+
+specs = finalize_mx_specs({'w_elem_format': 'fp8_e4m3', 'a_elem_format': 'fp8_e4m3', 'block_size': 32, 'bfloat': 16})
+with warnings.catch_warnings(record=True) as seen:
+    warnings.simplefilter("always")
+    mx_mapping.inject_pyt_ops(specs)
+    mx_mapping.inject_pyt_ops(specs)                       # injecting twice wraps torch's classes, not the wrappers
+assert len(seen) == 2 and all(issubclass(w.category, mx_mapping.UnportedOpWarning) for w in seen)
+assert "torch.add" in str(seen[0].message) and "torch.square" in str(seen[0].message)
+
+with warnings.catch_warnings(record=True) as seen:
+    warnings.simplefilter("always")
+    bn = torch.nn.BatchNorm2d(8)
+    lin = torch.nn.Linear(32, 32)                          # provided: no warning
+    y = F.group_norm(torch.randn(2, 8, 4), 2)
+names = [str(w.message).split(":")[0] for w in seen]
+assert names == ["torch.nn.BatchNorm2d", "torch.nn.functional.group_norm"], names
+assert isinstance(bn, torch.nn.modules.batchnorm.BatchNorm2d) and type(bn).__mro__[1].__name__ == "BatchNorm2d"
+assert bn(torch.randn(2, 8, 4, 4)).shape == (2, 8, 4, 4) and y.shape == (2, 8, 4)
+assert type(lin).__name__ == "Linear_inj"
+
+mx_mapping.inject_pyt_ops(specs, unported="raise")
+for make in (lambda: torch.nn.LSTM(4, 4), lambda: torch.nn.GroupNorm(2, 8), lambda: F.batch_norm(torch.randn(2, 3), None, None, training=True)):
+    try:
+        make()
+    except NotImplementedError as e:
+        assert "unquantized" in str(e)
+    else:
+        raise AssertionError("no error")
+
+with warnings.catch_warnings(record=True) as seen:
+    warnings.simplefilter("always")
+    mx_mapping.inject_pyt_ops(specs, unported="ignore")
+assert not seen
+print("OK")
+'''
+
+
+def test_injection_names_the_ops_it_does_not_provide():
+    """The reference's inject_pyt_ops also rebinds batch / group norm, transposed convolution, pooling, LSTM
+    and the tensor-level simd ops (mx/mx_mapping.py:68-122).  This package does not restate them; a model
+    that uses them must hear about it (or fail, with unported='raise') instead of running them unquantized
+    in silence."""
+    res = subprocess.run([sys.executable, "-c", UNPORTED_SCRIPT % {"root": ROOT_DIR}], capture_output=True, text=True,
+                         timeout=600)
+    assert res.returncode == 0 and "OK" in res.stdout, res.stdout + res.stderr
