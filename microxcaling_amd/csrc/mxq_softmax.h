@@ -165,8 +165,11 @@ __global__ __launch_bounds__(TPB) void softmax_row_kernel(const void* __restrict
                     uint32_t dw = packed(x[e] - m, x[e + 1] - m);
                     if (p.exp_mode == 2) dw = packed(1.4453125f * low_of(dw), 1.4453125f * high_of(dw));
                     // arguments in [-85, 0] (2^x: [-123, 0]): the results are normal numbers, which the
-                    // hardware exponential (v_exp_f32, 1 ulp, flushes subnormal results only) returns
-                    // without the range handling of expf / exp2f
+                    // hardware exponential (v_exp_f32: about 1 ulp, flushes subnormal results only) returns
+                    // without the range handling of expf / exp2f.  For e^x the fp32 product x * log2(e) in
+                    // front of it is rounded at magnitudes up to 123 (half an ulp there is 2^-18), which
+                    // moves the result by up to 2.6e-6 of its value -- about 45 fp32 ulps at x = -85, not
+                    // the 1-2 ulps of expf, and a 1500th of the bfloat16 rounding step that follows.
                     const uint32_t ew = p.exp_mode == 0 ? packed(fast_exp2(1.44269504f * low_of(dw)), fast_exp2(1.44269504f * high_of(dw)))
                                                         : packed(fast_exp2(low_of(dw)), fast_exp2(high_of(dw)));
                     x[e] = low_of(ew);

@@ -161,7 +161,13 @@ class Linear(torch.nn.Linear):
         GEMM reads it directly: 1 + 1/32 bytes per weight (1/2 + 1/32 when both formats are fp4)
         against 2.  keep_dense=False also drops the bf16 weight once its codes exist (weight.data
         becomes an empty tensor): the layer then holds a half to a quarter of the bytes and serves
-        GPU inputs through the fused GEMM only."""
+        bf16 GPU inputs through the fused GEMM only (anything else raises).  The codes and scales
+        then are buffers of the module (weight_codes, weight_scales, weight_code_kind): they move
+        with .to() / .cuda() and are part of state_dict(), and a fresh layer loads such a state.
+        The cached form of a kept weight follows the weight's version counter and device; after
+        changing weight.data in place (which bumps no counter) call prequantize_weights() again."""
+        if self._dense_dropped():
+            raise RuntimeError("prequantize_weights: the dense weight of this layer has been dropped already")
         self._keep_dense = keep_dense
         self._packed_weight = None
         if self.mx_none:
@@ -182,16 +188,23 @@ class Linear(torch.nn.Linear):
                     round=self.mx_specs["round_weight"]).to(torch.bfloat16)
         self.prequantized_weights = True
 
+    def _dense_dropped(self):
+        return getattr(self, "weight_codes", None) is not None
+
     def _packed(self, inputs):
-        """The cached MX form of the prequantized weight for this input, or None."""
+        """The MX form of the prequantized weight for this input, or None."""
         from . import fused
         from .gemm import fused_enabled
         if not (self.prequantized_weights and fused_enabled() and inputs.is_cuda
                 and inputs.dtype == torch.bfloat16):
             return None
+        if self._dense_dropped():
+            if self.weight_codes.device != inputs.device:
+                return None
+            return (self.weight_codes, self.weight_scales, int(self.weight_code_kind))
         w = self.weight
         key = (w.data_ptr(), w._version, w.device, tuple(w.shape))
-        if self._packed_weight is None or (w.numel() and self._packed_weight[0] != key):
+        if self._packed_weight is None or self._packed_weight[0] != key:
             if not w.is_cuda or w.numel() == 0:
                 return None
             packed = fused.pack_weight(w.data, self.mx_specs["a_elem_format"], self.mx_specs["w_elem_format"],
@@ -199,18 +212,42 @@ class Linear(torch.nn.Linear):
             if packed is None:
                 return None
             if not self._keep_dense:
+                codes, scales, kind = packed
+                self.register_buffer("weight_codes", codes)
+                self.register_buffer("weight_scales", scales)
+                self.register_buffer("weight_code_kind", torch.tensor(int(kind), dtype=torch.int32))
                 with torch.no_grad():
                     self.weight.data = torch.empty(0, dtype=w.dtype, device=w.device)
-                key = None
+                self._packed_weight = None
+                return packed
             self._packed_weight = (key, packed)
         return self._packed_weight[1]
 
     def packed_weight_bytes(self):
-        """Bytes of the cached MX form (codes + scales), 0 before the first GPU forward pass."""
+        """Bytes of the MX form the layer holds (codes + scales), 0 before the first GPU forward pass."""
+        if self._dense_dropped():
+            return self.weight_codes.numel() + self.weight_scales.numel()
         if getattr(self, "_packed_weight", None) is None:
             return 0
         codes, scales, _ = self._packed_weight[1]
         return codes.numel() + scales.numel()
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        # a state saved after prequantize_weights(keep_dense=False): codes and scales instead of the weight
+        codes = state_dict.get(prefix + "weight_codes")
+        if codes is not None and not self._dense_dropped():
+            dev = self.weight.device
+            self.register_buffer("weight_codes", torch.empty_like(codes, device=dev))
+            self.register_buffer("weight_scales", torch.empty_like(state_dict[prefix + "weight_scales"], device=dev))
+            self.register_buffer("weight_code_kind", torch.zeros((), dtype=torch.int32))
+            with torch.no_grad():
+                self.weight.data = torch.empty(0, dtype=torch.bfloat16, device=dev)
+                if self.bias is not None:
+                    self.bias.data = self.bias.data.to(torch.bfloat16)
+            self.prequantized_weights = True
+            self._keep_dense = False
+            self._packed_weight = None
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def forward(self, inputs):
         if self.mx_none:
@@ -219,5 +256,10 @@ class Linear(torch.nn.Linear):
         if self.prequantized_weights:
             assert self.training == False, "Cannot use prequantized weights when training!"
             packed = self._packed(inputs)
+            if packed is None and self._dense_dropped():
+                raise RuntimeError(
+                    "Linear: this layer dropped its dense weight (prequantize_weights(keep_dense=False)) and holds "
+                    "only MX codes on %s: it serves bfloat16 inputs on that device through the fused GEMM "
+                    "(gemm.set_fused(True)), not a %s input on %s" % (self.weight_codes.device, inputs.dtype, inputs.device))
         return linear(input=inputs, weight=self.weight, bias=self.bias, mx_specs=self.mx_specs,
                       prequantized_weights=self.prequantized_weights, name=self.name, packed_weight=packed)
