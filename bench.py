@@ -452,13 +452,27 @@ MFMA_PEAK_TFLOPS = {"fp8": 5000.0, "fp4": 10100.0}
 
 
 def measured_traffic(workload):
-    """HBM bytes per launch of the workload's dominant kernel, measured separately with
-    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (the summaries are in profiles/)."""
-    tfile = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
+    """HBM bytes per launch of the workload's dominant kernel, measured separately with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE (the summaries are in profiles/) -- but only while the kernel's source files
+    are the ones that summary was taken with: a figure from another build of the kernel is not this
+    build's traffic.  -> (bytes or None, where the last measurement is and whether it is current)"""
+    import hashlib
+    here = os.path.dirname(os.path.abspath(__file__))
+    tfile = os.path.join(here, "profiles", "traffic.json")
     if not os.path.exists(tfile):
-        return None
+        return None, None
     with open(tfile) as f:
-        return json.load(f).get(workload)
+        entry = json.load(f).get(workload)
+    if not isinstance(entry, dict):
+        return None, None
+    h = hashlib.sha256()
+    for name in entry["sources"]:
+        with open(os.path.join(here, "microxcaling_amd", "csrc", name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read() + b"\0")
+    current = not entry["sources"] or h.hexdigest() == entry["sources_sha256"]
+    note = {"last_measured_bytes": entry["bytes"], "summary": entry["profile"],
+            "kernel_sources_unchanged_since": current}
+    return (entry["bytes"] if current else None), note
 
 
 METRIC = "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s"
@@ -503,7 +517,7 @@ def flops_report(name, wl, steps, warmup, ms_per_step, step_gpu_ms, kernel_ms, c
     if kernel_ms is not None:
         achieved = wl["gemm_flops"] / (kernel_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": measured_traffic(name),
+                "frac": round(achieved / peak, 4), "traffic": measured_traffic(name)[0], "traffic_source": measured_traffic(name)[1],
                 "kernel": wl["gemm_kernel"], "launch_ms_avg": round(kernel_ms, 5),
                 "step_gpu_ms_avg": round(step_gpu_ms, 5),
                 "note": "GEMM kernel alone (operands packed beforehand) over the dense %s MFMA peak; the whole "
@@ -513,7 +527,7 @@ def flops_report(name, wl, steps, warmup, ms_per_step, step_gpu_ms, kernel_ms, c
     else:
         achieved = wl["flops"] / (step_gpu_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": measured_traffic(name),
+                "frac": round(achieved / peak, 4), "traffic": measured_traffic(name)[0], "traffic_source": measured_traffic(name)[1],
                 "step_gpu_ms_avg": round(step_gpu_ms, 5),
                 "note": "whole step (all launches) over the dense %s MFMA peak" % wl.get("peak", "fp8")}
     out = {"metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps,
@@ -550,7 +564,7 @@ def bytes_report(name, wl, steps, warmup, ms_per_step, kern_avg_ms, cpu):
                    "algorithmic_bytes_per_step": wl["bytes"],
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(name),
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(name)[0], "traffic_source": measured_traffic(name)[1],
                      "launch_ms_avg": round(kern_avg_ms, 5),
                      "launches_per_step": wl.get("launches", 1)},
     }
