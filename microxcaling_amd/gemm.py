@@ -31,6 +31,22 @@ def fused_enabled():
     return _use_fused
 
 
+_defer_scores = True
+
+
+def set_deferred_scores(enabled):
+    """mx.bmm on attention-shaped inference operands returns its product unevaluated (bmm.DeferredProduct)
+    so that an mx.softmax over the last axis right after it can run product and softmax as one kernel;
+    anything else that touches the result evaluates the product first.  enabled=False: mx.bmm always
+    evaluates at once."""
+    global _defer_scores
+    _defer_scores = bool(enabled)
+
+
+def deferred_scores_enabled():
+    return _use_fused and _defer_scores
+
+
 def _epilogue_mode(mx_specs, round, dtype):
     """How the layers' "elementwise-quantize the product (, add the bias, quantize again)" can ride
     in the fused GEMM's epilogue: 0 = the quantizer is the identity (plain rounding to the tensor

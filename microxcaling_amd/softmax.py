@@ -124,7 +124,11 @@ def softmax(input, dim=-1, mx_specs=None, name=None):
     if mx_specs is None:
         return f_softmax(input, dim=dim)
     mx_specs = apply_mx_specs(mx_specs)
-    return SoftmaxFunction.apply(input, dim, mx_specs, name)
+    from .bmm import evaluated, softmax_of_deferred
+    out = softmax_of_deferred(input, dim, mx_specs)          # mx.bmm's product, still pending: one kernel for both
+    if out is not None:
+        return out
+    return SoftmaxFunction.apply(evaluated(input), dim, mx_specs, name)
 
 
 class Softmax(nn.Softmax):

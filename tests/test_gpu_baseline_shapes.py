@@ -22,6 +22,16 @@ from oracle import mx_oracle as O
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture(autouse=True)
+def products_evaluated_at_once():
+    """mx.bmm as a kernel of its own in this file: the tests here compare the separate kernels with each other
+    and with mx.bmm_softmax (the deferred product of mx.bmm has tests/test_zv_deferred_product_gpu.py)."""
+    from microxcaling_amd import gemm
+    gemm.set_deferred_scores(False)
+    yield
+    gemm.set_deferred_scores(True)
+
 ROUNDS = ["nearest", "floor", "even"]
 BF16_MAX = 2 ** 127 * 255 / 128
 

@@ -6,6 +6,16 @@ from helpers import assert_bits_equal
 from oracle import mx_oracle as O
 
 pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def products_evaluated_at_once():
+    """mx.bmm as a kernel of its own in this file: the tests here compare the separate kernels with each other
+    and with mx.bmm_softmax (the deferred product of mx.bmm has tests/test_zv_deferred_product_gpu.py)."""
+    from microxcaling_amd import gemm
+    gemm.set_deferred_scores(False)
+    yield
+    gemm.set_deferred_scores(True)
 PACKABLE = ["fp8_e4m3", "fp8_e5m2", "fp6_e3m2", "fp6_e2m3", "fp4_e2m1"]
 
 

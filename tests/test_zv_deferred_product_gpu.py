@@ -1,0 +1,75 @@
+"""mx.softmax(mx.bmm(q, k^T), dim=-1) on the GPU -- the reference's own call sequence for attention scores
+(mx/bmm.py:138-145, mx/softmax.py:91-97) -- through mx.bmm's deferred product: the one-launch kernel is
+reached, with the results of mx.bmm_softmax bit for bit; anything else done to the product gives what the
+separate kernels give.  The laziness itself is tested on CPU tensors in tests/test_deferred_product.py."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _specs(**kw):
+    from microxcaling_amd.specs import finalize_mx_specs
+    return finalize_mx_specs(dict(kw), early_exit=False)
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need a GPU"
+    return torch.device("cuda:0")
+
+
+@pytest.mark.parametrize("shape", [(4, 256, 2048), (3, 33, 544), (130, 32, 32)])
+@pytest.mark.parametrize("fmt,exp2", [("fp6_e2m3", False), ("fp8_e4m3", True)])
+def test_softmax_of_bmm_is_the_one_launch_kernel(dev, shape, fmt, exp2):
+    from microxcaling_amd import gemm
+    from microxcaling_amd.bmm import DeferredProduct, bmm, bmm_softmax
+    from microxcaling_amd.softmax import Softmax, softmax
+    B, M, N = shape
+    specs = _specs(a_elem_format=fmt, block_size=32, bfloat=16, softmax_exp2=exp2, custom_cuda=True)
+    g = torch.Generator().manual_seed(B + M + N)
+    q = torch.randn(B, M, 128, generator=g).to(torch.bfloat16).to(dev)
+    kt = torch.randn(B, N, 128, generator=g).to(torch.bfloat16).to(dev).transpose(-1, -2)
+    want = bmm_softmax(q, kt, mx_specs=specs)
+    with torch.no_grad():
+        prod = bmm(q, kt, mx_specs=specs)
+        assert type(prod) is DeferredProduct and prod.shape == (B, M, N)
+        got = softmax(prod, dim=-1, mx_specs=specs)
+        assert prod.pending() is not None                                    # the logits were never written
+        via_module = Softmax(dim=-1, mx_specs=specs)(bmm(q, kt, mx_specs=specs))
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(via_module.view(torch.int16), want.view(torch.int16))
+    # the product as a tensor: what the GEMM kernel gives when mx.bmm evaluates at once
+    gemm.set_deferred_scores(False)
+    try:
+        eager = bmm(q, kt, mx_specs=specs)
+        assert type(eager) is torch.Tensor
+        two = softmax(eager, dim=-1, mx_specs=specs)
+    finally:
+        gemm.set_deferred_scores(True)
+    assert torch.equal((prod + 0).view(torch.int16), eager.view(torch.int16)) and prod.pending() is None
+    # a mask between product and softmax: the separate kernels, bit for bit
+    mask = torch.zeros(M, N, device=dev, dtype=torch.bfloat16)
+    mask[:, N // 2:] = float("-inf")
+    masked = softmax(bmm(q, kt, mx_specs=specs) + mask, dim=-1, mx_specs=specs)
+    assert torch.equal(masked.view(torch.int16), softmax(eager + mask, dim=-1, mx_specs=specs).view(torch.int16))
+    # and the two forms agree within one step of the quantizer's grid
+    d = (got.float() - two.float()).abs()
+    assert bool((d <= 2 ** -5 * two.float().abs() + 2.0 ** -132).all())
+
+
+def test_products_that_do_not_qualify_are_plain_tensors(dev):
+    from microxcaling_amd.bmm import bmm
+    specs = _specs(a_elem_format="fp6_e2m3", block_size=32, bfloat=16, custom_cuda=True)
+    g = torch.Generator().manual_seed(3)
+    for shape_q, shape_k, dt, grad in (((2, 40, 64), (2, 96, 64), torch.bfloat16, False),      # head_dim 64
+                                       ((2, 40, 128), (2, 100, 128), torch.bfloat16, False),   # N % 32 != 0
+                                       ((2, 40, 128), (2, 96, 128), torch.float32, False),
+                                       ((2, 40, 128), (2, 96, 128), torch.bfloat16, True)):    # a gradient is wanted
+        q = torch.randn(*shape_q, generator=g).to(dt).to(dev).requires_grad_(grad)
+        k = torch.randn(*shape_k, generator=g).to(dt).to(dev)
+        assert type(bmm(q, k.transpose(-1, -2), mx_specs=specs)) is torch.Tensor
+    v = torch.randn(2, 96, 128, generator=g).to(torch.bfloat16).to(dev)
+    p = torch.randn(2, 40, 96, generator=g).to(torch.bfloat16).to(dev)
+    assert type(bmm(p, v, mx_specs=specs)) is torch.Tensor                   # in2 not a transposed view
