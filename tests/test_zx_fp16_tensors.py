@@ -184,3 +184,59 @@ def test_fp16_dither_with_the_reference_noise_on_the_gpu():
         assert_bits_equal(got, want, "%s %s %d" % (kind, name, case_no))
         n += 1
     assert n == 13
+
+
+# ---- the layers on fp16 tensors (tests/golden/gen_reference_fp16_layer_vectors.py) ---------------------
+def _fp16_layer_fixture():
+    import importlib.util
+    import os
+    spec = importlib.util.spec_from_file_location("gen_reference_fp16_layer_vectors",
+                                                  os.path.join(GOLDEN, "gen_reference_fp16_layer_vectors.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return np.load(os.path.join(GOLDEN, "reference_fp16_layer_vectors.npz")), mod
+
+
+@pytest.mark.parametrize("case", ["mxfp8_bfloat16", "mxfp6_fp16", "mxfp4_floor"])
+def test_layers_on_fp16_tensors_reproduce_the_reference(case):
+    """linear, bmm, softmax, LayerNorm and RMSNorm on CPU fp16 tensors: forward outputs and every gradient
+    as the reference's own layers return them, bit for bit (host-library quantizers + torch's GEMM)."""
+    from microxcaling_amd.bmm import bmm
+    from microxcaling_amd.layernorm import LayerNorm, RMSNorm
+    from microxcaling_amd.linear import linear
+    from microxcaling_amd.softmax import softmax
+    from microxcaling_amd.specs import finalize_mx_specs
+    z, gen = _fp16_layer_fixture()
+    t = gen.inputs()
+    specs = finalize_mx_specs(dict(dict(gen.SPEC_CASES)[case], quantize_backprop=True, custom_cuda=False))
+    want = lambda name: from_bits(z[name], torch.float16)
+    threads = torch.get_num_threads()
+    torch.set_num_threads(1)                       # the summation order of torch's CPU GEMM the fixtures were written with
+    try:
+        xi, wi, bi = (t[k].clone().requires_grad_(True) for k in ("x", "w", "b"))
+        out = linear(xi, wi, bi, mx_specs=specs)
+        out.backward(t["go"])
+        for k, v in (("out", out), ("gx", xi.grad), ("gw", wi.grad), ("gb", bi.grad)):
+            assert_bits_equal(v, want("linear/%s/%s" % (case, k)), "linear " + k)
+        ai, bi2 = t["x"].clone().requires_grad_(True), t["a2"].clone().requires_grad_(True)
+        out = bmm(ai, bi2, mx_specs=specs)
+        out.backward(t["go"])
+        for k, v in (("out", out), ("g1", ai.grad), ("g2", bi2.grad)):
+            assert_bits_equal(v, want("bmm/%s/%s" % (case, k)), "bmm " + k)
+        si = t["sx"].clone().requires_grad_(True)
+        out = softmax(si, dim=-1, mx_specs=specs)
+        out.backward(t["sgo"])
+        assert_bits_equal(out, want("softmax/%s/out" % case), "softmax out")
+        assert_bits_equal(si.grad, want("softmax/%s/gx" % case), "softmax gx")
+        for lname, cls in (("layernorm", LayerNorm), ("rmsnorm", RMSNorm)):
+            m = cls(64, eps=1e-5, mx_specs=specs).to(torch.float16)
+            with torch.no_grad():
+                m.weight.copy_(t["nw"])
+                m.bias.copy_(t["nb"])
+            xi = t["nx"].clone().requires_grad_(True)
+            out = m(xi)
+            out.backward(t["ngo"])
+            for k, v in (("out", out), ("gx", xi.grad), ("gw", m.weight.grad), ("gb", m.bias.grad)):
+                assert_bits_equal(v, want("%s/%s/%s" % (lname, case, k)), "%s %s" % (lname, k))
+    finally:
+        torch.set_num_threads(threads)
