@@ -91,6 +91,9 @@ class DeferredProduct(torch.Tensor):
     tensor, so the object behaves like the logits tensor in every respect but one: the operands must
     not be modified in place before the product has been used (that raises)."""
 
+    # results of ops on it are ordinary tensors (no re-wrapping by torch's default __torch_function__)
+    __torch_function__ = torch._C._disabled_torch_function_impl
+
     @staticmethod
     def __new__(cls, in1, in2, specs, name):
         shape = in1.shape[:-1] + (in2.shape[-1],)
