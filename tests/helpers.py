@@ -125,3 +125,18 @@ class PackageImpl:
                                     saturate_normals=saturate_normals, allow_denorm=allow_denorm,
                                     custom_cuda=self.device == "cuda")
         return y.cpu()
+
+
+def integration_stub():
+    """The replacement for the reference's mx/custom_extensions.py printed in INTEGRATION.md, as a module."""
+    import re
+    import types
+    from microxcaling_amd import _lib
+    text = open(os.path.join(ROOT_DIR, "INTEGRATION.md")).read()
+    m = re.search(r"```python\n(# mx/custom_extensions.py  \(replacement.*?)```", text, re.S)
+    assert m, "the stub is no longer in INTEGRATION.md"
+    code = m.group(1).replace("/path/to/libmxq_gfx950.so", _lib.GPU_LIB_PATH).replace("/path/to/libmxq_host.so",
+                                                                                     _lib.HOST_LIB_PATH)
+    mod = types.ModuleType("reference_side_stub")
+    exec(compile(code, "INTEGRATION.md", "exec"), mod.__dict__)
+    return mod

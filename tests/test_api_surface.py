@@ -252,3 +252,26 @@ def test_bench_refuses_more_than_one_gpu_and_needs_one():
                              capture_output=True, text=True, timeout=300)
         assert res.returncode != 0
         assert '"metric"' not in res.stdout
+
+
+def test_the_reference_side_stub_of_the_integration_notes():
+    """The ctypes binding a maintainer of the reference would drop in for mx/custom_extensions.py is real
+    code: it loads both libraries, offers the seven names of mx/cpp/funcs.cpp:234-242, and its CPU
+    functions return what the reference's pure path returns (here: the oracle)."""
+    from oracle import mx_oracle as O
+    from helpers import integration_stub
+    stub = integration_stub()
+    assert sorted(vars(stub.funcs)) == sorted([
+        "quantize_mx_func_cpp", "quantize_elemwise_func_cpp", "quantize_mx_func_cuda", "quantize_mx_by_tile_func_cuda",
+        "quantize_elemwise_func_cuda", "reduce_sum_inner_dim", "reduce_max_inner_dim"])
+    g = torch.Generator().manual_seed(4)
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        x = (torch.randn(6, 96, generator=g) * 4).to(dtype)
+        blocks = x.view(6, 3, 32)
+        mx = blocks.abs().max(dim=2, keepdim=True).values
+        got = stub.funcs.quantize_mx_func_cpp(blocks, 8, 4, 5, 448.0, mx, 2, False, 0).view(6, 96)
+        assert_bits_equal(got, O.quantize_mx(x, 8, "fp8_e4m3", axes=[-1], block_size=32), "mx %s" % dtype)
+        got = stub.funcs.quantize_elemwise_func_cpp(x, 9, 8, 2 ** 127 * 255 / 128, 2, False, True)
+        assert_bits_equal(got, O.quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128, round="even"), "elem %s" % dtype)
+    with pytest.raises(RuntimeError, match="scale_bits"):
+        stub.funcs.quantize_mx_func_cpp(torch.zeros(1, 32), 0, 4, 5, 448.0, torch.zeros(1, 1), 1, False)
