@@ -1035,8 +1035,9 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     fetch_advance();
     scale_place(0);
     first_operands(lds);
+    // what the two groups behind a barrier would have issued of step 1's copy
 #pragma unroll
-    for (int i = 0; i < 6; ++i) fetch_part(1, f_fs, i);
+    for (int i = 0; i < mxq_addr::large_copy_first(0, NG); ++i) fetch_part(1, f_fs, i);
 
     int t = 0;
     while (true) {

@@ -142,7 +142,9 @@ MXQ_ADDR_FN int large_frag_row_b(int fi, bool pair) {
 // workgroup meets at the one barrier of the step; after it the wave reads the next stage (operands of
 // the next step's first group).  Behind the MFMAs of a group the wave issues copy instructions
 // first .. first + count - 1 (0-3 A codes, 4-7 B codes, 8 scales) of the flat step `ahead` steps after
-// the current one.  All nine are issued between two consecutive barriers.
+// the current one.  All nine are issued between two consecutive barriers: those of the groups behind
+// the barrier (loads 0 .. large_copy_first(0, ng) - 1) first, the rest from group 0 on.  Before the first
+// step the kernel issues the former share of step 1's copy itself.
 MXQ_ADDR_FN constexpr int large_barrier_group(int ng) { return ng - 3; }
 MXQ_ADDR_FN constexpr int large_copy_first(int gi, int ng) {
     return gi == 0 ? 6 : gi == 1 ? 8 : gi > large_barrier_group(ng) ? (gi - large_barrier_group(ng) - 1) * 3 : 0;

@@ -416,7 +416,7 @@ struct LargeModel {
             return true;
         };
         if (!first_operands(0, Where{tiles[0], 0}, 0, &bfh, &sb0, afh, sa, 0, -1)) return false;
-        for (int i = 0; i < 6; ++i)
+        for (int i = 0; i < large_copy_first(0, ng); ++i)       // what the groups behind a barrier would have issued
             if (!fetch_part(1, f_fs, i, -1)) return false;
 
         int t = 0;
