@@ -1009,9 +1009,15 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
             }
             // this group's share of the tile copy: loads 0 .. 5 of the step after next in the two groups
             // behind the barrier, loads 6 .. 8 of what is then the next step in the first two groups
+            if (!mxq_addr::large_copy_by_phase() || wave < 4) {
 #pragma unroll
-            for (int i = 0; i < mxq_addr::large_copy_count(gi, NG); ++i)
-                fetch_part(t + mxq_addr::large_copy_ahead(gi, NG), f_fs, mxq_addr::large_copy_first(gi, NG) + i);
+                for (int i = 0; i < mxq_addr::large_copy_count(gi, NG, 0); ++i)
+                    fetch_part(t + mxq_addr::large_copy_ahead(gi, NG), f_fs, mxq_addr::large_copy_first(gi, NG, 0) + i);
+            } else {
+#pragma unroll
+                for (int i = 0; i < mxq_addr::large_copy_count(gi, NG, 1); ++i)
+                    fetch_part(t + mxq_addr::large_copy_ahead(gi, NG), f_fs, mxq_addr::large_copy_first(gi, NG, 1) + i);
+            }
             __builtin_amdgcn_sched_barrier(0);
             bfh = bfh_next;
             afh[0] = afh_next[0];
@@ -1036,8 +1042,13 @@ __global__ __launch_bounds__(512, 1) void mx_gemm_nt_kernel_256p(GemmArgs g, int
     scale_place(0);
     first_operands(lds);
     // what the two groups behind a barrier would have issued of step 1's copy
+    if (!mxq_addr::large_copy_by_phase() || wave < 4) {
 #pragma unroll
-    for (int i = 0; i < mxq_addr::large_copy_first(0, NG); ++i) fetch_part(1, f_fs, i);
+        for (int i = 0; i < mxq_addr::large_copy_behind_barrier(NG, 0); ++i) fetch_part(1, f_fs, i);
+    } else {
+#pragma unroll
+        for (int i = 0; i < mxq_addr::large_copy_behind_barrier(NG, 1); ++i) fetch_part(1, f_fs, i);
+    }
 
     int t = 0;
     while (true) {

@@ -143,16 +143,30 @@ MXQ_ADDR_FN int large_frag_row_b(int fi, bool pair) {
 // the next step's first group).  Behind the MFMAs of a group the wave issues copy instructions
 // first .. first + count - 1 (0-3 A codes, 4-7 B codes, 8 scales) of the flat step `ahead` steps after
 // the current one.  All nine are issued between two consecutive barriers: those of the groups behind
-// the barrier (loads 0 .. large_copy_first(0, ng) - 1) first, the rest from group 0 on.  Before the first
-// step the kernel issues the former share of step 1's copy itself.
+// the barrier first, the rest from group 0 on.  Before the first step the kernel issues the former share
+// of step 1's copy itself.
 MXQ_ADDR_FN constexpr int large_barrier_group(int ng) { return ng - 3; }
-MXQ_ADDR_FN constexpr int large_copy_first(int gi, int ng) {
+// `phase` (0: waves 0-3, 1: waves 4-7) lets a schedule give the two waves of a SIMD (w and w + 4) different
+// places for their copy instructions; the one below does not (large_copy_by_phase() = false: the kernel
+// then never asks for phase 1).  Every wave issues each of its nine loads exactly once between two
+// barriers, in order.
+MXQ_ADDR_FN constexpr bool large_copy_by_phase() { return false; }
+MXQ_ADDR_FN constexpr int large_copy_first(int gi, int ng, int phase) {
+    (void)phase;
     return gi == 0 ? 6 : gi == 1 ? 8 : gi > large_barrier_group(ng) ? (gi - large_barrier_group(ng) - 1) * 3 : 0;
 }
-MXQ_ADDR_FN constexpr int large_copy_count(int gi, int ng) {
+MXQ_ADDR_FN constexpr int large_copy_count(int gi, int ng, int phase) {
+    (void)phase;
     return gi == 0 ? 2 : gi == 1 ? 1 : gi > large_barrier_group(ng) ? 3 : 0;
 }
 MXQ_ADDR_FN constexpr int large_copy_ahead(int gi, int ng) { return gi > large_barrier_group(ng) ? 2 : 1; }
+// loads of the next step that the groups behind a barrier issue (the kernel's prologue issues them itself
+// for step 1)
+MXQ_ADDR_FN constexpr int large_copy_behind_barrier(int ng, int phase) {
+    int n = 0;
+    for (int gi = large_barrier_group(ng) + 1; gi < ng; ++gi) n += large_copy_count(gi, ng, phase);
+    return n;
+}
 
 // ---- output elements of a lane, 256 x 256 kernel ----------------------------------------------------------
 // A 32 x 32 accumulator: lane L, register v holds C[row L % 32][fragment row 8 (v / 4) + 4 (L / 32) + v % 4]

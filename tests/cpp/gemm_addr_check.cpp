@@ -196,7 +196,8 @@ struct LargeModel {
     long long n_reads = 0, n_copies = 0;
     bool ok = true;
     // fetch side (uniform over the workgroup)
-    int f_logical = 0, f_fs = 0, f_groups = 0, f_kstart = 0, f_m0 = 0, f_n0 = 0, f_bz = 0;
+    int f_logical = 0, f_fs = 0, f_kstart = 0, f_m0 = 0, f_n0 = 0, f_bz = 0;
+    int f_groups[2] = {0, 0};                        // scale groups fetched so far, per phase (waves 0-3 / 4-7)
     // compute side
     int c_groups = 0, c_slot = 0, sc_base = 0;
     bool tail = false;
@@ -266,14 +267,14 @@ struct LargeModel {
         }
         return true;
     }
-    // load instruction i of every wave for flat step t, K step fs of the fetch-side tile (fetch_part)
-    bool fetch_part(int t, int fs, int i, int gi) {
+    // load instruction i of the waves of a phase for flat step t, K step fs of the fetch-side tile (fetch_part)
+    bool fetch_part(int t, int fs, int i, int gi, int phase) {
         const int k0 = large_kidx(f_kstart, fs, nk) * BK;
         const int64_t a_size = s.batch * s.M * (int64_t)kbytes, b_size = s.batch * s.N * (int64_t)kbytes;
         const int64_t sa_size = s.batch * s.M * (int64_t)kb, sb_size = s.batch * s.N * (int64_t)kb;
         const int64_t fa = f_bz * ((int64_t)s.M * kbytes) + (int64_t)f_m0 * kbytes;
         const int64_t fb = f_bz * ((int64_t)s.N * kbytes) + (int64_t)f_n0 * kbytes;
-        for (int wave = 0; wave < 8; ++wave) {
+        for (int wave = 4 * phase; wave < 4 * phase + 4; ++wave) {
             const bool s_is_b = wave >= 4;
             const int64_t fs_base = s_is_b ? f_bz * ((int64_t)s.N * kb) + (int64_t)f_n0 * kb
                                            : f_bz * ((int64_t)s.M * kb) + (int64_t)f_m0 * kb;
@@ -296,8 +297,8 @@ struct LargeModel {
                     const int64_t size = s_is_b ? sb_size : sa_size;
                     if (fs < nfull) {
                         if (fs % gs == 0) {
-                            const int lo = L_SCALE_OFF + (f_groups & 1) * L_SCALE_GROUP;
-                            if (!land(large_lds_scale_group_dst(f_groups, wave), 16, lane, kind, so, size, lo,
+                            const int lo = L_SCALE_OFF + (f_groups[phase] & 1) * L_SCALE_GROUP;
+                            if (!land(large_lds_scale_group_dst(f_groups[phase], wave), 16, lane, kind, so, size, lo,
                                       lo + L_SCALE_GROUP, t, gi, wave))
                                 return false;
                         }
@@ -312,7 +313,7 @@ struct LargeModel {
                 }
             }
         }
-        if (i == 8 && fs < nfull && fs % gs == 0) ++f_groups;
+        if (i == 8 && fs < nfull && fs % gs == 0) ++f_groups[phase];
         return true;
     }
 
@@ -395,8 +396,9 @@ struct LargeModel {
         // when it stops early (max_tiles) the fetch side simply runs on into tiles nobody multiplies here.
         fetch_tile(wg);
         f_fs = 0;
-        for (int i = 0; i < 9; ++i)
-            if (!fetch_part(0, 0, i, -1)) return false;
+        for (int phase = 0; phase < 2; ++phase)
+            for (int i = 0; i < 9; ++i)
+                if (!fetch_part(0, 0, i, -1, phase)) return false;
         ++epoch;                                             // s_waitcnt vmcnt(0); __syncthreads()
         fetch_advance();
         scale_place(0);
@@ -416,8 +418,9 @@ struct LargeModel {
             return true;
         };
         if (!first_operands(0, Where{tiles[0], 0}, 0, &bfh, &sb0, afh, sa, 0, -1)) return false;
-        for (int i = 0; i < large_copy_first(0, ng); ++i)       // what the groups behind a barrier would have issued
-            if (!fetch_part(1, f_fs, i, -1)) return false;
+        for (int phase = 0; phase < 2; ++phase)                  // what the groups behind a barrier would have issued
+            for (int i = 0; i < large_copy_behind_barrier(ng, large_copy_by_phase() ? phase : 0); ++i)
+                if (!fetch_part(1, f_fs, i, -1, phase)) return false;
 
         int t = 0;
         for (size_t ti_ = 0; ti_ < tiles.size(); ++ti_) {
@@ -468,8 +471,12 @@ struct LargeModel {
                         scale_place(next_cs);
                         if (!first_operands(nxt, nxt_w, t + 1, &bfh_n, &sb0_n, afh_n, sa_n, t, gi)) return false;
                     }
-                    for (int i = 0; i < large_copy_count(gi, ng); ++i)
-                        if (!fetch_part(t + large_copy_ahead(gi, ng), f_fs, large_copy_first(gi, ng) + i, gi)) return false;
+                    for (int phase = 0; phase < 2; ++phase) {
+                        const int ph = large_copy_by_phase() ? phase : 0;
+                        for (int i = 0; i < large_copy_count(gi, ng, ph); ++i)
+                            if (!fetch_part(t + large_copy_ahead(gi, ng), f_fs, large_copy_first(gi, ng, ph) + i, gi, phase))
+                                return false;
+                    }
                     bfh = bfh_next;
                     afh[0] = afh_next[0];
                     afh[1] = afh_next[1];

@@ -485,7 +485,8 @@ def test_gemm_copies_lds_image_schedule_and_stores_on_the_host(tmp_path):
     ("copies behind the barrier aimed at the stage still being read",
      "return gi > large_barrier_group(ng) ? 2 : 1; }", "return 1; }", "LDS MODEL: copy issued into bytes that are read"),
     ("a copy instruction short per step",
-     "gi > large_barrier_group(ng) ? 3 : 0;", "gi > large_barrier_group(ng) ? 2 : 0;", "LDS MODEL: a fragment read returns the wrong bytes"),
+     "return gi == 0 ? 2 : gi == 1 ? 1 : gi > large_barrier_group(ng) ? 3 : 0;",
+     "return gi == 0 ? 2 : gi == 1 ? 1 : gi > large_barrier_group(ng) ? 2 : 0;", "LDS MODEL: a fragment read returns the wrong bytes"),
     ("code rows landing one row down",
      "(wave * 32 + (i & 3) * 8) * 128);", "(wave * 32 + (i & 3) * 8 + 1) * 128);", "LDS MODEL: copy lands outside its LDS region"),
     ("the exchanged pieces stored at the wrong columns",
