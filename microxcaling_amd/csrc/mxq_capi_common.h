@@ -34,13 +34,14 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 // ---- dispatch over (dtype, rounding mode, element zone, lean) ------------------------------------
 // F is a functor template: F<DT, RMODE, ZONE_ELEM, LEAN>::run(args...).  The op-by-op form always
-// consults the zone table, so it exists once per rounding mode, and only bf16 tensors need it.
+// consults the zone table, so it exists once per rounding mode (bf16 tensors with wide formats; any
+// dtype for the two parameter corners of lean_ok).
 template <template <int, int, bool, bool> class F, int DT, typename... A>
 void dispatch_round(int rmode, bool zone_elem, bool lean, A... a) {
-    if (DT == MXQ_BF16 && !lean) {
-        if (rmode == MXQ_ROUND_FLOOR) F<MXQ_BF16, MXQ_FLOOR, true, false>::run(a...);
-        else if (rmode == MXQ_ROUND_NEAREST) F<MXQ_BF16, MXQ_NEAREST, true, false>::run(a...);
-        else F<MXQ_BF16, MXQ_EVEN, true, false>::run(a...);
+    if (!lean) {
+        if (rmode == MXQ_ROUND_FLOOR) F<DT, MXQ_FLOOR, true, false>::run(a...);
+        else if (rmode == MXQ_ROUND_NEAREST) F<DT, MXQ_NEAREST, true, false>::run(a...);
+        else F<DT, MXQ_EVEN, true, false>::run(a...);
         return;
     }
     if (rmode == MXQ_ROUND_FLOOR) {

@@ -293,6 +293,9 @@ MXQ_HD float mxq_round_every_op(float a, const MxqFmt& f, bool saturate, const u
         if (e >= (DT == MXQ_F16OPS ? 16 : 128)) return mxq_float(MXQ_QNAN_BITS);
     }
     float s = mxq_round_dt<DT>(ldexpf(mxq_float(ua), -e));  // out / 2**e
+    // sign(.) is taken of this quotient: where it underflowed to zero (e = 1 and the smallest subnormal)
+    // the result is +0 like for a zero input
+    const bool nonzero = s != 0.0f;
     s = mxq_round_dt<DT>(ldexpf(s, f.t));                   // * 2**(bits-2)
     float r;
     if (RMODE == MXQ_FLOOR) {
@@ -311,7 +314,7 @@ MXQ_HD float mxq_round_every_op(float a, const MxqFmt& f, bool saturate, const u
     y = mxq_round_dt<DT>(ldexpf(y, e));
     uint32_t uy = mxq_bits(y) & 0x7FFFFFFFu;
     if (uy > f.max_bits) uy = (saturate || f.ebits == 0) ? f.max_bits : MXQ_INF_BITS;
-    return mxq_float(uy | (ua != 0u ? (ba & 0x80000000u) : 0u));
+    return mxq_float(uy | (nonzero ? (ba & 0x80000000u) : 0u));
 }
 
 // One element of an MX block: x / 2^se -> round -> * 2^se  (mx/mx_ops.py:285-292).  The result

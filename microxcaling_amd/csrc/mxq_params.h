@@ -103,6 +103,10 @@ inline int make_fmt(int dtype, int flags, int ebits, int mbits, float max_norm, 
     fmt->min_exp = ebits ? 2 - (1 << (ebits - 1)) : 0;
     // torch casts the clamp bound to the tensor dtype (65504 becomes 65536 for a bf16 tensor)
     fmt->max_bits = mxq_bits(dtype == MXQ_DTYPE_BF16 ? mxq_round_bf16(max_norm) : max_norm);
+    // a clamp bound beyond the largest bf16 number: torch.clamp refuses the conversion (mx/elemwise_ops.py:154)
+    if (dtype == MXQ_DTYPE_BF16 && clamps && max_norm > 3.3895313892515355e38f)
+        return fail(MXQ_ERR_ARGUMENT, "%s: max_norm %g cannot be converted to bfloat16 without overflow "
+                    "(the clamp of a bfloat16 tensor needs its bound in bfloat16)", who, (double)max_norm);
     if (f16_ops(dtype, flags)) {
         // a bound beyond the fp16 range: torch.clamp refuses to convert it (mx/elemwise_ops.py:154
         // raises), the comparison of the non-saturating branch (156) sees it as Inf
@@ -143,6 +147,16 @@ inline void zone_for(int dtype, int flags, int* row, int* zshift) {
 // never have more than 6 fraction bits.
 // fp16 tensors evaluated op by op (f16_ops) always take the op-by-op form; callers test that first.
 inline bool lean_ok(int dtype, const MxqFmt& f, int rmode, bool elementwise) {
+    // Two parameter corners take the op-by-op form on every dtype.  One exponent bit: min_exp is 1, and
+    // x / 2**1 underflows to zero for the smallest subnormal, which then comes out as +0 (the lean form
+    // scales by 2**(t - e) in one exact step and would keep the sign).  An integer format whose max_norm
+    // is 2 or more (none of the named ones): the lean form lets |x| >= 2 take its own exponent, knowing
+    // that the clamp to a max_norm below 2 erases the difference.
+    if (f.ebits == 1 || (f.ebits == 0 && f.max_bits >= 0x40000000u)) return false;
+    // MX with an 8-bit element exponent (no named format has one): the block scale puts the maximum into
+    // the top binade, where floor(log2(x)) can come out as 128 and 2**128 = inf makes the element NaN;
+    // the elementwise quantizer handles that with a threshold of its own (nan_from), the lean MX form does not
+    if (!elementwise && f.ebits == 8) return false;
     return dtype != MXQ_DTYPE_BF16 || f.t <= 6 || (elementwise && rmode != MXQ_ROUND_EVEN);
 }
 

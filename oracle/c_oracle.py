@@ -28,13 +28,18 @@ def lib():
 _RMODE = {"nearest": 0, "floor": 1, "even": 2}
 
 
+def _clamp_bound_must_fit(dtype, max_norm):
+    """torch.clamp converts its bounds to the tensor dtype and refuses one that overflows it
+    (mx/elemwise_ops.py:154 on an fp16 / bf16 tensor)."""
+    if dtype in (torch.float16, torch.bfloat16) and max_norm > torch.finfo(dtype).max:
+        raise RuntimeError("value cannot be converted to type %s without overflow" % dtype)
+
+
 def quantize_elemwise_core(A, bits, exp_bits, max_norm, round="nearest", saturate_normals=False,
                            allow_denorm=True):
     A = A.contiguous()
-    if A.dtype == torch.float16 and (saturate_normals or exp_bits == 0) and max_norm > 65504.0:
-        # torch.clamp converts its bounds to the tensor dtype and refuses one that overflows it
-        # (mx/elemwise_ops.py:154 on an fp16 tensor)
-        raise RuntimeError("value cannot be converted to type at::Half without overflow")
+    if saturate_normals or exp_bits == 0:
+        _clamp_bound_must_fit(A.dtype, max_norm)
     out = torch.empty_like(A)
     lib().oracle_quantize_elemwise(A.data_ptr(), out.data_ptr(), _DT[A.dtype], A.numel(), bits,
                                    exp_bits, max_norm, _RMODE[round], int(saturate_normals),
@@ -54,6 +59,7 @@ def quantize_mx(A, scale_bits, elem_format, axes, block_size=0, round="nearest",
     for n in A.shape[axis + 1:]:
         post *= n
     ebits, mbits, emax, max_norm, _ = format_params(elem_format)
+    _clamp_bound_must_fit(A.dtype, max_norm)            # elements are saturated (mx/mx_ops.py:287-290)
     out = torch.empty_like(A)
     lib().oracle_quantize_mx(A.data_ptr(), out.data_ptr(), _DT[A.dtype], pre, A.shape[axis], post,
                              scale_bits, ebits, mbits, emax, max_norm, block_size,
