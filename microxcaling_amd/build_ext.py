@@ -101,6 +101,57 @@ def check_sources(verbose=False):
           os.path.join(CSRC, "mxq_host.cpp")], verbose)
 
 
+def kernel_resources(path=GPU_LIB):
+    """What the compiler recorded for every gfx950 kernel of the built library: a list of dicts with
+    name, vgprs, agprs, sgprs, lds (static bytes), scratch (bytes of private memory per lane), vgpr_spills,
+    sgpr_spills, max_workgroup.  Read from the AMDGPU metadata note of each code object in the library's
+    offload bundles (no GPU and no external tool needed) -- the build's own statement of whether a
+    kernel spills, how much LDS it declares and how many waves can share a SIMD."""
+    import struct
+    import msgpack
+    with open(path, "rb") as f:
+        blob = f.read()
+    magic, out, pos = b"__CLANG_OFFLOAD_BUNDLE__", [], 0
+    while True:
+        start = blob.find(magic, pos)
+        if start < 0:
+            break
+        pos = start + len(magic)
+        (n_entries,) = struct.unpack_from("<Q", blob, pos)
+        p = pos + 8
+        for _ in range(n_entries):
+            offset, size, triple_len = struct.unpack_from("<QQQ", blob, p)
+            triple = blob[p + 24:p + 24 + triple_len].decode()
+            p += 24 + triple_len
+            if "gfx950" not in triple or size == 0:
+                continue
+            elf = blob[start + offset:start + offset + size]
+            (shoff,) = struct.unpack_from("<Q", elf, 0x28)
+            shentsize, shnum = struct.unpack_from("<HH", elf, 0x3A)
+            for k in range(shnum):
+                (sh_type,) = struct.unpack_from("<I", elf, shoff + k * shentsize + 4)
+                sec_off, sec_size = struct.unpack_from("<QQ", elf, shoff + k * shentsize + 0x18)
+                if sh_type != 7:                                         # SHT_NOTE
+                    continue
+                q = sec_off
+                while q < sec_off + sec_size:
+                    namesz, descsz, ntype = struct.unpack_from("<III", elf, q)
+                    q += 12 + ((namesz + 3) & ~3)
+                    desc = elf[q:q + descsz]
+                    q += (descsz + 3) & ~3
+                    if ntype != 32:                                      # NT_AMDGPU_METADATA
+                        continue
+                    for kern in msgpack.unpackb(desc, raw=False, strict_map_key=False)["amdhsa.kernels"]:
+                        out.append({"name": kern[".name"], "vgprs": kern[".vgpr_count"],
+                                    "agprs": kern.get(".agpr_count", 0), "sgprs": kern[".sgpr_count"],
+                                    "lds": kern[".group_segment_fixed_size"],
+                                    "scratch": kern[".private_segment_fixed_size"],
+                                    "vgpr_spills": kern.get(".vgpr_spill_count", 0),
+                                    "sgpr_spills": kern.get(".sgpr_spill_count", 0),
+                                    "max_workgroup": kern[".max_flat_workgroup_size"]})
+    return out
+
+
 def build_all(verbose=True):
     return build_gpu(verbose), build_host(verbose)
 

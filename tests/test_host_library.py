@@ -64,6 +64,39 @@ def test_the_libraries_in_the_tree_are_built_from_the_sources_in_the_tree():
     assert _lib.host().mxq_host_build_digest() == want, "libmxq_host.so is stale: rebuild it"
 
 
+def test_kernels_of_the_built_library_fit_their_launch_shape():
+    """From the code objects' own metadata: registers leave room for the waves each launch shape puts on
+    a SIMD (512 per lane and SIMD, arch + accumulation), static LDS fits the 160 KB of a CU, and only the
+    kernels named here keep anything in private (scratch) memory -- the streaming quantizers, packers,
+    reductions and row kernels must not spill, since a spill in them is paid per element."""
+    import re
+    from microxcaling_amd import build_ext
+    kernels = build_ext.kernel_resources()
+    assert len(kernels) > 900
+
+    def plain(k):                                        # _ZN12_GLOBAL__N_1<length><name>... -> name
+        m = re.match(r"_ZN12_GLOBAL__N_1(\d+)", k["name"])
+        return k["name"][m.end():m.end() + int(m.group(1))]
+
+    names = {plain(k) for k in kernels}
+    for want in ("mx_lastaxis_kernel", "mx_strided_kernel", "mx_strided_tile_kernel", "mx_axes_kernel", "elemwise_kernel",
+                 "mx_pack_kernel", "mx_pack_t_kernel", "mx_unpack_kernel", "reduce_outer_kernel", "softmax_row_kernel",
+                 "mx_gemm_nt_kernel", "mx_gemm_nt_kernel_256p", "mx_bmm_softmax_kernel"):
+        assert want in names, want
+    # name prefix -> bytes of private memory per lane that are known and accounted for: the large GEMM's fp32
+    # epilogue keeps 8 loop-invariant address pairs there (written once per workgroup, read per tile after the
+    # K loop), the scores kernel 6, one fp32 instantiation of the norm backward row kernel its row buffer
+    allowed = {"mx_gemm_nt_kernel_256p": 68, "mx_bmm_softmax_kernel": 48, "norm_backward_row_kernel": 272}
+    for k in kernels:
+        name = plain(k)
+        waves_per_simd = max(1, k["max_workgroup"] // 256)
+        assert k["vgprs"] + k["agprs"] <= 512 // waves_per_simd, k
+        assert k["lds"] <= 160 * 1024, k
+        assert k["scratch"] <= allowed.get(name, 0), k
+        if k["scratch"] == 0:
+            assert k["vgpr_spills"] == 0, k
+
+
 def test_gpu_entry_points_reject_bad_arguments_without_a_gpu():
     lib = _lib.gpu()
     assert lib.mxq_version() >= 100
