@@ -254,6 +254,48 @@ def test_bench_refuses_more_than_one_gpu_and_needs_one():
         assert '"metric"' not in res.stdout
 
 
+def test_bench_reports_carry_the_contract_fields():
+    """Everything of bench.py that needs no GPU: the two default workloads build, their CPU legs run on a
+    sample, and the report functions turn timings into the JSON line of the contract (metric, value, unit,
+    config.workload, roofline with bound / achieved / peak / frac / traffic, cpu_baseline)."""
+    import importlib.util
+    import json
+    import os
+    from helpers import ROOT_DIR
+    spec = importlib.util.spec_from_file_location("bench_under_test", os.path.join(ROOT_DIR, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+
+    with open(os.path.join(ROOT_DIR, "profiles", "traffic.json")) as f:
+        names = [k for k, v in json.load(f).items() if isinstance(v, dict)]
+    assert bench.HEADLINE in names and bench.SECONDARY in names and "mx_bmm_softmax" in names
+    for name in names:
+        measured, note = bench.measured_traffic(name)
+        assert note["summary"].startswith("profiles/") and os.path.exists(os.path.join(ROOT_DIR, note["summary"])), name
+        assert (measured == note["last_measured_bytes"]) if note["kernel_sources_unchanged_since"] else measured is None
+
+    wl = bench.make_workload(bench.HEADLINE)
+    assert wl["bytes"] == 8192 * 8192 * 8 and wl["x"].shape == (8192, 8192)
+    assert wl["cpu"](wl["x"][:64, :64].contiguous()).shape == (64, 64)
+    line = bench.bytes_report(bench.HEADLINE, wl, 200, 50, 0.0831, 0.0807, False)
+    line["cpu_baseline"] = {"value": 1.0, "unit": "GB/s", "cores": 1, "kind": "port", "sample": "-"}
+    sec_wl = bench.make_workload(bench.SECONDARY)
+    assert sec_wl["flops"] == 2 * 16384 * 14336 * 4096
+    sec_wl["cpu_rows"] = 64                                     # a smaller sample than the bench run takes
+    sec = bench.flops_report(bench.SECONDARY, sec_wl, 200, 50, 0.95, 0.94, 0.85, True)
+    for rep, unit, bound in ((line, "GB/s", "hbm"), (sec, "TFLOP/s", "mfma")):
+        rep = json.loads(json.dumps(rep))
+        assert rep["metric"] == bench.METRIC and rep["unit"] == unit and rep["n_gpus"] == 1
+        assert rep["higher_is_better"] is True and rep["vs_baseline"] is None and rep["data"] == "synthetic"
+        assert "workload" in rep["config"] and "model" not in rep["config"]
+        roof = rep["roofline"]
+        assert roof["bound"] == bound and roof["unit"] == unit and "traffic" in roof
+        assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
+        assert set(rep["cpu_baseline"]) >= {"value", "unit", "cores", "kind", "sample"}
+    assert abs(line["roofline"]["achieved"] - 536870912 / 0.0807e-3 / 1e9) < 1.0
+    assert abs(sec["roofline"]["achieved"] - 1924145348608 / 0.85e-3 / 1e12) < 0.1 and sec["cpu_baseline"]["value"] > 0
+
+
 def test_the_reference_side_stub_of_the_integration_notes():
     """The ctypes binding a maintainer of the reference would drop in for mx/custom_extensions.py is real
     code: it loads both libraries, offers the seven names of mx/cpp/funcs.cpp:234-242, and its CPU

@@ -48,7 +48,7 @@ def test_softmax_of_bmm_is_the_one_launch_kernel(dev, shape, fmt, exp2):
         two = softmax(eager, dim=-1, mx_specs=specs)
     finally:
         gemm.set_deferred_scores(True)
-    assert torch.equal((prod + 0).view(torch.int16), eager.view(torch.int16)) and prod.pending() is None
+    assert torch.equal(prod.clone().view(torch.int16), eager.view(torch.int16)) and prod.pending() is None
     # a mask between product and softmax: the separate kernels, bit for bit
     mask = torch.zeros(M, N, device=dev, dtype=torch.bfloat16)
     mask[:, N // 2:] = float("-inf")
