@@ -20,6 +20,25 @@ from .formats import ElemFormat, RoundingMode, _get_format_params
 from .elemwise_ops import _native_round
 
 
+def _dither_noise(A, axes, block_size):
+    """One uniform [0, 1) number per element, the ones the reference's torch.rand_like hands the same
+    elements under the same generator state.  The reference draws inside the element quantizer, i.e. for
+    the tensor already padded to whole blocks (mx/mx_ops.py:226-229, 285-288, mx/elemwise_ops.py:58): when
+    an axis is not a multiple of block_size the draw has the padded shape -- the padding's numbers are
+    drawn and dropped, so that every real element meets the same number as there (on a GPU the number an
+    element gets depends on the size of the draw, not only on its position)."""
+    shape = list(A.shape)
+    if block_size > 0:
+        for ax in axes:
+            shape[ax] = -(-shape[ax] // block_size) * block_size
+    if shape == list(A.shape):
+        return torch.rand_like(A, requires_grad=False)
+    noise = torch.rand(shape, dtype=A.dtype, device=A.device)
+    for ax in axes:
+        noise = noise.narrow(ax, 0, A.shape[ax])
+    return noise.contiguous()
+
+
 def _quantize_mx(A, scale_bits, elem_format, shared_exp_method="max", axes=None, block_size=0,
                  round="nearest", flush_fp32_subnorms=False, custom_cuda=False):
     """Same contract as mx/mx_ops.py:173-298."""
@@ -55,7 +74,7 @@ def _quantize_mx(A, scale_bits, elem_format, shared_exp_method="max", axes=None,
             raise NotImplementedError("round='dither' with an exponent shared over several axes")
         if A.device.type not in ("cuda", "cpu"):
             raise ValueError("Unrecognized device type %s" % A.device.type)
-        return ce.funcs.quantize_mx_dither_by_tile_func(A, torch.rand_like(A, requires_grad=False), scale_bits,
+        return ce.funcs.quantize_mx_dither_by_tile_func(A, _dither_noise(A, axes, block_size), scale_bits,
                                                         ebits, mbits, max_norm, tile, axes[-1], flush_fp32_subnorms)
     if len(axes) > 1 and tile != 1:          # one exponent per tile of tile x tile (x tile) elements
         fn = {"cuda": ce.funcs.quantize_mx_axes_func_cuda, "cpu": ce.funcs.quantize_mx_axes_func_cpp}.get(A.device.type)

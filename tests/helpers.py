@@ -98,6 +98,18 @@ def dither_cases():
             yield "elem", name, dtype, n, 2000 + n, case, x, from_bits(z["elem_%s_%d" % (name, n)], dtype)
 
 
+def reference_noise(kind, case, x):
+    """The uniform numbers the reference hands the elements of x in a stored dither case, drawn on the CPU
+    under the current torch seed: torch.rand_like of the tensor the element quantizer sees, which for MX is
+    x padded to whole blocks along the block axis (mx/mx_ops.py:226-229; the padding's numbers are dropped)."""
+    if kind != "mx" or case[2] <= 0 or x.shape[case[1]] % case[2] == 0:
+        return torch.rand_like(x)
+    _, axis, bs = case
+    shape = list(x.shape)
+    shape[axis] = -(-shape[axis] // bs) * bs
+    return torch.rand(shape, dtype=x.dtype).narrow(axis % x.ndim, 0, x.shape[axis]).contiguous()
+
+
 class PackageImpl:
     """This package's own entry points behind the call signature of the oracles, so that one test
     body can run against an oracle, against the host library (CPU tensors -> libmxq_host.so) and

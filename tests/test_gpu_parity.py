@@ -257,14 +257,14 @@ def test_mx_several_axes(dev, shape, axes, bs, dtype):
 def test_dither_with_the_reference_noise(dev):
     """round='dither' on the GPU with the noise the reference drew (torch.rand_like under the stored
     seed, regenerated on the CPU and copied over): the reference's outputs bit for bit."""
-    from helpers import dither_cases
+    from helpers import dither_cases, reference_noise
     from microxcaling_amd.custom_extensions import funcs
     from microxcaling_amd.formats import _get_format_params
     for kind, name, dtype, case_no, seed, case, x, want in dither_cases():
         if dtype == torch.float16:
             continue                                  # tests/test_zx_fp16_tensors.py
         torch.manual_seed(seed)
-        noise = torch.rand_like(x).to(dev)
+        noise = reference_noise(kind, case, x).to(dev)
         if kind == "mx":
             fmt, axis, bs = case
             ebits, mbits, _, max_norm, _ = _get_format_params(fmt)

@@ -389,7 +389,8 @@ def test_golden_exhaustive_bf16_digests():
 def test_golden_dither():
     """round='dither' (mx/elemwise_ops.py:57-59): under the same torch seed the torch oracle draws
     the noise the reference drew and reproduces its outputs bit for bit (no test of the reference
-    covers this mode; the C oracle has no generator and does not take it)."""
+    covers this mode; the C oracle has no generator and does not take it).  Three of the ten MX cases have
+    blocks that do not divide the axis: the reference draws for the padded tensor there."""
     n = 0
     for kind, name, dtype, case_no, seed, case, x, want in dither_cases():
         torch.manual_seed(seed)
@@ -401,4 +402,4 @@ def test_golden_dither():
             got = O.quantize_elemwise_core(x.clone(), bits, eb, mn, round="dither", saturate_normals=sat)
         assert_bits_equal(got, want, "%s %s %d" % (kind, name, case_no))
         n += 1
-    assert n == 39
+    assert n == 48

@@ -161,7 +161,7 @@ def test_fp16_tensors_on_the_gpu():
 def test_fp16_dither_with_the_reference_noise_on_the_gpu():
     """round='dither' on fp16 tensors with the noise the reference drew (regenerated on the CPU under
     the stored seed and copied over): the reference's outputs bit for bit."""
-    from helpers import dither_cases
+    from helpers import dither_cases, reference_noise
     from microxcaling_amd.custom_extensions import funcs
     from microxcaling_amd.formats import _get_format_params
     assert torch.cuda.is_available(), "this test needs a GPU"
@@ -171,7 +171,7 @@ def test_fp16_dither_with_the_reference_noise_on_the_gpu():
         if dtype != torch.float16:
             continue
         torch.manual_seed(seed)
-        noise = torch.rand_like(x).to(dev)
+        noise = reference_noise(kind, case, x).to(dev)
         if kind == "mx":
             fmt, axis, bs = case
             ebits, mbits, _, max_norm, _ = _get_format_params(fmt)
