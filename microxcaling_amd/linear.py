@@ -94,7 +94,7 @@ class LinearFunction(torch.autograd.Function):
         # number of blocks, no block straddles two batch entries and the tensors can be flattened to
         # 2-D first (one GEMM over all examples); block_size 0 means one block per batch entry
         block = specs["block_size"]
-        if input.dim() == 2 or (block > 0 and input.shape[-2] % block == 0):
+        if input.dim() == 2 or (input.dim() > 2 and block > 0 and input.shape[-2] % block == 0):
             grad_weight = mx_grad_contract(
                 grad_output.reshape(-1, out_dim), specs["a_elem_format_bp_ex"],
                 specs["round_mx_grad_output_grad_weight"], True,

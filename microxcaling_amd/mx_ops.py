@@ -50,6 +50,9 @@ def _quantize_mx(A, scale_bits, elem_format, shared_exp_method="max", axes=None,
                         "block size to")
     axes = [axes] if type(axes) == int else list(axes)
     axes = [x + A.ndim if x < 0 else x for x in axes]
+    # the reference normalizes a negative axis a second time further down (mx/mx_ops.py:193-194, 105): axes=[-2]
+    # on a 1-D tensor, which its linear layer's backward pass asks for (mx/linear.py:124-137), means axis 0
+    axes = [x + A.ndim if -A.ndim <= x < 0 else x for x in axes]
     axes = sorted(axes)
     if len(axes) == 0 or len(set(axes)) != len(axes):
         raise ValueError("axes must name at least one dimension, each once")
