@@ -9,6 +9,7 @@ from .specs import (MxSpecs, get_default_mx_specs, get_backwards_mx_specs, apply
 from .formats import ElemFormat, RoundingMode
 from .mx_ops import quantize_mx_op
 from .elemwise_ops import quantize_elemwise_op
+from .quantize import quantize_bfloat
 from .linear import Linear, linear
 from .matmul import matmul
 from .bmm import bmm, bmm_softmax

@@ -4,7 +4,8 @@ for each gradient (mx/specs.py:84-91), every ``round_*`` key (mx/specs.py:104-11
 widths, bfloat_subnorms, quantize_backprop, block size, scale bits, flush, softmax_exp2 /
 vec_use_exp2 / vec_use_recip -- so that a layer applying the wrong role's format or rounding
 anywhere in forward or backward produces other bits.  Per case: linear, matmul (+bias), bmm, softmax,
-LayerNorm, RMSNorm, gelu, sigmoid, Conv2d -- outputs and every gradient, fp32 and bf16 tensors, as
+LayerNorm, RMSNorm, seven activations, quantize_bfloat, Conv2d -- outputs and every gradient, fp32 and
+bf16 tensors, as
 SHA-256 digests; the first four cases are also stored in full.
 
 Run once where the reference checkout exists:
@@ -171,6 +172,12 @@ def run_case(mx, raw, inp, dt):
     ran("rmsnorm", norm_("rmsnorm", mx.RMSNorm))
     ran("gelu", act_("gelu", mx.gelu))
     ran("sigmoid", act_("sigmoid", mx.sigmoid))
+    ran("tanh", act_("tanh", mx.tanh))
+    ran("silu", act_("silu", mx.silu))
+    ran("relu6", act_("relu6", mx.relu6))
+    ran("leaky_relu", act_("leaky_relu", lambda x, mx_specs: mx.leaky_relu(x, 0.05, mx_specs=mx_specs)))
+    ran("gelu1", act_("gelu1", lambda x, mx_specs: mx.gelu(x, mx_specs=mx_specs, first_order_gelu=True)))
+    ran("quantize_bfloat", act_("quantize_bfloat", lambda x, mx_specs: mx.quantize_bfloat(x, mx_specs)))
     if dt == torch.float32:
         ran("conv2d", conv_)
     return out
