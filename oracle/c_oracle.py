@@ -51,7 +51,10 @@ def quantize_mx(A, scale_bits, elem_format, axes, block_size=0, round="nearest",
                 flush_fp32_subnorms=False):
     A = A.contiguous()
     (axis,) = [axes] if isinstance(axes, int) else axes
-    axis = axis + A.ndim if axis < 0 else axis
+    for _ in range(2):             # the reference normalizes a negative axis twice (mx/mx_ops.py:193-194, 105)
+        axis = axis + A.ndim if axis < 0 else axis
+    if not 0 <= axis < A.ndim:
+        raise IndexError("axis out of range for a tensor of %d dimensions" % A.ndim)
     pre = 1
     for n in A.shape[:axis]:
         pre *= n
