@@ -4,6 +4,7 @@ libmxq_host.so) is bit-identical to the oracle on exhaustive sweeps; the round-u
 agree with torch's CPU log2 on this machine.  No GPU compute happens here."""
 import ctypes
 import os
+import subprocess
 import re
 
 import numpy as np
@@ -475,6 +476,23 @@ def test_fp16_conversions_of_the_scalar_core(tmp_path, compiler):
     got_f = torch.from_numpy(np.fromfile(fb, dtype=np.float32))
     assert_bits_equal(got_h, x.half(), "fp32 -> fp16")
     assert_bits_equal(got_f, x.half().float(), "fp16 -> fp32")
+
+
+def test_host_quantizers_under_address_and_undefined_behaviour_sanitizers(tmp_path):
+    """tests/cpp/host_abi_sanitize.cpp + mxq_host.cpp compiled with -fsanitize=address,undefined: eight
+    seconds of random calls (empty and ragged shapes, tiles longer than the axis, several shared axes, all
+    dtypes / formats / flags) on buffers of exactly the described size; any read or write past an operand,
+    signed overflow or misaligned access ends the run with a report."""
+    exe = str(tmp_path / "host_abi_sanitize")
+    subprocess.run(["/opt/rocm/lib/llvm/bin/clang++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined",
+                    "-fno-sanitize-recover=undefined", "-ffp-contract=off", "-I" + os.path.join(ROOT_DIR, "include"),
+                    "-I" + os.path.join(ROOT_DIR, "microxcaling_amd", "csrc"),
+                    os.path.join(ROOT_DIR, "tests", "cpp", "host_abi_sanitize.cpp"),
+                    os.path.join(ROOT_DIR, "microxcaling_amd", "csrc", "mxq_host.cpp"), "-o", exe],
+                   check=True, capture_output=True, text=True, timeout=600)
+    res = subprocess.run([exe, "8"], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0 and res.stdout.startswith("ok "), (res.stdout[-2000:], res.stderr[-4000:])
+    assert int(res.stdout.split()[1]) > 1000
 
 
 def _build_gemm_addr_check(tmp_path, include_dir=None):
