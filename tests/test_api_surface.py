@@ -317,3 +317,27 @@ def test_the_reference_side_stub_of_the_integration_notes():
         assert_bits_equal(got, O.quantize_elemwise_core(x, 9, 8, 2 ** 127 * 255 / 128, round="even"), "elem %s" % dtype)
     with pytest.raises(RuntimeError, match="scale_bits"):
         stub.funcs.quantize_mx_func_cpp(torch.zeros(1, 32), 0, 4, 5, 448.0, torch.zeros(1, 1), 1, False)
+
+
+@pytest.mark.parametrize("name", ["sigmoid", "tanh", "relu", "leaky_relu", "silu", "gelu", "softmax", "linear", "matmul",
+                                  "bmm", "conv1d", "conv2d", "conv3d"])
+def test_finite_differences_without_mx_specs(name):
+    """mx/tests/test_gradcheck.py:25-89: with mx_specs None every function is torch's own and passes
+    torch.autograd.gradcheck in float64 (a wrapper that dropped or reordered an argument would not)."""
+    import microxcaling_amd as mx
+    fn = getattr(mx, name)
+    g = torch.Generator().manual_seed(0xBEEF)
+    r = lambda *s: torch.randn(*s, dtype=torch.float64, generator=g).requires_grad_(True)
+    if name in ("linear", "matmul"):
+        args = (r(3, 8, 8), r(8, 8))
+    elif name == "bmm":
+        args = (r(3, 8, 8), r(3, 8, 8))
+    elif name.startswith("conv"):
+        nd = int(name[4])
+        args = (r(2, 8, *([3] * nd)), r(2, 8, *([1] * nd)))
+    elif name == "softmax":
+        args = (r(64),)
+        fn = lambda x: mx.softmax(x, dim=-1)
+    else:
+        args = (r(64),)
+    assert torch.autograd.gradcheck(fn, args)
