@@ -341,3 +341,31 @@ def test_finite_differences_without_mx_specs(name):
     else:
         args = (r(64),)
     assert torch.autograd.gradcheck(fn, args)
+
+
+def test_the_written_notes_name_things_that_exist():
+    """Every test, source file, profile summary, kernel and C symbol that the Markdown notes at the repository
+    root mention in code quotes exists in the tree (notes drift when code is renamed)."""
+    import glob
+    import os
+    import re
+    from helpers import ROOT_DIR
+    tests = {os.path.basename(f): open(f).read() for f in glob.glob(os.path.join(ROOT_DIR, "tests", "*.py"))}
+    sources = "\n".join(open(f).read() for f in glob.glob(os.path.join(ROOT_DIR, "microxcaling_amd", "**", "*"), recursive=True)
+                        if os.path.isfile(f) and f.endswith((".py", ".h", ".hip", ".cpp")))
+    sources += open(os.path.join(ROOT_DIR, "include", "mxq.h")).read()
+    missing = []
+    for doc in ("DESIGN", "README", "INTEGRATION"):
+        text = open(os.path.join(ROOT_DIR, doc + ".md")).read()
+        for path, name in re.findall(r"(tests/[\w/]+\.(?:py|cpp))(?:::([\w…]+))?", text):
+            if not os.path.exists(os.path.join(ROOT_DIR, path)):
+                missing.append((doc, path))
+            elif name and path.endswith(".py") and ("def " + name.rstrip("…")) not in tests[os.path.basename(path)]:
+                missing.append((doc, path, name))
+        for path in re.findall(r"`((?:profiles|include|microxcaling_amd)/[\w/.+-]+)`", text):
+            if not os.path.exists(os.path.join(ROOT_DIR, path)):
+                missing.append((doc, path))
+        for name in set(re.findall(r"`(\w+_kernel(?:_256p)?|mxq_\w+)`", text)):
+            if name not in sources:
+                missing.append((doc, name))
+    assert not missing, missing
