@@ -263,6 +263,8 @@ def test_dither_with_the_reference_noise(dev):
     for kind, name, dtype, case_no, seed, case, x, want in dither_cases():
         if dtype == torch.float16:
             continue                                  # tests/test_zx_fp16_tensors.py
+        if kind == "mx" and case[2] > 0 and x.shape[case[1]] % case[2] != 0:
+            continue                                  # ragged blocks: tests/test_zt_uncommon_parameters.py
         torch.manual_seed(seed)
         noise = reference_noise(kind, case, x).to(dev)
         if kind == "mx":

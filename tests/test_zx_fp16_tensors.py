@@ -170,6 +170,8 @@ def test_fp16_dither_with_the_reference_noise_on_the_gpu():
     for kind, name, dtype, case_no, seed, case, x, want in dither_cases():
         if dtype != torch.float16:
             continue
+        if kind == "mx" and case[2] > 0 and x.shape[case[1]] % case[2] != 0:
+            continue                                  # ragged blocks: tests/test_zt_uncommon_parameters.py
         torch.manual_seed(seed)
         noise = reference_noise(kind, case, x).to(dev)
         if kind == "mx":
