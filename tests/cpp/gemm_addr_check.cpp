@@ -23,6 +23,7 @@
 //
 //   usage: gemm_addr_check            (prints one line per shape and check; exit status 1 on the first
 //                                      violation)
+//          gemm_addr_check --plans    (prints which kernel and K split the rules restated here give each shape)
 //
 // The launch rules restated here (which kernel a shape takes, grid sizes, K splits) are those of
 // mxq_capi_gemm.hip / mxq_capi_scores.hip; the loop skeletons are those of mxq_gemm.h / mxq_bmm_softmax.h.
@@ -30,6 +31,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <deque>
+#include <string>
 #include <vector>
 
 #include "mxq_gemm_addr.h"
@@ -784,7 +786,7 @@ int k_splits(const Shape& s) {
 
 }  // namespace
 
-int main() {
+int main(int argc, char** argv) {
     const Shape shapes[] = {
         {1, 16384, 14336, 4096, false, "config 4 (MXFP8)"},
         {1, 16384, 14336, 4096, true, "config 4 (MXFP4 nibbles)"},
@@ -807,6 +809,14 @@ int main() {
         {6, 200, 264, 128, false, "batched attention scores, ragged"},
         {2, 300, 257, 3328, true, "nibbles, 13 K steps, split"},
     };
+    if (argc > 1 && std::string(argv[1]) == "--plans") {
+        // the launch rules as restated above, one line per shape, for comparison with what the library itself
+        // reports (mxq_gemm_plan, mxq_gemm_workspace_bytes): batch M N K nibbles large-tiles K-splits
+        for (const Shape& s : shapes)
+            std::printf("%lld %lld %lld %lld %d %d %d\n", (long long)s.batch, (long long)s.M, (long long)s.N,
+                        (long long)s.K, s.nibbles ? 1 : 0, takes_large(s) ? 1 : 0, k_splits(s));
+        return 0;
+    }
     bool ok = true;
     // the attention-score kernel: config 5, ragged rows, an odd number of tiles, the narrowest and widest rows
     const int scores[][3] = {{128, 2048, 2048}, {3, 100, 1056}, {1, 32, 32}, {2, 33, 64}, {1, 2048, 96}, {5, 70, 2016}};

@@ -529,6 +529,32 @@ def test_gemm_copies_lds_image_schedule_and_stores_on_the_host(tmp_path):
     assert out.count("each once and in place") == 33 and out.count("scores kernel") == 6
 
 
+def test_the_host_check_replays_the_kernels_the_library_would_launch(tmp_path):
+    """tests/cpp/gemm_addr_check.cpp restates the launch rules (which shapes take the 256 x 256 kernel, how
+    many K splits the others get) to know what to replay; the library answers the same questions without a
+    GPU (mxq_gemm_plan, mxq_gemm_workspace_bytes).  For every shape of the check both must agree, or the
+    replay would vouch for a kernel that is not the one launched."""
+    exe = _build_gemm_addr_check(tmp_path)
+    res = subprocess.run([exe, "--plans"], capture_output=True, text=True, timeout=60)
+    assert res.returncode == 0
+    lib = _lib.gpu()
+    lib.mxq_gemm_plan.restype = ctypes.c_int
+    lib.mxq_gemm_plan.argtypes = [ctypes.c_int64] * 4 + [ctypes.c_int]
+    lib.mxq_gemm_workspace_bytes.restype = ctypes.c_int64
+    lib.mxq_gemm_workspace_bytes.argtypes = [ctypes.c_int64] * 4 + [ctypes.c_int]
+    E4M3, E2M1, LARGE, SPLIT, ONE_STEP, SMALL = 0, 4, 2, 1, 3, 0
+    n = 0
+    for line in res.stdout.splitlines():
+        batch, M, N, K, nib, large, splits = (int(v) for v in line.split())
+        kind = E2M1 if nib else E4M3
+        plan = lib.mxq_gemm_plan(batch, M, N, K, kind)
+        want = LARGE if large else SPLIT if splits > 1 else ONE_STEP if (K // 2 if nib else K) == 128 else SMALL
+        assert plan == want, (line, plan)
+        assert lib.mxq_gemm_workspace_bytes(batch, M, N, K, kind) == (0 if splits == 1 else splits * batch * M * N * 4), line
+        n += 1
+    assert n == 20
+
+
 @pytest.mark.parametrize("what, old, new, says", [
     ("the step's barrier one group later",
      "constexpr int large_barrier_group(int ng) { return ng - 3; }",
