@@ -459,8 +459,10 @@ MFMA_PEAK_TFLOPS = {"fp8": 5000.0, "fp4": 10100.0}
 def measured_traffic(workload):
     """HBM bytes per launch of the workload's dominant kernel, measured separately with rocprofv3 --pmc
     FETCH_SIZE / WRITE_SIZE (the summaries are in profiles/) -- but only while the kernel's source files
-    are the ones that summary was taken with: a figure from another build of the kernel is not this
-    build's traffic.  -> (bytes or None, where the last measurement is and whether it is current)"""
+    are the ones that summary was taken with, or ones for which the kernel's generated code has been compared
+    with that of the measured build and found identical (profiles/traffic.json says which): a figure from
+    another build of the kernel is not this build's traffic.
+    -> (bytes or None, where the last measurement is and whether it is current)"""
     import hashlib
     here = os.path.dirname(os.path.abspath(__file__))
     tfile = os.path.join(here, "profiles", "traffic.json")
@@ -474,10 +476,13 @@ def measured_traffic(workload):
     for name in entry["sources"]:
         with open(os.path.join(here, "microxcaling_amd", "csrc", name), "rb") as f:
             h.update(name.encode() + b"\0" + f.read() + b"\0")
-    current = not entry["sources"] or h.hexdigest() == entry["sources_sha256"]
+    unchanged = not entry["sources"] or h.hexdigest() == entry["sources_sha256"]
+    # ... or the files are in the state for which the measured kernel's generated code was compared with the
+    # code of the measurement's sources and found identical
+    same_code = h.hexdigest() == entry.get("same_code_checked", {}).get("sources_sha256")
     note = {"last_measured_bytes": entry["bytes"], "summary": entry["profile"],
-            "kernel_sources_unchanged_since": current}
-    return (entry["bytes"] if current else None), note
+            "kernel_sources_unchanged_since": unchanged, "kernel_code_compared_identical": same_code}
+    return (entry["bytes"] if unchanged or same_code else None), note
 
 
 METRIC = "MX quantize GB/s + % HBM peak (8192² fp32 MXFP8); fused MX-linear TFLOP/s"

@@ -272,7 +272,8 @@ def test_bench_reports_carry_the_contract_fields():
     for name in names:
         measured, note = bench.measured_traffic(name)
         assert note["summary"].startswith("profiles/") and os.path.exists(os.path.join(ROOT_DIR, note["summary"])), name
-        assert (measured == note["last_measured_bytes"]) if note["kernel_sources_unchanged_since"] else measured is None
+        current = note["kernel_sources_unchanged_since"] or note["kernel_code_compared_identical"]
+        assert (measured == note["last_measured_bytes"]) if current else measured is None
 
     wl = bench.make_workload(bench.HEADLINE)
     assert wl["bytes"] == 8192 * 8192 * 8 and wl["x"].shape == (8192, 8192)
