@@ -79,8 +79,12 @@ def build_gpu(verbose=True):
     return GPU_LIB
 
 
+# floor / rint as instructions (SSE4.1, any x86-64 CPU since 2008) instead of calls into libm; threads
+HOST_FLAGS = ["-msse4.1", "-pthread"]
+
+
 def build_host(verbose=True):
-    cmd = [os.path.join(ROCM, "lib", "llvm", "bin", "clang++"), *COMMON, _digest_flag(), "-o", HOST_LIB,
+    cmd = [os.path.join(ROCM, "lib", "llvm", "bin", "clang++"), *COMMON, *HOST_FLAGS, _digest_flag(), "-o", HOST_LIB,
            os.path.join(CSRC, "mxq_host.cpp")]
     _run(cmd, verbose)
     return HOST_LIB
@@ -97,8 +101,8 @@ def check_sources(verbose=False):
         jobs = [pool.submit(_run, [hipcc, *flags, os.path.join(CSRC, src)], verbose) for src in GPU_SOURCES]
         for job in jobs:
             job.result()
-    _run([os.path.join(ROCM, "lib", "llvm", "bin", "clang++"), *[f for f in COMMON if f != "-shared"], "-fsyntax-only",
-          os.path.join(CSRC, "mxq_host.cpp")], verbose)
+    _run([os.path.join(ROCM, "lib", "llvm", "bin", "clang++"), *[f for f in COMMON if f != "-shared"], *HOST_FLAGS,
+          "-fsyntax-only", os.path.join(CSRC, "mxq_host.cpp")], verbose)
 
 
 def kernel_resources(path=GPU_LIB):

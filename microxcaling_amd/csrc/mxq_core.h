@@ -36,6 +36,18 @@ enum MxqRound { MXQ_NEAREST = 0, MXQ_FLOOR = 1, MXQ_EVEN = 2 };   // mx/formats.
 MXQ_HD uint32_t mxq_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
 MXQ_HD float mxq_float(uint32_t u) { return __builtin_bit_cast(float, u); }
 
+// x * 2^n, exact unless the result is subnormal (then rounded to nearest even once) or overflows.
+// Device: ldexpf (one v_ldexp_f32).  Host: for n in [-126, 127] a multiplication by the power of two
+// built from its bit pattern -- the same correctly rounded result without a call into libm.
+MXQ_HD float mxq_ldexp(float x, int n) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return ldexpf(x, n);
+#else
+    if ((unsigned)(n + 126) <= 253u) return x * mxq_float((uint32_t)(n + 127) << 23);
+    return ldexpf(x, n);
+#endif
+}
+
 // ---- dtype rounding ---------------------------------------------------------------------------
 // fp32 -> bf16 -> fp32, round to nearest even, subnormals kept (what torch's CPU bf16 kernels do
 // after every op).
@@ -78,7 +90,7 @@ MXQ_HD unsigned short mxq_f16_bits(float f) {
 }
 MXQ_HD float mxq_f16_value(unsigned short h) {
     const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 31u, m = h & 1023u;
-    if (e == 0u) return mxq_float(sign | mxq_bits(ldexpf((float)m, -24)));
+    if (e == 0u) return mxq_float(sign | mxq_bits(mxq_ldexp((float)m, -24)));
     if (e == 31u) return mxq_float(sign | MXQ_INF_BITS | (m << 13));
     return mxq_float(sign | ((e + 112u) << 23) | (m << 13));
 }
@@ -182,8 +194,8 @@ MXQ_HD MxqScale mxq_block_scale(uint32_t um, int emax, int scale_emax, bool flus
     se = se < -scale_emax ? -scale_emax : se;
     se = se > 127 ? 127 : se;
     MxqScale r;
-    r.scale = nan ? mxq_float(MXQ_QNAN_BITS) : ldexpf(1.0f, se);
-    r.inv_scale = (flush_subnorms && E <= -127) ? 0.0f : ldexpf(1.0f, -se);
+    r.scale = nan ? mxq_float(MXQ_QNAN_BITS) : mxq_ldexp(1.0f, se);
+    r.inv_scale = (flush_subnorms && E <= -127) ? 0.0f : mxq_ldexp(1.0f, -se);
     return r;
 }
 
@@ -206,8 +218,8 @@ MXQ_HD MxqScale mxq_block_scale_f16ops(uint32_t um, int emax, int scale_emax, co
     nan = nan || se >= 16 || se <= -25;
     se = se < -25 ? -25 : (se > 16 ? 16 : se);
     MxqScale r;
-    r.scale = nan ? mxq_float(MXQ_QNAN_BITS) : ldexpf(1.0f, se);
-    r.inv_scale = ldexpf(1.0f, -se);
+    r.scale = nan ? mxq_float(MXQ_QNAN_BITS) : mxq_ldexp(1.0f, se);
+    r.inv_scale = mxq_ldexp(1.0f, -se);
     return r;
 }
 
@@ -243,7 +255,7 @@ MXQ_HD float mxq_round_lean(float a, float sign_src, const MxqFmt& f, bool satur
     // max_norm with either exponent and are clamped to it
     const uint32_t ebc = eb > f.min_eb ? eb : f.min_eb;
     const int n = f.t127 - (int)ebc;
-    const float s = ldexpf(mxq_float(ua), n);   // exact
+    const float s = mxq_ldexp(mxq_float(ua), n);   // exact
     float r;
     if (RMODE == MXQ_FLOOR) {
         r = floorf(s);
@@ -257,7 +269,7 @@ MXQ_HD float mxq_round_lean(float a, float sign_src, const MxqFmt& f, bool satur
         r = __builtin_rintf(s);                 // ties to even (default rounding mode)
         r = (s == f.tie_fix) ? 1.0f : r;
     }
-    const float y = ldexpf(r, -n);              // exact
+    const float y = mxq_ldexp(r, -n);              // exact
     uint32_t uy = mxq_bits(y);
     if (saturate) uy = uy < f.max_bits ? uy : f.max_bits;
     else uy = uy > f.max_bits ? MXQ_INF_BITS : uy;
@@ -292,11 +304,11 @@ MXQ_HD float mxq_round_every_op(float a, const MxqFmt& f, bool saturate, const u
         // 2**e = inf (fp16: from 2^16) -> x / inf = 0 and 0 * inf
         if (e >= (DT == MXQ_F16OPS ? 16 : 128)) return mxq_float(MXQ_QNAN_BITS);
     }
-    float s = mxq_round_dt<DT>(ldexpf(mxq_float(ua), -e));  // out / 2**e
+    float s = mxq_round_dt<DT>(mxq_ldexp(mxq_float(ua), -e));  // out / 2**e
     // sign(.) is taken of this quotient: where it underflowed to zero (e = 1 and the smallest subnormal)
     // the result is +0 like for a zero input
     const bool nonzero = s != 0.0f;
-    s = mxq_round_dt<DT>(ldexpf(s, f.t));                   // * 2**(bits-2)
+    s = mxq_round_dt<DT>(mxq_ldexp(s, f.t));                   // * 2**(bits-2)
     float r;
     if (RMODE == MXQ_FLOOR) {
         r = floorf(s);
@@ -310,8 +322,8 @@ MXQ_HD float mxq_round_every_op(float a, const MxqFmt& f, bool saturate, const u
         float tie = (h == floorf(h)) ? 1.0f : 0.0f;         // (|v| - 0.5) % 2 == 0
         r = floorf(mxq_round_dt<DT>(s + 0.5f)) - tie;
     }
-    float y = mxq_round_dt<DT>(ldexpf(r, -f.t));
-    y = mxq_round_dt<DT>(ldexpf(y, e));
+    float y = mxq_round_dt<DT>(mxq_ldexp(r, -f.t));
+    y = mxq_round_dt<DT>(mxq_ldexp(y, e));
     uint32_t uy = mxq_bits(y) & 0x7FFFFFFFu;
     if (uy > f.max_bits) uy = (saturate || f.ebits == 0) ? f.max_bits : MXQ_INF_BITS;
     return mxq_float(uy | (nonzero ? (ba & 0x80000000u) : 0u));
@@ -364,7 +376,7 @@ MXQ_HD uint32_t mxq_quant_mx_code(float x, const MxqScale& sc, const MxqFmt& f, 
     const uint32_t ua = mxq_bits(a) & 0x7FFFFFFFu;
     const uint32_t eb = ua >> 23;
     const uint32_t ebc = eb > f.min_eb ? eb : f.min_eb;
-    const float s = ldexpf(mxq_float(ua), f.t127 - (int)ebc);   // exact
+    const float s = mxq_ldexp(mxq_float(ua), f.t127 - (int)ebc);   // exact
     float r;
     if (RMODE == MXQ_FLOOR) {
         r = floorf(s);
@@ -405,12 +417,12 @@ MXQ_HD uint32_t mxq_encode_e5m2(float y) {
 }
 MXQ_HD float mxq_decode_e4m3(uint32_t c) {
     const uint32_t e = (c >> 3) & 15u, m = c & 7u;
-    const float v = e ? ldexpf((float)(8u + m), (int)e - 10) : ldexpf((float)m, -9);
+    const float v = e ? mxq_ldexp((float)(8u + m), (int)e - 10) : mxq_ldexp((float)m, -9);
     return (c & 0x80u) ? -v : v;
 }
 MXQ_HD float mxq_decode_e5m2(uint32_t c) {
     const uint32_t e = (c >> 2) & 31u, m = c & 3u;
-    const float v = e ? ldexpf((float)(4u + m), (int)e - 17) : ldexpf((float)m, -16);
+    const float v = e ? mxq_ldexp((float)(4u + m), (int)e - 17) : mxq_ldexp((float)m, -16);
     return (c & 0x80u) ? -v : v;
 }
 
@@ -423,7 +435,7 @@ MXQ_HD uint32_t mxq_encode_e2m1(float y) {
 }
 MXQ_HD float mxq_decode_e2m1(uint32_t c) {
     const uint32_t e = (c >> 1) & 3u, m = c & 1u;
-    const float v = e ? ldexpf((float)(2u + m), (int)e - 2) : 0.5f * (float)m;
+    const float v = e ? mxq_ldexp((float)(2u + m), (int)e - 2) : 0.5f * (float)m;
     return (c & 0x8u) ? -v : v;
 }
 
@@ -440,8 +452,8 @@ MXQ_HD uint32_t mxq_encode_fp6(float y) {
 template <int MANT, int BIAS>
 MXQ_HD float mxq_decode_fp6(uint32_t c) {
     const uint32_t e = (c >> MANT) & ((1u << (5 - MANT)) - 1u), m = c & ((1u << MANT) - 1u);
-    const float v = e ? ldexpf((float)((1u << MANT) + m), (int)e - BIAS - MANT)
-                      : ldexpf((float)m, 1 - BIAS - MANT);
+    const float v = e ? mxq_ldexp((float)((1u << MANT) + m), (int)e - BIAS - MANT)
+                      : mxq_ldexp((float)m, 1 - BIAS - MANT);
     return (c & 0x20u) ? -v : v;
 }
 

@@ -2,8 +2,8 @@
 // under AddressSanitizer and UndefinedBehaviorSanitizer: random shapes (empty, one element, ragged last
 // tiles, tiles longer than the axis, several shared axes), all dtypes, formats, roundings and flags, with
 // every buffer allocated at exactly the size the call describes, so that an index past the end of an
-// operand is reported instead of reading a neighbour.  Also checked: the input is not written, and a call
-// that returns an error leaves the output untouched.
+// operand is reported instead of reading a neighbour.  One call in 150 is large enough for the library's
+// threads to start.  Also checked: a call that returns an error leaves the output untouched.
 //
 //   usage: host_abi_sanitize [seconds]      exit status 0 and "ok <calls>" when nothing was reported
 #include <chrono>
@@ -70,8 +70,11 @@ void one_call() {
     std::vector<unsigned char>*in = nullptr, *aux = nullptr;
     int rc = 0;
     std::vector<unsigned char>* out = nullptr;
+    // now and then a call large enough for the library to spread it over several threads
+    const bool big = pick(0, 150) == 0;
     if (kind <= 2) {                                                          // by tile, given max, dither by tile
-        const int64_t pre = pick(0, 5), axis = pick(0, 70), post = pick(0, 9);
+        const int64_t pre = big ? pick(1, 40) : pick(0, 5), axis = big ? pick(200, 2000) : pick(0, 70),
+                      post = big ? pick(1, 12) : pick(0, 9);
         int64_t tile = pick(-1, 80);
         n = pre * axis * post;
         in = random_tensor(n, dtype);
@@ -93,7 +96,7 @@ void one_call() {
         int64_t ext[7];
         n = 1;
         for (int i = 0; i <= 2 * n_axes; ++i) {
-            ext[i] = (i % 2 == 0) ? pick(1, 3) : pick(1, 40);
+            ext[i] = (i % 2 == 0) ? pick(1, 3) : pick(1, big ? 90 : 40);
             if (pick(0, 40) == 0) ext[i] = 0;
             n *= ext[i];
         }
@@ -102,7 +105,7 @@ void one_call() {
         rc = mxq_host_quantize_mx_axes(in->data(), out->data(), dtype, n_axes, ext, scale_bits, f.ebits, f.mbits,
                                        f.max_norm, pick(-1, 48), flush, rmode, flags);
     } else {                                                                  // elementwise, plain and dither
-        n = pick(0, 3000);
+        n = big ? pick(200000, 600000) : pick(0, 3000);
         const int bits = (int)pick(2, 24), exp_bits = (int)pick(0, 8), sat = (int)pick(0, 1), den = (int)pick(0, 1);
         const float max_norm = pick(0, 1) ? f.max_norm : 1.5f * (float)(1 << pick(0, 20));
         in = random_tensor(n, dtype);
@@ -133,7 +136,7 @@ int main(int argc, char** argv) {
     const double seconds = argc > 1 ? atof(argv[1]) : 20.0;
     const auto t0 = std::chrono::steady_clock::now();
     while (std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() < seconds)
-        for (int i = 0; i < 200; ++i) one_call();
+        for (int i = 0; i < 20; ++i) one_call();
     check(refused * 2 < calls, "more than half of the calls were refused: the driver's parameters are off");
     printf("ok %ld calls, %ld refused with a message\n", calls, refused);
     return 0;

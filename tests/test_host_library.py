@@ -481,11 +481,12 @@ def test_fp16_conversions_of_the_scalar_core(tmp_path, compiler):
 def test_host_quantizers_under_address_and_undefined_behaviour_sanitizers(tmp_path):
     """tests/cpp/host_abi_sanitize.cpp + mxq_host.cpp compiled with -fsanitize=address,undefined: eight
     seconds of random calls (empty and ragged shapes, tiles longer than the axis, several shared axes, all
-    dtypes / formats / flags) on buffers of exactly the described size; any read or write past an operand,
-    signed overflow or misaligned access ends the run with a report."""
+    dtypes / formats / flags, now and then a call large enough for the library's threads to start) on buffers
+    of exactly the described size; any read or write past an operand, signed overflow or misaligned access
+    ends the run with a report.  (The same driver under -fsanitize=thread reports no race.)"""
     exe = str(tmp_path / "host_abi_sanitize")
-    subprocess.run(["/opt/rocm/lib/llvm/bin/clang++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined",
-                    "-fno-sanitize-recover=undefined", "-ffp-contract=off", "-I" + os.path.join(ROOT_DIR, "include"),
+    subprocess.run(["/opt/rocm/lib/llvm/bin/clang++", "-std=c++17", "-O1", "-gline-tables-only", "-fsanitize=address,undefined",
+                    "-fno-sanitize-recover=undefined", "-ffp-contract=off", "-pthread", "-I" + os.path.join(ROOT_DIR, "include"),
                     "-I" + os.path.join(ROOT_DIR, "microxcaling_amd", "csrc"),
                     os.path.join(ROOT_DIR, "tests", "cpp", "host_abi_sanitize.cpp"),
                     os.path.join(ROOT_DIR, "microxcaling_amd", "csrc", "mxq_host.cpp"), "-o", exe],
