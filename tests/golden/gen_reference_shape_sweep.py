@@ -28,27 +28,28 @@ SETTINGS = [
 ]
 
 
-def cases():
-    """[(kind, parameters)] -- plain lists and ints, stored in the fixture as they are."""
+def cases(mult=1):
+    """[(kind, parameters)] -- plain lists and ints, stored in the fixture as they are.  mult: that many times
+    as many cases of every kind (a longer sweep; the committed fixture is mult = 1)."""
     rng = np.random.default_rng(271828)
     r = lambda lo, hi: int(rng.integers(lo, hi + 1))
     out = []
-    for _ in range(10):                                   # linear: input rank 1..4, ragged K and N
+    for _ in range(10 * mult):                                   # linear: input rank 1..4, ragged K and N
         lead = [r(1, 5) for _ in range(r(0, 3))]
         out.append(("linear", dict(lead=lead, k=r(1, 150), n=r(1, 90), bias=bool(r(0, 1)))))
-    for _ in range(8):                                    # matmul: (..., m, k) x (k, n) or batched second operand
+    for _ in range(8 * mult):                                    # matmul: (..., m, k) x (k, n) or batched second operand
         lead = [r(1, 4) for _ in range(r(0, 2))]
         out.append(("matmul", dict(lead=lead, m=r(1, 40), k=r(1, 130), n=r(1, 70), batched2=bool(r(0, 1)) and bool(lead),
                                    bias=bool(r(0, 1)), mode=["aa", "aw", "wa"][r(0, 2)])))
-    for _ in range(6):                                    # bmm
+    for _ in range(6 * mult):                                    # bmm
         out.append(("bmm", dict(b=r(1, 5), m=r(1, 40), k=r(1, 130), n=r(1, 70))))
-    for _ in range(6):                                    # softmax over any axis
+    for _ in range(6 * mult):                                    # softmax over any axis
         shape = [r(1, 12) for _ in range(r(1, 4))]
         out.append(("softmax", dict(shape=shape, dim=r(-len(shape), len(shape) - 1))))
-    for _ in range(6):                                    # layer norm / rms norm widths
+    for _ in range(6 * mult):                                    # layer norm / rms norm widths
         out.append(("norm", dict(lead=[r(1, 6) for _ in range(r(1, 2))], width=r(1, 200), rms=bool(r(0, 1)))))
     for nd in (1, 2, 3):                                  # convolutions
-        for _ in range(3):
+        for _ in range(3 * mult):
             groups = [1, 1, 2, 4][r(0, 3)]
             cin, cout = groups * r(1, 12), groups * r(1, 6)
             size = [r(5, 9) for _ in range(nd)]
@@ -131,13 +132,13 @@ def run_case(mx, kind, prm, setting, dt, seed):
     return res
 
 
-def main(ref_root):
+def main(ref_root, mult=1, out_dir=HERE):
     sys.path.insert(0, ref_root)
     import mx                                            # noqa: E402
     torch.set_num_threads(1)                             # fixed summation order inside torch's CPU GEMM
-    meta = {"torch": torch.__version__, "cases": [[k, p] for k, p in cases()], "settings": SETTINGS, "digests": {}}
+    meta = {"torch": torch.__version__, "cases": [[k, p] for k, p in cases(mult)], "settings": SETTINGS, "digests": {}}
     n_raised = 0
-    for ci, (kind, prm) in enumerate(cases()):
+    for ci, (kind, prm) in enumerate(cases(mult)):
         for si, setting in enumerate(SETTINGS):
             for dname, dt in DTYPES.items():
                 if kind == "conv" and dname == "bf16":
@@ -150,10 +151,11 @@ def main(ref_root):
                         n_raised += 1
                     else:
                         meta["digests"][key] = digest(v)
-    with open(os.path.join(HERE, "reference_shape_sweep.json"), "w") as f:
+    with open(os.path.join(out_dir, "reference_shape_sweep.json"), "w") as f:
         json.dump(meta, f, indent=1, sort_keys=True)
     print("wrote", len(meta["digests"]), "digests,", n_raised, "raising runs")
 
 
 if __name__ == "__main__":
-    main(sys.argv[1] if len(sys.argv) > 1 else "/root/reference")
+    main(sys.argv[1] if len(sys.argv) > 1 else "/root/reference",
+         int(sys.argv[2]) if len(sys.argv) > 2 else 1, sys.argv[3] if len(sys.argv) > 3 else HERE)

@@ -30,12 +30,12 @@ N_STORED = 4
 DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16}
 
 
-def spec_cases():
+def spec_cases(n_cases=N_CASES):
     """The sweep's settings (plain dicts, before finalize_mx_specs)."""
     rng = np.random.default_rng(314159)
     pick = lambda seq: seq[int(rng.integers(len(seq)))]
     cases = []
-    for i in range(N_CASES):
+    for i in range(n_cases):
         d = {"custom_cuda": False}
         d["w_elem_format"] = pick(FORMATS)
         d["a_elem_format"] = pick(FORMATS)
@@ -183,13 +183,15 @@ def run_case(mx, raw, inp, dt):
     return out
 
 
-def main(ref_root):
+def main(ref_root, n_cases=N_CASES, out_dir=HERE):
+    """n_cases / out_dir other than the defaults: a longer sweep written somewhere else (digests only are
+    compared by whoever reads it; the committed fixture is the default run)."""
     sys.path.insert(0, ref_root)
     import mx                                            # noqa: E402
     torch.set_num_threads(1)                             # fixed summation order inside torch's CPU GEMM
     inp = inputs()
     arrays = {"in/" + k: bits_of(v) for k, v in inp.items()}
-    meta = {"torch": torch.__version__, "cases": spec_cases(), "digests": {}}
+    meta = {"torch": torch.__version__, "cases": spec_cases(n_cases), "digests": {}}
     n_raised = 0
     for i, raw in enumerate(meta["cases"]):
         for dname, dt in DTYPES.items():
@@ -203,11 +205,12 @@ def main(ref_root):
                 meta["digests"][key] = digest(v)
                 if i < N_STORED:
                     arrays[key] = bits_of(v)
-    np.savez_compressed(os.path.join(HERE, "reference_spec_sweep.npz"), **arrays)
-    with open(os.path.join(HERE, "reference_spec_sweep.json"), "w") as f:
+    np.savez_compressed(os.path.join(out_dir, "reference_spec_sweep.npz"), **arrays)
+    with open(os.path.join(out_dir, "reference_spec_sweep.json"), "w") as f:
         json.dump(meta, f, indent=1, sort_keys=True)
     print("wrote", len(meta["digests"]), "digests,", n_raised, "raising layer runs,", len(arrays), "arrays")
 
 
 if __name__ == "__main__":
-    main(sys.argv[1] if len(sys.argv) > 1 else "/root/reference")
+    main(sys.argv[1] if len(sys.argv) > 1 else "/root/reference",
+         int(sys.argv[2]) if len(sys.argv) > 2 else N_CASES, sys.argv[3] if len(sys.argv) > 3 else HERE)
