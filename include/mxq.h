@@ -330,8 +330,8 @@ int mxq_gemm_plan(int64_t batch, int64_t M, int64_t N, int64_t K, int a_kind);
  * (mx/cpp/funcs.cpp:117-149) take CPU tensors; these are their stand-ins.  Pointers are host
  * pointers and a call returns when the work is done.  A call with more than about 128 K elements is
  * spread over up to 16 threads of its own (blocks are independent and each is computed by exactly one
- * thread, so the result does not depend on their number); MXQ_HOST_THREADS in the environment sets
- * another upper limit, 1 keeps everything on the calling thread.  The by-tile variant has no
+ * thread, so the result does not depend on their number); MXQ_HOST_THREADS in the environment (read once
+ * per process) sets another upper limit, 1 keeps everything on the calling thread.  The by-tile variant has no
  * CPU counterpart in the reference; it mirrors mxq_quantize_mx_by_tile so the kernel arithmetic
  * can be checked on a machine without a GPU.  mxq_host_quantize_mx_axes mirrors mxq_quantize_mx_axes. */
 #define MXQ_HOST_FLAG_ROUND_EVERY_OP 2 /* bf16: round to bf16 after every op, no shortcuts */

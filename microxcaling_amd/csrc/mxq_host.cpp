@@ -99,21 +99,26 @@ MxqScale block_scale(int dtype, int flags, uint32_t um, const MxParams& p, const
 // body(begin, end) over the n independent work items of a call (blocks, tiles, chunks of elements), on up
 // to 16 threads -- fewer when the call is small: a thread is started per 64 K elements of work.  Every item
 // is computed by exactly one thread with the same arithmetic, so the result does not depend on the number of
-// threads.  MXQ_HOST_THREADS in the environment sets the upper limit (1: everything on the calling thread).
-int64_t thread_limit() {
-    int64_t n = (int64_t)std::thread::hardware_concurrency();
-    if (n > 16) n = 16;
-    if (const char* env = getenv("MXQ_HOST_THREADS")) {
-        const long v = strtol(env, nullptr, 10);
-        if (v >= 1) n = v < 64 ? v : 64;
-    }
-    return n < 1 ? 1 : n;
+// threads.  MXQ_HOST_THREADS in the environment, read at the first large call, sets the upper limit (1:
+// everything on the calling thread).
+int64_t thread_limit() {                                  // read once per process
+    static const int64_t limit = [] {
+        int64_t n = (int64_t)std::thread::hardware_concurrency();
+        if (n > 16) n = 16;
+        if (const char* env = getenv("MXQ_HOST_THREADS")) {
+            const long v = strtol(env, nullptr, 10);
+            if (v >= 1) n = v < 64 ? v : 64;
+        }
+        return n < 1 ? (int64_t)1 : n;
+    }();
+    return limit;
 }
 template <class Body>
 void parallel_for(int64_t n, int64_t elements_per_item, const Body& body) {
     const int64_t per_item = elements_per_item < 1 ? 1 : elements_per_item;
-    int64_t threads = std::min(thread_limit(), n);
+    int64_t threads = n;
     if (n > 0 && per_item <= INT64_MAX / n) threads = std::min(threads, n * per_item / 65536);
+    if (threads > 1) threads = std::min(threads, thread_limit());
     if (threads <= 1) {
         body((int64_t)0, n);
         return;

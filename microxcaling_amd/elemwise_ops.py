@@ -11,15 +11,16 @@ Differences from the reference, on purpose:
 """
 import torch
 
-from .formats import RoundingMode, _get_format_params, _get_max_norm
+from .formats import ROUNDING_VALUES, RoundingMode, _get_format_params, _get_max_norm
 
 
 def _native_round(round):
-    if round not in RoundingMode.string_enums():
+    value = ROUNDING_VALUES.get(round) if type(round) is str else None
+    if value is None:
         raise NotImplementedError(
             "rounding mode %r is not implemented by the native kernels (supported: %s)"
             % (round, ", ".join(RoundingMode.string_enums())))
-    return int(RoundingMode[round])
+    return value
 
 
 def _quantize_elemwise_core(A, bits, exp_bits, max_norm, round='nearest',

@@ -13,7 +13,11 @@ class RoundingMode(IntEnum):
 
     @staticmethod
     def string_enums():
-        return [m.name for m in RoundingMode]
+        return list(_ROUNDING_NAMES)
+
+
+_ROUNDING_NAMES = tuple(m.name for m in RoundingMode)
+ROUNDING_VALUES = {m.name: int(m) for m in RoundingMode}          # name -> what crosses the native boundary
 
 
 class ElemFormat(Enum):
@@ -69,7 +73,11 @@ _FORMAT_CACHE = {}
 def _get_format_params(fmt):
     """(ebits, mbits, emax, max_norm, min_norm), as mx/formats.py:61-125."""
     if type(fmt) is str:
-        fmt = ElemFormat.from_str(fmt)
+        hit = _FORMAT_CACHE.get(fmt)              # layers pass the same few names over and over
+        if hit is not None:
+            return hit
+        _FORMAT_CACHE[fmt] = _get_format_params(ElemFormat.from_str(fmt))
+        return _FORMAT_CACHE[fmt]
     if fmt in _FORMAT_CACHE:
         return _FORMAT_CACHE[fmt]
     if fmt not in _LAYOUT:

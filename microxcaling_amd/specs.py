@@ -49,16 +49,21 @@ _SPEC_TABLE = collections.OrderedDict([
 ])
 
 
+_DEFAULTS = {k: default for k, (default, _) in _SPEC_TABLE.items()}
+_HELP_STRINGS = {k: h for k, (_, h) in _SPEC_TABLE.items()}
+
+
 class MxSpecs(collections.UserDict):
     """Dict of quantization parameters; unknown keys are rejected, missing keys get defaults."""
 
     def __init__(self, *args, **kwargs):
         super().__init__(*args, **kwargs)
-        self.help_strings = {k: h for k, (_, h) in _SPEC_TABLE.items()}
-        for k, (default, _) in _SPEC_TABLE.items():
-            self.data.setdefault(k, default)
-        for k in self.data:
-            assert k in _SPEC_TABLE, "unknown mx spec %r" % k
+        self.help_strings = _HELP_STRINGS
+        given, self.data = self.data, dict(_DEFAULTS)
+        self.data.update(given)
+        if len(self.data) != len(_DEFAULTS):
+            for k in self.data:
+                assert k in _SPEC_TABLE, "unknown mx spec %r" % k
 
     def safe_json(self, indent=None):
         return json.dumps(self.data, indent=indent,
@@ -92,11 +97,12 @@ def apply_mx_specs(mx_specs, default_mx_specs=None):
         default_mx_specs = get_default_mx_specs()
     if not mx_specs:
         return default_mx_specs
-    for k in mx_specs:
-        if mx_specs[k] != None:
+    given = mx_specs.data if isinstance(mx_specs, MxSpecs) else mx_specs
+    for k, v in given.items():
+        if v != None:
             if k not in default_mx_specs:
                 raise KeyError(f"Unknown key '{k}' passed to mx specs")
-            default_mx_specs[k] = mx_specs[k]
+            default_mx_specs[k] = v
     return default_mx_specs
 
 
