@@ -4,6 +4,7 @@
     libmxq_host.so     the same scalar arithmetic for CPU tensors            (ROCm clang++)
 
 Usage:  python -m microxcaling_amd.build_ext
+        python -m microxcaling_amd.build_ext --compare-with <commit>    (generated code, kernel by kernel)
 hipcc cross-compiles, so no GPU is needed to build.
 """
 import concurrent.futures
@@ -156,10 +157,80 @@ def kernel_resources(path=GPU_LIB):
     return out
 
 
+def device_kernels(src_root=ROOT, verbose=False):
+    """{mangled kernel name: [instructions]} of the gfx950 code hipcc generates from the sources under
+    src_root (a checkout of this repository), every translation unit, with what does not change what a
+    kernel does normalized away: branch-label numbers and the offsets at which kernel arguments are loaded."""
+    import re
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    csrc = os.path.join(src_root, "microxcaling_amd", "csrc")
+    flags = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-O3", "-std=c++17",
+             "-fPIC", "-ffp-contract=off", "-fvisibility=hidden", "-I" + os.path.join(src_root, "include"), "-I" + csrc,
+             "-S", "--cuda-device-only"]
+    out = {}
+    with tempfile.TemporaryDirectory(prefix="mxq_asm_") as tmp:
+        units = [u for u in GPU_SOURCES if os.path.exists(os.path.join(csrc, u))]
+        with concurrent.futures.ThreadPoolExecutor(max_workers=len(units)) as pool:
+            jobs = [pool.submit(_run, [hipcc, *flags, "-o", os.path.join(tmp, u + ".s"), os.path.join(csrc, u)], verbose)
+                    for u in units]
+            for job in jobs:
+                job.result()
+        for u in units:
+            name = None
+            with open(os.path.join(tmp, u + ".s"), errors="replace") as f:
+                for line in f:
+                    m = re.match(r"^(_Z\w+):", line)
+                    if m:
+                        name = m.group(1)
+                        out[name] = []
+                    elif line.startswith(".Lfunc_end"):
+                        name = None
+                    elif name is not None:
+                        text = line.split(";")[0].strip()
+                        if text and not text.startswith("."):
+                            text = re.sub(r"\.LBB\d+_", ".LBB_", text)
+                            if text.startswith("s_load_dword"):
+                                text = re.sub(r"(s\[0:1\]), 0x[0-9a-f]+$", r"\1, <kernarg>", text)
+                            out[name].append(text)
+    return {k: v for k, v in out.items() if "s_endpgm" in v}  # kernels only (data symbols have no instructions)
+
+
+def compare_kernels_with(commit, verbose=False):
+    """Which kernels' generated code differs between `commit` (its sources are taken from git into a
+    temporary folder) and the working tree: {kernel family: [identical, different, only there, only here]}.
+    Two builds of a kernel that compare identical execute the same instructions on the same operands; a
+    measurement or a test run of the one holds for the other."""
+    import collections
+    import re
+    with tempfile.TemporaryDirectory(prefix="mxq_src_") as tmp:
+        tar = subprocess.run(["git", "-C", ROOT, "archive", commit, "microxcaling_amd/csrc", "include"],
+                             stdout=subprocess.PIPE, check=True).stdout
+        subprocess.run(["tar", "-x", "-C", tmp], input=tar, check=True)
+        old = device_kernels(tmp, verbose)
+    new = device_kernels(ROOT, verbose)
+
+    def family(name):
+        m = re.match(r"_ZN12_GLOBAL__N_1(\d+)", name)
+        return name[m.end():m.end() + int(m.group(1))] if m else name
+    table = collections.defaultdict(lambda: [0, 0, 0, 0])
+    for name, code in old.items():
+        table[family(name)][2 if name not in new else 0 if new[name] == code else 1] += 1
+    for name in new:
+        if name not in old:
+            table[family(name)][3] += 1
+    return dict(table)
+
+
 def build_all(verbose=True):
     return build_gpu(verbose), build_host(verbose)
 
 
 if __name__ == "__main__":
-    build_all(verbose=True)
-    print("built", GPU_LIB, HOST_LIB)
+    if len(sys.argv) == 3 and sys.argv[1] == "--compare-with":
+        # python -m microxcaling_amd.build_ext --compare-with <commit>: generated code, kernel by kernel
+        print("%-34s %9s %9s %10s %9s" % ("kernel", "identical", "different", "only there", "only here"))
+        for fam, row in sorted(compare_kernels_with(sys.argv[2]).items()):
+            print("%-34s %9d %9d %10d %9d" % (fam, *row))
+    else:
+        build_all(verbose=True)
+        print("built", GPU_LIB, HOST_LIB)
