@@ -1,0 +1,91 @@
+"""The HIP kernels of the quantizer translation unit, executed on the CPU.
+
+microxcaling_amd/csrc/mxq_capi.hip (with mxq_kernels.h: MX quantization along any axis and over several
+axes, given-max, elementwise, dither, the reductions, the closed-form bf16 kernel) is compiled for the host
+behind tests/cpp/emu/hip/hip_runtime.h -- kernel launches rewritten into calls that run the workgroups
+one after another, the 256 lanes of a workgroup as 256 threads meeting at __syncthreads and at the DPP /
+shuffle / vote exchanges of a wave -- and the GPU-marked parity tests of those kernels then run against
+that library (tests/hip_on_host_plugin.py): same .hip source, same launch geometry and kernel selection,
+same ctypes signatures as libmxq_gfx950.so, checked bit for bit against the oracle and the reference's
+fixtures.  What this cannot show is what only the hardware decides (its IEEE arithmetic and conversions,
+which the kernels assume and the GPU runs of the same tests confirm); what it does show is that the
+kernels' own logic -- vector packing, lane exchanges, ragged tiles, dispatch -- is right for every
+instantiation the tests reach, including those that no GPU has run yet.
+
+By default a selection that takes about two minutes; MXQ_KERNELS_ON_HOST=all runs every GPU-marked
+quantizer test that fits (about ten minutes)."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+from helpers import ROOT_DIR
+
+FILES = ["tests/test_zt_uncommon_parameters.py", "tests/test_zx_fp16_tensors.py", "tests/test_gpu_parity.py",
+         "tests/test_oracle_pins.py"]
+# full-size shapes are out of reach of 256 threads on a few cores; one test checks that CPU tensors are refused
+TOO_LARGE = "not headline and not config1 and not config3 and not baseline and not errors_are_raised"
+SLOW = " and not every_code and not config2 and not reduce_reference and not several_axes and not dither_with_the_reference"
+
+
+def rewrite_launches(src):
+    """kernel<...><<<grid, block, 0, stream>>>(args)  ->  emu::launch(grid, [&] { kernel<...>(args); })"""
+    out, i = [], 0
+    while True:
+        j = src.find("<<<", i)
+        if j < 0:
+            out.append(src[i:])
+            return "".join(out)
+        k, depth = j - 1, 0                                # back over the template argument list
+        assert src[k] == ">", src[j - 60:j + 10]
+        while True:
+            depth += {">": 1, "<": -1}.get(src[k], 0)
+            if depth == 0:
+                break
+            k -= 1
+        start = k
+        while src[start - 1].isalnum() or src[start - 1] == "_":
+            start -= 1
+        end = src.find(">>>", j)
+        grid = src[j + 3:end].rsplit(",", 3)[0].strip()     # grid, block, shared memory, stream
+        assert src[end + 3] == "("
+        p, depth = end + 3, 0
+        while True:
+            depth += {"(": 1, ")": -1}.get(src[p], 0)
+            if depth == 0:
+                break
+            p += 1
+        out.append(src[i:start])
+        out.append("emu::launch(%s, [&] { %s(%s); })" % (grid, src[start:j], src[end + 4:p]))
+        i = p + 1
+
+
+@pytest.fixture(scope="module")
+def host_build(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("hip_on_host")
+    csrc = os.path.join(ROOT_DIR, "microxcaling_amd", "csrc")
+    with open(os.path.join(csrc, "mxq_capi.hip")) as f:
+        text = rewrite_launches(f.read())
+    assert text.count("emu::launch(") >= 25 and "<<<" not in text
+    cpp, lib = str(tmp / "mxq_capi_on_host.cpp"), str(tmp / "libmxq_hip_on_host.so")
+    with open(cpp, "w") as f:
+        f.write(text)
+    subprocess.run(["/opt/rocm/lib/llvm/bin/clang++", "-std=c++20", "-O0", "-fPIC", "-shared", "-ffp-contract=off",
+                    "-pthread", "-msse4.1", "-I" + os.path.join(ROOT_DIR, "tests", "cpp", "emu"),
+                    "-I" + os.path.join(ROOT_DIR, "include"), "-I" + csrc, "-o", lib, cpp],
+                   check=True, capture_output=True, text=True, timeout=1200)
+    return lib
+
+
+def test_gpu_parity_tests_pass_on_the_kernels_compiled_for_the_host(host_build):
+    everything = os.environ.get("MXQ_KERNELS_ON_HOST") == "all"
+    env = dict(os.environ, MXQ_HIP_ON_HOST_LIB=host_build,
+               PYTHONPATH=os.path.join(ROOT_DIR, "tests") + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    res = subprocess.run([sys.executable, "-m", "pytest", "-p", "hip_on_host_plugin", "-p", "no:cacheprovider", "-q", "-x",
+                          "-m", "gpu", "-k", TOO_LARGE + ("" if everything else SLOW), *FILES],
+                         cwd=ROOT_DIR, env=env, capture_output=True, text=True, timeout=3400)
+    tail = res.stdout[-3000:] + res.stderr[-2000:]
+    assert res.returncode == 0, tail
+    assert " passed" in res.stdout and "failed" not in res.stdout, tail
+    assert int(res.stdout.rsplit(" passed", 1)[0].split()[-1]) >= (190 if everything else 140), tail
