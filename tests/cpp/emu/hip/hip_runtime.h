@@ -1,21 +1,28 @@
-// A stand-in for <hip/hip_runtime.h> that lets the HIP sources of this package's *quantizer* translation
-// unit (mxq_kernels.h, mxq_capi.hip) be compiled for the host and executed there, for tests on machines
-// without a GPU.  A kernel launch runs the workgroups one after another; the 256 lanes of a workgroup are
-// 256 host threads (kept for the life of the process) that meet where the hardware's lanes exchange data or wait for each other:
-// __syncthreads (all 256), and the lane exchanges of a wave of 64 (DPP, __shfl_xor, __all).  A lane that
-// has left the kernel counts as inactive: it no longer takes part in barriers, and an exchange that would
-// read from it returns what the instruction returns for a disabled lane.  Nothing here knows about MFMA,
-// LDS copies or inline assembly: the GEMM and row kernels cannot be run this way.
+// A stand-in for <hip/hip_runtime.h> that lets HIP sources of this package be compiled for the host and
+// executed there, for tests on machines without a GPU.  A kernel launch runs the workgroups one after
+// another; the lanes of a workgroup (up to 512) are host threads, kept for the life of the process, that
+// meet where the hardware's lanes exchange data or wait for each other: __syncthreads (all of them), and the
+// collective instructions of a wave of 64 (DPP moves, shuffles, votes, permlane swaps, readfirstlane, the
+// scaled matrix instructions).  A lane that has left the kernel counts as inactive: it no longer takes part
+// in barriers, and an exchange that would read from it returns what the instruction returns for a disabled
+// lane.  What is modelled is what the instructions compute, not when: a copy from memory into LDS lands at
+// once (one of the orders the hardware allows), waits and scheduling hints do nothing, and the matrix
+// instruction accumulates in double precision and rounds once (the hardware's own order of additions is
+// not public; the tests that use it carry a tolerance).
 #pragma once
+#include <math.h>
 #include <stdint.h>
 #include <string.h>
+#include <sys/mman.h>
 
 #include <atomic>
 #include <barrier>
 #include <condition_variable>
 #include <functional>
+#include <memory>
 #include <mutex>
 #include <thread>
+#include <vector>
 
 #define __global__
 #define __device__
@@ -34,36 +41,67 @@ struct dim3 {
 typedef void* hipStream_t;
 typedef int hipError_t;
 constexpr hipError_t hipSuccess = 0;
+enum { hipFuncAttributeMaxDynamicSharedMemorySize = 8, hipDeviceAttributeMultiprocessorCount = 63 };
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline const char* hipGetErrorString(hipError_t) { return "no error"; }
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
 inline hipError_t hipGetSymbolAddress(void** p, const void* symbol) { *p = const_cast<void*>(symbol); return hipSuccess; }
+inline hipError_t hipFuncSetAttribute(const void*, int, int) { return hipSuccess; }
+// a small "device": few enough compute units that a persistent kernel gives every workgroup several tiles
+inline hipError_t hipDeviceGetAttribute(int* value, int, int) { *value = 8; return hipSuccess; }
 
 namespace emu {
 
-constexpr int kLanes = 256, kWave = 64;
+constexpr int kMaxLanes = 512, kWave = 64, kMaxWaves = kMaxLanes / kWave;
+constexpr size_t kDynamicLds = 160 * 1024;
+
 struct Block {
-    std::barrier<> all{kLanes};
-    std::barrier<> wave[kLanes / kWave] = {std::barrier<>(kWave), std::barrier<>(kWave), std::barrier<>(kWave),
-                                           std::barrier<>(kWave)};
-    uint64_t slot[kLanes];                   // what a lane offers in an exchange
-    std::atomic<bool> active[kLanes];
+    explicit Block(int lanes) : all(lanes) {
+        for (int w = 0; w < kMaxWaves; ++w) wave[w] = std::make_unique<std::barrier<>>(kWave);
+        for (auto& a : active) a.store(true);
+    }
+    std::barrier<> all;
+    std::unique_ptr<std::barrier<>> wave[kMaxWaves];
+    uint64_t slot[kMaxLanes];                // what a lane offers in an exchange
+    const void* operand[kMaxLanes][2];       // ... and the operands of a matrix instruction
+    int scale[kMaxLanes][2];
+    std::atomic<bool> active[kMaxLanes];
 };
 inline Block*& block() { static Block* b = nullptr; return b; }
 inline thread_local dim3 t_thread, t_block;
 inline dim3 g_grid, g_blockdim;
 
-// 256 threads that live as long as the process; a workgroup is one job for each of them
+// LDS of a launch with dynamic shared memory: mapped below 4 GB, so that the 32-bit LDS addresses the
+// kernels compute from pointers (the value the hardware wants in m0) convert back to the same pointers
+inline unsigned char* dynamic_lds() {
+    static unsigned char* p = [] {
+        void* m = mmap(nullptr, kDynamicLds, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_32BIT, -1, 0);
+        if (m == MAP_FAILED) __builtin_trap();
+        return static_cast<unsigned char*>(m);
+    }();
+    return p;
+}
+// a 32-bit LDS address back to a pointer: dynamic LDS as above; a static __shared__ array lies in this
+// library's data, whose upper address bits are those of `anchor`
+inline unsigned char* lds_pointer(uint32_t addr) {
+    static unsigned char anchor;
+    const uintptr_t low = reinterpret_cast<uintptr_t>(dynamic_lds());
+    if (addr >= low && addr < low + kDynamicLds) return reinterpret_cast<unsigned char*>((uintptr_t)addr);
+    return reinterpret_cast<unsigned char*>((reinterpret_cast<uintptr_t>(&anchor) & ~(uintptr_t)0xFFFFFFFFu) | addr);
+}
+
+// threads that live as long as the process; a workgroup is one job for each of its lanes
 class Lanes {
   public:
     static Lanes& get() {
         static Lanes* pool = new Lanes;      // never destroyed: its threads wait on it until the process ends
         return *pool;
     }
-    void run(const std::function<void(int)>& job) {
+    void run(int lanes, const std::function<void(int)>& job) {
         std::unique_lock<std::mutex> lock(m_);
         job_ = &job;
-        pending_ = kLanes;
+        lanes_ = lanes;
+        pending_ = lanes;
         ++generation_;
         start_.notify_all();
         done_.wait(lock, [&] { return pending_ == 0; });
@@ -72,7 +110,7 @@ class Lanes {
 
   private:
     Lanes() {
-        for (int t = 0; t < kLanes; ++t) std::thread([this, t] { work(t); }).detach();
+        for (int t = 0; t < kMaxLanes; ++t) std::thread([this, t] { work(t); }).detach();
     }
     void work(int t) {
         uint64_t seen = 0;
@@ -82,6 +120,7 @@ class Lanes {
                 std::unique_lock<std::mutex> lock(m_);
                 start_.wait(lock, [&] { return generation_ != seen; });
                 seen = generation_;
+                if (t >= lanes_) continue;                   // this launch has fewer lanes
                 job = job_;
             }
             (*job)(t);
@@ -93,44 +132,117 @@ class Lanes {
     std::condition_variable start_, done_;
     const std::function<void(int)>* job_ = nullptr;
     uint64_t generation_ = 0;
-    int pending_ = 0;
+    int pending_ = 0, lanes_ = 0;
 };
 
-// the workgroups of a launch one after another, each on the 256 lane threads
+// the workgroups of a launch one after another (dynamic_lds_bytes: as in <<<grid, block, bytes, stream>>>)
 template <class Body>
-void launch(dim3 grid, const Body& body) {
+void launch(dim3 grid, dim3 blockdim, size_t dynamic_lds_bytes, const Body& body) {
     static std::mutex one_launch_at_a_time;
     std::lock_guard<std::mutex> guard(one_launch_at_a_time);
+    const int lanes = (int)blockdim.x;
+    if (lanes < 1 || lanes > kMaxLanes || lanes % kWave != 0 || blockdim.y != 1 || blockdim.z != 1 ||
+        dynamic_lds_bytes > kDynamicLds)
+        __builtin_trap();
     g_grid = grid;
-    g_blockdim = dim3(kLanes);
-    for (unsigned by = 0; by < grid.y; ++by)
-        for (unsigned bx = 0; bx < grid.x; ++bx) {
-            Block b;
-            for (auto& a : b.active) a.store(true);
-            block() = &b;
-            const std::function<void(int)> lane = [&](int t) {
-                t_thread = dim3((unsigned)t);
-                t_block = dim3(bx, by);
-                body();
-                b.active[t].store(false);                // leaves: no longer expected at any barrier
-                b.wave[t / kWave].arrive_and_drop();
-                b.all.arrive_and_drop();
-            };
-            Lanes::get().run(lane);
-            block() = nullptr;
-        }
+    g_blockdim = blockdim;
+    for (unsigned bz = 0; bz < grid.z; ++bz)
+        for (unsigned by = 0; by < grid.y; ++by)
+            for (unsigned bx = 0; bx < grid.x; ++bx) {
+                Block b(lanes);
+                block() = &b;
+                const std::function<void(int)> lane = [&](int t) {
+                    t_thread = dim3((unsigned)t);
+                    t_block = dim3(bx, by, bz);
+                    body();
+                    b.active[t].store(false);            // leaves: no longer expected at any barrier
+                    b.wave[t / kWave]->arrive_and_drop();
+                    b.all.arrive_and_drop();
+                };
+                Lanes::get().run(lanes, lane);
+                block() = nullptr;
+            }
 }
+
+inline int lane_in_block() { return (int)t_thread.x; }
+inline int lane_in_wave() { return (int)t_thread.x % kWave; }
+inline void wave_meet() { block()->wave[lane_in_block() / kWave]->arrive_and_wait(); }
 
 // every active lane of the wave offers `mine`; returns what lane `from` offered, or `inactive` if it has left
 inline uint64_t exchange(uint64_t mine, int from, uint64_t inactive) {
     Block& b = *block();
-    const int lane = (int)t_thread.x, w = lane / kWave;
+    const int lane = lane_in_block(), w = lane / kWave;
     b.slot[lane] = mine;
-    b.wave[w].arrive_and_wait();
+    wave_meet();
     const int src = w * kWave + from;
     const uint64_t got = b.active[src].load() ? b.slot[src] : inactive;
-    b.wave[w].arrive_and_wait();                        // nobody overwrites a slot that is still being read
+    wave_meet();                                         // nobody overwrites a slot that is still being read
     return got;
+}
+
+// global_load_lds_dword / _dwordx4: lane L of the wave copies `bytes` bytes from base + offset to LDS address
+// lds_base + bytes * L
+inline void global_load_lds(int bytes, uint32_t lds_base, uint32_t offset, const unsigned char* base) {
+    memcpy(lds_pointer(lds_base + (uint32_t)(bytes * lane_in_wave())), base + offset, (size_t)bytes);
+}
+
+// ---- element formats of the scaled matrix instructions (cbsz / blgp): 0 e4m3, 1 e5m2, 4 e2m1 ---------------
+inline double decode8(unsigned char c, int fmt) {
+    const int ebits = fmt == 0 ? 4 : 5, mbits = 7 - ebits, bias = fmt == 0 ? 7 : 15;
+    const int e = (c >> mbits) & ((1 << ebits) - 1), m = c & ((1 << mbits) - 1);
+    const double sign = (c & 0x80) ? -1.0 : 1.0;
+    if (fmt == 0 && e == 15 && m == 7) return NAN;                           // e4m3: S.1111.111
+    if (fmt == 1 && e == 31) return m ? NAN : sign * INFINITY;
+    if (e == 0) return sign * ldexp((double)m, 1 - bias - mbits);
+    return sign * ldexp((double)((1 << mbits) + m), e - bias - mbits);
+}
+inline double decode4(unsigned char nibble) {                                // e2m1
+    static const double mag[8] = {0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0};
+    return (nibble & 8) ? -mag[nibble & 7] : mag[nibble & 7];
+}
+// K value k (0..31) of the 32 a lane supplies
+inline double element(const void* regs, int k, int fmt) {
+    const unsigned char* p = static_cast<const unsigned char*>(regs);
+    if (fmt == 4) return decode4((p[k >> 1] >> (4 * (k & 1))) & 15);
+    if (fmt == 0 || fmt == 1) return decode8(p[k], fmt);
+    __builtin_trap();                                                        // 6-bit formats: not used
+}
+inline double e8m0(int scale_reg, int opsel) {
+    const int s = (scale_reg >> (8 * opsel)) & 255;
+    return s == 255 ? NAN : ldexp(1.0, s - 127);
+}
+
+// v_mfma_scale_f32_{32x32x64,16x16x128}_f8f6f4: D = A x B + C with A (rows x K) from the first operand, B
+// (K x columns) from the second.  Lane l supplies row (column) l % DIM, K block l / DIM (32 consecutive K
+// values in its 8 registers, 4 for e2m1) and the E8M0 scale of that block (byte `opsel` of its scale register);
+// it receives column l % DIM, rows 8 (r / 4) + 4 (l / 32) + r % 4 (32 x 32, r = 0..15) or 4 (l / 16) + r (16 x 16).
+template <int DIM, class VI, class VF>
+VF mfma_scale(const VI& a, const VI& b, const VF& c, int fmt_a, int fmt_b, int opsel_a, int scale_a, int opsel_b,
+              int scale_b) {
+    Block& blk = *block();
+    const int lane = lane_in_block(), w0 = lane / kWave * kWave, l = lane % kWave;
+    constexpr int KB = kWave / DIM, NOUT = DIM * DIM / kWave;
+    blk.operand[lane][0] = &a;
+    blk.operand[lane][1] = &b;
+    blk.scale[lane][0] = (scale_a >> (8 * opsel_a)) & 255;
+    blk.scale[lane][1] = (scale_b >> (8 * opsel_b)) & 255;
+    wave_meet();
+    VF d = c;
+    const int j = l % DIM;
+    for (int r = 0; r < NOUT; ++r) {
+        const int i = DIM == 32 ? 8 * (r / 4) + 4 * (l / 32) + r % 4 : 4 * (l / 16) + r;
+        double sum = 0.0;
+        for (int kb = 0; kb < KB; ++kb) {
+            const int la = w0 + i + DIM * kb, lb = w0 + j + DIM * kb;
+            if (!blk.active[la].load() || !blk.active[lb].load()) __builtin_trap();   // MFMA needs the whole wave
+            double part = 0.0;
+            for (int k = 0; k < 32; ++k) part += element(blk.operand[la][0], k, fmt_a) * element(blk.operand[lb][1], k, fmt_b);
+            sum += part * e8m0(blk.scale[la][0], 0) * e8m0(blk.scale[lb][1], 0);
+        }
+        d[r] = (float)((double)c[r] + sum);
+    }
+    wave_meet();                                          // operands stay in place until every lane has read them
+    return d;
 }
 
 }  // namespace emu
@@ -152,12 +264,14 @@ inline unsigned long min(unsigned long a, unsigned long b) { return a < b ? a : 
 
 inline void __syncthreads() { emu::block()->all.arrive_and_wait(); }
 
-// v_mov_b32_dpp with row_mask = bank_mask = 0xF: quad_perm (ctrl 0x00-0xFF), row_mirror (0x140),
-// row_half_mirror (0x141); a disabled source lane leaves `old` in the destination (bound_ctrl false) or 0
+// v_mov_b32_dpp with row_mask = bank_mask = 0xF: quad_perm (ctrl 0x00-0xFF), row_ror:n (0x121-0x12F),
+// row_mirror (0x140), row_half_mirror (0x141); a disabled source lane leaves `old` in the destination
+// (bound_ctrl false) or 0
 inline int emu_update_dpp(int old, int src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
-    const int lane = (int)emu::t_thread.x % emu::kWave;
+    const int lane = emu::lane_in_wave();
     int from;
     if (ctrl >= 0 && ctrl <= 0xFF) from = (lane & ~3) | ((ctrl >> (2 * (lane & 3))) & 3);
+    else if (ctrl >= 0x121 && ctrl <= 0x12F) from = (lane & ~15) | ((lane + (ctrl & 15)) & 15);
     else if (ctrl == 0x140) from = (lane & ~15) | (15 - (lane & 15));
     else if (ctrl == 0x141) from = (lane & ~7) | (7 - (lane & 7));
     else __builtin_trap();                                // a control this stand-in does not know
@@ -167,26 +281,81 @@ inline int emu_update_dpp(int old, int src, int ctrl, int row_mask, int bank_mas
 #define __builtin_amdgcn_update_dpp emu_update_dpp
 
 template <class T>
-inline T __shfl_xor(T v, int mask, int width = 64) {
-    if (width != 64) __builtin_trap();
+inline T emu_shuffle(T v, int from) {
     static_assert(sizeof(T) <= 8, "exchange slot is 64 bits");
     uint64_t bits = 0;
     memcpy(&bits, &v, sizeof(T));
-    const int lane = (int)emu::t_thread.x % emu::kWave;
-    const uint64_t got = emu::exchange(bits, lane ^ mask, bits);   // an inactive source: the lane's own value
+    const uint64_t got = (from >= 0 && from < emu::kWave) ? emu::exchange(bits, from, bits) : emu::exchange(bits, emu::lane_in_wave(), bits);
     T out;
     memcpy(&out, &got, sizeof(T));
     return out;
 }
+template <class T>
+inline T __shfl_xor(T v, int mask, int width = 64) {
+    if (width != 64) __builtin_trap();
+    return emu_shuffle(v, emu::lane_in_wave() ^ mask);    // an inactive source: the lane's own value
+}
+template <class T>
+inline T __shfl_down(T v, unsigned delta, int width = 64) {
+    if (width != 64) __builtin_trap();
+    return emu_shuffle(v, emu::lane_in_wave() + (int)delta);   // past the end of the wave: the lane's own value
+}
 
 inline int __all(int pred) {                               // over the lanes of the wave that are still there
     emu::Block& b = *emu::block();
-    const int lane = (int)emu::t_thread.x, w = lane / emu::kWave;
+    const int lane = emu::lane_in_block(), w = lane / emu::kWave;
     b.slot[lane] = pred ? 1 : 0;
-    b.wave[w].arrive_and_wait();
+    emu::wave_meet();
     int all = 1;
     for (int l = w * emu::kWave; l < (w + 1) * emu::kWave; ++l)
         if (b.active[l].load() && b.slot[l] == 0) all = 0;
-    b.wave[w].arrive_and_wait();
+    emu::wave_meet();
     return all;
 }
+
+// v_readfirstlane_b32: the value of the first lane of the wave that is still there
+inline int emu_readfirstlane(int v) {
+    emu::Block& b = *emu::block();
+    const int lane = emu::lane_in_block(), w = lane / emu::kWave;
+    b.slot[lane] = (uint32_t)v;
+    emu::wave_meet();
+    int got = v;
+    for (int l = w * emu::kWave; l < (w + 1) * emu::kWave; ++l)
+        if (b.active[l].load()) {
+            got = (int)(uint32_t)b.slot[l];
+            break;
+        }
+    emu::wave_meet();
+    return got;
+}
+#define __builtin_amdgcn_readfirstlane emu_readfirstlane
+#define __builtin_amdgcn_sched_barrier(mask) ((void)0)
+
+// v_permlane16_swap_b32: the first operand of the lanes 16-31 / 48-63 trades places with the second operand of
+// the lanes 0-15 / 32-47 (lane L + 16 with lane L)
+struct emu_pair {
+    unsigned v[2];
+    unsigned operator[](int i) const { return v[i]; }
+};
+inline emu_pair emu_permlane16_swap(unsigned a, unsigned b, bool, bool) {
+    const int lane = emu::lane_in_wave();
+    const bool upper = (lane & 16) != 0;
+    const uint64_t mine = upper ? a : b;                  // what this lane gives away
+    const unsigned got = (unsigned)emu::exchange(mine, upper ? lane - 16 : lane + 16, mine);
+    return upper ? emu_pair{{got, b}} : emu_pair{{a, got}};
+}
+#define __builtin_amdgcn_permlane16_swap emu_permlane16_swap
+
+// (object-like macros: the kernels pass braced vectors, whose commas a function-like macro would split)
+template <class VI, class VF>
+inline VF emu_mfma_32x32x64(const VI& a, const VI& b, const VF& c, int cbsz, int blgp, int opsel_a, int scale_a, int opsel_b,
+                            int scale_b) {
+    return emu::mfma_scale<32>(a, b, c, cbsz, blgp, opsel_a, scale_a, opsel_b, scale_b);
+}
+template <class VI, class VF>
+inline VF emu_mfma_16x16x128(const VI& a, const VI& b, const VF& c, int cbsz, int blgp, int opsel_a, int scale_a, int opsel_b,
+                             int scale_b) {
+    return emu::mfma_scale<16>(a, b, c, cbsz, blgp, opsel_a, scale_a, opsel_b, scale_b);
+}
+#define __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4 emu_mfma_32x32x64
+#define __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4 emu_mfma_16x16x128

@@ -30,7 +30,7 @@ SLOW = " and not every_code and not config2 and not reduce_reference and not sev
 
 
 def rewrite_launches(src):
-    """kernel<...><<<grid, block, 0, stream>>>(args)  ->  emu::launch(grid, [&] { kernel<...>(args); })"""
+    """kernel<...><<<grid, block, lds, stream>>>(args)  ->  emu::launch(grid, block, lds, [&] { kernel<...>(args); })"""
     out, i = [], 0
     while True:
         j = src.find("<<<", i)
@@ -48,7 +48,7 @@ def rewrite_launches(src):
         while src[start - 1].isalnum() or src[start - 1] == "_":
             start -= 1
         end = src.find(">>>", j)
-        grid = src[j + 3:end].rsplit(",", 3)[0].strip()     # grid, block, shared memory, stream
+        grid, blockdim, lds_bytes, _ = (part.strip() for part in src[j + 3:end].rsplit(",", 3))   # ..., stream
         assert src[end + 3] == "("
         p, depth = end + 3, 0
         while True:
@@ -57,7 +57,7 @@ def rewrite_launches(src):
                 break
             p += 1
         out.append(src[i:start])
-        out.append("emu::launch(%s, [&] { %s(%s); })" % (grid, src[start:j], src[end + 4:p]))
+        out.append("emu::launch(%s, %s, %s, [&] { %s(%s); })" % (grid, blockdim, lds_bytes, src[start:j], src[end + 4:p]))
         i = p + 1
 
 
