@@ -186,60 +186,47 @@ inline void global_load_lds(int bytes, uint32_t lds_base, uint32_t offset, const
     memcpy(lds_pointer(lds_base + (uint32_t)(bytes * lane_in_wave())), base + offset, (size_t)bytes);
 }
 
-// ---- element formats of the scaled matrix instructions (cbsz / blgp): 0 e4m3, 1 e5m2, 4 e2m1 ---------------
-inline double decode8(unsigned char c, int fmt) {
-    const int ebits = fmt == 0 ? 4 : 5, mbits = 7 - ebits, bias = fmt == 0 ? 7 : 15;
-    const int e = (c >> mbits) & ((1 << ebits) - 1), m = c & ((1 << mbits) - 1);
-    const double sign = (c & 0x80) ? -1.0 : 1.0;
-    if (fmt == 0 && e == 15 && m == 7) return NAN;                           // e4m3: S.1111.111
-    if (fmt == 1 && e == 31) return m ? NAN : sign * INFINITY;
-    if (e == 0) return sign * ldexp((double)m, 1 - bias - mbits);
-    return sign * ldexp((double)((1 << mbits) + m), e - bias - mbits);
-}
-inline double decode4(unsigned char nibble) {                                // e2m1
-    static const double mag[8] = {0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0};
-    return (nibble & 8) ? -mag[nibble & 7] : mag[nibble & 7];
-}
-// K value k (0..31) of the 32 a lane supplies
-inline double element(const void* regs, int k, int fmt) {
-    const unsigned char* p = static_cast<const unsigned char*>(regs);
-    if (fmt == 4) return decode4((p[k >> 1] >> (4 * (k & 1))) & 15);
-    if (fmt == 0 || fmt == 1) return decode8(p[k], fmt);
-    __builtin_trap();                                                        // 6-bit formats: not used
-}
-inline double e8m0(int scale_reg, int opsel) {
-    const int s = (scale_reg >> (8 * opsel)) & 255;
-    return s == 255 ? NAN : ldexp(1.0, s - 127);
-}
+// the arithmetic of the matrix instruction (emu_math.cpp)
+void decode_row(const void* const* regs, int groups, int fmt, double* out);
+double scaled_dot(const double* a, const double* b, const int* scale_a, const int* scale_b, int groups);
 
 // v_mfma_scale_f32_{32x32x64,16x16x128}_f8f6f4: D = A x B + C with A (rows x K) from the first operand, B
-// (K x columns) from the second.  Lane l supplies row (column) l % DIM, K block l / DIM (32 consecutive K
-// values in its 8 registers, 4 for e2m1) and the E8M0 scale of that block (byte `opsel` of its scale register);
-// it receives column l % DIM, rows 8 (r / 4) + 4 (l / 32) + r % 4 (32 x 32, r = 0..15) or 4 (l / 16) + r (16 x 16).
+// (K x columns) from the second, K = 64 (32 x 32) or 128 (16 x 16); formats (cbsz / blgp) 0 e4m3, 1 e5m2, 4 e2m1.
+// Lane l belongs to row (column) l % DIM and to group g = l / DIM; which K values its registers hold:
+// emu_math.cpp.  Its scale register (byte `opsel`) is the E8M0 scale of K block g (32 g .. 32 g + 31) of its row,
+// whichever lane holds those values.  It receives column l % DIM, rows 8 (r / 4) + 4 (l / 32) + r % 4 (32 x 32,
+// r = 0..15) or 4 (l / 16) + r (16 x 16, r = 0..3).
 template <int DIM, class VI, class VF>
 VF mfma_scale(const VI& a, const VI& b, const VF& c, int fmt_a, int fmt_b, int opsel_a, int scale_a, int opsel_b,
               int scale_b) {
     Block& blk = *block();
     const int lane = lane_in_block(), w0 = lane / kWave * kWave, l = lane % kWave;
-    constexpr int KB = kWave / DIM, NOUT = DIM * DIM / kWave;
+    constexpr int GROUPS = kWave / DIM, KTOT = 32 * GROUPS, NOUT = DIM * DIM / kWave;
     blk.operand[lane][0] = &a;
     blk.operand[lane][1] = &b;
     blk.scale[lane][0] = (scale_a >> (8 * opsel_a)) & 255;
     blk.scale[lane][1] = (scale_b >> (8 * opsel_b)) & 255;
     wave_meet();
-    VF d = c;
+    for (int other = w0; other < w0 + kWave; ++other)
+        if (!blk.active[other].load()) __builtin_trap();   // the instruction needs the whole wave
     const int j = l % DIM;
+    const void* regs[GROUPS];
+    double col[KTOT], row[KTOT];
+    int scale_col[GROUPS], scale_row[GROUPS];
+    for (int g = 0; g < GROUPS; ++g) {
+        regs[g] = blk.operand[w0 + j + DIM * g][1];
+        scale_col[g] = blk.scale[w0 + j + DIM * g][1];
+    }
+    decode_row(regs, GROUPS, fmt_b, col);
+    VF d = c;
     for (int r = 0; r < NOUT; ++r) {
         const int i = DIM == 32 ? 8 * (r / 4) + 4 * (l / 32) + r % 4 : 4 * (l / 16) + r;
-        double sum = 0.0;
-        for (int kb = 0; kb < KB; ++kb) {
-            const int la = w0 + i + DIM * kb, lb = w0 + j + DIM * kb;
-            if (!blk.active[la].load() || !blk.active[lb].load()) __builtin_trap();   // MFMA needs the whole wave
-            double part = 0.0;
-            for (int k = 0; k < 32; ++k) part += element(blk.operand[la][0], k, fmt_a) * element(blk.operand[lb][1], k, fmt_b);
-            sum += part * e8m0(blk.scale[la][0], 0) * e8m0(blk.scale[lb][1], 0);
+        for (int g = 0; g < GROUPS; ++g) {
+            regs[g] = blk.operand[w0 + i + DIM * g][0];
+            scale_row[g] = blk.scale[w0 + i + DIM * g][0];
         }
-        d[r] = (float)((double)c[r] + sum);
+        decode_row(regs, GROUPS, fmt_a, row);
+        d[r] = (float)((double)c[r] + scaled_dot(row, col, scale_row, scale_col, GROUPS));
     }
     wave_meet();                                          // operands stay in place until every lane has read them
     return d;
@@ -261,6 +248,9 @@ inline int min(int a, int b) { return a < b ? a : b; }
 inline unsigned min(unsigned a, unsigned b) { return a < b ? a : b; }
 inline long min(long a, long b) { return a < b ? a : b; }
 inline unsigned long min(unsigned long a, unsigned long b) { return a < b ? a : b; }
+
+inline unsigned __float_as_uint(float f) { return __builtin_bit_cast(unsigned, f); }
+inline float __uint_as_float(unsigned u) { return __builtin_bit_cast(float, u); }
 
 inline void __syncthreads() { emu::block()->all.arrive_and_wait(); }
 

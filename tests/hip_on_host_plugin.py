@@ -34,6 +34,9 @@ def _contiguous_only(t, name, who):
 
 ce._check_gpu_input = _contiguous_only
 ce._stream = lambda t: None
+from microxcaling_amd import fused  # noqa: E402  (its own names for the two, imported from custom_extensions)
+fused._check_gpu_input = _contiguous_only
+fused._stream = lambda t: None
 torch.cuda.device = lambda *a, **k: contextlib.nullcontext()
 
 # CPU tensors take the GPU entry points (their pointers are host pointers, which is what the host build reads)

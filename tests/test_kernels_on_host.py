@@ -61,20 +61,52 @@ def rewrite_launches(src):
         i = p + 1
 
 
+def rewrite_assembly(text):
+    """The inline assembly of mxq_gemm.h in terms of the stand-in: the copies from memory into LDS as calls,
+    waits and register pins as nothing, the dynamic LDS array as a pointer to the stand-in's buffer."""
+    import re
+    text, copies = re.subn(r'asm volatile\("s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dword(x4)? %1, %2"\s*::\s*'
+                           r'"s"\((\w+)\),\s*"v"\((\w+)\),\s*"s"\((\w+)\)\s*:\s*"memory"\);',
+                           lambda m: "emu::global_load_lds(%d, %s, %s, %s);" % (16 if m.group(1) else 4, m.group(2),
+                                                                                m.group(3), m.group(4)), text)
+    text = re.sub(r'asm volatile\("s_waitcnt[^"]*"\s*:::\s*"memory"\);', ";", text)
+    text = re.sub(r'asm volatile\(""\s*:[^;]*\);', ";", text)
+    text, lds = re.subn(r"extern __shared__ __attribute__\(\(aligned\(16\)\)\) unsigned char (\w+)\[\];",
+                        r"unsigned char* \1 = emu::dynamic_lds();", text)
+    assert "asm volatile" not in text, "inline assembly the stand-in has no counterpart for"
+    return text, copies, lds
+
+
 @pytest.fixture(scope="module")
 def host_build(tmp_path_factory):
+    """libmxq_hip_on_host.so: mxq_capi.hip (quantizers, reductions) and mxq_capi_gemm.hip (pack, unpack, both GEMM
+    kernels) with their headers, compiled for the host behind the stand-in runtime."""
     tmp = tmp_path_factory.mktemp("hip_on_host")
     csrc = os.path.join(ROOT_DIR, "microxcaling_amd", "csrc")
-    with open(os.path.join(csrc, "mxq_capi.hip")) as f:
-        text = rewrite_launches(f.read())
-    assert text.count("emu::launch(") >= 25 and "<<<" not in text
-    cpp, lib = str(tmp / "mxq_capi_on_host.cpp"), str(tmp / "libmxq_hip_on_host.so")
-    with open(cpp, "w") as f:
-        f.write(text)
-    subprocess.run(["/opt/rocm/lib/llvm/bin/clang++", "-std=c++20", "-O0", "-fPIC", "-shared", "-ffp-contract=off",
-                    "-pthread", "-msse4.1", "-I" + os.path.join(ROOT_DIR, "tests", "cpp", "emu"),
-                    "-I" + os.path.join(ROOT_DIR, "include"), "-I" + csrc, "-o", lib, cpp],
-                   check=True, capture_output=True, text=True, timeout=1200)
+    with open(os.path.join(csrc, "mxq_gemm.h")) as f:
+        header, copies, lds = rewrite_assembly(f.read())
+    assert copies == 2 and lds == 1
+    with open(str(tmp / "mxq_gemm.h"), "w") as f:                # found before the original on the include path
+        f.write(header)
+    sources, launches = [], 0
+    for unit in ("mxq_capi.hip", "mxq_capi_gemm.hip"):
+        with open(os.path.join(csrc, unit)) as f:
+            text = rewrite_launches(f.read())
+        assert "<<<" not in text
+        launches += text.count("emu::launch(")
+        sources.append(str(tmp / (unit[:-4] + "_on_host.cpp")))
+        with open(sources[-1], "w") as f:
+            f.write(text)
+    assert launches >= 39
+    lib, emu = str(tmp / "libmxq_hip_on_host.so"), os.path.join(ROOT_DIR, "tests", "cpp", "emu")
+    clang = ["/opt/rocm/lib/llvm/bin/clang++", "-std=c++20", "-fPIC", "-ffp-contract=off", "-pthread", "-msse4.1"]
+    # the kernels without optimization (hundreds of instantiations: seconds instead of minutes), the arithmetic
+    # of the stand-in's matrix instruction with
+    subprocess.run([*clang, "-O2", "-c", os.path.join(emu, "emu_math.cpp"), "-o", str(tmp / "emu_math.o")],
+                   check=True, capture_output=True, text=True, timeout=600)
+    subprocess.run([*clang, "-O0", "-shared", "-I" + str(tmp), "-I" + emu, "-I" + os.path.join(ROOT_DIR, "include"),
+                    "-I" + csrc, "-o", lib, *sources, str(tmp / "emu_math.o")],
+                   check=True, capture_output=True, text=True, timeout=1800)
     return lib
 
 
