@@ -149,4 +149,4 @@ class Softmax(nn.Softmax):
     def forward(self, input):
         if self.mx_none:
             return super().forward(input)
-        return SoftmaxFunction.apply(input, self.dim, self.mx_specs, self.name)
+        return softmax(input, dim=self.dim, mx_specs=self.mx_specs, name=self.name)   # (sees a deferred mx.bmm product)

@@ -319,6 +319,19 @@ inline int emu_readfirstlane(int v) {
     return got;
 }
 #define __builtin_amdgcn_readfirstlane emu_readfirstlane
+
+// v_exp_f32 / v_rcp_f32: results below the smallest normal number are flushed to zero, as the instructions do
+// (accuracy: the C library's instead of the hardware's 1 ulp)
+inline float emu_exp2f(float x) {
+    const float r = exp2f(x);
+    return fabsf(r) < 1.17549435e-38f ? 0.0f : r;
+}
+inline float emu_rcpf(float x) {
+    const float r = 1.0f / x;
+    return fabsf(r) < 1.17549435e-38f ? copysignf(0.0f, r) : r;
+}
+#define __builtin_amdgcn_exp2f emu_exp2f
+#define __builtin_amdgcn_rcpf emu_rcpf
 #define __builtin_amdgcn_sched_barrier(mask) ((void)0)
 
 // v_permlane16_swap_b32: the first operand of the lanes 16-31 / 48-63 trades places with the second operand of

@@ -6,12 +6,13 @@ behind tests/cpp/emu/hip/hip_runtime.h: every kernel launch runs its workgroups 
 lanes of a workgroup as 256 threads that meet at __syncthreads and at the lane exchanges of a wave.  This
 plugin maps every cuda device to the CPU (as tests/cpu_dry_run_plugin.py does) and makes the package's
 entry points for GPU *and* CPU tensors call that library through the same ctypes signatures as
-libmxq_gfx950.so -- so the arithmetic, the vector handling, the lane exchanges and the launch geometry that
+libmxq_gfx950.so (tensors report is_cuda, so the layers take their fused paths) -- so the arithmetic, the vector handling, the lane exchanges and the launch geometry that
 the tests exercise are those of the .hip sources, not of the host library.  Used by
 tests/test_kernels_on_host.py only."""
 import contextlib
 import ctypes
 import os
+import types
 
 import cpu_dry_run_plugin  # noqa: F401  (cuda -> cpu)
 import torch
@@ -38,6 +39,10 @@ from microxcaling_amd import fused  # noqa: E402  (its own names for the two, im
 fused._check_gpu_input = _contiguous_only
 fused._stream = lambda t: None
 torch.cuda.device = lambda *a, **k: contextlib.nullcontext()
+torch.cuda.current_stream = lambda *a, **k: types.SimpleNamespace(cuda_stream=None)
+# the layers choose their fused paths (packed operands, the MFMA GEMM, the attention-score kernel) by
+# tensor.is_cuda: every tensor says yes, and the entry points behind those paths are the host build's
+torch.Tensor.is_cuda = property(lambda self: True)
 
 # CPU tensors take the GPU entry points (their pointers are host pointers, which is what the host build reads)
 ce.funcs.quantize_mx_by_tile_func_cpp = lambda A, *a, round_every_op=False, **k: ce.quantize_mx_by_tile_func_cuda(A, *a, **k)

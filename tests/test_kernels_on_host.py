@@ -62,14 +62,23 @@ def rewrite_launches(src):
 
 
 def rewrite_assembly(text):
-    """The inline assembly of mxq_gemm.h in terms of the stand-in: the copies from memory into LDS as calls,
-    waits and register pins as nothing, the dynamic LDS array as a pointer to the stand-in's buffer."""
+    """The inline assembly of mxq_gemm.h / mxq_bmm_softmax.h in terms of the stand-in: the copies from memory into
+    LDS as calls, waits as meeting points of the wave, register pins as nothing, the dynamic LDS array as a pointer
+    to the stand-in's buffer."""
     import re
     text, copies = re.subn(r'asm volatile\("s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dword(x4)? %1, %2"\s*::\s*'
                            r'"s"\((\w+)\),\s*"v"\((\w+)\),\s*"s"\((\w+)\)\s*:\s*"memory"\);',
                            lambda m: "emu::global_load_lds(%d, %s, %s, %s);" % (16 if m.group(1) else 4, m.group(2),
                                                                                 m.group(3), m.group(4)), text)
-    text = re.sub(r'asm volatile\("s_waitcnt[^"]*"\s*:::\s*"memory"\);', ";", text)
+    # a wait for the wave's own copies or LDS reads: on the hardware the lanes of a wave pass it together, and the
+    # kernels count on that where one lane reads LDS bytes another lane of its wave has just fetched
+    text = re.sub(r'asm volatile\("s_waitcnt[^"]*"\s*:::\s*"memory"\);', "emu::wave_meet();", text)
+    # ... and in the one place where lanes of a wave hand data to each other through LDS with no wait in the source
+    # (the attention-score kernel stages its output rows): a meeting point between the writes and the reads
+    staged = "            const bool second = t0 + 1 < ntiles;"
+    if staged in text:
+        assert text.count(staged) == 1
+        text = text.replace(staged, "            emu::wave_meet();\n" + staged)
     text = re.sub(r'asm volatile\(""\s*:[^;]*\);', ";", text)
     text, lds = re.subn(r"extern __shared__ __attribute__\(\(aligned\(16\)\)\) unsigned char (\w+)\[\];",
                         r"unsigned char* \1 = emu::dynamic_lds();", text)
@@ -79,17 +88,24 @@ def rewrite_assembly(text):
 
 @pytest.fixture(scope="module")
 def host_build(tmp_path_factory):
-    """libmxq_hip_on_host.so: mxq_capi.hip (quantizers, reductions) and mxq_capi_gemm.hip (pack, unpack, both GEMM
-    kernels) with their headers, compiled for the host behind the stand-in runtime."""
+    """libmxq_hip_on_host.so: mxq_capi.hip (quantizers, reductions), mxq_capi_gemm.hip (pack, unpack, both GEMM
+    kernels), mxq_capi_scores.hip (the attention-score kernel), mxq_capi_chain.hip and mxq_capi_norm.hip (softmax,
+    activation, vector-op and normalization kernels) with their headers: every kernel of libmxq_gfx950.so, compiled
+    for the host behind the stand-in runtime."""
     tmp = tmp_path_factory.mktemp("hip_on_host")
     csrc = os.path.join(ROOT_DIR, "microxcaling_amd", "csrc")
-    with open(os.path.join(csrc, "mxq_gemm.h")) as f:
-        header, copies, lds = rewrite_assembly(f.read())
-    assert copies == 2 and lds == 1
-    with open(str(tmp / "mxq_gemm.h"), "w") as f:                # found before the original on the include path
-        f.write(header)
-    sources, launches = [], 0
-    for unit in ("mxq_capi.hip", "mxq_capi_gemm.hip"):
+    for name, expect in (("mxq_gemm.h", (2, 1)), ("mxq_bmm_softmax.h", (0, 0))):
+        with open(os.path.join(csrc, name)) as f:
+            header, copies, lds = rewrite_assembly(f.read())
+        assert (copies, lds) == expect, name
+        with open(str(tmp / name), "w") as f:                    # found before the original on the include path
+            f.write(header)
+    with open(os.path.join(csrc, "mxq_capi_chain.h")) as f:       # launch macros shared by two translation units
+        text = rewrite_launches(f.read())
+    with open(str(tmp / "mxq_capi_chain.h"), "w") as f:
+        f.write(text)
+    sources, launches = [], text.count("emu::launch(")
+    for unit in ("mxq_capi.hip", "mxq_capi_gemm.hip", "mxq_capi_scores.hip", "mxq_capi_chain.hip", "mxq_capi_norm.hip"):
         with open(os.path.join(csrc, unit)) as f:
             text = rewrite_launches(f.read())
         assert "<<<" not in text
@@ -97,7 +113,7 @@ def host_build(tmp_path_factory):
         sources.append(str(tmp / (unit[:-4] + "_on_host.cpp")))
         with open(sources[-1], "w") as f:
             f.write(text)
-    assert launches >= 39
+    assert launches >= 50
     lib, emu = str(tmp / "libmxq_hip_on_host.so"), os.path.join(ROOT_DIR, "tests", "cpp", "emu")
     clang = ["/opt/rocm/lib/llvm/bin/clang++", "-std=c++20", "-fPIC", "-ffp-contract=off", "-pthread", "-msse4.1"]
     # the kernels without optimization (hundreds of instantiations: seconds instead of minutes), the arithmetic
