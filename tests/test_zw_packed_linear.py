@@ -107,7 +107,8 @@ def test_a_codes_only_layer_moves_saves_and_reloads_on_the_gpu():
         with pytest.raises(RuntimeError, match="dropped its dense weight"):
             lin(x.float())
         lin.cpu()
-        with pytest.raises(RuntimeError, match="dropped its dense weight"):
-            lin(x)
+        if x.device.type == "cuda":                     # (a dry run on CPU tensors has one device only)
+            with pytest.raises(RuntimeError, match="dropped its dense weight"):
+                lin(x)
         lin.to(dev)
         assert torch.equal(lin(x).view(torch.int16), first.view(torch.int16))
