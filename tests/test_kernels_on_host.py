@@ -41,6 +41,8 @@ ESSENTIAL = [
      "(scaled_mfma and fp8_e4m3-fp8_e4m3 and (128-128-128-1 or 2048-2048-512-2))"),
     # the attention-score kernel behind mx.softmax(mx.bmm(...)), with the softmax row kernel and the GEMM beside it
     (["tests/test_zv_deferred_product_gpu.py"], "not_qualify or (shape1 and fp6_e2m3)"),
+    # the reduction that allocates nothing (static scratch array) against the one with a workspace
+    (["tests/test_zz_no_alloc.py"], ""),
 ]
 # with MXQ_KERNELS_ON_HOST=all: every GPU-marked test that fits.  Full-size shapes are out of reach of a few
 # hundred threads on a few cores; one test checks that CPU tensors are refused; one replays a HIP graph
@@ -48,7 +50,8 @@ EVERYTHING = [
     (["tests/test_zt_uncommon_parameters.py", "tests/test_zx_fp16_tensors.py", "tests/test_gpu_parity.py",
       "tests/test_oracle_pins.py"],
      "not headline and not config1 and not config3 and not baseline and not errors_are_raised"),
-    (["tests/test_zv_deferred_product_gpu.py", "tests/test_zw_packed_linear.py"], ""),
+    (["tests/test_zv_deferred_product_gpu.py", "tests/test_zw_packed_linear.py", "tests/test_zz_no_alloc.py",
+      "tests/test_gpu_layers.py"], ""),
     (["tests/test_gpu_fused.py"],
      "not hip_graph and not thousands_of_tiles and not 4096 and not 2050 and not 1100 and not 600-520 and not 1024-"),
 ]
