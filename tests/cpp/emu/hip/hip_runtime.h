@@ -12,6 +12,7 @@
 #pragma once
 #include <math.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 #include <sys/mman.h>
 
@@ -90,6 +91,16 @@ inline unsigned char* lds_pointer(uint32_t addr) {
     return reinterpret_cast<unsigned char*>((reinterpret_cast<uintptr_t>(&anchor) & ~(uintptr_t)0xFFFFFFFFu) | addr);
 }
 
+// copies into LDS that have been issued and not yet carried out (see global_load_lds)
+struct PendingCopy {
+    unsigned char* dst;
+    const unsigned char* src;
+    int bytes;
+};
+inline std::vector<PendingCopy>& pending_copies() {
+    static thread_local std::vector<PendingCopy> q;
+    return q;
+}
 // threads that live as long as the process; a workgroup is one job for each of its lanes
 class Lanes {
   public:
@@ -155,6 +166,8 @@ void launch(dim3 grid, dim3 blockdim, size_t dynamic_lds_bytes, const Body& body
                     t_thread = dim3((unsigned)t);
                     t_block = dim3(bx, by, bz);
                     body();
+                    for (const PendingCopy& c : pending_copies()) memcpy(c.dst, c.src, (size_t)c.bytes);
+                    pending_copies().clear();
                     b.active[t].store(false);            // leaves: no longer expected at any barrier
                     b.wave[t / kWave]->arrive_and_drop();
                     b.all.arrive_and_drop();
@@ -181,9 +194,32 @@ inline uint64_t exchange(uint64_t mine, int from, uint64_t inactive) {
 }
 
 // global_load_lds_dword / _dwordx4: lane L of the wave copies `bytes` bytes from base + offset to LDS address
-// lds_base + bytes * L
+// lds_base + bytes * L.  The hardware performs the copy some time between the instruction and the s_waitcnt
+// vmcnt(n) that leaves at most n later copies outstanding; a kernel is right only if it is right for every such
+// time.  Two extremes can be run: at once (default), or as late as the waits allow (MXQ_EMU_COPIES=late in the
+// environment): the copy is queued and carried out by the wait that no longer tolerates it.
+inline bool copies_land_late() {
+    static const bool late = [] {
+        const char* e = getenv("MXQ_EMU_COPIES");
+        return e != nullptr && strcmp(e, "late") == 0;
+    }();
+    return late;
+}
 inline void global_load_lds(int bytes, uint32_t lds_base, uint32_t offset, const unsigned char* base) {
-    memcpy(lds_pointer(lds_base + (uint32_t)(bytes * lane_in_wave())), base + offset, (size_t)bytes);
+    unsigned char* dst = lds_pointer(lds_base + (uint32_t)(bytes * lane_in_wave()));
+    if (copies_land_late()) pending_copies().push_back(PendingCopy{dst, base + offset, bytes});
+    else memcpy(dst, base + offset, (size_t)bytes);
+}
+// s_waitcnt vmcnt(n) (n < 0: the wait does not concern vmcnt): the oldest copies until n are left, then the wave
+// meets (its lanes pass a wait together, and the kernels count on that)
+inline void wait_for_copies(int n) {
+    std::vector<PendingCopy>& q = pending_copies();
+    if (n >= 0 && (int)q.size() > n) {
+        const size_t done = q.size() - (size_t)n;
+        for (size_t i = 0; i < done; ++i) memcpy(q[i].dst, q[i].src, (size_t)q[i].bytes);
+        q.erase(q.begin(), q.begin() + (long)done);
+    }
+    wave_meet();
 }
 
 // the arithmetic of the matrix instruction (emu_math.cpp)
