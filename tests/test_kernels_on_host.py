@@ -43,8 +43,6 @@ ESSENTIAL = [
     # the attention-score kernel behind mx.softmax(mx.bmm(...)), with the softmax row kernel and the GEMM beside it
     # (also with the copies into LDS landing as late as the waits allow: see LATE)
     (["tests/test_zv_deferred_product_gpu.py"], "not_qualify or (shape1 and fp6_e2m3)"),
-    # the reduction that allocates nothing (static scratch array) against the one with a workspace
-    (["tests/test_zz_no_alloc.py"], ""),
 ]
 # with MXQ_KERNELS_ON_HOST=all: every GPU-marked test that fits.  Full-size shapes are out of reach of a few
 # hundred threads on a few cores; one test checks that CPU tensors are refused; one replays a HIP graph
