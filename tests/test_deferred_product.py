@@ -88,6 +88,25 @@ def test_a_pending_product_goes_to_the_one_launch_kernel(monkeypatch):
     assert len(calls) == 2 and d.pending() is None
 
 
+def test_the_softmax_module_and_injected_names_meet_a_pending_product_too(monkeypatch):
+    """mx.Softmax (what inject_pyt_ops binds torch.nn.Softmax to) takes the same path as mx.softmax: a layer that
+    called the autograd function directly would evaluate the product and never reach the one-launch kernel."""
+    import importlib
+    B = importlib.import_module("microxcaling_amd.bmm")
+    from microxcaling_amd.softmax import Softmax
+    specs = _specs(**SPECS)
+    q, kt = _operands()
+    calls = []
+
+    def stand_in(in1, in2, sp):
+        calls.append(1)
+        return torch.full(in1.shape[:-1] + (in2.shape[-1],), 0.25, dtype=in1.dtype)
+    monkeypatch.setattr(B, "_scores_in_one_launch", stand_in)
+    d = B.DeferredProduct(q, kt, specs, None)
+    out = Softmax(dim=-1, mx_specs=specs)(d)
+    assert calls == [1] and d.pending() is not None and bool((out == 0.25).all())
+
+
 def test_modifying_an_operand_before_the_product_is_used_raises():
     from microxcaling_amd.bmm import DeferredProduct
     specs = _specs(**SPECS)
